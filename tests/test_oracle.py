@@ -1,0 +1,376 @@
+"""Pins the CPU oracle before anything is compared with it (runs without a GPU).
+
+Each oracle function is checked against something that is NOT a retyping of its own
+loop: a library routine it must reduce to (torch unfold / fold / max_pool2d / conv2d,
+numpy float64 matmul), closed forms and invariants, and the generators the reference's
+own tests use (integer ramps and cycles, tests/integration_tests.rs:291-305,
+:1499-1628), on which every float sum is exact.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle as orc
+from refgrid import DOT_SIZES, POOL_SHAPES, cases, conv_options, input_shapes, BATCH_IN_OUT
+
+
+def bf16_bits_torch(x):
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+
+
+# ---------------------------------------------------------------- bf16 ----
+def test_bf16_roundtrip_all_patterns():
+    bits = np.arange(65536, dtype=np.uint16)
+    f = orc.bf16_to_f32(bits)
+    back = orc.f32_to_bf16(f)
+    nan = (bits & 0x7FFF) > 0x7F80
+    assert np.array_equal(back[~nan], bits[~nan])
+    # NaNs come back quiet with the payload kept
+    assert np.array_equal(back[nan], bits[nan] | 0x40)
+    # widening is a plain shift for every non-NaN pattern
+    assert np.array_equal(f[~nan].view(np.uint32), bits[~nan].astype(np.uint32) << 16)
+
+
+def test_bf16_rne_matches_torch_and_closed_form():
+    rng = np.random.default_rng(0)
+    # every exponent, random mantissas, plus exact ties and their neighbours
+    u = rng.integers(0, 2**32, size=400000, dtype=np.uint64).astype(np.uint32)
+    ties = (rng.integers(0, 2**16, size=20000, dtype=np.uint32) << 16) | 0x8000
+    u = np.concatenate([u, ties, ties + 1, ties - 1, np.array([0, 0x80000000, 0x7F7FFFFF, 0x7F800000, 0xFF800000, 0x00000001, 0x00008000, 0x00018000], dtype=np.uint32)])
+    f = u.view(np.float32)
+    finite = ~np.isnan(f)
+    got = orc.f32_to_bf16(f)
+    assert np.array_equal(got[finite], bf16_bits_torch(f)[finite])
+    # closed form: nearest representable, ties to even, computed in integer arithmetic
+    lo = (u >> 16).astype(np.uint32)
+    rem = u & 0xFFFF
+    up = (rem > 0x8000) | ((rem == 0x8000) & ((lo & 1) == 1))
+    want = (lo + up).astype(np.uint16)
+    assert np.array_equal(got[finite], want[finite])
+    assert np.all((got[~finite] & 0x7FC0) == 0x7FC0)
+
+
+# -------------------------------------------------------------- shapes ----
+def test_shape_formulas_against_torch():
+    for f, p, s, d in conv_options():
+        for ih, iw in input_shapes(f, p, s, d):
+            y = F.conv2d(torch.zeros(1, 1, ih, iw), torch.zeros(1, 1, *f), padding=p, stride=s, dilation=d)
+            oh, ow = orc.conv_out(ih, f[0], p[0], s[0], d[0]), orc.conv_out(iw, f[1], p[1], s[1], d[1])
+            assert (oh, ow) == tuple(y.shape[2:])
+            # col2im's output formula inverts it whenever the stride divides evenly
+            if (ih + 2 * p[0] - d[0] * (f[0] - 1) - 1) % s[0] == 0:
+                assert orc.col2im_out(oh, f[0], p[0], s[0], d[0]) == ih
+    for i, x, s in [(4, 2, 2), (24, 2, 2), (7, 3, 2), (9, 3, 1), (5, 2, 3)]:
+        assert orc.pool_out(i, x, s) == F.max_pool2d(torch.zeros(1, 1, i, i), x, s).shape[-1]
+
+
+# -------------------------------------------------------------- im2col ----
+def torch_im2col(x, f, p, s, d):
+    bs, c = x.shape[:2]
+    u = F.unfold(torch.from_numpy(x), f, dilation=d, padding=p, stride=s)  # [bs, c*fh*fw, L]
+    return u.transpose(1, 2).reshape(-1, c * f[0] * f[1]).numpy()
+
+
+def test_im2col_reference_grid_vs_unfold():
+    n = 0
+    for bs, c, ih, iw, f, p, s, d in cases():
+        x = np.arange(1, bs * c * ih * iw + 1, dtype=np.float32).reshape(bs, c, ih, iw)  # ramp, :1505
+        y = orc.im2col_conv2(x, f, p, s, d)
+        assert np.array_equal(y, torch_im2col(x, f, p, s, d)), (bs, c, ih, iw, f, p, s, d)
+        # 16-bit elements move the same way
+        xb = orc.f32_to_bf16(x)
+        assert np.array_equal(orc.im2col_conv2(xb, f, p, s, d), orc.f32_to_bf16(y))
+        n += 1
+    assert n > 1000
+
+
+def test_im2col_mixed_options_random():
+    rng = np.random.default_rng(1)
+    for (bs, c, ih, iw, f, p, s, d) in [(2, 3, 9, 11, (3, 2), (1, 2), (2, 1), (1, 2)), (1, 5, 14, 9, (5, 3), (2, 0), (3, 2), (2, 1)), (3, 2, 6, 6, (2, 2), (0, 0), (2, 2), (1, 1))]:
+        x = rng.standard_normal((bs, c, ih, iw)).astype(np.float32)
+        assert np.array_equal(orc.im2col_conv2(x, f, p, s, d).view(np.uint32), torch_im2col(x, f, p, s, d).view(np.uint32))
+
+
+# -------------------------------------------------------------- col2im ----
+def torch_col2im(cols, bs, c, out_hw, f, p, s, d):
+    L = cols.shape[0] // bs
+    t = torch.from_numpy(cols.astype(np.float64)).reshape(bs, L, c * f[0] * f[1]).transpose(1, 2)
+    return F.fold(t, out_hw, f, dilation=d, padding=p, stride=s).numpy()
+
+
+def test_col2im_reference_grid_exact_integers():
+    for bs, c, ih, iw, f, p, s, d in cases():
+        oh, ow = orc.conv_out(ih, f[0], p[0], s[0], d[0]), orc.conv_out(iw, f[1], p[1], s[1], d[1])
+        rows, cols = bs * oh * ow, c * f[0] * f[1]
+        dy = np.arange(1, rows * cols + 1, dtype=np.float32).reshape(rows, cols)  # ramp, :1535-1538
+        if dy.max() * f[0] * f[1] >= 2**24:
+            continue
+        dx = orc.col2im_conv2(dy, (oh, ow), f, p, s, d)
+        out_hw = (orc.col2im_out(oh, f[0], p[0], s[0], d[0]), orc.col2im_out(ow, f[1], p[1], s[1], d[1]))
+        assert dx.shape == (bs, c) + out_hw
+        want = torch_col2im(dy, bs, c, out_hw, f, p, s, d)
+        assert np.array_equal(dx.astype(np.float64), want), (bs, c, ih, iw, f, p, s, d)
+
+
+def test_col2im_of_ones_counts_windows():
+    # col2im(im2col(1)) = how many patches cover each pixel
+    for (ih, iw, f, p, s, d) in [(7, 9, (3, 3), (1, 1), (1, 1), (1, 1)), (8, 8, (2, 2), (0, 0), (2, 2), (1, 1)), (9, 7, (3, 2), (0, 1), (2, 1), (1, 2))]:
+        ones = np.ones((2, 3, ih, iw), dtype=np.float32)
+        cols = orc.im2col_conv2(ones, f, p, s, d)
+        oh, ow = orc.conv_out(ih, f[0], p[0], s[0], d[0]), orc.conv_out(iw, f[1], p[1], s[1], d[1])
+        cnt = orc.col2im_conv2(cols, (oh, ow), f, p, s, d)
+        want = torch_col2im(cols, 2, 3, cnt.shape[2:], f, p, s, d)
+        assert np.array_equal(cnt, want)
+        # bf16 accumulates the same small integers exactly
+        cntb = orc.col2im_conv2(orc.f32_to_bf16(cols), (oh, ow), f, p, s, d)
+        assert np.array_equal(orc.bf16_to_f32(cntb), cnt)
+
+
+def test_col2im_bf16_rounds_after_every_add_in_host_order():
+    # One output pixel, three contributions a, b, c chosen so that
+    # rn(rn(a+b)+c) != rn(a+(b+c)) != rn_f32sum: 256 + 1 + 1 in bf16 (8 significant bits).
+    # 1x3 filter over a 1x3 grid, padding 1: the centre output pixel w=1 receives
+    # (wid=0,fj=2), (wid=1,fj=1), (wid=2,fj=0) in that order (wid ascending).
+    f, p = (1, 3), (0, 1)
+    cols = np.zeros((3, 3), dtype=np.float32)
+    cols[0, 2], cols[1, 1], cols[2, 0] = 256.0, 1.0, 1.0
+    y = orc.bf16_to_f32(orc.col2im_conv2(orc.f32_to_bf16(cols), (1, 3), f, p))
+    assert y.shape == (1, 1, 1, 3)
+    assert y[0, 0, 0, 1] == 256.0  # (256+1 -> 256) + 1 -> 256 ; an f32 accumulator would give 258
+    cols[0, 2], cols[1, 1], cols[2, 0] = 1.0, 1.0, 256.0
+    y = orc.bf16_to_f32(orc.col2im_conv2(orc.f32_to_bf16(cols), (1, 3), f, p))
+    assert y[0, 0, 0, 1] == 258.0  # (1+1) + 256 is exact
+    # f32 path keeps f32 sums
+    y32 = orc.col2im_conv2(cols, (1, 3), f, p)
+    assert y32[0, 0, 0, 1] == 258.0
+
+
+def test_col2im_f32_order_is_hid_then_wid():
+    # 3 values whose f32 sum depends on the order: big, -big, small
+    big, small = np.float32(2**25), np.float32(1.0)
+    f, p = (3, 1), (1, 0)  # vertical 3-tap: centre pixel h=1 gets hid=0 (fi=2), hid=1 (fi=1), hid=2 (fi=0)
+    cols = np.zeros((3, 3), dtype=np.float32)
+    cols[0, 2], cols[1, 1], cols[2, 0] = small, big, -big
+    y = orc.col2im_conv2(cols, (3, 1), f, p)
+    assert y[0, 0, 1, 0] == 0.0  # ((0+1)+2^25)-2^25 = 0
+    cols[0, 2], cols[1, 1], cols[2, 0] = big, -big, small
+    y = orc.col2im_conv2(cols, (3, 1), f, p)
+    assert y[0, 0, 1, 0] == 1.0
+
+
+# ------------------------------------------------------------ max pool ----
+def cyc(shape, dtype=np.float32):
+    n = int(np.prod(shape))
+    return (np.arange(n) % 10).astype(dtype).reshape(shape)  # (0..10).cycle(), :1556-1560
+
+
+def test_max_pool2_reference_shapes_vs_torch():
+    for shape in POOL_SHAPES:
+        x = cyc(shape)
+        y = orc.max_pool2(x, (2, 2))
+        want, idx = F.max_pool2d(torch.from_numpy(x), 2, 2, return_indices=True)
+        assert np.array_equal(y, want.numpy())
+        dy = np.arange(y.size, dtype=np.float32).reshape(y.shape)  # 0..len ramp, :1605-1608
+        dx = orc.max_pool2_backward(x, dy, (2, 2))
+        # the cycling data contains ties inside windows; the first maximum in row-major
+        # window order must win, which is what torch reports as the index
+        want_dx = np.zeros(x.size, dtype=np.float32).reshape(shape[0] * shape[1], -1)
+        flat_idx = idx.numpy().reshape(shape[0] * shape[1], -1)
+        for pl in range(want_dx.shape[0]):
+            want_dx[pl, flat_idx[pl]] = dy.reshape(shape[0] * shape[1], -1)[pl]
+        assert np.array_equal(dx, want_dx.reshape(shape))
+        yb = orc.max_pool2(orc.f32_to_bf16(x), (2, 2))
+        assert np.array_equal(orc.bf16_to_f32(yb), y)
+        dxb = orc.max_pool2_backward(orc.f32_to_bf16(x), orc.f32_to_bf16(dy), (2, 2))
+        assert np.array_equal(orc.bf16_to_f32(dxb), orc.bf16_to_f32(orc.f32_to_bf16(dx)))
+
+
+def test_max_pool2_first_max_wins_on_ties():
+    x = np.array([[[[5, 5], [5, 5]]]], dtype=np.float32)
+    dx = orc.max_pool2_backward(x, np.array([[[[7.0]]]], dtype=np.float32), (2, 2))
+    assert np.array_equal(dx, np.array([[[[7, 0], [0, 0]]]], dtype=np.float32))
+    x = np.array([[[[1, 9], [9, 3]]]], dtype=np.float32)
+    dx = orc.max_pool2_backward(x, np.array([[[[2.0]]]], dtype=np.float32), (2, 2))
+    assert np.array_equal(dx, np.array([[[[0, 2], [0, 0]]]], dtype=np.float32))
+
+
+def test_max_pool2_special_values():
+    nan = np.float32(np.nan)
+    # leading NaN sticks (nothing is > NaN); a later NaN never replaces
+    x = np.array([[[[nan, 3], [4, 5]]]], dtype=np.float32)
+    assert np.isnan(orc.max_pool2(x, (2, 2))[0, 0, 0, 0])
+    x = np.array([[[[1, nan], [4, 2]]]], dtype=np.float32)
+    assert orc.max_pool2(x, (2, 2))[0, 0, 0, 0] == 4
+    # -0 first, +0 later: +0 > -0 is false, so -0 is kept bit for bit
+    x = np.array([[[[-0.0, 0.0], [0.0, -0.0]]]], dtype=np.float32)
+    assert orc.max_pool2(x, (2, 2)).view(np.uint32)[0, 0, 0, 0] == 0x80000000
+    xb = orc.f32_to_bf16(x)
+    assert orc.max_pool2(xb, (2, 2))[0, 0, 0, 0] == 0x8000
+    # backward: 0 + (-0) = +0
+    dx = orc.max_pool2_backward(np.ones((1, 1, 2, 2), np.float32), np.array([[[[-0.0]]]], np.float32), (2, 2))
+    assert dx.view(np.uint32)[0, 0, 0, 0] == 0
+
+
+def test_max_pool2_general_windows_vs_torch_and_uncovered_cells():
+    rng = np.random.default_rng(3)
+    for (shape, size, st) in [((2, 3, 7, 9), (3, 2), (3, 2)), ((1, 2, 11, 10), (2, 3), (4, 5)), ((2, 2, 9, 9), (3, 3), (2, 2)), ((1, 1, 8, 8), (3, 3), (1, 1))]:
+        x = rng.permutation(int(np.prod(shape))).astype(np.float32).reshape(shape)  # all distinct
+        y = orc.max_pool2(x, size, st)
+        want = F.max_pool2d(torch.from_numpy(x), size, st)
+        assert np.array_equal(y, want.numpy())
+    # stride > window: cells between windows keep their x value after backward
+    x = rng.permutation(2 * 7 * 7).astype(np.float32).reshape(1, 2, 7, 7) + 1
+    dy = rng.standard_normal((1, 2, 2, 2)).astype(np.float32)
+    dx = orc.max_pool2_backward(x, dy, (2, 2), (4, 4))
+    covered = np.zeros((7, 7), bool)
+    for h0 in (0, 4):
+        for w0 in (0, 4):
+            covered[h0:h0 + 2, w0:w0 + 2] = True
+    assert np.array_equal(dx[..., ~covered], x[..., ~covered])
+    _, idx = F.max_pool2d(torch.from_numpy(x), 2, 4, return_indices=True)
+    want = np.zeros((2, 49), np.float32)
+    for pl in range(2):
+        want[pl, idx.numpy().reshape(2, -1)[pl]] = dy.reshape(2, -1)[pl]
+    assert np.array_equal(dx[..., covered], want.reshape(1, 2, 7, 7)[..., covered])
+
+
+def test_max_pool2_backward_overlapping_windows_is_sequential():
+    # 1x3 input, window 1x2 stride 1: window 0 zeroes cells 0,1 and puts dy0 at its
+    # argmax; window 1 then reads the UPDATED cell 1.
+    x = np.array([[[[1.0, 5.0, 2.0]]]], dtype=np.float32)
+    dy = np.array([[[[10.0, 1.0]]]], dtype=np.float32)
+    dx = orc.max_pool2_backward(x, dy, (1, 2), (1, 1))
+    # w0: argmax cell1 -> cells (0,10,2); w1 sees (10,2): argmax cell1, zero both, cell1 = 0+1
+    assert np.array_equal(dx, np.array([[[[0.0, 1.0, 0.0]]]], dtype=np.float32))
+
+
+# ---------------------------------------------------------- relu / bias ----
+def test_relu_rules():
+    x = (np.arange(-10, 10).astype(np.float32))  # (-10..10).cycle(), :1632-1636
+    assert np.array_equal(orc.relu(x), np.maximum(x, 0))
+    sp = np.array([-0.0, np.nan, np.inf, -np.inf, 1e-45], dtype=np.float32)
+    r = orc.relu(sp)
+    assert r.view(np.uint32)[0] == 0x80000000 and r[1] == 0 and r[2] == np.inf and r[3] == 0 and r[4] == sp[4]
+    rb = orc.relu(orc.f32_to_bf16(sp))
+    assert rb[0] == 0x8000 and rb[1] == 0 and rb[3] == 0
+    dy = np.arange(20, dtype=np.float32)
+    assert np.array_equal(orc.relu_backward(x, dy), np.where(x >= 0, dy, 0))
+
+
+def test_bias_add():
+    rng = np.random.default_rng(4)
+    y = rng.standard_normal((5, 7)).astype(np.float32)
+    b = rng.standard_normal(7).astype(np.float32)
+    assert np.array_equal(orc.bias_add_rows(y, b), b[None, :] + y)
+    yb, bb = orc.f32_to_bf16(y), orc.f32_to_bf16(b)
+    want = orc.f32_to_bf16(orc.bf16_to_f32(bb)[None, :] + orc.bf16_to_f32(yb))
+    assert np.array_equal(orc.bias_add_rows(yb, bb), want)
+
+
+# ---------------------------------------------------------------- gemm ----
+def gen_array(shape):  # values 1..9 cycling, integration_tests.rs:291-305
+    n = shape[0] * shape[1]
+    return ((np.arange(n) % 9) + 1).astype(np.float32).reshape(shape)
+
+
+@pytest.mark.parametrize("n", DOT_SIZES)
+def test_gemm_checkers_exact_on_reference_generator(n):
+    for ta in (False, True):
+        for tb in (False, True):
+            a = gen_array((n, n))
+            b = gen_array((n, n))
+            av, bv = (a.T if ta else a), (b.T if tb else b)
+            want = av.astype(np.float64) @ bv.astype(np.float64)
+            assert np.array_equal(orc.gemm_f64acc(av, bv), want)
+            assert np.array_equal(orc.gemm_f32_host(av, bv).astype(np.float64), want)
+            ab, bb = orc.f32_to_bf16(a), orc.f32_to_bf16(b)
+            abv, bbv = (ab.T if ta else ab), (bb.T if tb else bb)
+            assert np.array_equal(orc.gemm_f64acc(abv, bbv), want)
+            got = orc.bf16_to_f32(orc.gemm_bf16_f32acc(abv, bbv))
+            assert np.array_equal(got, orc.bf16_to_f32(orc.f32_to_bf16(want.astype(np.float32))))
+            if n <= 32:
+                # host fold rounds every step: within the reference's own epsilon = k (:356-361)
+                fold = orc.bf16_to_f32(orc.gemm_bf16_hostfold(abv, bbv))
+                assert np.all(np.abs(fold - want) <= n * np.maximum(1, np.abs(want) * 2**-8 * n))
+
+
+def test_gemm_strided_views_offsets_alpha_beta():
+    rng = np.random.default_rng(5)
+    big_a = rng.uniform(-1, 1, (40, 50)).astype(np.float32)
+    big_b = rng.uniform(-1, 1, (60, 45)).astype(np.float32)
+    a = big_a[3:36:2, 5:44:3]          # 17 x 13, strides (100, 3), offset
+    b = big_b[40:1:-3, 44:10:-3]       # 13 x 12, negative row and column strides
+    c = rng.uniform(-1, 1, (17, 12)).astype(np.float32)
+    want = 0.5 * (a.astype(np.float64) @ b.astype(np.float64)) + 2.0 * c
+    assert np.allclose(orc.gemm_f64acc(a, b, 0.5, 2.0, c), want, rtol=1e-14, atol=1e-14)
+    got = orc.gemm_f32_host(a, b, 0.5, 2.0, c)
+    assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(13) * np.max(np.abs(want))
+    # beta == 0 must not read C (NaN-poisoned C stays out of the result)
+    poison = np.full((17, 12), np.nan, dtype=np.float32)
+    assert np.isfinite(orc.gemm_f32_host(a, b, 1.0, 0.0, poison)).all()
+
+
+def test_gemm_f32_host_blocking_edges_vs_float64():
+    rng = np.random.default_rng(6)
+    for (m, k, n) in [(1, 1, 1), (7, 300, 9), (65, 257, 1030), (130, 513, 17)]:
+        a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        for av, bv in [(a, b), (np.asfortranarray(a), b), (a, np.asfortranarray(b))]:
+            got = orc.gemm_f32_host(av, bv, threads=3)
+            assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(k) * max(1.0, np.max(np.abs(want)))
+
+
+def test_gemm_bf16_f32acc_vs_float64():
+    rng = np.random.default_rng(7)
+    a = orc.f32_to_bf16(rng.normal(0, 0.02, (33, 200)).astype(np.float32))
+    b = orc.f32_to_bf16(rng.normal(0, 0.02, (200, 29)).astype(np.float32))
+    want = orc.bf16_to_f32(a).astype(np.float64) @ orc.bf16_to_f32(b).astype(np.float64)
+    assert np.allclose(orc.gemm_f64acc(a, b), want, rtol=1e-13, atol=0)
+    got = orc.bf16_to_f32(orc.gemm_bf16_f32acc(a, b)).astype(np.float64)
+    ulp = np.abs(want) * 2.0**-7
+    assert np.all(np.abs(got - want) <= ulp + 1e-2 * np.abs(want))
+
+
+# ---------------------------------------------------------------- conv ----
+def test_conv2_naive_vs_torch_conv2d_reference_generator():
+    # x, w = (1..=10).cycle(), integration_tests.rs:1190-1207 ; all sums exact
+    k = 0
+    for f, p, s, d in conv_options():
+        for ih, iw in list(input_shapes(f, p, s, d))[::5]:
+            for bs, ic, oc in BATCH_IN_OUT[::3]:
+                x = ((np.arange(bs * ic * ih * iw) % 10) + 1).astype(np.float32).reshape(bs, ic, ih, iw)
+                w = ((np.arange(oc * ic * f[0] * f[1]) % 10) + 1).astype(np.float32).reshape(oc, ic, *f)
+                y = orc.conv2_naive_f64(x, w, p, s, d)
+                want = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), padding=p, stride=s, dilation=d).numpy()
+                assert np.array_equal(y, want)
+                # conv2_im2col chain (layer.rs:950-1005) built from oracle parts equals it
+                cols = orc.im2col_conv2(x, f, p, s, d)
+                wm = w.reshape(oc, -1)
+                om = orc.gemm_f64acc(cols, wm.T)
+                oh, ow = y.shape[2:]
+                assert np.array_equal(om.reshape(bs, oh, ow, oc).transpose(0, 3, 1, 2), want)
+                k += 1
+    assert k > 100
+
+
+def test_lenet5_forward_vs_torch():
+    rng = np.random.default_rng(8)
+    bs = 6
+    x = rng.uniform(0, 1, (bs, 1, 28, 28)).astype(np.float32)
+
+    def he(shape, fan_in):  # Uniform(-a, a), a = sqrt(2/fan_in): layer.rs:345-349, :463-467
+        a = np.sqrt(2.0 / fan_in)
+        return rng.uniform(-a, a, shape).astype(np.float32)
+
+    w1, w2 = he((6, 1, 5, 5), 25), he((16, 6, 5, 5), 150)
+    wd1, wd2, wd3, b3 = he((256, 128), 256), he((128, 84), 128), he((84, 10), 84), he((10,), 84)
+    got = orc.lenet5_forward_f32(x, w1, w2, wd1, wd2, wd3, b3)
+    t = torch.from_numpy
+    h = F.max_pool2d(F.relu(F.conv2d(t(x).double(), t(w1).double())), 2)
+    h = F.max_pool2d(F.relu(F.conv2d(h, t(w2).double())), 2).flatten(1)
+    h = F.relu(h @ t(wd1).double())
+    h = F.relu(h @ t(wd2).double())
+    want = (h @ t(wd3).double() + t(b3).double()).numpy()
+    assert np.max(np.abs(got - want)) < 1e-4 * max(1.0, np.max(np.abs(want)))
