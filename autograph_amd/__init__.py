@@ -1,0 +1,17 @@
+"""MI355X-native device backend for autograph's dense-contraction hot path.
+
+The package is a thin host layer over libautograph_hip.so; importing it fails loudly when
+the library has not been built.
+"""
+from ._ffi import LIB_PATH, AghError, lib  # noqa: F401
+from .tensor import (  # noqa: F401
+    BF16,
+    F32,
+    Buffer,
+    Col2ImConv2Options,
+    Device,
+    Im2ColConv2Options,
+    MaxPool2Options,
+    Tensor,
+    gemm,
+)

@@ -1,0 +1,212 @@
+#include <stdlib.h>
+#include <string.h>
+// Host side of the GEMM entry points: argument checks (the reference's bail!s at
+// src/tensor/linalg.rs:256-279), orientation / loader / tile selection, split-K planning
+// (the job of linalg.rs:306-340) and the launches.  Included once per element type.
+#pragma once
+#include "agh_gemm_kernel.h"
+
+namespace agh {
+namespace gemm {
+
+struct TileCfg {
+    int bp, bq;
+    float eff;       // relative MFMA efficiency of the tile shape (bigger tiles reuse operands more)
+    int wgs_per_cu;  // workgroups a CU can hold (LDS / register bound)
+    bool scalar_ok;  // has instantiations with the element-wise loader
+};
+
+// index = config id used by launch_cfg below
+static const TileCfg kCfgs[] = {
+    {256, 256, 1.00f, 1, false},
+    {128, 256, 0.85f, 1, false},
+    {256, 128, 0.85f, 1, false},
+    {128, 128, 0.70f, 2, false},
+    {64, 64, 0.35f, 4, true},
+    {32, 128, 0.28f, 4, true},
+    {128, 32, 0.28f, 4, true},
+};
+static constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
+
+template <typename T, int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
+int launch_one(const Args &g, int splits) {
+    auto kern = gemm_kernel<T, BP, BQ, WGP, WGQ, LP, LQ>;
+    constexpr size_t smem = 2 * (size_t)(BP + BQ) * 128;
+    static bool attr_done = false;
+    if (!attr_done) {
+        if (smem > 48 * 1024)
+            AGH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_done = true;
+    }
+    dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits);
+    hipLaunchKernelGGL(kern, grid, dim3(WGP * WGQ * 64), smem, stream(), g);
+    AGH_LAUNCH_CHECK("gemm kernel launch");
+    return AGH_OK;
+}
+
+template <typename T, int BP, int BQ, int WGP, int WGQ, bool SCALAR_OK>
+int launch_loaders(const Args &g, int splits, int lp, int lq) {
+    switch (lp * 3 + lq) {
+        case LD_K * 3 + LD_K: return launch_one<T, BP, BQ, WGP, WGQ, LD_K, LD_K>(g, splits);
+        case LD_K * 3 + LD_R: return launch_one<T, BP, BQ, WGP, WGQ, LD_K, LD_R>(g, splits);
+        case LD_R * 3 + LD_K: return launch_one<T, BP, BQ, WGP, WGQ, LD_R, LD_K>(g, splits);
+        case LD_R * 3 + LD_R: return launch_one<T, BP, BQ, WGP, WGQ, LD_R, LD_R>(g, splits);
+        default: break;
+    }
+    if constexpr (SCALAR_OK) {
+        switch (lp * 3 + lq) {
+            case LD_K * 3 + LD_S: return launch_one<T, BP, BQ, WGP, WGQ, LD_K, LD_S>(g, splits);
+            case LD_R * 3 + LD_S: return launch_one<T, BP, BQ, WGP, WGQ, LD_R, LD_S>(g, splits);
+            case LD_S * 3 + LD_K: return launch_one<T, BP, BQ, WGP, WGQ, LD_S, LD_K>(g, splits);
+            case LD_S * 3 + LD_R: return launch_one<T, BP, BQ, WGP, WGQ, LD_S, LD_R>(g, splits);
+            case LD_S * 3 + LD_S: return launch_one<T, BP, BQ, WGP, WGQ, LD_S, LD_S>(g, splits);
+            default: break;
+        }
+    }
+    return fail(AGH_EINVAL, "gemm: no kernel for loader pair (%d,%d)", lp, lq);
+}
+
+template <typename T>
+int launch_cfg(int cfg, const Args &g, int splits, int lp, int lq) {
+    switch (cfg) {
+        case 0: return launch_loaders<T, 256, 256, 2, 2, false>(g, splits, lp, lq);
+        case 1: return launch_loaders<T, 128, 256, 2, 2, false>(g, splits, lp, lq);
+        case 2: return launch_loaders<T, 256, 128, 2, 2, false>(g, splits, lp, lq);
+        case 3: return launch_loaders<T, 128, 128, 2, 2, false>(g, splits, lp, lq);
+        case 4: return launch_loaders<T, 64, 64, 2, 2, true>(g, splits, lp, lq);
+        case 5: return launch_loaders<T, 32, 128, 1, 4, true>(g, splits, lp, lq);
+        case 6: return launch_loaders<T, 128, 32, 4, 1, true>(g, splits, lp, lq);
+        default: return fail(AGH_EINVAL, "gemm: bad tile config %d", cfg);
+    }
+}
+
+inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+// Which loader can serve an operand seen as NR rows x K with element strides (rs, ks).
+template <typename T>
+int pick_loader(const void *base, int64_t rs, int64_t ks, int NR, int K) {
+    constexpr int EPC = Geo<T>::EPC;
+    if (!aligned(base, 16)) return LD_S;
+    if (ks == 1 && K % EPC == 0 && (rs % EPC == 0 || NR == 1)) return LD_K;
+    if (rs == 1 && NR % EPC == 0 && (ks % EPC == 0 || K == 1)) return LD_R;
+    return LD_S;
+}
+
+// Optional override for experiments: AGH_GEMM_CFG=<config id>, AGH_GEMM_SPLITS=<n>.
+inline int env_int(const char *name, int dflt) {
+    const char *s = getenv(name);
+    return (s && *s) ? atoi(s) : dflt;
+}
+
+template <typename T>
+int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, const void *a, int64_t off_a,
+               int64_t rsa, int64_t csa, const void *b, int64_t off_b, int64_t rsb, int64_t csb, float beta, void *c,
+               int64_t off_c, int64_t rsc, int64_t csc, const void *bias, int64_t off_bias, int64_t bias_stride,
+               int act) {
+    AGH_API_ENTER();
+    if (m < 0 || k < 0 || n < 0) return fail(AGH_EINVAL, "%s: negative dimension", name);
+    const int64_t lim = ((int64_t)1 << 31) - 512;
+    if (m > lim || k > lim || n > lim) return fail(AGH_ERANGE, "%s: dimension does not fit 31 bits", name);
+    if (act != AGH_ACT_NONE && act != AGH_ACT_RELU) return fail(AGH_EINVAL, "%s: unknown activation %d", name, act);
+    if (m == 0 || n == 0) return AGH_OK;
+    if (!c) return fail(AGH_ENULL, "%s: null c", name);
+    if (k > 0 && (!a || !b)) return fail(AGH_ENULL, "%s: null a or b", name);
+    if (m > 1 && rsc == 0) return fail(AGH_EINVAL, "%s: c row stride is 0", name);
+    if (n > 1 && csc == 0) return fail(AGH_EINVAL, "%s: c column stride is 0", name);
+    constexpr int EPC = Geo<T>::EPC;
+    constexpr int BK = 8 * EPC;
+
+    const T *A = (const T *)a + off_a;
+    const T *B = (const T *)b + off_b;
+    T *C = (T *)c + off_c;
+
+    Args g;
+    memset(&g, 0, sizeof(g));
+    // p runs along C's unit-stride axis when it has one (rows of C otherwise: p = n axis)
+    const bool p_is_n = !(rsc == 1 && csc != 1);
+    if (p_is_n) {
+        g.P = B; g.ps = csb; g.pk = rsb; g.NP = (int)n;
+        g.Q = A; g.qs = rsa; g.qk = csa; g.NQ = (int)m;
+        g.dp = csc; g.dq = rsc;
+        g.bias_on_p = 1;
+    } else {
+        g.P = A; g.ps = rsa; g.pk = csa; g.NP = (int)m;
+        g.Q = B; g.qs = csb; g.qk = rsb; g.NQ = (int)n;
+        g.dp = rsc; g.dq = csc;
+        g.bias_on_p = 0;
+    }
+    g.D = C;
+    g.K = (int)k;
+    g.alpha = alpha;
+    g.beta = beta;
+    g.has_bias = bias != nullptr;
+    g.bias = bias ? (const void *)((const T *)bias + off_bias) : nullptr;
+    g.bias_stride = bias_stride;
+    g.act = act;
+    g.NPpad = (g.NP + 3) & ~3;
+
+    int lp = k > 0 ? pick_loader<T>(g.P, g.ps, g.pk, g.NP, g.K) : LD_S;
+    int lq = k > 0 ? pick_loader<T>(g.Q, g.qs, g.qk, g.NQ, g.K) : LD_S;
+    const bool any_scalar = (lp == LD_S || lq == LD_S);
+    const bool vec_store = g.dp == 1 && g.NP % 4 == 0 && (g.dq % 4 == 0 || g.NQ == 1) && aligned(C, 4 * sizeof(T));
+
+    // ---- tile shape: minimise (rounds of workgroups) x (tile area) / efficiency ----
+    const int cus = compute_units() > 0 ? compute_units() : 256;
+    int best = -1;
+    double best_cost = 0;
+    for (int i = 0; i < kNumCfgs; ++i) {
+        const TileCfg &t = kCfgs[i];
+        if (any_scalar && !t.scalar_ok) continue;
+        const int64_t tiles = (int64_t)((g.NP + t.bp - 1) / t.bp) * ((g.NQ + t.bq - 1) / t.bq);
+        if (tiles > 0x7FFFFFFF) continue;
+        // a CU works through ceil(tiles / CUs) tiles; co-resident workgroups share its MFMA rate
+        const int64_t rounds = (tiles + cus - 1) / cus;
+        const double cost = (double)rounds * t.bp * t.bq / t.eff;
+        if (best < 0 || cost < best_cost) { best = i; best_cost = cost; }
+    }
+    best = env_int("AGH_GEMM_CFG", best);
+    if (best < 0 || best >= kNumCfgs || (any_scalar && !kCfgs[best].scalar_ok))
+        return fail(AGH_ERANGE, "%s: no tile configuration for this shape", name);
+    const TileCfg &t = kCfgs[best];
+    g.tiles_p = (g.NP + t.bp - 1) / t.bp;
+    g.tiles_q = (g.NQ + t.bq - 1) / t.bq;
+
+    // ---- split-K when the tile grid cannot fill the chip and k is long ----
+    const int64_t tiles = (int64_t)g.tiles_p * g.tiles_q;
+    const int64_t slots = (int64_t)cus;
+    int splits = 1;
+    const int ktiles = (g.K + BK - 1) / BK;
+    if (tiles * 2 <= slots && ktiles >= 8) {
+        int64_t s = slots / tiles;
+        if (s > ktiles / 4) s = ktiles / 4;
+        if (s > 64) s = 64;
+        if (s > 1) splits = (int)s;
+    }
+    splits = env_int("AGH_GEMM_SPLITS", splits);
+    if (splits < 1) splits = 1;
+    if (splits > ktiles && ktiles > 0) splits = ktiles;
+    if (ktiles == 0) splits = 1;
+    int tiles_per_split = ktiles > 0 ? (ktiles + splits - 1) / splits : 1;
+    splits = ktiles > 0 ? (ktiles + tiles_per_split - 1) / tiles_per_split : 1;
+    g.k_per_split = tiles_per_split * BK;
+
+    if (splits > 1) {
+        void *ws = nullptr;
+        const size_t bytes = (size_t)splits * g.NQ * g.NPpad * sizeof(float);
+        if (int rc = workspace(bytes, &ws)) return rc;
+        g.ws = (float *)ws;
+        g.store_mode = ST_SPLITK;
+        if (int rc = launch_cfg<T>(best, g, splits, lp, lq)) return rc;
+        const size_t total = (size_t)g.NQ * g.NP;
+        const size_t blocks = (total + 255) / 256;
+        if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: output too large for split-K", name);
+        hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream(), g, splits);
+        AGH_LAUNCH_CHECK("split-K reduce launch");
+        return AGH_OK;
+    }
+    g.store_mode = vec_store ? ST_VEC : ST_SCALAR;
+    return launch_cfg<T>(best, g, 1, lp, lq);
+}
+
+}  // namespace gemm
+}  // namespace agh

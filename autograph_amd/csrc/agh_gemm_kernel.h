@@ -1,0 +1,388 @@
+// MFMA GEMM for gfx950 behind agh_gemm_{f32,bf16}[_bias_act].
+//
+// Formulation.  The host rewrites C = alpha*A*B + beta*C as
+//     D[p][q] = sum_k P[p][k] * Q[q][k]
+// where P and Q are the two operands seen as "row index x k" matrices with arbitrary
+// signed element strides (row stride rs, k stride ks).  Which of A, B becomes P is chosen
+// so that p runs along the unit-stride axis of C: the 32x32 MFMA accumulator holds four
+// consecutive p per lane, so C is written with 8/16-byte stores.  Transposed views are
+// therefore never materialised; they only change which loader a side uses:
+//     LD_K  k is unit stride      -> 16-byte global loads along k
+//     LD_R  rows are unit stride  -> 16-byte global loads along rows + in-register transpose
+//     LD_S  anything else         -> guarded element loads (any stride, any size)
+//
+// LDS layout (both operands, both element types): tile rows of 128 bytes = 8 chunks of 16
+// bytes (64 bf16 or 32 f32 of k).  Chunk c of row r lives at chunk slot c ^ swz(r) with
+// swz(r) = (r & 7) ^ ((r >> 3) & 1): sixteen consecutive rows reading the same logical
+// chunk touch sixteen different 16-byte bank groups, whether the LDS is viewed as 32 or
+// as 64 banks wide, and so do the 8-lane row writes of the loaders.
+//
+// MFMA operand mapping.  A 16-byte chunk is exactly one lane's operand:
+//   bf16: v_mfma_f32_32x32x16_bf16, lane l supplies row l%32, the 8 k of chunk 2s + l/32.
+//   f32 : v_mfma_f32_32x32x2_f32 four times per chunk pair; MFMA e takes element e of the
+//         chunk, i.e. k = {4(2s)+e, 4(2s+1)+e} - a permutation of k that is the same on
+//         both operands, so the dot products are unchanged.
+// Accumulator element r of lane l is D[p0 + 8*(r/4) + 4*(l/32) + r%4][q0 + l%32].
+//
+// Pipeline: global loads for k-tile t+1 are issued into registers before the MFMA loop
+// over k-tile t, and written to the other LDS stage after it; one barrier per k-tile.
+#pragma once
+#include "agh_internal.h"
+
+namespace agh {
+namespace gemm {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+enum { LD_K = 0, LD_R = 1, LD_S = 2 };
+enum { ST_SCALAR = 0, ST_VEC = 1, ST_SPLITK = 2 };
+
+struct Args {
+    const void *P;
+    const void *Q;
+    void *D;
+    const void *bias;
+    float *ws;  // split-K partials [splits][NQ][NPpad]
+    int64_t ps, pk, qs, qk, dp, dq, bias_stride;
+    int NP, NQ, K, NPpad;
+    int tiles_p, tiles_q;
+    int k_per_split;  // multiple of the k-tile
+    float alpha, beta;
+    int bias_on_p, has_bias, act;
+    int store_mode;
+};
+
+template <typename T> struct Geo;
+template <> struct Geo<uint16_t> { static constexpr int EPC = 8; };
+template <> struct Geo<float> { static constexpr int EPC = 4; };
+
+__device__ __forceinline__ uint32_t swz(uint32_t r) { return (r & 7u) ^ ((r >> 3) & 1u); }
+__device__ __forceinline__ uint32_t lds_off(uint32_t r, uint32_t c) { return r * 128u + ((c ^ swz(r)) << 4); }
+
+// ---- epilogue arithmetic in the order the reference's separate ops round ----
+template <typename T>
+__device__ __forceinline__ T finish(float acc, float alpha, float beta, T cold, bool has_bias, T bias, int act) {
+    float v = alpha * acc;
+    if (beta != 0.0f) v = v + beta * Elem<T>::to_f32(cold);
+    T r = Elem<T>::from_f32(v);
+    if (has_bias) r = Elem<T>::from_f32(Elem<T>::to_f32(bias) + Elem<T>::to_f32(r));
+    if (act == AGH_ACT_RELU) r = (Elem<T>::to_f32(r) >= 0.0f) ? r : Elem<T>::zero();
+    return r;
+}
+
+// ---- global -> register loaders (one operand tile of BR rows x 8 chunks) ----
+template <typename T, int MODE, int BR, int NT>
+struct Loader {
+    static constexpr int EPC = Geo<T>::EPC;
+    static constexpr int TOTAL = BR * 8;                   // chunks in the tile
+    static constexpr int NREG = (TOTAL + NT - 1) / NT;     // 16-byte registers per thread
+    static constexpr int NBLK_TOTAL = 8 * (BR / EPC);      // LD_R: EPC x EPC blocks in the tile
+    static constexpr int NBLK = (NBLK_TOTAL + NT - 1) / NT;
+
+    // base: element pointer of the operand; r0: first tile row; NR: rows in the operand;
+    // k0: first k of the tile; kend: one past the last valid k.
+    static __device__ __forceinline__ void load(uint4 (&reg)[NREG > NBLK * EPC ? NREG : NBLK * EPC], const T *base,
+                                                int64_t rs, int64_t ks, int r0, int NR, int k0, int kend, int tid) {
+        if constexpr (MODE == LD_K) {
+#pragma unroll
+            for (int i = 0; i < NREG; ++i) {
+                int id = tid + i * NT;
+                int r = id >> 3, c = id & 7;
+                int row = min(r0 + r, NR - 1);
+                int kk = k0 + c * EPC;
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if ((TOTAL % NT == 0 || id < TOTAL) && kk < kend) v = *(const uint4 *)(base + (int64_t)row * rs + kk);
+                reg[i] = v;
+            }
+        } else if constexpr (MODE == LD_R) {
+#pragma unroll
+            for (int i = 0; i < NBLK; ++i) {
+                int id = tid + i * NT;
+                int kb = id & 7, rb = id >> 3;
+                int row = r0 + rb * EPC;
+                if (row >= NR) row = NR - EPC;  // NR is a multiple of EPC on this path
+                bool live = (NBLK_TOTAL % NT == 0 || id < NBLK_TOTAL);
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) {
+                    int kk = k0 + kb * EPC + e;
+                    uint4 v = make_uint4(0, 0, 0, 0);
+                    if (live && kk < kend) v = *(const uint4 *)(base + (int64_t)kk * ks + row);
+                    reg[i * EPC + e] = v;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NREG; ++i) {
+                int id = tid + i * NT;
+                int r = id >> 3, c = id & 7;
+                int row = r0 + r;
+                bool rok = (TOTAL % NT == 0 || id < TOTAL) && row < NR;
+                const T *src = base + (int64_t)row * rs;
+                T tmp[EPC];
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) {
+                    int kk = k0 + c * EPC + e;
+                    T v = 0;
+                    if (rok && kk < kend) v = src[(int64_t)kk * ks];
+                    tmp[e] = v;
+                }
+                uint4 v;
+                if constexpr (sizeof(T) == 2) {
+                    v.x = (uint32_t)tmp[0] | ((uint32_t)tmp[1] << 16);
+                    v.y = (uint32_t)tmp[2] | ((uint32_t)tmp[3] << 16);
+                    v.z = (uint32_t)tmp[4] | ((uint32_t)tmp[5] << 16);
+                    v.w = (uint32_t)tmp[6] | ((uint32_t)tmp[7] << 16);
+                } else {
+                    v.x = __float_as_uint(tmp[0]);
+                    v.y = __float_as_uint(tmp[1]);
+                    v.z = __float_as_uint(tmp[2]);
+                    v.w = __float_as_uint(tmp[3]);
+                }
+                reg[i] = v;
+            }
+        }
+    }
+
+    // registers -> LDS stage (tile base address `lds`, bytes)
+    static __device__ __forceinline__ void store(const uint4 (&reg)[NREG > NBLK * EPC ? NREG : NBLK * EPC],
+                                                 unsigned char *lds, int tid) {
+        if constexpr (MODE == LD_R) {
+#pragma unroll
+            for (int i = 0; i < NBLK; ++i) {
+                int id = tid + i * NT;
+                int kb = id & 7, rb = id >> 3;
+                if (!(NBLK_TOTAL % NT == 0 || id < NBLK_TOTAL)) continue;
+                const uint4 *in = &reg[i * EPC];  // in[e] = EPC rows at k = kb*EPC + e
+                if constexpr (sizeof(T) == 4) {
+                    // 4x4 transpose of 32-bit values: pure register renaming
+                    uint4 o0 = make_uint4(in[0].x, in[1].x, in[2].x, in[3].x);
+                    uint4 o1 = make_uint4(in[0].y, in[1].y, in[2].y, in[3].y);
+                    uint4 o2 = make_uint4(in[0].z, in[1].z, in[2].z, in[3].z);
+                    uint4 o3 = make_uint4(in[0].w, in[1].w, in[2].w, in[3].w);
+                    uint32_t r = rb * 4;
+                    *(uint4 *)(lds + lds_off(r + 0, kb)) = o0;
+                    *(uint4 *)(lds + lds_off(r + 1, kb)) = o1;
+                    *(uint4 *)(lds + lds_off(r + 2, kb)) = o2;
+                    *(uint4 *)(lds + lds_off(r + 3, kb)) = o3;
+                } else {
+                    // 8x8 transpose of 16-bit values: one half-word interleave per output word,
+                    // the 32- and 64-bit levels are register renaming
+                    uint32_t w[8][4];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const uint4 &s = in[e];
+                        w[e][0] = s.x; w[e][1] = s.y; w[e][2] = s.z; w[e][3] = s.w;
+                    }
+                    uint32_t r = rb * 8;
+#pragma unroll
+                    for (int rr = 0; rr < 8; ++rr) {
+                        uint32_t o[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            uint32_t lo = w[2 * q][rr >> 1], hi = w[2 * q + 1][rr >> 1];
+                            o[q] = (rr & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
+                        }
+                        *(uint4 *)(lds + lds_off(r + rr, kb)) = make_uint4(o[0], o[1], o[2], o[3]);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NREG; ++i) {
+                int id = tid + i * NT;
+                int r = id >> 3, c = id & 7;
+                if (TOTAL % NT == 0 || id < TOTAL) *(uint4 *)(lds + lds_off(r, c)) = reg[i];
+            }
+        }
+    }
+};
+
+template <typename T> struct Mma;
+template <> struct Mma<uint16_t> {
+    static __device__ __forceinline__ void run(f32x16 &acc, const uint4 &a, const uint4 &b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                      acc, 0, 0, 0);
+    }
+};
+template <> struct Mma<float> {
+    static __device__ __forceinline__ void run(f32x16 &acc, const uint4 &a, const uint4 &b) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), acc, 0, 0, 0);
+    }
+};
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD a
+// contiguous run of tile ids, and walk tiles in panels of GROUP_P tile rows so that tiles
+// running together on an XCD share operand panels.
+__device__ __forceinline__ void tile_coords(int bid, int tiles_p, int tiles_q, int &tp, int &tq) {
+    const int nb = tiles_p * tiles_q;
+    int id = bid;
+    if ((nb & 7) == 0) id = (bid & 7) * (nb >> 3) + (bid >> 3);
+    constexpr int GROUP_P = 8;
+    const int per_group = GROUP_P * tiles_q;
+    const int group = id / per_group;
+    const int first_p = group * GROUP_P;
+    const int gsz = min(tiles_p - first_p, GROUP_P);
+    const int in_group = id - group * per_group;
+    tp = first_p + in_group % gsz;
+    tq = in_group / gsz;
+}
+
+template <typename T, int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
+__global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
+    constexpr int NT = WGP * WGQ * 64;
+    constexpr int EPC = Geo<T>::EPC;
+    constexpr int BK = 8 * EPC;
+    constexpr int TP = BP / WGP / 32, TQ = BQ / WGQ / 32;
+    static_assert(TP >= 1 && TQ >= 1, "wave tile must hold at least one 32x32 MFMA tile");
+    constexpr int STAGE_BYTES = (BP + BQ) * 128;
+    typedef Loader<T, LP, BP, NT> LdP;
+    typedef Loader<T, LQ, BQ, NT> LdQ;
+    constexpr int NRP = LdP::NREG > LdP::NBLK * EPC ? LdP::NREG : LdP::NBLK * EPC;
+    constexpr int NRQ = LdQ::NREG > LdQ::NBLK * EPC ? LdQ::NREG : LdQ::NBLK * EPC;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wp = wave % WGP, wq = wave / WGP;
+    int tp, tq;
+    tile_coords(blockIdx.x, g.tiles_p, g.tiles_q, tp, tq);
+    const int p0 = tp * BP, q0 = tq * BQ;
+    const int split = blockIdx.y;
+    const int kbeg = split * g.k_per_split;
+    const int kend = min(g.K, kbeg + g.k_per_split);
+    const int KT = kend > kbeg ? (kend - kbeg + BK - 1) / BK : 0;
+
+    const T *P = (const T *)g.P;
+    const T *Q = (const T *)g.Q;
+
+    f32x16 acc[TP][TQ];
+#pragma unroll
+    for (int i = 0; i < TP; ++i)
+#pragma unroll
+        for (int j = 0; j < TQ; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    uint4 rp[NRP], rq[NRQ];
+    if (KT > 0) {
+        LdP::load(rp, P, g.ps, g.pk, p0, g.NP, kbeg, kend, tid);
+        LdQ::load(rq, Q, g.qs, g.qk, q0, g.NQ, kbeg, kend, tid);
+        LdP::store(rp, smem, tid);
+        LdQ::store(rq, smem + BP * 128, tid);
+    }
+    __syncthreads();
+
+    // per-lane read offsets: row = lane%32 inside a 32-row MFMA tile, chunk = 2s + lane/32
+    const uint32_t lrow = lane & 31, lg = lane >> 5;
+    const uint32_t lane_off = lrow * 128u + ((lg ^ swz(lrow)) << 4);  // tile row bases are multiples of 32
+
+    for (int kt = 0; kt < KT; ++kt) {
+        const bool more = kt + 1 < KT;
+        if (more) {
+            const int k0 = kbeg + (kt + 1) * BK;
+            LdP::load(rp, P, g.ps, g.pk, p0, g.NP, k0, kend, tid);
+            LdQ::load(rq, Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
+        }
+        const unsigned char *sp = smem + (kt & 1) * STAGE_BYTES + (wp * TP * 32) * 128;
+        const unsigned char *sq = smem + (kt & 1) * STAGE_BYTES + BP * 128 + (wq * TQ * 32) * 128;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            uint4 pf[TP], qf[TQ];
+            const uint32_t off = lane_off ^ (uint32_t)(s << 5);
+#pragma unroll
+            for (int i = 0; i < TP; ++i) pf[i] = *(const uint4 *)(sp + i * 32 * 128 + off);
+#pragma unroll
+            for (int j = 0; j < TQ; ++j) qf[j] = *(const uint4 *)(sq + j * 32 * 128 + off);
+#pragma unroll
+            for (int i = 0; i < TP; ++i)
+#pragma unroll
+                for (int j = 0; j < TQ; ++j) Mma<T>::run(acc[i][j], pf[i], qf[j]);
+        }
+        if (more) {
+            unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
+            LdP::store(rp, nxt, tid);
+            LdQ::store(rq, nxt + BP * 128, tid);
+        }
+        __syncthreads();
+    }
+
+    // ------------------------------------------------------------ epilogue ----
+    const int pw0 = p0 + wp * TP * 32, qw0 = q0 + wq * TQ * 32;
+    T *D = (T *)g.D;
+    const T *bias = (const T *)g.bias;
+#pragma unroll
+    for (int i = 0; i < TP; ++i)
+#pragma unroll
+        for (int j = 0; j < TQ; ++j) {
+            const int q = qw0 + j * 32 + (int)lrow;
+            if (q >= g.NQ) continue;
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk) {
+                const int p = pw0 + i * 32 + blk * 8 + (int)lg * 4;
+                float v[4] = {acc[i][j][blk * 4 + 0], acc[i][j][blk * 4 + 1], acc[i][j][blk * 4 + 2],
+                              acc[i][j][blk * 4 + 3]};
+                if (g.store_mode == ST_SPLITK) {
+                    if (p < g.NPpad)
+                        *(float4 *)(g.ws + ((size_t)split * g.NQ + q) * g.NPpad + p) = make_float4(v[0], v[1], v[2], v[3]);
+                } else if (g.store_mode == ST_VEC) {
+                    if (p >= g.NP) continue;  // NP is a multiple of 4 on this path
+                    T *dst = D + (int64_t)q * g.dq + p;
+                    __align__(16) T old[4] = {0, 0, 0, 0};
+                    if (g.beta != 0.0f) {
+                        if constexpr (sizeof(T) == 4) *(uint4 *)old = *(const uint4 *)dst;
+                        else *(uint2 *)old = *(const uint2 *)dst;
+                    }
+                    T bq = 0;
+                    if (g.has_bias && !g.bias_on_p) bq = bias[(int64_t)q * g.bias_stride];
+                    __align__(16) T out[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        T bv = bq;
+                        if (g.has_bias && g.bias_on_p) bv = bias[(int64_t)(p + e) * g.bias_stride];
+                        out[e] = finish<T>(v[e], g.alpha, g.beta, old[e], g.has_bias != 0, bv, g.act);
+                    }
+                    if constexpr (sizeof(T) == 4) *(uint4 *)dst = *(const uint4 *)out;
+                    else *(uint2 *)dst = *(const uint2 *)out;
+                } else {
+                    T bq = 0;
+                    if (g.has_bias && !g.bias_on_p) bq = bias[(int64_t)q * g.bias_stride];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (p + e >= g.NP) continue;
+                        T *dst = D + (int64_t)(p + e) * g.dp + (int64_t)q * g.dq;
+                        T old = 0;
+                        if (g.beta != 0.0f) old = *dst;
+                        T bv = bq;
+                        if (g.has_bias && g.bias_on_p) bv = bias[(int64_t)(p + e) * g.bias_stride];
+                        *dst = finish<T>(v[e], g.alpha, g.beta, old, g.has_bias != 0, bv, g.act);
+                    }
+                }
+            }
+        }
+}
+
+// Second pass of split-K: sum the partials in split order (deterministic), then the same
+// epilogue as the single-pass kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(Args g, int splits) {
+    const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t total = (size_t)g.NQ * g.NP;
+    if (e >= total) return;
+    const int q = (int)(e / g.NP), p = (int)(e - (size_t)q * g.NP);
+    float s = 0.0f;
+    for (int z = 0; z < splits; ++z) s += g.ws[((size_t)z * g.NQ + q) * g.NPpad + p];
+    T *dst = (T *)g.D + (int64_t)p * g.dp + (int64_t)q * g.dq;
+    T old = 0;
+    if (g.beta != 0.0f) old = *dst;
+    T bv = 0;
+    if (g.has_bias) bv = ((const T *)g.bias)[(int64_t)(g.bias_on_p ? p : q) * g.bias_stride];
+    *dst = finish<T>(s, g.alpha, g.beta, old, g.has_bias != 0, bv, g.act);
+}
+
+}  // namespace gemm
+}  // namespace agh

@@ -1,0 +1,90 @@
+// Shared internals of the C-ABI library: error reporting, the single stream, the
+// library-owned workspace, argument checks and device-side bf16 helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <mutex>
+
+#include "../../include/autograph_hip.h"
+
+namespace agh {
+
+// One lock serialises every entry point (the reference's tensors are Send + Sync and
+// krnl queues work in order per device).
+std::recursive_mutex &api_mutex();
+hipStream_t stream();
+bool initialized();
+int compute_units();
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char *what);
+// Scratch owned by the library (split-K partials); grows on demand, never shrinks.
+int workspace(size_t bytes, void **ptr);
+
+#define AGH_API_ENTER()                                           \
+    std::lock_guard<std::recursive_mutex> _agh_lock(agh::api_mutex()); \
+    if (!agh::initialized()) return agh::fail(AGH_ENOINIT, "%s: agh_init has not been called", __func__)
+
+#define AGH_HIP(expr)                                                  \
+    do {                                                               \
+        hipError_t _e = (expr);                                        \
+        if (_e != hipSuccess) return agh::hip_fail(_e, #expr);         \
+    } while (0)
+
+#define AGH_LAUNCH_CHECK(name)                                         \
+    do {                                                               \
+        hipError_t _e = hipGetLastError();                             \
+        if (_e != hipSuccess) return agh::hip_fail(_e, name);          \
+    } while (0)
+
+// Division by a launch-constant divisor d (1 <= d < 2^31) of values n < 2^31 with one
+// multiply-high, an add and a shift.
+struct FastDiv {
+    uint32_t d, magic, shift;
+    FastDiv() : d(1), magic(0), shift(0) {}
+    explicit FastDiv(uint32_t div) : d(div) {
+        for (shift = 0; shift < 32; ++shift)
+            if ((1u << shift) >= d) break;
+        uint64_t one = 1;
+        magic = (uint32_t)(((one << 32) * ((one << shift) - d)) / d + 1);
+    }
+    __host__ __device__ __forceinline__ uint32_t div(uint32_t n) const {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return (__umulhi(n, magic) + n) >> shift;
+#else
+        return (uint32_t)((((uint64_t)n * magic) >> 32) + n) >> shift;
+#endif
+    }
+    __host__ __device__ __forceinline__ void divmod(uint32_t n, uint32_t &q, uint32_t &r) const {
+        q = div(n);
+        r = n - q * d;
+    }
+};
+
+// ---- bf16 <-> f32 exactly as the `half` crate does it (the reference's bf16 type) ----
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+    uint32_t x = (uint32_t)h << 16;
+    if ((h & 0x7FFFu) > 0x7F80u) x |= 0x00400000u;  // NaN: set the quiet bit
+    return __uint_as_float(x);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    uint32_t x = __float_as_uint(f);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    // round to nearest even: up iff the round bit is set and (sticky or lsb) is set
+    uint32_t up = ((x & 0x00008000u) != 0 && (x & 0x00017FFFu) != 0) ? 1u : 0u;
+    return (uint16_t)((x >> 16) + up);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+    static __device__ __forceinline__ float from_f32(float v) { return v; }
+    static __device__ __forceinline__ float zero() { return 0.0f; }
+};
+template <> struct Elem<uint16_t> {
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return bf16_to_f32(v); }
+    static __device__ __forceinline__ uint16_t from_f32(float v) { return f32_to_bf16(v); }
+    static __device__ __forceinline__ uint16_t zero() { return 0; }
+};
+
+}  // namespace agh

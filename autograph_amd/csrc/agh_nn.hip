@@ -1,0 +1,548 @@
+// Memory-bound kernels of the hot path: im2col / col2im for Conv2, MaxPool2 forward and
+// backward, ReLU, byte fill.  All of them are bounded by HBM traffic, so the work is laid
+// out for coalesced 16-byte stores and single-pass reads; index arithmetic is kept off
+// the critical path with launch-constant multiply-high division.
+#include "agh_internal.h"
+
+using namespace agh;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+inline int64_t conv_out(int64_t i, int64_t f, int64_t p, int64_t s, int64_t d) {
+    return (i + 2 * p - d * (f - 1) - 1) / s + 1;
+}
+inline int64_t col2im_out(int64_t i, int64_t f, int64_t p, int64_t s, int64_t d) {
+    return (i - 1) * s + d * (f - 1) + 1 - 2 * p;
+}
+
+// ------------------------------------------------------------------- fill ----
+__global__ __launch_bounds__(kThreads) void fill_bytes_kernel(uint8_t *dst, uint32_t pattern, size_t bytes) {
+    // head/tail bytes individually, the aligned middle as 16-byte stores
+    size_t addr = (size_t)dst;
+    size_t head = (16 - (addr & 15)) & 15;
+    if (head > bytes) head = bytes;
+    size_t body = (bytes - head) / 16;
+    size_t tail = bytes - head - body * 16;
+    size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint4 v = make_uint4(pattern, pattern, pattern, pattern);
+    uint4 *mid = (uint4 *)(dst + head);
+    for (size_t i = tid; i < body; i += stride) mid[i] = v;
+    if (tid < head) dst[tid] = (uint8_t)pattern;
+    if (tid < tail) dst[head + body * 16 + tid] = (uint8_t)pattern;
+}
+
+// ----------------------------------------------------------------- im2col ----
+//
+// One workgroup produces the patch rows of one (image b, output row ho) for a chunk of
+// CC channels: it stages the fh input rows those patches touch, for every channel of the
+// chunk, in LDS (zero-filled where the window hangs over the border), then streams the
+// patch matrix out.  For a fixed ho the rows (b, ho, wo = 0..ow-1) are adjacent in y, so
+// when the chunk is all channels the workgroup writes ONE contiguous block of
+// ow * c*fh*fw elements with 16-byte stores; the input is read once per (ho, fi) pair and
+// re-reads across neighbouring ho hit L2.
+struct Im2colParams {
+    int bs, c, ih, iw, oh, ow;
+    int fh, fw, ph, pw, sh, sw, dh, dw;
+    int cc;        // channels per workgroup
+    int nchunk;    // ceil(c / cc)
+    int span;      // input columns a row of patches touches: (ow-1)*sw + (fw-1)*dw + 1
+    int span_pad;  // LDS row pitch (elements)
+    int ktot;      // c*fh*fw
+    FastDiv div_l, div_ff, div_fw, div_nchunk, div_oh;
+};
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kThreads) void im2col_lds_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                               Im2colParams p) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    // layout: int tab[Lmax rounded to 4] | T tile[cc*fh*span_pad]
+    uint32_t bid = blockIdx.x;
+    uint32_t t0, chunk, b, ho;
+    p.div_nchunk.divmod(bid, t0, chunk);
+    p.div_oh.divmod(t0, b, ho);
+    const int c0 = chunk * p.cc;
+    const int ccur = p.cc;  // cc divides c
+    const int ff = p.fh * p.fw;
+    const int L = ccur * ff;             // columns this workgroup writes per patch row
+    const int Lmax = p.cc * ff;
+    int *tab = (int *)smem_raw;
+    T *tile = (T *)(smem_raw + (size_t)((Lmax + 3) & ~3) * sizeof(int));
+
+    // column j = (cl, fi, fj)  ->  LDS offset of its element for wo = 0
+    for (int j = threadIdx.x; j < L; j += kThreads) {
+        uint32_t cl, r, fi, fj;
+        p.div_ff.divmod(j, cl, r);
+        p.div_fw.divmod(r, fi, fj);
+        tab[j] = (cl * p.fh + fi) * p.span_pad + fj * p.dw;
+    }
+    // stage rows: one wave per (channel, fi) row, lanes along the row
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = kThreads >> 6;
+    const int nrows = ccur * p.fh;
+    for (int r = wave; r < nrows; r += nwave) {
+        int cl = r / p.fh, fi = r - cl * p.fh;
+        int hidx = -p.ph + fi * p.dh + p.sh * (int)ho;
+        bool hok = hidx >= 0 && hidx < p.ih;
+        const T *src = x + (((size_t)b * p.c + c0 + cl) * p.ih + (hok ? hidx : 0)) * (size_t)p.iw;
+        T *dst = tile + (size_t)r * p.span_pad;
+        for (int j = lane; j < p.span; j += 64) {
+            int widx = j - p.pw;
+            T v = 0;
+            if (hok && widx >= 0 && widx < p.iw) v = src[widx];
+            dst[j] = v;
+        }
+    }
+    __syncthreads();
+
+    const size_t row0 = ((size_t)b * p.oh + ho) * p.ow;  // first patch row of this workgroup
+    T *ybase = y + row0 * p.ktot + (size_t)c0 * ff;
+    const uint32_t total = (uint32_t)p.ow * L;
+    if (VEC > 1) {
+        // every patch-row segment starts 16-byte aligned and has a length that is a multiple of VEC
+        for (uint32_t e = threadIdx.x * VEC; e < total; e += kThreads * VEC) {
+            uint32_t wo, j;
+            p.div_l.divmod(e, wo, j);
+            const int base = wo * p.sw;
+            __align__(16) T vals[VEC];
+#pragma unroll
+            for (int u = 0; u < VEC; u += 4) {
+                int4 o = *(const int4 *)(tab + j + u);
+                vals[u + 0] = tile[o.x + base];
+                vals[u + 1] = tile[o.y + base];
+                vals[u + 2] = tile[o.z + base];
+                vals[u + 3] = tile[o.w + base];
+            }
+            *(uint4 *)(ybase + (size_t)wo * p.ktot + j) = *(const uint4 *)vals;
+        }
+    } else {
+        for (uint32_t e = threadIdx.x; e < total; e += kThreads) {
+            uint32_t wo, j;
+            p.div_l.divmod(e, wo, j);
+            ybase[(size_t)wo * p.ktot + j] = tile[tab[j] + wo * p.sw];
+        }
+    }
+}
+
+// Fallback for geometries whose staged rows do not fit in LDS: one thread per output
+// element, consecutive threads along a patch row.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void im2col_direct_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                                  Im2colParams p, size_t total) {
+    size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    size_t row = e / p.ktot;
+    int j = (int)(e - row * p.ktot);
+    int wo = (int)(row % p.ow);
+    size_t t = row / p.ow;
+    int ho = (int)(t % p.oh);
+    size_t b = t / p.oh;
+    int ff = p.fh * p.fw;
+    int ci = j / ff, r = j - ci * ff;
+    int fi = r / p.fw, fj = r - fi * p.fw;
+    int hidx = -p.ph + fi * p.dh + p.sh * ho;
+    int widx = -p.pw + fj * p.dw + p.sw * wo;
+    T v = 0;
+    if (hidx >= 0 && hidx < p.ih && widx >= 0 && widx < p.iw)
+        v = x[((b * p.c + ci) * p.ih + hidx) * (size_t)p.iw + widx];
+    y[e] = v;
+}
+
+template <typename T>
+int im2col_launch(const char *name, const void *x, void *y, int64_t bs, int64_t c, int64_t ih, int64_t iw,
+                  int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t sh, int64_t sw, int64_t dh, int64_t dw) {
+    AGH_API_ENTER();
+    if (bs < 0 || c < 0 || ih < 0 || iw < 0 || fh < 1 || fw < 1 || ph < 0 || pw < 0 || sh < 1 || sw < 1 || dh < 1 || dw < 1)
+        return fail(AGH_EINVAL, "%s: invalid shape/options", name);
+    if (ih + 2 * ph < dh * (fh - 1) + 1 || iw + 2 * pw < dw * (fw - 1) + 1)
+        return fail(AGH_EINVAL, "%s: filter (with dilation) larger than the padded input", name);
+    const int64_t oh = conv_out(ih, fh, ph, sh, dh), ow = conv_out(iw, fw, pw, sw, dw);
+    const int64_t lim = (int64_t)1 << 30;
+    if (bs > lim || c > lim || ih > lim || iw > lim || fh > lim || fw > lim || ph > lim || pw > lim || sh > lim ||
+        sw > lim || dh > lim || dw > lim || c * fh * fw > lim || bs * oh > lim)
+        return fail(AGH_ERANGE, "%s: dimension too large", name);
+    const size_t total = (size_t)bs * oh * ow * c * fh * fw;
+    if (total == 0) return AGH_OK;
+    if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+
+    Im2colParams p;
+    p.bs = bs; p.c = c; p.ih = ih; p.iw = iw; p.oh = oh; p.ow = ow;
+    p.fh = fh; p.fw = fw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+    p.ktot = c * fh * fw;
+    const int64_t span = (ow - 1) * sw + (fw - 1) * dw + 1;
+    const int64_t span_pad = span | 1;  // odd pitch spreads the rows over the LDS banks
+    const int ff = fh * fw;
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int64_t kLdsBudget = 48 * 1024;
+    auto lds_bytes = [&](int64_t cc) {
+        return (int64_t)((cc * ff + 3) & ~3) * 4 + cc * fh * span_pad * (int64_t)sizeof(T);
+    };
+    // Channels per workgroup: the largest divisor of c whose staged rows fit the LDS budget.
+    // Vector stores need every patch-row segment to start 16-byte aligned and to hold a
+    // multiple of VEC elements, i.e. ktot and cc*ff multiples of VEC.
+    auto pick = [&](bool vec) -> int64_t {
+        for (int64_t d = c; d >= 1; --d) {
+            if (c % d != 0) continue;
+            if (vec && (d * ff) % VEC != 0) continue;
+            if (lds_bytes(d) <= kLdsBudget && ow * d * ff < ((int64_t)1 << 31)) return d;
+        }
+        return 0;
+    };
+    bool vec = (p.ktot % VEC == 0);
+    int64_t cc = vec ? pick(true) : 0;
+    if (cc == 0) { vec = false; cc = pick(false); }
+    if (cc == 0) {
+        size_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
+        hipLaunchKernelGGL(im2col_direct_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(),
+                           (const T *)x, (T *)y, p, total);
+        AGH_LAUNCH_CHECK(name);
+        return AGH_OK;
+    }
+    p.cc = cc;
+    p.nchunk = c / cc;
+    p.span = span;
+    p.span_pad = span_pad;
+    p.div_l = FastDiv((uint32_t)(cc * ff));
+    p.div_ff = FastDiv((uint32_t)ff);
+    p.div_fw = FastDiv((uint32_t)fw);
+    p.div_nchunk = FastDiv((uint32_t)p.nchunk);
+    p.div_oh = FastDiv((uint32_t)oh);
+    const int64_t nblocks = bs * oh * p.nchunk;
+    if (nblocks > 0x7FFFFFFFll) return fail(AGH_ERANGE, "%s: too many workgroups", name);
+    const size_t smem = (size_t)lds_bytes(cc);
+    if (vec)
+        hipLaunchKernelGGL((im2col_lds_kernel<T, VEC>), dim3((unsigned)nblocks), dim3(kThreads), smem, stream(),
+                           (const T *)x, (T *)y, p);
+    else
+        hipLaunchKernelGGL((im2col_lds_kernel<T, 1>), dim3((unsigned)nblocks), dim3(kThreads), smem, stream(),
+                           (const T *)x, (T *)y, p);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+// ----------------------------------------------------------------- col2im ----
+//
+// Gather form: one thread owns one output pixel y[b,ci,hy,wy] and adds the patch entries
+// that map onto it in the order the host loop meets them: patch row hi ascending, then
+// patch column wi ascending (filter taps fi, fj therefore DEscending).  The accumulator has
+// the element type, so a bf16 sum is rounded after every add, exactly like the host.
+struct Col2imParams {
+    int bs, c, ih, iw, oh, ow;  // ih, iw: patch grid; oh, ow: image
+    int fh, fw, ph, pw, sh, sw, dh, dw;
+    int ktot;
+    FastDiv div_ow, div_oh, div_c, div_sh, div_sw;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void col2im_gather_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                                  Col2imParams p, size_t total) {
+    size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    // e = ((b*c + ci)*oh + hy)*ow + wy ; planes < 2^31 checked on the host
+    const size_t plane_sz = (size_t)p.oh * p.ow;
+    const uint32_t plane = (uint32_t)(e / plane_sz);
+    const uint32_t rem = (uint32_t)(e - (size_t)plane * plane_sz);
+    uint32_t hy, wy, b, ci;
+    p.div_ow.divmod(rem, hy, wy);
+    p.div_c.divmod(plane, b, ci);
+    const int ff = p.fh * p.fw;
+    const T *xb = x + (size_t)b * p.ih * p.iw * p.ktot + (size_t)ci * ff;
+    T acc = Elem<T>::zero();
+    for (int fi = p.fh - 1; fi >= 0; --fi) {
+        int th = (int)hy + p.ph - fi * p.dh;
+        if (th < 0) continue;
+        uint32_t hid, rh;
+        p.div_sh.divmod((uint32_t)th, hid, rh);
+        if (rh != 0 || hid >= (uint32_t)p.ih) continue;
+        for (int fj = p.fw - 1; fj >= 0; --fj) {
+            int tw = (int)wy + p.pw - fj * p.dw;
+            if (tw < 0) continue;
+            uint32_t wid, rw;
+            p.div_sw.divmod((uint32_t)tw, wid, rw);
+            if (rw != 0 || wid >= (uint32_t)p.iw) continue;
+            T v = xb[((size_t)hid * p.iw + wid) * p.ktot + fi * p.fw + fj];
+            acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(v));
+        }
+    }
+    y[e] = acc;
+}
+
+template <typename T>
+int col2im_launch(const char *name, const void *x, void *y, int64_t bs, int64_t c, int64_t ih, int64_t iw,
+                  int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t sh, int64_t sw, int64_t dh, int64_t dw) {
+    AGH_API_ENTER();
+    if (bs < 0 || c < 0 || ih < 0 || iw < 0 || fh < 1 || fw < 1 || ph < 0 || pw < 0 || sh < 1 || sw < 1 || dh < 1 || dw < 1)
+        return fail(AGH_EINVAL, "%s: invalid shape/options", name);
+    if (bs == 0 || c == 0 || ih == 0 || iw == 0) return AGH_OK;
+    const int64_t oh = col2im_out(ih, fh, ph, sh, dh), ow = col2im_out(iw, fw, pw, sw, dw);
+    if (oh < 1 || ow < 1) return fail(AGH_EINVAL, "%s: padding larger than the reconstructed image", name);
+    const int64_t lim = (int64_t)1 << 30;
+    if (bs > lim || c > lim || ih > lim || iw > lim || oh > lim || ow > lim || fh > lim || fw > lim || ph > lim ||
+        pw > lim || sh > lim || sw > lim || dh > lim || dw > lim || c * fh * fw > lim || bs * c > lim ||
+        oh * ow > lim || oh + ph > lim || ow + pw > lim)
+        return fail(AGH_ERANGE, "%s: dimension too large", name);
+    if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+    Col2imParams p;
+    p.bs = bs; p.c = c; p.ih = ih; p.iw = iw; p.oh = oh; p.ow = ow;
+    p.fh = fh; p.fw = fw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+    p.ktot = c * fh * fw;
+    p.div_ow = FastDiv((uint32_t)ow);
+    p.div_oh = FastDiv((uint32_t)oh);
+    p.div_c = FastDiv((uint32_t)c);
+    p.div_sh = FastDiv((uint32_t)sh);
+    p.div_sw = FastDiv((uint32_t)sw);
+    const size_t total = (size_t)bs * c * oh * ow;
+    size_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
+    hipLaunchKernelGGL(col2im_gather_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(), (const T *)x,
+                       (T *)y, p, total);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+// --------------------------------------------------------------- max pool ----
+struct PoolParams {
+    int ih, iw, oh, ow, h, w, sh, sw;
+    FastDiv div_ow, div_oh;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void max_pool2_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                              PoolParams p, size_t total) {
+    size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    const size_t osz = (size_t)p.oh * p.ow;
+    const size_t plane = e / osz;
+    const uint32_t rem = (uint32_t)(e - plane * osz);
+    uint32_t ho, wo;
+    p.div_ow.divmod(rem, ho, wo);
+    const T *src = x + (plane * p.ih + (size_t)ho * p.sh) * p.iw + (size_t)wo * p.sw;
+    T m = src[0];
+    float mf = Elem<T>::to_f32(m);
+    for (int fi = 0; fi < p.h; ++fi)
+        for (int fj = 0; fj < p.w; ++fj) {
+            T v = src[(size_t)fi * p.iw + fj];
+            float vf = Elem<T>::to_f32(v);
+            if (vf > mf) { m = v; mf = vf; }
+        }
+    y[e] = m;
+}
+
+// Disjoint windows (sh >= h and sw >= w): one thread per window, in place.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void max_pool2_backward_kernel(T *__restrict__ dx, const T *__restrict__ dy,
+                                                                       PoolParams p, size_t total) {
+    size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    const size_t osz = (size_t)p.oh * p.ow;
+    const size_t plane = e / osz;
+    const uint32_t rem = (uint32_t)(e - plane * osz);
+    uint32_t ho, wo;
+    p.div_ow.divmod(rem, ho, wo);
+    T *win = dx + (plane * p.ih + (size_t)ho * p.sh) * p.iw + (size_t)wo * p.sw;
+    float mf = Elem<T>::to_f32(win[0]);
+    int am = 0;
+    for (int fi = 0; fi < p.h; ++fi)
+        for (int fj = 0; fj < p.w; ++fj) {
+            int off = fi * p.iw + fj;
+            float vf = Elem<T>::to_f32(win[off]);
+            if (vf > mf) { mf = vf; am = off; }
+        }
+    // `0 + dy` in T, as the host's `+=` on the zeroed cell computes it
+    const T g = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(dy[e]));
+    for (int fi = 0; fi < p.h; ++fi)
+        for (int fj = 0; fj < p.w; ++fj) {
+            int off = fi * p.iw + fj;
+            win[off] = (off == am) ? g : Elem<T>::zero();
+        }
+}
+
+// Overlapping windows: the host visits windows of a plane one after another and each sees
+// what the previous ones wrote, so a plane is walked by a single thread.
+template <typename T>
+__global__ __launch_bounds__(64) void max_pool2_backward_seq_kernel(T *__restrict__ dx, const T *__restrict__ dy,
+                                                                     PoolParams p, size_t planes) {
+    size_t plane = (size_t)blockIdx.x * 64 + threadIdx.x;
+    if (plane >= planes) return;
+    T *d = dx + plane * (size_t)p.ih * p.iw;
+    const T *g = dy + plane * (size_t)p.oh * p.ow;
+    for (int ho = 0; ho < p.oh; ++ho)
+        for (int wo = 0; wo < p.ow; ++wo) {
+            T *win = d + (size_t)ho * p.sh * p.iw + (size_t)wo * p.sw;
+            float mf = Elem<T>::to_f32(win[0]);
+            int am = 0;
+            for (int fi = 0; fi < p.h; ++fi)
+                for (int fj = 0; fj < p.w; ++fj) {
+                    int off = fi * p.iw + fj;
+                    float vf = Elem<T>::to_f32(win[off]);
+                    if (vf > mf) { mf = vf; am = off; }
+                    win[off] = Elem<T>::zero();
+                }
+            win[am] = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(g[(size_t)ho * p.ow + wo]));
+        }
+}
+
+int pool_check(const char *name, int64_t bc, int64_t ih, int64_t iw, int64_t h, int64_t w, int64_t sh, int64_t sw,
+               PoolParams &p) {
+    if (bc < 0 || ih < 0 || iw < 0 || h < 1 || w < 1 || sh < 1 || sw < 1)
+        return fail(AGH_EINVAL, "%s: invalid shape/options", name);
+    if (h > ih || w > iw) return fail(AGH_EINVAL, "%s: window larger than the input", name);
+    const int64_t lim = (int64_t)1 << 30;
+    if (ih > lim || iw > lim || h > lim || w > lim || sh > lim || sw > lim || ih * iw > lim)
+        return fail(AGH_ERANGE, "%s: dimension too large", name);
+    p.ih = ih; p.iw = iw; p.h = h; p.w = w; p.sh = sh; p.sw = sw;
+    p.oh = (ih - h) / sh + 1;
+    p.ow = (iw - w) / sw + 1;
+    p.div_ow = FastDiv((uint32_t)p.ow);
+    p.div_oh = FastDiv((uint32_t)p.oh);
+    return AGH_OK;
+}
+
+template <typename T>
+int max_pool2_launch(const char *name, const void *x, void *y, int64_t bc, int64_t ih, int64_t iw, int64_t h,
+                     int64_t w, int64_t sh, int64_t sw) {
+    AGH_API_ENTER();
+    PoolParams p;
+    if (int rc = pool_check(name, bc, ih, iw, h, w, sh, sw, p)) return rc;
+    const size_t total = (size_t)bc * p.oh * p.ow;
+    if (total == 0) return AGH_OK;
+    if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+    size_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
+    hipLaunchKernelGGL(max_pool2_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(), (const T *)x,
+                       (T *)y, p, total);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+template <typename T>
+int max_pool2_backward_launch(const char *name, void *dx, const void *dy, int64_t bc, int64_t ih, int64_t iw,
+                              int64_t h, int64_t w, int64_t sh, int64_t sw) {
+    AGH_API_ENTER();
+    PoolParams p;
+    if (int rc = pool_check(name, bc, ih, iw, h, w, sh, sw, p)) return rc;
+    const size_t total = (size_t)bc * p.oh * p.ow;
+    if (total == 0) return AGH_OK;
+    if (!dx || !dy) return fail(AGH_ENULL, "%s: null buffer", name);
+    if (sh >= h && sw >= w) {
+        size_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
+        hipLaunchKernelGGL(max_pool2_backward_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(),
+                           (T *)dx, (const T *)dy, p, total);
+    } else {
+        size_t blocks = ((size_t)bc + 63) / 64;
+        if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many planes", name);
+        hipLaunchKernelGGL(max_pool2_backward_seq_kernel<T>, dim3((unsigned)blocks), dim3(64), 0, stream(), (T *)dx,
+                           (const T *)dy, p, (size_t)bc);
+    }
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+// ------------------------------------------------------------------- relu ----
+template <typename T>
+__global__ __launch_bounds__(kThreads) void relu_kernel(const T *x, T *y, size_t n) {
+    size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * kThreads;
+    for (; i < n; i += stride) {
+        T v = x[i];
+        y[i] = Elem<T>::to_f32(v) >= 0.0f ? v : Elem<T>::zero();
+    }
+}
+template <typename T>
+__global__ __launch_bounds__(kThreads) void relu_backward_kernel(const T *x, const T *dy, T *dx, size_t n) {
+    size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * kThreads;
+    for (; i < n; i += stride) dx[i] = Elem<T>::to_f32(x[i]) >= 0.0f ? dy[i] : Elem<T>::zero();
+}
+
+unsigned grid_for(size_t n) {
+    size_t blocks = (n + kThreads - 1) / kThreads;
+    size_t cap = (size_t)compute_units() * 32;
+    if (cap == 0) cap = 8192;
+    return (unsigned)(blocks < cap ? blocks : cap);
+}
+
+template <typename T>
+int relu_launch(const char *name, const void *x, void *y, int64_t n) {
+    AGH_API_ENTER();
+    if (n < 0) return fail(AGH_EINVAL, "%s: negative length", name);
+    if (n == 0) return AGH_OK;
+    if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+    hipLaunchKernelGGL(relu_kernel<T>, dim3(grid_for(n)), dim3(kThreads), 0, stream(), (const T *)x, (T *)y, (size_t)n);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+template <typename T>
+int relu_backward_launch(const char *name, const void *x, const void *dy, void *dx, int64_t n) {
+    AGH_API_ENTER();
+    if (n < 0) return fail(AGH_EINVAL, "%s: negative length", name);
+    if (n == 0) return AGH_OK;
+    if (!x || !dy || !dx) return fail(AGH_ENULL, "%s: null buffer", name);
+    hipLaunchKernelGGL(relu_backward_kernel<T>, dim3(grid_for(n)), dim3(kThreads), 0, stream(), (const T *)x,
+                       (const T *)dy, (T *)dx, (size_t)n);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int agh_memset(void *dst, int byte_value, size_t bytes) {
+    AGH_API_ENTER();
+    if (bytes == 0) return AGH_OK;
+    if (!dst) return fail(AGH_ENULL, "agh_memset: null pointer");
+    uint32_t b = (uint32_t)(byte_value & 0xFF);
+    uint32_t pattern = b | (b << 8) | (b << 16) | (b << 24);
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3(grid_for(bytes / 16 + 16)), dim3(kThreads), 0, stream(),
+                       (uint8_t *)dst, pattern, bytes);
+    AGH_LAUNCH_CHECK("agh_memset");
+    return AGH_OK;
+}
+
+#define AGH_CONV_ARGS int64_t bs, int64_t c, int64_t ih, int64_t iw, int64_t fh, int64_t fw, int64_t ph, int64_t pw, \
+                      int64_t sh, int64_t sw, int64_t dh, int64_t dw
+#define AGH_CONV_PASS bs, c, ih, iw, fh, fw, ph, pw, sh, sw, dh, dw
+
+int agh_im2col_conv2_f32(const void *x, void *y, AGH_CONV_ARGS) {
+    return im2col_launch<uint32_t>("agh_im2col_conv2_f32", x, y, AGH_CONV_PASS);
+}
+int agh_im2col_conv2_bf16(const void *x, void *y, AGH_CONV_ARGS) {
+    return im2col_launch<uint16_t>("agh_im2col_conv2_bf16", x, y, AGH_CONV_PASS);
+}
+int agh_col2im_conv2_f32(const void *x, void *y, AGH_CONV_ARGS) {
+    return col2im_launch<float>("agh_col2im_conv2_f32", x, y, AGH_CONV_PASS);
+}
+int agh_col2im_conv2_bf16(const void *x, void *y, AGH_CONV_ARGS) {
+    return col2im_launch<uint16_t>("agh_col2im_conv2_bf16", x, y, AGH_CONV_PASS);
+}
+
+#define AGH_POOL_ARGS int64_t bc, int64_t ih, int64_t iw, int64_t h, int64_t w, int64_t sh, int64_t sw
+#define AGH_POOL_PASS bc, ih, iw, h, w, sh, sw
+
+int agh_max_pool2_f32(const void *x, void *y, AGH_POOL_ARGS) {
+    return max_pool2_launch<float>("agh_max_pool2_f32", x, y, AGH_POOL_PASS);
+}
+int agh_max_pool2_bf16(const void *x, void *y, AGH_POOL_ARGS) {
+    return max_pool2_launch<uint16_t>("agh_max_pool2_bf16", x, y, AGH_POOL_PASS);
+}
+int agh_max_pool2_backward_f32(void *dx, const void *dy, AGH_POOL_ARGS) {
+    return max_pool2_backward_launch<float>("agh_max_pool2_backward_f32", dx, dy, AGH_POOL_PASS);
+}
+int agh_max_pool2_backward_bf16(void *dx, const void *dy, AGH_POOL_ARGS) {
+    return max_pool2_backward_launch<uint16_t>("agh_max_pool2_backward_bf16", dx, dy, AGH_POOL_PASS);
+}
+
+int agh_relu_f32(const void *x, void *y, int64_t n) { return relu_launch<float>("agh_relu_f32", x, y, n); }
+int agh_relu_bf16(const void *x, void *y, int64_t n) { return relu_launch<uint16_t>("agh_relu_bf16", x, y, n); }
+int agh_relu_backward_f32(const void *x, const void *dy, void *dx, int64_t n) {
+    return relu_backward_launch<float>("agh_relu_backward_f32", x, dy, dx, n);
+}
+int agh_relu_backward_bf16(const void *x, const void *dy, void *dx, int64_t n) {
+    return relu_backward_launch<uint16_t>("agh_relu_backward_bf16", x, dy, dx, n);
+}
+
+}  // extern "C"

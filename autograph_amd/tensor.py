@@ -1,0 +1,292 @@
+"""Host-side mirror of the reference's tensor interface for the hot path.
+
+`Device`, `Buffer` and `Tensor` carry exactly what the reference's device branches hand
+to a kernel: a device allocation, an element offset, dims and signed element strides
+(src/tensor.rs:327-332, :796-804).  Every operation below forwards to one C-ABI entry
+point of libautograph_hip.so; nothing is computed on the host.
+
+bf16 tensors travel as numpy ``uint16`` arrays of raw bit patterns.
+"""
+import ctypes as C
+from dataclasses import dataclass, field
+from typing import Tuple
+
+import numpy as np
+
+from ._ffi import AghError, check, lib
+
+F32 = "f32"
+BF16 = "bf16"
+_ITEMSIZE = {F32: 4, BF16: 2}
+_NPTYPE = {F32: np.float32, BF16: np.uint16}
+
+
+def _dtype_of(array):
+    if array.dtype == np.float32:
+        return F32
+    if array.dtype == np.uint16:
+        return BF16
+    raise TypeError(f"unsupported dtype {array.dtype}: use float32, or uint16 for bf16 bit patterns")
+
+
+class Device:
+    """`Device::builder().index(i).build()` (tests/integration_tests.rs:27-30)."""
+
+    def __init__(self, index=0):
+        check(lib.agh_init(index))
+        self.index = index
+
+    def info(self):
+        name = C.create_string_buffer(256)
+        cus = C.c_int()
+        mem = C.c_size_t()
+        check(lib.agh_device_info(name, 256, C.byref(cus), C.byref(mem)))
+        return {"name": name.value.decode(), "compute_units": cus.value, "total_mem": mem.value}
+
+    def wait(self):
+        """`device.wait()` (src/tensor/linalg.rs:549)."""
+        check(lib.agh_sync())
+
+
+class Buffer:
+    """Owning device allocation (krnl `Buffer`); freed when dropped."""
+
+    def __init__(self, nbytes):
+        p = C.c_void_p()
+        check(lib.agh_malloc(C.byref(p), nbytes))
+        self.ptr = p.value
+        self.nbytes = nbytes
+
+    def __del__(self):
+        ptr, self.ptr = getattr(self, "ptr", None), None
+        if ptr:
+            try:
+                lib.agh_free(ptr)
+            except Exception:
+                pass
+
+
+# ---- option structs, src/ops.rs:9-108 ----
+@dataclass
+class Im2ColConv2Options:
+    filter: Tuple[int, int] = (0, 0)
+    padding: Tuple[int, int] = (0, 0)
+    stride: Tuple[int, int] = (1, 1)
+    dilation: Tuple[int, int] = (1, 1)
+
+    def output_shape(self, input_shape):
+        return tuple((a + 2 * p - d * (f - 1) - 1) // s + 1
+                     for a, f, p, s, d in zip(input_shape, self.filter, self.padding, self.stride, self.dilation))
+
+
+@dataclass
+class Col2ImConv2Options:
+    shape: Tuple[int, int] = (0, 0)
+    filter: Tuple[int, int] = (0, 0)
+    padding: Tuple[int, int] = (0, 0)
+    stride: Tuple[int, int] = (1, 1)
+    dilation: Tuple[int, int] = (1, 1)
+
+    def output_shape(self):
+        return tuple((a - 1) * s + d * (f - 1) + 1 - 2 * p
+                     for a, f, p, s, d in zip(self.shape, self.filter, self.padding, self.stride, self.dilation))
+
+
+@dataclass
+class MaxPool2Options:
+    size: Tuple[int, int] = (2, 2)
+    strides: Tuple[int, int] = (2, 2)
+
+    def output_shape(self, input_shape):
+        return tuple((a - x) // s + 1 for a, x, s in zip(input_shape, self.size, self.strides))
+
+
+def _std_strides(shape):
+    strides, acc = [], 1
+    for d in reversed(shape):
+        strides.append(acc)
+        acc *= d
+    return tuple(reversed(strides))
+
+
+class Tensor:
+    """`TensorBase` = {dim, strides, buffer, offset} (src/tensor.rs:327-332) on the device."""
+
+    def __init__(self, buffer, shape, strides, offset, dtype):
+        self.buffer, self.shape, self.strides, self.offset, self.dtype = buffer, tuple(shape), tuple(strides), offset, dtype
+
+    # -- construction / transfer (src/tensor.rs:1377-1416, :1775-1833, :1923-1934) --
+    @classmethod
+    def uninit(cls, shape, dtype):
+        n = int(np.prod(shape)) if len(shape) else 1
+        return cls(Buffer(n * _ITEMSIZE[dtype]), shape, _std_strides(shape), 0, dtype)
+
+    @classmethod
+    def zeros(cls, shape, dtype):
+        t = cls.uninit(shape, dtype)
+        check(lib.agh_memset(t.buffer.ptr, 0, t.buffer.nbytes))
+        return t
+
+    @classmethod
+    def from_array(cls, array):
+        """`Tensor::from(array).into_device(device)`: copies in standard layout."""
+        a = np.ascontiguousarray(array)
+        t = cls.uninit(a.shape, _dtype_of(a))
+        check(lib.agh_memcpy_h2d(t.buffer.ptr, a.ctypes.data, a.nbytes))
+        check(lib.agh_sync())  # `a` may be a temporary
+        return t
+
+    def into_array(self):
+        """`into_array()`: blocking copy of the whole buffer, then the same strided view."""
+        raw = np.empty(self.buffer.nbytes // _ITEMSIZE[self.dtype], dtype=_NPTYPE[self.dtype])
+        check(lib.agh_memcpy_d2h(raw.ctypes.data, self.buffer.ptr, self.buffer.nbytes))
+        es = raw.itemsize
+        view = np.lib.stride_tricks.as_strided(raw[self.offset:], shape=self.shape,
+                                               strides=tuple(s * es for s in self.strides))
+        return np.array(view, order="C", copy=True)
+
+    # -- views (src/tensor.rs:695-703, :103-122) --
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    def __len__(self):
+        return int(np.prod(self.shape))
+
+    def is_standard_layout(self):
+        return all(d == 1 or s == e for d, s, e in zip(self.shape, self.strides, _std_strides(self.shape)))
+
+    def t(self):
+        return Tensor(self.buffer, self.shape[::-1], self.strides[::-1], self.offset, self.dtype)
+
+    def permuted_axes(self, axes):
+        return Tensor(self.buffer, [self.shape[a] for a in axes], [self.strides[a] for a in axes], self.offset, self.dtype)
+
+    def into_shape(self, shape):
+        if not self.is_standard_layout():
+            raise AghError(-1, "into_shape: tensor is not in standard layout")  # tensor.rs:103-122
+        if int(np.prod(shape)) != len(self):
+            raise AghError(-1, f"into_shape: incompatible shapes {self.shape} -> {tuple(shape)}")
+        return Tensor(self.buffer, shape, _std_strides(shape), self.offset, self.dtype)
+
+    def slice_rows(self, start, stop, step=1):
+        """Row slice of a 2-D tensor; a negative step gives the negative-stride views ndarray allows."""
+        assert self.ndim == 2
+        idx = range(self.shape[0])[start:stop:step]
+        off = self.offset + (idx.start if len(idx) else 0) * self.strides[0]
+        return Tensor(self.buffer, (len(idx), self.shape[1]), (self.strides[0] * step, self.strides[1]), off, self.dtype)
+
+    def _ptr(self):
+        return self.buffer.ptr
+
+    def _fn(self, stem):
+        return getattr(lib, f"{stem}_{self.dtype}")
+
+    # -- Dot, src/tensor/linalg.rs:362-468 --
+    def dot(self, rhs, bias=None, relu=False):
+        """`self.dot(&rhs)`; with `bias`/`relu` the Dense epilogue is fused into the same launch."""
+        if self.dtype != rhs.dtype:
+            raise AghError(-1, f"Can not dot tensors of different types {self.dtype} != {rhs.dtype}!")  # linalg.rs:428-434
+        if self.ndim != 2 or rhs.ndim != 2:
+            raise AghError(-1, "dot: both operands must be 2-D")
+        m, k = self.shape
+        k2, n = rhs.shape
+        if k != k2:
+            raise AghError(-1, f"a_cols != b_rows, {k} != {k2}")  # linalg.rs:274-276
+        out = Tensor.uninit((m, n), self.dtype)
+        gemm(1.0, self, rhs, 0.0, out, bias=bias, relu=relu)
+        return out
+
+    # -- Im2ColConv2 / Col2ImConv2, src/tensor/ops.rs:831-888, :982-1037 --
+    def im2col_conv2(self, options):
+        x = self.as_standard_layout()
+        bs, c, ih, iw = x.shape
+        oh, ow = options.output_shape((ih, iw))
+        (fh, fw), (ph, pw), (sh, sw), (dh, dw) = options.filter, options.padding, options.stride, options.dilation
+        y = Tensor.uninit((bs * oh * ow, c * fh * fw), self.dtype)
+        check(self._fn("agh_im2col_conv2")(x._data_ptr(), y._ptr(), bs, c, ih, iw, fh, fw, ph, pw, sh, sw, dh, dw))
+        return y
+
+    def col2im_conv2(self, options):
+        x = self.as_standard_layout()
+        rows, cols = x.shape
+        ih, iw = options.shape
+        (fh, fw), (ph, pw), (sh, sw), (dh, dw) = options.filter, options.padding, options.stride, options.dilation
+        bs, c = rows // (ih * iw), cols // (fh * fw)
+        oh, ow = options.output_shape()
+        y = Tensor.uninit((bs, c, oh, ow), self.dtype)
+        check(self._fn("agh_col2im_conv2")(x._data_ptr(), y._ptr(), bs, c, ih, iw, fh, fw, ph, pw, sh, sw, dh, dw))
+        return y
+
+    # -- MaxPool2 / MaxPool2Backward, src/tensor/ops.rs:1106-1141, :1228-1275 --
+    def max_pool2(self, options):
+        x = self.as_standard_layout()
+        bs, c, ih, iw = x.shape
+        oh, ow = options.output_shape((ih, iw))
+        y = Tensor.uninit((bs, c, oh, ow), self.dtype)
+        check(self._fn("agh_max_pool2")(x._data_ptr(), y._ptr(), bs * c, ih, iw, *options.size, *options.strides))
+        return y
+
+    def max_pool2_backward(self, output_grad, options):
+        """In place: `self` holds x on entry and dx on return (layer.rs:1203-1211 clones x first)."""
+        if self.dtype != output_grad.dtype:
+            raise AghError(-1, f"Expected {self.dtype} found {output_grad.dtype}")  # ops.rs:1236-1242
+        if not self.is_standard_layout():
+            raise AghError(-1, "max_pool2_backward: input gradient must be in standard layout")
+        dy = output_grad.as_standard_layout()
+        bs, c, ih, iw = self.shape
+        check(self._fn("agh_max_pool2_backward")(self._data_ptr(), dy._data_ptr(), bs * c, ih, iw,
+                                                 *options.size, *options.strides))
+
+    # -- relu, layer.rs:1269-1510 --
+    def relu(self):
+        x = self.as_standard_layout()
+        y = Tensor.uninit(x.shape, x.dtype)
+        check(self._fn("agh_relu")(x._data_ptr(), y._ptr(), len(x)))
+        return y
+
+    def relu_backward(self, output_grad):
+        x, dy = self.as_standard_layout(), output_grad.as_standard_layout()
+        dx = Tensor.uninit(x.shape, x.dtype)
+        check(self._fn("agh_relu_backward")(x._data_ptr(), dy._data_ptr(), dx._ptr(), len(x)))
+        return dx
+
+    # -- helpers --
+    def _data_ptr(self):
+        return self.buffer.ptr + self.offset * _ITEMSIZE[self.dtype]
+
+    def clone(self):
+        assert self.is_standard_layout()
+        out = Tensor.uninit(self.shape, self.dtype)
+        check(lib.agh_memcpy_d2d(out._ptr(), self._data_ptr(), len(self) * _ITEMSIZE[self.dtype]))
+        return out
+
+    def as_standard_layout(self):
+        if self.is_standard_layout():
+            return self
+        raise AghError(-1, "as_standard_layout: strided copy kernels are not part of this build; "
+                           "pass a standard-layout tensor")
+
+
+def gemm(alpha, a, b, beta, c, bias=None, relu=False):
+    """`fn gemm(alpha, a, b, beta, c)` with the reference's checks (src/tensor/linalg.rs:249-299)."""
+    if a.dtype != b.dtype:
+        raise AghError(-1, f"a_scalar_type != b_scalar_type, {a.dtype} != {b.dtype}")
+    if a.dtype != c.dtype:
+        raise AghError(-1, f"a_scalar_type != c_scalar_type, {a.dtype} != {c.dtype}")
+    (m, k), (k2, n), (m2, n2) = a.shape, b.shape, c.shape
+    if m != m2:
+        raise AghError(-1, f"a_rows != c_rows, {m} != {m2}")
+    if k != k2:
+        raise AghError(-1, f"a_cols != b_rows, {k} != {k2}")
+    if n != n2:
+        raise AghError(-1, f"b_cols != c_rows, {n} != {n2}")
+    common = (m, k, n, alpha, a._ptr(), a.offset, a.strides[0], a.strides[1], b._ptr(), b.offset, b.strides[0],
+              b.strides[1], beta, c._ptr(), c.offset, c.strides[0], c.strides[1])
+    if bias is None and not relu:
+        check(getattr(lib, f"agh_gemm_{c.dtype}")(*common))
+    else:
+        if bias is not None and (bias.dtype != c.dtype or bias.shape != (n,)):
+            raise AghError(-1, f"bias must be a {c.dtype} vector of length {n}")
+        bp, bo, bs_ = (bias._ptr(), bias.offset, bias.strides[0]) if bias is not None else (None, 0, 0)
+        check(getattr(lib, f"agh_gemm_{c.dtype}_bias_act")(*common, bp, bo, bs_, 1 if relu else 0))

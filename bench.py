@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Headline benchmark: bf16 GEMM at 8192^3 on one MI355X, plus the other BASELINE configs
+as `extras`, the MFMA roofline of the dominant kernel and the CPU host-path baseline.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one pass of the hot path (one GEMM launch) over operands already resident in
+HBM.  Prints ONE JSON line on stdout.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3     # MI355X f32 matrix
+PEAK_HBM_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Timer:
+    """HIP events on the library's stream, through the C ABI."""
+
+    def __init__(self, ag):
+        self.ag = ag
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        ag._ffi.check(ag.lib.agh_event_create(C.byref(self.e0)))
+        ag._ffi.check(ag.lib.agh_event_create(C.byref(self.e1)))
+
+    def time(self, fn, steps, warmup):
+        """Returns (wall ms per step, device ms per launch)."""
+        ag = self.ag
+        for _ in range(warmup):
+            fn()
+        ag._ffi.check(ag.lib.agh_sync())
+        t0 = time.perf_counter()
+        ag._ffi.check(ag.lib.agh_event_record(self.e0))
+        for _ in range(steps):
+            fn()
+        ag._ffi.check(ag.lib.agh_event_record(self.e1))
+        ag._ffi.check(ag.lib.agh_sync())
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        ms = C.c_float()
+        ag._ffi.check(ag.lib.agh_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
+        return wall, ms.value / steps
+
+
+def rand_bf16(orc, rng, shape, std=0.02):
+    out = np.empty(shape, dtype=np.uint16)
+    rows = shape[0]
+    step = max(1, (1 << 24) // max(1, int(np.prod(shape[1:]))))
+    for r in range(0, rows, step):  # chunked: keeps the f32 temporaries small
+        out[r:r + step] = orc.f32_to_bf16(rng.standard_normal((min(step, rows - r),) + tuple(shape[1:]), dtype=np.float32) * np.float32(std))
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here runs across GPUs")
+
+    import autograph_amd as ag
+    import autograph_amd._ffi  # noqa: F401
+    import oracle as orc  # cpu_baseline leg + synthetic-data helpers only
+
+    dev = ag.Device(0)
+    info = dev.info()
+    log("device:", info)
+    timer = Timer(ag)
+    rng = np.random.default_rng(2024)
+    extras = {}
+
+    # ---------------- headline: bf16 GEMM 8192^3, f32 accumulate, bf16 out ----------------
+    n = 8192
+    a = ag.Tensor.from_array(rand_bf16(orc, rng, (n, n)))
+    b = ag.Tensor.from_array(rand_bf16(orc, rng, (n, n)))
+    c = ag.Tensor.uninit((n, n), "bf16")
+    wall_ms, dev_ms = timer.time(lambda: ag.gemm(1.0, a, b, 0.0, c), args.steps, args.warmup)
+    flop = 2.0 * n * n * n
+    value = flop / (wall_ms * 1e-3) / 1e12
+    achieved = flop / (dev_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": "gemm_kernel<bf16,256x256> (v_mfma_f32_32x32x16_bf16)",
+                "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "algorithmic_flop_per_launch": flop, "avg_launch_ms": round(dev_ms, 4)}
+    log(f"bf16 gemm 8192^3: {dev_ms:.3f} ms/launch  {achieved:.1f} TFLOP/s ({100 * achieved / PEAK_BF16_TFLOPS:.1f}% of peak)")
+    del c
+
+    if not args.no_extras:
+        ks, kw = max(3, args.steps // 4), 2
+
+        def run(name, fn, work, unit, peak, steps=ks):
+            try:
+                _, ms = timer.time(fn, steps, kw)
+                rate = work / (ms * 1e-3) / (1e12 if unit == "TFLOP/s" else 1e9)
+                extras[name] = {"ms": round(ms, 4), "rate": round(rate, 2), "unit": unit, "frac_of_peak": round(rate / peak, 4)}
+                log(f"{name}: {ms:.3f} ms  {rate:.1f} {unit} ({100 * rate / peak:.1f}%)")
+            except Exception as e:  # an extra must not lose the headline line
+                extras[name] = {"error": str(e)}
+                log(f"{name}: FAILED {e}")
+
+        # bf16 A^T*B / A*B^T at 8192^3 (same operands, transposed views)
+        c = ag.Tensor.uninit((n, n), "bf16")
+        run("gemm_bf16_8192_tn", lambda: ag.gemm(1.0, a.t(), b, 0.0, c), flop, "TFLOP/s", PEAK_BF16_TFLOPS)
+        run("gemm_bf16_8192_nt", lambda: ag.gemm(1.0, a, b.t(), 0.0, c), flop, "TFLOP/s", PEAK_BF16_TFLOPS)
+        del c
+        # Dense-shaped bf16: 16384 x 4096 x 4096 with fused bias + ReLU
+        xd = ag.Tensor.from_array(rand_bf16(orc, rng, (16384, 4096)))
+        wd = ag.Tensor.from_array(rand_bf16(orc, rng, (4096, 4096)))
+        bd = ag.Tensor.from_array(rand_bf16(orc, rng, (4096,)))
+        yd = ag.Tensor.uninit((16384, 4096), "bf16")
+        run("dense_bf16_16384x4096x4096_bias_relu", lambda: ag.gemm(1.0, xd, wd, 0.0, yd, bias=bd, relu=True),
+            2.0 * 16384 * 4096 * 4096, "TFLOP/s", PEAK_BF16_TFLOPS)
+        del xd, wd, bd, yd, a, b
+
+        # f32 GEMMs: 1024, 4096 (+ transposed variants), 8192
+        for sz in (1024, 4096, 8192):
+            af = ag.Tensor.from_array(rng.uniform(-1, 1, (sz, sz)).astype(np.float32))
+            bf = ag.Tensor.from_array(rng.uniform(-1, 1, (sz, sz)).astype(np.float32))
+            cf = ag.Tensor.uninit((sz, sz), "f32")
+            w = 2.0 * sz ** 3
+            run(f"gemm_f32_{sz}", lambda: ag.gemm(1.0, af, bf, 0.0, cf), w, "TFLOP/s", PEAK_F32_TFLOPS)
+            if sz == 4096:
+                run("gemm_f32_4096_tn", lambda: ag.gemm(1.0, af.t(), bf, 0.0, cf), w, "TFLOP/s", PEAK_F32_TFLOPS)
+                run("gemm_f32_4096_nt", lambda: ag.gemm(1.0, af, bf.t(), 0.0, cf), w, "TFLOP/s", PEAK_F32_TFLOPS)
+            del af, bf, cf
+
+        # Conv2 config: im2col / col2im / conv gemm, batch 256, 64->128 ch, 56x56, 3x3 s1 p1
+        bs, ci, co, hw = 256, 64, 128, 56
+        for dt, es in (("f32", 4), ("bf16", 2)):
+            if dt == "f32":
+                x = ag.Tensor.from_array(rng.standard_normal((bs, ci, hw, hw), dtype=np.float32))
+                wt = ag.Tensor.from_array((rng.standard_normal((co, ci * 9), dtype=np.float32) * np.float32(np.sqrt(2.0 / 576))))
+            else:
+                x = ag.Tensor.from_array(rand_bf16(orc, rng, (bs, ci, hw, hw), 1.0))
+                wt = ag.Tensor.from_array(rand_bf16(orc, rng, (co, ci * 9), np.sqrt(2.0 / 576)))
+            opts = ag.Im2ColConv2Options(filter=(3, 3), padding=(1, 1))
+            cols = ag.Tensor.uninit((bs * hw * hw, ci * 9), dt)
+            fn_i = getattr(ag.lib, f"agh_im2col_conv2_{dt}")
+            fn_c = getattr(ag.lib, f"agh_col2im_conv2_{dt}")
+            bytes_ = es * (bs * ci * hw * hw + bs * hw * hw * ci * 9)
+            run(f"im2col_{dt}_conv3x3_b256", lambda: ag._ffi.check(fn_i(x._ptr(), cols._ptr(), bs, ci, hw, hw, 3, 3, 1, 1, 1, 1, 1, 1)),
+                bytes_, "GB/s", PEAK_HBM_GBS)
+            y = ag.Tensor.uninit((bs * hw * hw, co), dt)
+            run(f"conv_gemm_{dt}_802816x576x128", lambda: ag.gemm(1.0, cols, wt.t(), 0.0, y), 2.0 * bs * hw * hw * 576 * co,
+                "TFLOP/s", PEAK_F32_TFLOPS if dt == "f32" else PEAK_BF16_TFLOPS)
+            del y
+            dx = ag.Tensor.uninit((bs, ci, hw, hw), dt)
+            run(f"col2im_{dt}_conv3x3_b256", lambda: ag._ffi.check(fn_c(cols._ptr(), dx._ptr(), bs, ci, hw, hw, 3, 3, 1, 1, 1, 1, 1, 1)),
+                bytes_, "GB/s", PEAK_HBM_GBS)
+            # MaxPool2 2x2/2 on the conv-sized activation
+            py = ag.Tensor.uninit((bs, ci, hw // 2, hw // 2), dt)
+            fn_p = getattr(ag.lib, f"agh_max_pool2_{dt}")
+            fn_pb = getattr(ag.lib, f"agh_max_pool2_backward_{dt}")
+            nx, ny = bs * ci * hw * hw, bs * ci * (hw // 2) ** 2
+            run(f"max_pool2_{dt}_b256x64x56x56", lambda: ag._ffi.check(fn_p(x._ptr(), py._ptr(), bs * ci, hw, hw, 2, 2, 2, 2)),
+                es * (nx + ny), "GB/s", PEAK_HBM_GBS)
+            run(f"max_pool2_backward_{dt}_b256x64x56x56", lambda: ag._ffi.check(fn_pb(dx._ptr(), py._ptr(), bs * ci, hw, hw, 2, 2, 2, 2)),
+                es * (2 * nx + ny), "GB/s", PEAK_HBM_GBS)
+            del x, wt, cols, dx, py
+
+    # ---------------- CPU baseline: the oracle's restatement of the host path ----------------
+    cpu = None
+    if not args.no_cpu:
+        t0 = time.perf_counter()
+        s = 768  # bounded sample of the same workload: scalar bf16 fold is O(mnk) on one thread
+        ha, hb = rand_bf16(orc, rng, (s, s)), rand_bf16(orc, rng, (s, s))
+        t1 = time.perf_counter()
+        orc.gemm_bf16_hostfold(ha, hb)
+        dt_bf16 = time.perf_counter() - t1
+        sf = 2048
+        fa, fb = rng.uniform(-1, 1, (sf, sf)).astype(np.float32), rng.uniform(-1, 1, (sf, sf)).astype(np.float32)
+        threads = min(4, orc.max_threads())
+        orc.gemm_f32_host(fa[:256], fb, threads=threads)
+        t1 = time.perf_counter()
+        orc.gemm_f32_host(fa, fb, threads=threads)
+        dt_f32 = time.perf_counter() - t1
+        cpu = {"value": round(2.0 * s ** 3 / dt_bf16 / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+               "sample": f"bf16 {s}^3 GEMM, host path = scalar fold with per-op bf16 rounding, 1 thread ({dt_bf16:.2f} s); "
+                         f"the 8192^3 job is the same loop x{(8192 / s) ** 3:.0f}",
+               "f32_sgemm": {"value": round(2.0 * sf ** 3 / dt_f32 / 1e12, 4), "unit": "TFLOP/s", "cores": threads,
+                             "sample": f"f32 {sf}^3 blocked sgemm ({dt_f32:.2f} s)"},
+               "host_cores_visible": os.cpu_count()}
+        log(f"cpu baseline: bf16 fold {cpu['value']} TFLOP/s (1 thread), f32 sgemm {cpu['f32_sgemm']['value']} TFLOP/s ({threads} threads), {time.perf_counter() - t0:.1f} s")
+
+    line = {
+        "metric": "bf16/f32 GEMM TFLOP/s @8192^3 (% MFMA peak); LeNet5 b=1000 infer ms",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "bf16 GEMM C=A*B, M=N=K=8192, row-major, f32 accumulate, bf16 out (BASELINE configs[2])",
+                   "device": info["name"], "compute_units": info["compute_units"]},
+        "roofline": roofline, "cpu_baseline": cpu, "extras": extras,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,178 @@
+/*
+ * autograph_hip.h - C ABI of the MI355X (gfx950) device backend for autograph's
+ * dense-contraction hot path.
+ *
+ * The reference has no FFI layer of its own: its device backend is the krnl crate,
+ * reached from the `#[cfg(feature = "device")]` branch of every op.  Each entry point
+ * below replaces one of those device branches and takes exactly the plain values that
+ * branch extracts before dispatching a kernel (buffer, element offset, dims, signed
+ * element strides, option integers).  Citations are file:line in the reference tree.
+ *
+ * Conventions
+ *   - Every function returns 0 on success, a negative AGH_E* code for argument errors
+ *     (detected before anything is launched, like the reference's `bail!`s) and a
+ *     positive hipError_t value when HIP fails.  agh_last_error_string() describes the
+ *     last failure on the calling thread.  Nothing throws or aborts across the ABI.
+ *   - All device work is enqueued on ONE in-order stream owned by the library
+ *     (krnl's per-device queue).  Launch entry points return without waiting;
+ *     agh_memcpy_d2h and agh_sync wait.
+ *   - Pointers named x/y/a/b/c/dx/dy are DEVICE pointers from agh_malloc.  Offsets and
+ *     strides are in ELEMENTS (not bytes); strides may be negative or zero.
+ *   - bf16 data are raw 16-bit patterns (uint16_t).
+ *   - Outputs are caller-allocated and fully overwritten unless stated otherwise.
+ *     Kernels keep no pointer after they finish; the caller frees.
+ *   - Entry points may be called from any thread; calls are serialised internally.
+ */
+#ifndef AUTOGRAPH_HIP_H
+#define AUTOGRAPH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AGH_OK 0
+#define AGH_EINVAL (-1)   /* bad shape / stride / option value */
+#define AGH_ENOINIT (-2)  /* agh_init has not succeeded */
+#define AGH_ENULL (-3)    /* null pointer where data is required */
+#define AGH_ERANGE (-4)   /* size does not fit the kernel's index range */
+
+/* Epilogue activation of the fused Dense entry points. */
+#define AGH_ACT_NONE 0
+#define AGH_ACT_RELU 1
+
+/* ------------------------------------------------------------------ runtime ---- */
+
+/* Device::builder().index(i).build()  (tests/integration_tests.rs:27-30).  Selects the
+ * GPU, creates the stream.  Idempotent for the same index. */
+int agh_init(int device_index);
+/* Frees the library's own workspace and stream.  Buffers from agh_malloc stay valid
+ * until freed by the caller. */
+int agh_shutdown(void);
+const char *agh_last_error_string(void);
+/* Name, compute-unit count and memory size of the active device (krnl DeviceInfo). */
+int agh_device_info(char *name, size_t name_len, int *compute_units, size_t *total_mem_bytes);
+
+/* Buffer allocation: Tensor::uninit (src/tensor.rs:1377-1389) -> hipMalloc. */
+int agh_malloc(void **ptr, size_t bytes);
+int agh_free(void *ptr);
+/* into_device / to_device (src/tensor.rs:1775-1833): host -> device, enqueued on the stream.
+ * The host range must stay valid until the next agh_sync unless it is pageable memory. */
+int agh_memcpy_h2d(void *dst, const void *src, size_t bytes);
+/* into_array / into_vec (src/tensor.rs:1923-1934): blocks until the bytes are on the host. */
+int agh_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int agh_memcpy_d2d(void *dst, const void *src, size_t bytes);
+/* Tensor::zeros / fill for byte patterns (src/tensor.rs:1394-1416). */
+int agh_memset(void *dst, int byte_value, size_t bytes);
+/* device.wait() (src/tensor/linalg.rs:549). */
+int agh_sync(void);
+/* The hipStream_t all work is enqueued on (for callers that record their own events). */
+void *agh_stream(void);
+
+/* Timing helpers: hipEvent pairs recorded on the library's stream. */
+int agh_event_create(void **event);
+int agh_event_destroy(void *event);
+int agh_event_record(void *event);
+int agh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop` */
+
+/* --------------------------------------------------------------------- gemm ---- */
+
+/* fn gemm(alpha, a, b, beta, c)  (src/tensor/linalg.rs:249-360), reached from
+ * Tensor::dot (:410-421) and ScalarTensor::dot (:453-466).
+ *   c[off_c + i*rsc + j*csc] = alpha * sum_x a[off_a + i*rsa + x*csa] * b[off_b + x*rsb + j*csb]
+ *                              + beta * c[...]            for i < m, j < n
+ * Accumulation is f32 on the matrix cores; bf16 results are rounded once, to nearest
+ * even (linalg.rs:244, :217).  beta == 0 never reads c (linalg.rs:215).  a and b may
+ * alias each other; c must not overlap a or b, and its m*n elements must be distinct
+ * addresses (rsc, csc nonzero and non-overlapping).  m, n or k == 0 is allowed (k == 0
+ * yields beta*c).  dims must be < 2^31. */
+int agh_gemm_f32(int64_t m, int64_t k, int64_t n, float alpha,
+                 const void *a, int64_t off_a, int64_t rsa, int64_t csa,
+                 const void *b, int64_t off_b, int64_t rsb, int64_t csb,
+                 float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc);
+int agh_gemm_bf16(int64_t m, int64_t k, int64_t n, float alpha,
+                  const void *a, int64_t off_a, int64_t rsa, int64_t csa,
+                  const void *b, int64_t off_b, int64_t rsb, int64_t csb,
+                  float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc);
+
+/* Dense forward fused into one launch: `input.dot(&weight)` then `add_assign(bias)`
+ * (src/learn/neural_network/layer.rs:1134-1143, autograd.rs:571-599) then the Relu
+ * layer that follows it (layer.rs:1254-1267, rule x >= 0 ? x : 0 at :1526-1532).
+ * bias (may be null) has n elements at bias[off_bias + j*bias_stride] and is added to
+ * every row.  The epilogue rounds in the order the three separate reference ops do:
+ * T(dot) -> T(bias + .) -> relu, so bf16 results equal the unfused sequence bit for bit
+ * given the same f32 dot. */
+int agh_gemm_f32_bias_act(int64_t m, int64_t k, int64_t n, float alpha,
+                          const void *a, int64_t off_a, int64_t rsa, int64_t csa,
+                          const void *b, int64_t off_b, int64_t rsb, int64_t csb,
+                          float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc,
+                          const void *bias, int64_t off_bias, int64_t bias_stride, int act);
+int agh_gemm_bf16_bias_act(int64_t m, int64_t k, int64_t n, float alpha,
+                           const void *a, int64_t off_a, int64_t rsa, int64_t csa,
+                           const void *b, int64_t off_b, int64_t rsb, int64_t csb,
+                           float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc,
+                           const void *bias, int64_t off_bias, int64_t bias_stride, int act);
+
+/* ------------------------------------------------------------ im2col / col2im ---- */
+
+/* Im2ColConv2 device branch (src/tensor/ops.rs:842-880; semantics from the host impl
+ * :741-813).  x: [bs,c,ih,iw] standard layout.  y: [bs*oh*ow, c*fh*fw] row-major with
+ * o = (i + 2p - d(f-1) - 1)/s + 1 (src/ops.rs:35);
+ *   y[(b,ho,wo),(ci,fi,fj)] = x[b,ci,-ph+fi*dh+sh*ho,-pw+fj*dw+sw*wo], 0 outside x. */
+int agh_im2col_conv2_f32(const void *x, void *y, int64_t bs, int64_t c, int64_t ih, int64_t iw,
+                         int64_t fh, int64_t fw, int64_t ph, int64_t pw,
+                         int64_t sh, int64_t sw, int64_t dh, int64_t dw);
+int agh_im2col_conv2_bf16(const void *x, void *y, int64_t bs, int64_t c, int64_t ih, int64_t iw,
+                          int64_t fh, int64_t fw, int64_t ph, int64_t pw,
+                          int64_t sh, int64_t sw, int64_t dh, int64_t dw);
+
+/* Col2ImConv2 device branch (src/tensor/ops.rs:992-1030).  x: [bs*ih*iw, c*fh*fw] where
+ * (ih,iw) is the PATCH GRID (options.shape).  y: [bs,c,oh,ow] with
+ * o = (i-1)s + d(f-1) + 1 - 2p (src/ops.rs:75), fully overwritten.  Sums follow the
+ * reference's HOST loop (:913-960): accumulator of type T starting at +0, contributions
+ * added in (hi, wi) ascending order, every bf16 add rounded - so results are bit-identical
+ * to the host path (the reference's own device kernel accumulates in f32 instead). */
+int agh_col2im_conv2_f32(const void *x, void *y, int64_t bs, int64_t c, int64_t ih, int64_t iw,
+                         int64_t fh, int64_t fw, int64_t ph, int64_t pw,
+                         int64_t sh, int64_t sw, int64_t dh, int64_t dw);
+int agh_col2im_conv2_bf16(const void *x, void *y, int64_t bs, int64_t c, int64_t ih, int64_t iw,
+                          int64_t fh, int64_t fw, int64_t ph, int64_t pw,
+                          int64_t sh, int64_t sw, int64_t dh, int64_t dw);
+
+/* ---------------------------------------------------------------- max pool ---- */
+
+/* MaxPool2 device branch (src/tensor/ops.rs:1117-1133; rule from the host impl
+ * :1062-1084).  x: [bc, ih, iw] (bc = bs*c planes), y: [bc, oh, ow], o = (i - size)/s + 1
+ * (src/ops.rs:99).  The first element of the window is taken, a later one replaces it
+ * only if strictly greater; the result is a bit copy of that element. */
+int agh_max_pool2_f32(const void *x, void *y, int64_t bc, int64_t ih, int64_t iw,
+                      int64_t h, int64_t w, int64_t sh, int64_t sw);
+int agh_max_pool2_bf16(const void *x, void *y, int64_t bc, int64_t ih, int64_t iw,
+                       int64_t h, int64_t w, int64_t sh, int64_t sw);
+
+/* MaxPool2Backward device branch (src/tensor/ops.rs:1252-1264; host rule :1173-1201).
+ * dx_inout holds the forward input x on entry ([bc, ih, iw]) and the input gradient on
+ * return; dy is [bc, oh, ow].  Per window: every cell is zeroed and `0 + dy` lands on the
+ * first strict maximum; cells no window covers keep x.  Overlapping windows
+ * (sh < h or sw < w) are applied in the host's (ho, wo) order, one plane per thread. */
+int agh_max_pool2_backward_f32(void *dx_inout, const void *dy, int64_t bc, int64_t ih, int64_t iw,
+                               int64_t h, int64_t w, int64_t sh, int64_t sw);
+int agh_max_pool2_backward_bf16(void *dx_inout, const void *dy, int64_t bc, int64_t ih, int64_t iw,
+                                int64_t h, int64_t w, int64_t sh, int64_t sw);
+
+/* -------------------------------------------------------------------- relu ---- */
+
+/* relu / relu_mut (x == y allowed) and relu_backward / relu_backward_mut (dx == dy
+ * allowed) kernels (src/learn/neural_network/layer.rs:1542-1565) over n contiguous
+ * elements. */
+int agh_relu_f32(const void *x, void *y, int64_t n);
+int agh_relu_bf16(const void *x, void *y, int64_t n);
+int agh_relu_backward_f32(const void *x, const void *dy, void *dx, int64_t n);
+int agh_relu_backward_bf16(const void *x, const void *dy, void *dx, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AUTOGRAPH_HIP_H */

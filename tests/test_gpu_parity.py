@@ -1,0 +1,422 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on a real MI355X.
+
+Modelled on the reference's own device tests (tests/integration_tests.rs): the same
+generators (ramps, cycles), the same parameter grids, host result vs device result.
+Bars: im2col / col2im / pooling / relu bit-exact; f32 gemm within 1e-5*sqrt(K) relative;
+bf16 gemm within 1 bf16 ulp + 1e-2 relative of an f32-accumulated reference.
+"""
+import numpy as np
+import pytest
+
+import oracle as orc
+from refgrid import DOT_SIZES, POOL_SHAPES, cases
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ag():
+    import autograph_amd as ag
+    ag.Device(0)
+    return ag
+
+
+def to_dtype(x, dtype):
+    return orc.f32_to_bf16(x) if dtype == "bf16" else np.ascontiguousarray(x, dtype=np.float32)
+
+
+def as_f32(x):
+    return orc.bf16_to_f32(x) if x.dtype == np.uint16 else x
+
+
+# ------------------------------------------------------------------ tolerances ----
+def assert_f32_gemm_close(got, a, b, want64=None, k=None):
+    """|got - want| <= 1e-5*sqrt(K) * scale, with scale = max|want| (norm-wise) and, element-wise,
+    sum_k |a||b| (the quantity a rounding-error bound of a dot product is relative to)."""
+    k = k or a.shape[1]
+    want64 = orc.gemm_f64acc(a, b) if want64 is None else want64
+    absprod = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
+    err = np.abs(got.astype(np.float64) - want64)
+    tol = 1e-5 * np.sqrt(max(k, 1))
+    assert err.max() <= tol * max(np.abs(want64).max(), 1e-30), (err.max(), np.abs(want64).max())
+    assert np.all(err <= tol * absprod + 1e-30)
+
+
+def bf16_ulp(x):
+    x = np.abs(x.astype(np.float64))
+    e = np.floor(np.log2(np.maximum(x, 2.0**-126)))
+    return 2.0 ** (e - 7)
+
+
+def assert_bf16_gemm_close(got_bits, ref_bits, a_bits, b_bits):
+    """got within 1 bf16 ulp + 1e-2 relative of the f32-accumulated reference.  Two f32
+    accumulation orders can themselves differ by about sqrt(K)*2^-24*sum|a||b|, which matters
+    only where the true result cancels to ~0; that floor is added so such entries do not
+    decide the test."""
+    got, ref = orc.bf16_to_f32(got_bits).astype(np.float64), orc.bf16_to_f32(ref_bits).astype(np.float64)
+    a, b = orc.bf16_to_f32(a_bits).astype(np.float64), orc.bf16_to_f32(b_bits).astype(np.float64)
+    k = a.shape[1]
+    floor = 8 * np.sqrt(k) * 2.0**-24 * (np.abs(a) @ np.abs(b))
+    tol = bf16_ulp(ref) + 1e-2 * np.abs(ref) + floor
+    bad = np.abs(got - ref) > tol
+    assert not bad.any(), (np.argwhere(bad)[:5], got[bad][:5], ref[bad][:5])
+
+
+# ------------------------------------------------------------------------ dot ----
+def gen_array(shape):  # 1..9 cycling, integration_tests.rs:291-305
+    return ((np.arange(shape[0] * shape[1]) % 9) + 1).astype(np.float32).reshape(shape)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("n", DOT_SIZES)
+def test_tensor_dot_reference_cases(ag, dtype, n):
+    """tensor_dot_<T>_m{n}_k{n}_n{n}_{nn,tn,nt,tt} (integration_tests.rs:272-376): exact data."""
+    for ta in (False, True):
+        for tb in (False, True):
+            a1, a2 = to_dtype(gen_array((n, n)), dtype), to_dtype(gen_array((n, n)), dtype)
+            t1, t2 = ag.Tensor.from_array(a1), ag.Tensor.from_array(a2)
+            if ta:
+                a1, t1 = a1.T, t1.t()
+            if tb:
+                a2, t2 = a2.T, t2.t()
+            out = t1.dot(t2).into_array()
+            want = orc.gemm_f64acc(a1, a2)
+            if dtype == "f32":
+                assert np.array_equal(out.astype(np.float64), want), (n, ta, tb)
+            else:
+                assert np.array_equal(out, orc.gemm_bf16_f32acc(a1, a2)), (n, ta, tb)
+                assert np.all(np.abs(orc.bf16_to_f32(out) - want) <= n)  # the reference's own epsilon = k
+
+
+SHAPES = [(1, 1, 1), (3, 7, 5), (33, 17, 65), (100, 77, 53), (64, 64, 64), (129, 256, 130), (256, 512, 384),
+          (300, 1000, 20), (17, 2048, 9), (1000, 256, 128), (1000, 84, 10), (6400, 150, 16), (100, 25, 6)]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("mkn", SHAPES)
+def test_dot_seeded_all_transposes(ag, dtype, mkn):
+    m, k, n = mkn
+    rng = np.random.default_rng(hash((m, k, n)) % 2**32)
+    for ta in (False, True):
+        for tb in (False, True):
+            a = to_dtype(rng.uniform(-1, 1, (k, m) if ta else (m, k)), dtype)
+            b = to_dtype(rng.uniform(-1, 1, (n, k) if tb else (k, n)), dtype)
+            ta_, tb_ = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+            av, bv = (a.T if ta else a), (b.T if tb else b)
+            tav, tbv = (ta_.t() if ta else ta_), (tb_.t() if tb else tb_)
+            out = tav.dot(tbv).into_array()
+            if dtype == "f32":
+                assert_f32_gemm_close(out, av, bv)
+            else:
+                assert_bf16_gemm_close(out, orc.gemm_bf16_f32acc(av, bv), av, bv)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_gemm_strides_offsets_alpha_beta(ag, dtype):
+    """fn gemm with the full (offset, rs, cs) tuple for all three operands (linalg.rs:281-299):
+    sub-views with offsets, negative strides, a column-major C, alpha and beta."""
+    rng = np.random.default_rng(11)
+    big_a = to_dtype(rng.uniform(-1, 1, (90, 150)), dtype)
+    big_b = to_dtype(rng.uniform(-1, 1, (140, 120)), dtype)
+    big_c = to_dtype(rng.uniform(-1, 1, (80, 100)), dtype)
+    cases_ = [
+        (big_a[3:67:2, 5:125:3], big_b[100:20:-2, 110:2:-3], big_c[2:34, 10:46]),         # 32x40 @ 40x36
+        (big_a[10:74, 8:72], big_b[4:68, 16:80], big_c[0:64, 4:68]),                      # aligned 64^3 views
+        (big_a[0:80, 0:96].T[0:96:1, 0:80][:, ::-1], big_b[0:80, 0:40], big_c.T[0:96, 0:40]),  # A transposed + reversed, C col-major
+    ]
+    for av, bv, cv in cases_:
+        m, k = av.shape
+        k2, n = bv.shape
+        assert k == k2 and cv.shape == (m, n)
+        for alpha, beta in [(1.0, 0.0), (0.5, 2.0), (-1.25, 1.0)]:
+            ta, tb, tc = ag.Tensor.from_array(big_a), ag.Tensor.from_array(big_b), ag.Tensor.from_array(big_c)
+
+            def view(t, base, v):
+                _, off, rs, cs = orc._view(v)
+                return ag.Tensor(t.buffer, v.shape, (rs, cs), off, t.dtype)
+
+            tcv = view(tc, big_c, cv)
+            ag.gemm(alpha, view(ta, big_a, av), view(tb, big_b, bv), beta, tcv)
+            full = tc.into_array()
+            got = np.lib.stride_tricks.as_strided(full.reshape(-1)[orc._view(cv)[1]:], shape=cv.shape,
+                                                  strides=tuple(s * full.itemsize for s in orc._view(cv)[2:]))
+            want = orc.gemm_f64acc(av, bv, alpha, beta, cv)
+            # everything outside the C view is untouched
+            mask = np.ones(big_c.size, bool)
+            idx = (orc._view(cv)[1] + np.arange(m)[:, None] * orc._view(cv)[2] + np.arange(n)[None, :] * orc._view(cv)[3])
+            mask[idx.reshape(-1)] = False
+            assert np.array_equal(full.reshape(-1)[mask], big_c.reshape(-1)[mask])
+            if dtype == "f32":
+                absprod = abs(alpha) * (np.abs(av).astype(np.float64) @ np.abs(bv)) + abs(beta) * np.abs(cv)
+                assert np.all(np.abs(got - want) <= 1e-5 * np.sqrt(k) * absprod)
+            else:
+                gotf = orc.bf16_to_f32(np.ascontiguousarray(got)).astype(np.float64)
+                absprod = abs(alpha) * (np.abs(as_f32(np.ascontiguousarray(av))).astype(np.float64) @ np.abs(as_f32(np.ascontiguousarray(bv)))) + abs(beta) * np.abs(as_f32(np.ascontiguousarray(cv)))
+                assert np.all(np.abs(gotf - want) <= bf16_ulp(want) + 1e-2 * np.abs(want) + 1e-5 * absprod)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_gemm_beta_zero_never_reads_c_and_k_zero(ag, dtype):
+    rng = np.random.default_rng(12)
+    a, b = to_dtype(rng.uniform(-1, 1, (40, 24)), dtype), to_dtype(rng.uniform(-1, 1, (24, 48)), dtype)
+    poison = np.full((40, 48), np.nan, dtype=np.float32)
+    c = ag.Tensor.from_array(to_dtype(poison, dtype))
+    ag.gemm(1.0, ag.Tensor.from_array(a), ag.Tensor.from_array(b), 0.0, c)  # linalg.rs:215
+    assert np.isfinite(as_f32(c.into_array())).all()
+    # k == 0: C = beta*C
+    c0 = to_dtype(rng.uniform(-1, 1, (8, 12)), dtype)
+    c = ag.Tensor.from_array(c0)
+    ag.gemm(1.0, ag.Tensor.uninit((8, 0), dtype), ag.Tensor.uninit((0, 12), dtype), 2.0, c)
+    assert np.array_equal(as_f32(c.into_array()), as_f32(to_dtype(2.0 * as_f32(c0), dtype)))
+    # empty outputs are a no-op
+    assert ag.Tensor.uninit((0, 5), dtype).dot(ag.Tensor.uninit((5, 3), dtype)).shape == (0, 3)
+
+
+def test_split_k_shapes(ag):
+    """The weight-gradient shapes of the LeNet5 step (k >> m*n), which the reference splits along k
+    (linalg.rs:306-340): dW1 = dY^T * im2col (6 x 57600 x 25), dW2 (16 x 6400 x 150)."""
+    rng = np.random.default_rng(13)
+    for (m, k, n) in [(6, 57600, 25), (16, 6400, 150), (64, 16384, 64)]:
+        for dtype in ("f32", "bf16"):
+            dy = to_dtype(rng.normal(0, 1, (k, m)), dtype)
+            cols = to_dtype(rng.normal(0, 1, (k, n)), dtype)
+            out = ag.Tensor.from_array(dy).t().dot(ag.Tensor.from_array(cols)).into_array()
+            if dtype == "f32":
+                assert_f32_gemm_close(out, dy.T, cols)
+            else:
+                assert_bf16_gemm_close(out, orc.gemm_bf16_f32acc(dy.T, cols), dy.T, cols)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_dense_fused_bias_relu(ag, dtype):
+    """Dense::forward + Relu (layer.rs:1134-1143, :1254-1267) in one launch equals dot -> add_assign(bias)
+    -> relu done as three ops."""
+    # exact data: small integers, so the f32 dot is exact and the fused result must be bit-identical
+    x = ((np.arange(37 * 48) % 7) - 3).astype(np.float32).reshape(37, 48)
+    w = ((np.arange(48 * 20) % 5) - 2).astype(np.float32).reshape(48, 20)
+    bias = (np.arange(20) % 9 - 4).astype(np.float32) * 0.5
+    xd, wd, bd = to_dtype(x, dtype), to_dtype(w, dtype), to_dtype(bias, dtype)
+    got = ag.Tensor.from_array(xd).dot(ag.Tensor.from_array(wd), bias=ag.Tensor.from_array(bd), relu=True).into_array()
+    dot = orc.gemm_bf16_f32acc(xd, wd) if dtype == "bf16" else orc.gemm_f64acc(xd, wd).astype(np.float32)
+    want = orc.relu(orc.bias_add_rows(dot, bd))
+    assert np.array_equal(got, want)
+    # bias only (dense3 of LeNet5), relu only
+    got = ag.Tensor.from_array(xd).dot(ag.Tensor.from_array(wd), bias=ag.Tensor.from_array(bd)).into_array()
+    assert np.array_equal(got, orc.bias_add_rows(dot, bd))
+    got = ag.Tensor.from_array(xd).dot(ag.Tensor.from_array(wd), relu=True).into_array()
+    assert np.array_equal(got, orc.relu(dot))
+    # seeded real data at a Dense-like shape, tolerance of the unfused sequence
+    rng = np.random.default_rng(14)
+    x = to_dtype(rng.normal(0, 0.02, (512, 256)), dtype)
+    w = to_dtype(rng.normal(0, 0.02, (256, 384)), dtype)
+    b = to_dtype(rng.normal(0, 0.02, (384,)), dtype)
+    got = ag.Tensor.from_array(x).dot(ag.Tensor.from_array(w), bias=ag.Tensor.from_array(b), relu=True).into_array()
+    if dtype == "f32":
+        want = np.maximum(orc.gemm_f64acc(x, w) + b, 0)
+        assert np.all(np.abs(got - want) <= 1e-5 * 16 * (np.abs(x).astype(np.float64) @ np.abs(w) + np.abs(b)))
+    else:
+        ref = orc.relu(orc.bias_add_rows(orc.gemm_bf16_f32acc(x, w), b))
+        g, r = orc.bf16_to_f32(got).astype(np.float64), orc.bf16_to_f32(ref).astype(np.float64)
+        scale = np.abs(orc.bf16_to_f32(x)).astype(np.float64) @ np.abs(orc.bf16_to_f32(w)) + np.abs(orc.bf16_to_f32(b))
+        assert np.all(np.abs(g - r) <= 2 * bf16_ulp(np.maximum(np.abs(r), np.abs(g))) + 1e-2 * np.abs(r) + 1e-5 * scale)
+
+
+def test_dot_error_behaviour(ag):
+    a = ag.Tensor.from_array(np.zeros((4, 5), np.float32))
+    with pytest.raises(ag.AghError, match="different types"):
+        a.dot(ag.Tensor.from_array(np.zeros((5, 3), np.uint16)))
+    with pytest.raises(ag.AghError, match="a_cols != b_rows"):
+        a.dot(ag.Tensor.from_array(np.zeros((4, 3), np.float32)))
+    with pytest.raises(ag.AghError, match="a_rows != c_rows"):
+        ag.gemm(1.0, a, ag.Tensor.from_array(np.zeros((5, 3), np.float32)), 0.0, ag.Tensor.uninit((5, 3), "f32"))
+    # the C ABI itself rejects bad arguments with a status
+    assert ag.lib.agh_gemm_f32(-1, 1, 1, 1.0, None, 0, 1, 1, None, 0, 1, 1, 0.0, None, 0, 1, 1) == -1
+    assert ag.lib.agh_gemm_f32(2, 2, 2, 1.0, None, 0, 1, 1, None, 0, 1, 1, 0.0, None, 0, 1, 1) == -3
+    assert ag.lib.agh_im2col_conv2_f32(None, None, 1, 1, 2, 2, 3, 3, 0, 0, 1, 1, 1, 1) == -1  # filter > input
+    assert ag.lib.agh_max_pool2_f32(None, None, 1, 2, 2, 3, 3, 1, 1) == -1
+
+
+@pytest.mark.parametrize("dtype,shape", [("f32", (4096, 4096, 4096)), ("bf16", (8192, 8192, 8192)),
+                                         ("f32", (8192, 8192, 8192))])
+def test_gemm_full_size_sampled_entries_and_identity(ag, dtype, shape):
+    """BASELINE-size GEMMs: the oracle cannot run 10^12 flops, so check (1) 4096 sampled output
+    entries against f64 dot products of the corresponding row and column, for A*B, A^T*B and
+    A*B^T, and (2) A*I == A bit for bit."""
+    m, k, n = shape
+    rng = np.random.default_rng(15)
+    if dtype == "f32":
+        a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    else:
+        a = orc.f32_to_bf16(rng.normal(0, 0.02, (m, k)).astype(np.float32))
+        b = orc.f32_to_bf16(rng.normal(0, 0.02, (k, n)).astype(np.float32))
+    ta, tb = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+    ii, jj = rng.integers(0, m, 4096), rng.integers(0, n, 4096)
+    af, bf = as_f32(a), as_f32(b)
+
+    def check(out, av, bv):
+        want = np.einsum("ik,ki->i", av[ii].astype(np.float64), bv[:, jj].astype(np.float64))
+        scale = np.einsum("ik,ki->i", np.abs(av[ii]).astype(np.float64), np.abs(bv[:, jj]).astype(np.float64))
+        got = as_f32(out[ii, jj]).astype(np.float64)
+        if dtype == "f32":
+            assert np.all(np.abs(got - want) <= 1e-5 * np.sqrt(k) * scale)
+            assert np.abs(got - want).max() <= 1e-5 * np.sqrt(k) * np.abs(want).max()
+        else:
+            assert np.all(np.abs(got - want) <= bf16_ulp(want) + 1e-2 * np.abs(want) + 8 * np.sqrt(k) * 2.0**-24 * scale)
+
+    check(ta.dot(tb).into_array(), af, bf)
+    if m == k == n:
+        check(ta.t().dot(tb).into_array(), af.T, bf)
+        check(ta.dot(tb.t()).into_array(), af, bf.T)
+    eye = np.eye(k, n, dtype=np.float32)
+    out = ta.dot(ag.Tensor.from_array(to_dtype(eye, dtype))).into_array()
+    assert np.array_equal(out[:, :min(k, n)], a[:, :min(k, n)])
+
+
+# ------------------------------------------------------------- im2col / col2im ----
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_im2col_col2im_reference_grid(ag, dtype):
+    """im2col_conv2_<T>_<opts> and col2im_conv2_<T>_<opts> (integration_tests.rs:946-981, :1499-1552):
+    ramp inputs over the whole filter/padding/stride/dilation grid; host vs device, bit for bit."""
+    count = 0
+    for bs, c, ih, iw, f, p, s, d in cases():
+        x = to_dtype(np.arange(1, bs * c * ih * iw + 1, dtype=np.float32).reshape(bs, c, ih, iw), dtype)
+        opts = ag.Im2ColConv2Options(filter=f, padding=p, stride=s, dilation=d)
+        y = ag.Tensor.from_array(x).im2col_conv2(opts).into_array()
+        want = orc.im2col_conv2(x, f, p, s, d)
+        assert np.array_equal(y, want), ("im2col", bs, c, ih, iw, f, p, s, d)
+        oh, ow = opts.output_shape((ih, iw))
+        dy = to_dtype(np.arange(1, want.size + 1, dtype=np.float32).reshape(want.shape), dtype)
+        copts = ag.Col2ImConv2Options(shape=(oh, ow), filter=f, padding=p, stride=s, dilation=d)
+        dx = ag.Tensor.from_array(dy).col2im_conv2(copts).into_array()
+        assert np.array_equal(dx, orc.col2im_conv2(dy, (oh, ow), f, p, s, d)), ("col2im", bs, c, ih, iw, f, p, s, d)
+        count += 1
+    assert count > 1000
+
+
+IM2COL_SEEDED = [
+    # bs, c, ih, iw, filter, padding, stride, dilation
+    (4, 16, 28, 28, (3, 3), (1, 1), (1, 1), (1, 1)),      # vector-store path, all channels in one workgroup
+    (100, 1, 28, 28, (5, 5), (0, 0), (1, 1), (1, 1)),     # LeNet5 conv1 (25-wide rows, scalar stores)
+    (100, 6, 12, 12, (5, 5), (0, 0), (1, 1), (1, 1)),     # LeNet5 conv2
+    (2, 512, 14, 14, (3, 3), (1, 1), (1, 1), (1, 1)),     # channels split over several workgroups
+    (3, 8, 17, 23, (3, 5), (2, 1), (2, 3), (2, 1)),       # everything non-default at once
+    (1, 4, 6, 9000, (1, 3), (0, 1), (1, 1), (1, 1)),      # rows too wide for LDS: direct kernel
+    (2, 24, 9, 9, (2, 2), (0, 0), (2, 2), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("case", IM2COL_SEEDED)
+def test_im2col_col2im_seeded(ag, dtype, case):
+    bs, c, ih, iw, f, p, s, d = case
+    rng = np.random.default_rng(16)
+    x = to_dtype(rng.standard_normal((bs, c, ih, iw)), dtype)
+    opts = ag.Im2ColConv2Options(filter=f, padding=p, stride=s, dilation=d)
+    y = ag.Tensor.from_array(x).im2col_conv2(opts).into_array()
+    assert np.array_equal(y, orc.im2col_conv2(x, f, p, s, d))
+    oh, ow = opts.output_shape((ih, iw))
+    g = to_dtype(rng.standard_normal(y.shape), dtype)
+    dx = ag.Tensor.from_array(g).col2im_conv2(ag.Col2ImConv2Options((oh, ow), f, p, s, d)).into_array()
+    want = orc.col2im_conv2(g, (oh, ow), f, p, s, d)
+    assert np.array_equal(dx, want)  # bit-exact incl. bf16's per-add rounding in host order
+
+
+def test_col2im_bf16_rounding_order_case(ag):
+    f, p = (1, 3), (0, 1)
+    cols = np.zeros((3, 3), dtype=np.float32)
+    cols[0, 2], cols[1, 1], cols[2, 0] = 256.0, 1.0, 1.0
+    y = ag.Tensor.from_array(orc.f32_to_bf16(cols)).col2im_conv2(ag.Col2ImConv2Options((1, 3), f, p)).into_array()
+    assert orc.bf16_to_f32(y)[0, 0, 0, 1] == 256.0  # an f32 accumulator would give 258
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_im2col_col2im_config3_full_size(ag, dtype):
+    """Conv2 config: batch 256, 64 channels, 56x56, 3x3, stride 1, pad 1 - bit-exact against the
+    oracle at full size (the oracle is a threaded copy loop, it finishes in seconds)."""
+    rng = np.random.default_rng(17)
+    bs, c, ih, iw, f, p = 256, 64, 56, 56, (3, 3), (1, 1)
+    x = to_dtype(rng.standard_normal((bs, c, ih, iw), dtype=np.float32), dtype)
+    t = ag.Tensor.from_array(x).im2col_conv2(ag.Im2ColConv2Options(filter=f, padding=p))
+    y = t.into_array()
+    want = orc.im2col_conv2(x, f, p)
+    assert y.shape == (802816, 576)
+    assert np.array_equal(y, want)
+    del want
+    # col2im of the patch matrix itself (values repeat, sums still round): bit-exact vs the host order
+    dx = t.col2im_conv2(ag.Col2ImConv2Options((56, 56), f, p)).into_array()
+    assert np.array_equal(dx, orc.col2im_conv2(y, (56, 56), f, p))
+
+
+# ------------------------------------------------------------------- max pool ----
+def cyc(shape):
+    return (np.arange(int(np.prod(shape))) % 10).astype(np.float32).reshape(shape)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_max_pool2_reference_cases(ag, dtype):
+    """max_pool2_<T> / max_pool2_backward_<T> (integration_tests.rs:1038-1061, :1554-1628)."""
+    opts = ag.MaxPool2Options((2, 2), (2, 2))
+    for shape in POOL_SHAPES:
+        x = to_dtype(cyc(shape), dtype)
+        tx = ag.Tensor.from_array(x)
+        y = tx.max_pool2(opts).into_array()
+        assert np.array_equal(y, orc.max_pool2(x, (2, 2)))
+        dy = to_dtype(np.arange(y.size, dtype=np.float32).reshape(y.shape), dtype)
+        dx = tx.clone()
+        dx.max_pool2_backward(ag.Tensor.from_array(dy), opts)
+        assert np.array_equal(dx.into_array(), orc.max_pool2_backward(x, dy, (2, 2)))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("shape,size,strides", [
+    ((1000, 6, 24, 24), (2, 2), (2, 2)), ((1000, 16, 8, 8), (2, 2), (2, 2)), ((100, 6, 24, 24), (2, 2), (2, 2)),
+    ((3, 5, 17, 23), (3, 2), (3, 2)), ((2, 4, 19, 21), (2, 3), (4, 5)), ((2, 3, 15, 15), (3, 3), (2, 2)),
+    ((1, 2, 9, 11), (3, 3), (1, 1)), ((7, 3, 10, 33), (2, 2), (2, 1)),
+])
+def test_max_pool2_seeded(ag, dtype, shape, size, strides):
+    rng = np.random.default_rng(18)
+    # values drawn from a small set so windows contain ties; the first maximum must win
+    x = to_dtype(rng.integers(-4, 5, shape).astype(np.float32) * 0.5, dtype)
+    opts = ag.MaxPool2Options(size, strides)
+    tx = ag.Tensor.from_array(x)
+    y = tx.max_pool2(opts).into_array()
+    assert np.array_equal(y, orc.max_pool2(x, size, strides))
+    dy = to_dtype(rng.standard_normal(y.shape), dtype)
+    dx = tx.clone()
+    dx.max_pool2_backward(ag.Tensor.from_array(dy), opts)
+    assert np.array_equal(dx.into_array(), orc.max_pool2_backward(x, dy, size, strides))
+
+
+def test_max_pool2_special_values(ag):
+    nan = np.nan
+    x = np.array([[[[nan, 3, 1, nan], [4, 5, 4, 2], [-0.0, 0.0, 0.0, -0.0], [0.0, -0.0, -0.0, 0.0]]]], dtype=np.float32)
+    for dtype in ("f32", "bf16"):
+        xd = to_dtype(x, dtype)
+        opts = ag.MaxPool2Options((2, 2), (2, 2))
+        y = ag.Tensor.from_array(xd).max_pool2(opts).into_array()
+        assert np.array_equal(y.view(np.uint32 if dtype == "f32" else np.uint16),
+                              orc.max_pool2(xd, (2, 2)).view(np.uint32 if dtype == "f32" else np.uint16))
+        dy = to_dtype(np.array([[[[1.0, -0.0], [-0.0, 2.0]]]], dtype=np.float32), dtype)
+        dx = ag.Tensor.from_array(xd)
+        dx.max_pool2_backward(ag.Tensor.from_array(dy), opts)
+        got, want = dx.into_array(), orc.max_pool2_backward(xd, dy, (2, 2))
+        assert np.array_equal(got.view(np.uint32 if dtype == "f32" else np.uint16),
+                              want.view(np.uint32 if dtype == "f32" else np.uint16))
+
+
+# ----------------------------------------------------------------------- relu ----
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_relu_reference_cases(ag, dtype):
+    """relu_<T>, relu_backward_<T> (integration_tests.rs:1062-1078, :1630-1695)."""
+    for shape in [(1, 8), (15, 20)]:
+        n = shape[0] * shape[1]
+        x = to_dtype(((np.arange(n) % 20) - 10).astype(np.float32).reshape(shape), dtype)
+        assert np.array_equal(ag.Tensor.from_array(x).relu().into_array(), orc.relu(x))
+        yv = to_dtype(((np.arange(n) % 2) - 1).astype(np.float32).reshape(shape), dtype)
+        dy = to_dtype(np.arange(n, dtype=np.float32).reshape(shape), dtype)
+        got = ag.Tensor.from_array(yv).relu_backward(ag.Tensor.from_array(dy)).into_array()
+        assert np.array_equal(got, orc.relu_backward(yv, dy))
+    sp = to_dtype(np.array([[-0.0, np.nan, np.inf, -np.inf, 1e-30, -1e-30]], dtype=np.float32), dtype)
+    got = ag.Tensor.from_array(sp).relu().into_array()
+    assert np.array_equal(got.view(np.uint8), orc.relu(sp).view(np.uint8))
