@@ -27,12 +27,27 @@
 // Pipeline: global loads for k-tile t+1 are issued into registers before the MFMA loop
 // over k-tile t, and written to the other LDS stage after it; one barrier per k-tile.
 #pragma once
+#include <utility>
+
 #include "agh_internal.h"
 
 namespace agh {
 namespace gemm {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// Compile-time loop: the body is instantiated once per index, so accumulator registers are
+// only ever named by constants no matter how large the unrolled code gets (a `#pragma unroll`
+// loop that exceeds the unroller's size budget silently stays a loop, and an accumulator
+// array indexed by a loop variable is demoted to scratch memory).
+template <int... Is, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F &&f) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F &&>(f));
+}
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 enum { LD_K = 0, LD_R = 1, LD_S = 2 };
@@ -91,9 +106,12 @@ struct Loader {
                 int r = id >> 3, c = id & 7;
                 int row = min(r0 + r, NR - 1);
                 int kk = k0 + c * EPC;
+                // branch-free k tail: load a valid chunk, then zero it (K is a multiple of EPC here)
+                const bool ok = kk < kend;
+                if (!ok) kk = kend - EPC;
                 uint4 v = make_uint4(0, 0, 0, 0);
-                if ((TOTAL % NT == 0 || id < TOTAL) && kk < kend) v = *(const uint4 *)(base + (int64_t)row * rs + kk);
-                reg[i] = v;
+                if (TOTAL % NT == 0 || id < TOTAL) v = *(const uint4 *)(base + (int64_t)row * rs + kk);
+                reg[i] = ok ? v : make_uint4(0, 0, 0, 0);
             }
         } else if constexpr (MODE == LD_R) {
 #pragma unroll
@@ -106,9 +124,11 @@ struct Loader {
 #pragma unroll
                 for (int e = 0; e < EPC; ++e) {
                     int kk = k0 + kb * EPC + e;
+                    const bool ok = kk < kend;
+                    if (!ok) kk = kend - 1;
                     uint4 v = make_uint4(0, 0, 0, 0);
-                    if (live && kk < kend) v = *(const uint4 *)(base + (int64_t)kk * ks + row);
-                    reg[i * EPC + e] = v;
+                    if (live) v = *(const uint4 *)(base + (int64_t)kk * ks + row);
+                    reg[i * EPC + e] = ok ? v : make_uint4(0, 0, 0, 0);
                 }
             }
         } else {
@@ -312,58 +332,92 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     }
 
     // ------------------------------------------------------------ epilogue ----
-    const int pw0 = p0 + wp * TP * 32, qw0 = q0 + wq * TQ * 32;
+    // One loop nest per store mode, each small enough to unroll fully: the accumulators must
+    // only ever be indexed by compile-time constants or they would be demoted to scratch.
+    const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
     T *D = (T *)g.D;
     const T *bias = (const T *)g.bias;
-#pragma unroll
-    for (int i = 0; i < TP; ++i)
-#pragma unroll
-        for (int j = 0; j < TQ; ++j) {
-            const int q = qw0 + j * 32 + (int)lrow;
-            if (q >= g.NQ) continue;
-#pragma unroll
-            for (int blk = 0; blk < 4; ++blk) {
-                const int p = pw0 + i * 32 + blk * 8 + (int)lg * 4;
-                float v[4] = {acc[i][j][blk * 4 + 0], acc[i][j][blk * 4 + 1], acc[i][j][blk * 4 + 2],
-                              acc[i][j][blk * 4 + 3]};
-                if (g.store_mode == ST_SPLITK) {
-                    if (p < g.NPpad)
-                        *(float4 *)(g.ws + ((size_t)split * g.NQ + q) * g.NPpad + p) = make_float4(v[0], v[1], v[2], v[3]);
-                } else if (g.store_mode == ST_VEC) {
-                    if (p >= g.NP) continue;  // NP is a multiple of 4 on this path
-                    T *dst = D + (int64_t)q * g.dq + p;
-                    __align__(16) T old[4] = {0, 0, 0, 0};
-                    if (g.beta != 0.0f) {
-                        if constexpr (sizeof(T) == 4) *(uint4 *)old = *(const uint4 *)dst;
-                        else *(uint2 *)old = *(const uint2 *)dst;
+    const int mode = g.store_mode;
+    const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;
+    if (mode == ST_SPLITK) {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            float *wrow = g.ws + ((size_t)split * g.NQ + q) * g.NPpad;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<4>([&](auto bc) {
+                    constexpr int blk = decltype(bc)::value;
+                    const int p = pw0 + i * 32 + blk * 8;
+                    if (q < g.NQ && p < g.NPpad)
+                        *(float4 *)(wrow + p) = make_float4(acc[i][j][blk * 4 + 0], acc[i][j][blk * 4 + 1],
+                                                            acc[i][j][blk * 4 + 2], acc[i][j][blk * 4 + 3]);
+                });
+            });
+        });
+    } else if (mode == ST_VEC) {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            const bool qok = q < g.NQ;
+            T bq = 0;
+            if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
+            T *drow = D + (int64_t)q * g.dq;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<4>([&](auto bc) {
+                    constexpr int blk = decltype(bc)::value;
+                    const int p = pw0 + i * 32 + blk * 8;
+                    if (qok && p < g.NP) {  // NP is a multiple of 4 on this path
+                        T *dst = drow + p;
+                        __align__(16) T old[4] = {0, 0, 0, 0};
+                        if (g.beta != 0.0f) {
+                            if constexpr (sizeof(T) == 4) *(uint4 *)old = *(const uint4 *)dst;
+                            else *(uint2 *)old = *(const uint2 *)dst;
+                        }
+                        T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
+                        if (has_bias && bias_p) {
+                            b0 = bias[(int64_t)(p + 0) * g.bias_stride];
+                            b1 = bias[(int64_t)(p + 1) * g.bias_stride];
+                            b2 = bias[(int64_t)(p + 2) * g.bias_stride];
+                            b3 = bias[(int64_t)(p + 3) * g.bias_stride];
+                        }
+                        __align__(16) T out[4];
+                        out[0] = finish<T>(acc[i][j][blk * 4 + 0], g.alpha, g.beta, old[0], has_bias, b0, g.act);
+                        out[1] = finish<T>(acc[i][j][blk * 4 + 1], g.alpha, g.beta, old[1], has_bias, b1, g.act);
+                        out[2] = finish<T>(acc[i][j][blk * 4 + 2], g.alpha, g.beta, old[2], has_bias, b2, g.act);
+                        out[3] = finish<T>(acc[i][j][blk * 4 + 3], g.alpha, g.beta, old[3], has_bias, b3, g.act);
+                        if constexpr (sizeof(T) == 4) *(uint4 *)dst = *(const uint4 *)out;
+                        else *(uint2 *)dst = *(const uint2 *)out;
                     }
-                    T bq = 0;
-                    if (g.has_bias && !g.bias_on_p) bq = bias[(int64_t)q * g.bias_stride];
-                    __align__(16) T out[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        T bv = bq;
-                        if (g.has_bias && g.bias_on_p) bv = bias[(int64_t)(p + e) * g.bias_stride];
-                        out[e] = finish<T>(v[e], g.alpha, g.beta, old[e], g.has_bias != 0, bv, g.act);
-                    }
-                    if constexpr (sizeof(T) == 4) *(uint4 *)dst = *(const uint4 *)out;
-                    else *(uint2 *)dst = *(const uint2 *)out;
-                } else {
-                    T bq = 0;
-                    if (g.has_bias && !g.bias_on_p) bq = bias[(int64_t)q * g.bias_stride];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (p + e >= g.NP) continue;
-                        T *dst = D + (int64_t)(p + e) * g.dp + (int64_t)q * g.dq;
+                });
+            });
+        });
+    } else {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            const bool qok = q < g.NQ;
+            T bq = 0;
+            if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
+            T *drow = D + (int64_t)q * g.dq;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    const int p = pw0 + i * 32 + (r >> 2) * 8 + (r & 3);
+                    if (qok && p < g.NP) {
+                        T *dst = drow + (int64_t)p * g.dp;
                         T old = 0;
                         if (g.beta != 0.0f) old = *dst;
                         T bv = bq;
-                        if (g.has_bias && g.bias_on_p) bv = bias[(int64_t)(p + e) * g.bias_stride];
-                        *dst = finish<T>(v[e], g.alpha, g.beta, old, g.has_bias != 0, bv, g.act);
+                        if (has_bias && bias_p) bv = bias[(int64_t)p * g.bias_stride];
+                        *dst = finish<T>(acc[i][j][r], g.alpha, g.beta, old, has_bias, bv, g.act);
                     }
-                }
-            }
-        }
+                });
+            });
+        });
+    }
 }
 
 // Second pass of split-K: sum the partials in split order (deterministic), then the same
