@@ -22,6 +22,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3     # MI355X f32 matrix
 PEAK_HBM_GBS = 8000.0
+TRAFFIC_BYTES_BF16_8192 = 1.796e9  # profiles/gemm_bf16_8192_hbm_counters.md
 
 
 def log(*a):
@@ -71,6 +72,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib", action="store_true",
+                    help="also run a plain elementwise pass of known size (agh_relu_f32 over 2^28 floats: 1 GiB read, "
+                         "1 GiB written) so HBM byte counters of a profiler run can be scaled against it")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here runs across GPUs")
@@ -97,10 +101,22 @@ def main():
     achieved = flop / (dev_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": "gemm_kernel<bf16,256x256> (v_mfma_f32_32x32x16_bf16)",
                 "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/
+                # (scaled by a copy pass of known size); refreshed whenever the kernel changes
+                "traffic": TRAFFIC_BYTES_BF16_8192,
                 "algorithmic_flop_per_launch": flop, "avg_launch_ms": round(dev_ms, 4)}
     log(f"bf16 gemm 8192^3: {dev_ms:.3f} ms/launch  {achieved:.1f} TFLOP/s ({100 * achieved / PEAK_BF16_TFLOPS:.1f}% of peak)")
     del c
+
+    if args.calib:
+        ncal = 1 << 28
+        cx, cy = ag.Tensor.zeros((ncal,), "f32"), ag.Tensor.uninit((ncal,), "f32")
+        _, ms = timer.time(lambda: ag._ffi.check(ag.lib.agh_relu_f32(cx._ptr(), cy._ptr(), ncal)), 3, 1)
+        extras["calib_relu_f32_2^28"] = {"ms": round(ms, 4), "rate": round(8.0 * ncal / ms / 1e6, 1), "unit": "GB/s",
+                                         "bytes_read": 4 * ncal, "bytes_written": 4 * ncal}
+        log(f"calibration pass: {ms:.3f} ms  {8.0 * ncal / ms / 1e6:.0f} GB/s")
+        del cx, cy
 
     if not args.no_extras:
         ks, kw = max(3, args.steps // 4), 2
