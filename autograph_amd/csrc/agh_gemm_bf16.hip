@@ -1,4 +1,5 @@
 // bf16 GEMM entry points (v_mfma_f32_32x32x16_bf16, f32 accumulate, one RNE at the end).
+#define AGH_GEMM_WITH_BF16_DIRECT 1
 #include "agh_gemm_host.h"
 
 extern "C" {

@@ -1,0 +1,336 @@
+// bf16 GEMM fast path for gfx950: operand tiles go from global memory STRAIGHT into LDS
+// (global_load_lds_dwordx4, 16 bytes per lane, no VGPR staging, no ds_write), for both
+// operand layouts, and the transposition a row-contiguous operand needs is done by the
+// LDS read itself (ds_read_b64_tr_b16).  The k loop therefore contains only MFMAs, LDS
+// reads, the direct loads and one barrier.
+//
+// Same formulation as agh_gemm_kernel.h:  D[p][q] = sum_k P[p][k] * Q[q][k], 32x32x16 MFMAs,
+// accumulator element r of lane l = D[p0 + 8*(r/4) + 4*(l/32) + r%4][q0 + l%32].
+//
+// LDS tile of an operand with BR rows, k-tile of 64:
+//   LD_K (k contiguous in memory):   [row][64 k], 128-byte rows, 16-byte chunk c of row r at
+//        slot c ^ swz(r)  (the layout of agh_gemm_kernel.h); fragment = one ds_read_b128.
+//   LD_R (rows contiguous in memory): [k][BR rows], pitch 2*BR bytes.  A 32-byte group of 16
+//        rows (index m) of k-row kr sits at group slot  m ^ (kr&3) ^ ((m&1)<<2).
+//        Fragment = two ds_read_b64_tr_b16: within a 16-lane group, lanes 4j..4j+3 point at
+//        the 16 rows of k-row k0+j, and lane i receives the 4 k values of row i.  The slot
+//        function spreads the four k-rows a group touches (and the two row groups of a
+//        32-row MFMA tile) over distinct banks.
+// A direct load deposits lane L's 16 bytes at (wave-uniform LDS base) + 16*L, so the swizzles
+// are applied on the global side: each lane computes once which chunk of the tile belongs at
+// its LDS position.
+//
+// Requirements checked by the host: K (and every split's k range) a multiple of 64, operand
+// base pointers 16-byte aligned, unit stride along k (LD_K) or along rows (LD_R) with the
+// other stride a multiple of 8 elements, rows a multiple of 8 for LD_R.
+#pragma once
+#include "agh_gemm_kernel.h"
+
+namespace agh {
+namespace gemm {
+
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t rslot(uint32_t m, uint32_t kr) { return m ^ (kr & 3u) ^ ((m & 1u) << 2); }
+// inverse of rslot in m for a given kr
+__device__ __forceinline__ uint32_t rslot_inv(uint32_t ms, uint32_t kr) {
+    const uint32_t c = kr & 3u;
+    const uint32_t b0 = (ms ^ c) & 1u;
+    return ms ^ c ^ (b0 << 2);
+}
+
+// 16-byte direct load: lane L's data lands at LDS address lds_base + 16*L (lds_base is
+// wave-uniform and travels in M0).  Issued as inline assembly on purpose: the compiler's
+// wait-count pass treats an LDS-DMA it knows about as aliasing EVERY later LDS read and would
+// stall the fragment reads of the other stage until the load has landed.  Completion is
+// awaited explicitly (s_waitcnt vmcnt(0)) before the barrier that publishes the stage.
+__device__ __forceinline__ void direct_load16(const void *gptr, uint32_t lds_addr_uniform) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(lds_addr_uniform)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char *)p;
+}
+
+// Per-lane byte offsets (relative to the operand's tile origin for k-tile 0) of the NL direct
+// loads this wave issues for one operand tile.
+template <int MODE, int BR, int NWAVES>
+struct DirectLoad {
+    static constexpr int BYTES = BR * 128;
+    static constexpr int NL = BYTES / 1024 / NWAVES;  // instructions per wave per k-tile
+    static_assert(BYTES % (1024 * NWAVES) == 0, "tile must split evenly over the waves");
+    static constexpr int PITCH = BR * 2;              // LD_R: bytes per k-row
+    static constexpr int CPR = PITCH / 16;            // LD_R: 16-byte chunks per k-row
+    static constexpr int KRPI = 1024 / PITCH;         // LD_R: k-rows per instruction
+
+    static __device__ __forceinline__ void offsets(int64_t (&off)[NL], int64_t rs, int64_t ks, int r0, int NR,
+                                                   int wave, int lane) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const int inst = wave * NL + i;
+            if constexpr (MODE == LD_K) {
+                const int row = inst * 8 + (lane >> 3);
+                const int c = (lane & 7) ^ (int)swz((uint32_t)row);
+                const int rowg = min(r0 + row, NR - 1);
+                off[i] = ((int64_t)rowg * rs + c * 8) * 2;
+            } else {
+                const int kr = inst * KRPI + lane / CPR;
+                const int pc = lane % CPR;
+                const uint32_t m = rslot_inv((uint32_t)(pc >> 1), (uint32_t)kr);
+                int rowg = r0 + (int)(2 * m + (pc & 1)) * 8;
+                if (rowg >= NR) rowg = NR - 8;
+                off[i] = ((int64_t)kr * ks + rowg) * 2;
+            }
+        }
+    }
+};
+
+// Per-lane LDS byte offsets for the MFMA fragments of one operand (32-row tile index i).
+template <int MODE, int BR, int NTILE>
+struct FragRead {
+    static constexpr int PITCH = BR * 2;
+    // LD_K: off[i] as in agh_gemm_kernel.h (substep s toggles bits 5..6)
+    // LD_R: off[i] = ((8*(l/32) + j) * PITCH + 32*slot + 8*(l%4)), substep s / half h add (16s+4h)*PITCH
+    static __device__ __forceinline__ void offsets(uint32_t (&off)[NTILE], int row_base, int lane) {
+#pragma unroll
+        for (int i = 0; i < NTILE; ++i) {
+            const int rb = row_base + i * 32;
+            if constexpr (MODE == LD_K) {
+                const uint32_t lrow = lane & 31, lg = lane >> 5;
+                off[i] = (uint32_t)(rb + (int)lrow) * 128u + ((lg ^ swz(lrow)) << 4);
+            } else {
+                const uint32_t j = (lane & 15) >> 2;
+                const uint32_t m = (uint32_t)(rb >> 4) + ((lane >> 4) & 1);
+                off[i] = (8u * (lane >> 5) + j) * PITCH + 32u * rslot(m, j) + 8u * (lane & 3);
+            }
+        }
+    }
+    static __device__ __forceinline__ uint4 read(const unsigned char *tile, uint32_t off, int s) {
+        if constexpr (MODE == LD_K) {
+            return *(const uint4 *)(tile + (off ^ (uint32_t)(s << 5)));
+        } else {
+            const unsigned char *p = tile + off + s * 16 * PITCH;
+            s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3))) *)p);
+            s16x4_t hi =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3))) *)(p + 4 * PITCH));
+            uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+            return make_uint4(l2.x, l2.y, h2.x, h2.y);
+        }
+    }
+};
+
+template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
+__global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
+    typedef uint16_t T;
+    constexpr int NW = WGP * WGQ;
+    constexpr int BK = 64;
+    constexpr int TP = BP / WGP / 32, TQ = BQ / WGQ / 32;
+    constexpr int P_BYTES = BP * 128, Q_BYTES = BQ * 128, STAGE_BYTES = P_BYTES + Q_BYTES;
+    typedef DirectLoad<LP, BP, NW> DlP;
+    typedef DirectLoad<LQ, BQ, NW> DlQ;
+    typedef FragRead<LP, BP, TP> FrP;
+    typedef FragRead<LQ, BQ, TQ> FrQ;
+
+    // Two separately declared LDS stages: distinct objects, so the compiler knows a direct load
+    // into one stage cannot alias fragment reads of the other and does not wait for it.
+    __shared__ __align__(1024) unsigned char stage0[STAGE_BYTES];
+    __shared__ __align__(1024) unsigned char stage1[STAGE_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wp = wave % WGP, wq = wave / WGP;
+    int tp, tq;
+    tile_coords(blockIdx.x, g.tiles_p, g.tiles_q, tp, tq);
+    const int p0 = tp * BP, q0 = tq * BQ;
+    const int split = blockIdx.y;
+    const int kbeg = split * g.k_per_split;
+    const int kend = min(g.K, kbeg + g.k_per_split);
+    const int KT = kend > kbeg ? (kend - kbeg) / BK : 0;
+
+    // global source pointers of this lane's direct loads, advanced by one k-tile per iteration
+    int64_t offp[DlP::NL], offq[DlQ::NL];
+    DlP::offsets(offp, g.ps, g.pk, p0, g.NP, wave, lane);
+    DlQ::offsets(offq, g.qs, g.qk, q0, g.NQ, wave, lane);
+    const int64_t stepP = (int64_t)BK * g.pk * 2, stepQ = (int64_t)BK * g.qk * 2;
+    const unsigned char *gp[DlP::NL], *gq[DlQ::NL];
+#pragma unroll
+    for (int i = 0; i < DlP::NL; ++i) gp[i] = (const unsigned char *)g.P + offp[i] + (int64_t)kbeg * g.pk * 2;
+#pragma unroll
+    for (int i = 0; i < DlQ::NL; ++i) gq[i] = (const unsigned char *)g.Q + offq[i] + (int64_t)kbeg * g.qk * 2;
+
+    uint32_t fp[TP], fq[TQ];
+    FrP::offsets(fp, wp * TP * 32, lane);
+    FrQ::offsets(fq, wq * TQ * 32, lane);
+
+    f32x16 acc[TP][TQ];
+    static_for<TP>([&](auto ic) {
+        static_for<TQ>([&](auto jc) { acc[decltype(ic)::value][decltype(jc)::value] = (f32x16)(0.0f); });
+    });
+
+    auto issue_loads = [&](unsigned char *stage) {
+        const uint32_t sp = __builtin_amdgcn_readfirstlane(lds_address(stage) + wave * DlP::NL * 1024);
+        const uint32_t sq = __builtin_amdgcn_readfirstlane(lds_address(stage) + P_BYTES + wave * DlQ::NL * 1024);
+#pragma unroll
+        for (int i = 0; i < DlP::NL; ++i) {
+            direct_load16(gp[i], sp + i * 1024);
+            gp[i] += stepP;
+        }
+#pragma unroll
+        for (int i = 0; i < DlQ::NL; ++i) {
+            direct_load16(gq[i], sq + i * 1024);
+            gq[i] += stepQ;
+        }
+    };
+
+    // two fragment sets, named separately so every register index is a compile-time constant
+    uint4 pfa[TP], qfa[TQ], pfb[TP], qfb[TQ];
+    auto read_frags = [&](uint4 (&pf)[TP], uint4 (&qf)[TQ], const unsigned char *stage, auto sc) {
+        constexpr int s = decltype(sc)::value;
+        const unsigned char *sp = stage;
+        const unsigned char *sq = stage + P_BYTES;
+        static_for<TP>([&](auto ic) { pf[decltype(ic)::value] = FrP::read(sp, fp[decltype(ic)::value], s); });
+        static_for<TQ>([&](auto jc) { qf[decltype(jc)::value] = FrQ::read(sq, fq[decltype(jc)::value], s); });
+    };
+    auto mma = [&](const uint4 (&pf)[TP], const uint4 (&qf)[TQ]) {
+        static_for<TP>([&](auto ic) {
+            static_for<TQ>([&](auto jc) {
+                constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
+                Mma<T>::run(acc[i][j], pf[i], qf[j]);
+            });
+        });
+    };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
+
+    // One k-tile: multiply the tile in `cur` while the next one streams into `nxt`.
+    auto step = [&](unsigned char *cur, unsigned char *nxt, bool more) {
+        // sched_barrier(0) pins the phase order: each batch of LDS reads is issued one MFMA
+        // batch (16 MFMAs, ~512 cycles) before its first use
+        if (more) issue_loads(nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(pfb, qfb, cur, S1{});
+        __builtin_amdgcn_sched_barrier(0);
+        mma(pfa, qfa);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(pfa, qfa, cur, S2{});
+        __builtin_amdgcn_sched_barrier(0);
+        mma(pfb, qfb);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(pfb, qfb, cur, S3{});
+        __builtin_amdgcn_sched_barrier(0);
+        mma(pfa, qfa);
+        __builtin_amdgcn_sched_barrier(0);
+        // every wave has issued its last reads of `cur`; the next tile must have landed
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (more) read_frags(pfa, qfa, nxt, S0{});  // first fragments of the next tile, under the last MFMAs
+        __builtin_amdgcn_sched_barrier(0);
+        mma(pfb, qfb);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    if (KT > 0) {
+        issue_loads(stage0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        read_frags(pfa, qfa, stage0, S0{});
+    }
+    int kt = 0;
+    for (; kt + 2 <= KT; kt += 2) {
+        step(stage0, stage1, true);
+        step(stage1, stage0, kt + 2 < KT);
+    }
+    if (kt < KT) step(stage0, stage1, false);
+
+    // ------------------------------------------------------------ epilogue ----
+    const uint32_t lrow = lane & 31, lg = lane >> 5;
+    const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
+    T *D = (T *)g.D;
+    const T *bias = (const T *)g.bias;
+    const int mode = g.store_mode;
+    const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;
+    if (mode == ST_SPLITK) {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            float *wrow = g.ws + ((size_t)split * g.NQ + q) * g.NPpad;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<4>([&](auto bc) {
+                    constexpr int blk = decltype(bc)::value;
+                    const int p = pw0 + i * 32 + blk * 8;
+                    if (q < g.NQ && p < g.NPpad)
+                        *(float4 *)(wrow + p) = make_float4(acc[i][j][blk * 4 + 0], acc[i][j][blk * 4 + 1],
+                                                            acc[i][j][blk * 4 + 2], acc[i][j][blk * 4 + 3]);
+                });
+            });
+        });
+    } else if (mode == ST_VEC) {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            const bool qok = q < g.NQ;
+            T bq = 0;
+            if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
+            T *drow = D + (int64_t)q * g.dq;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<4>([&](auto bc) {
+                    constexpr int blk = decltype(bc)::value;
+                    const int p = pw0 + i * 32 + blk * 8;
+                    if (qok && p < g.NP) {
+                        T *dst = drow + p;
+                        __align__(8) T old[4] = {0, 0, 0, 0};
+                        if (g.beta != 0.0f) *(uint2 *)old = *(const uint2 *)dst;
+                        T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
+                        if (has_bias && bias_p) {
+                            b0 = bias[(int64_t)(p + 0) * g.bias_stride];
+                            b1 = bias[(int64_t)(p + 1) * g.bias_stride];
+                            b2 = bias[(int64_t)(p + 2) * g.bias_stride];
+                            b3 = bias[(int64_t)(p + 3) * g.bias_stride];
+                        }
+                        __align__(8) T out[4];
+                        out[0] = finish<T>(acc[i][j][blk * 4 + 0], g.alpha, g.beta, old[0], has_bias, b0, g.act);
+                        out[1] = finish<T>(acc[i][j][blk * 4 + 1], g.alpha, g.beta, old[1], has_bias, b1, g.act);
+                        out[2] = finish<T>(acc[i][j][blk * 4 + 2], g.alpha, g.beta, old[2], has_bias, b2, g.act);
+                        out[3] = finish<T>(acc[i][j][blk * 4 + 3], g.alpha, g.beta, old[3], has_bias, b3, g.act);
+                        *(uint2 *)dst = *(const uint2 *)out;
+                    }
+                });
+            });
+        });
+    } else {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            const bool qok = q < g.NQ;
+            T bq = 0;
+            if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
+            T *drow = D + (int64_t)q * g.dq;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    const int p = pw0 + i * 32 + (r >> 2) * 8 + (r & 3);
+                    if (qok && p < g.NP) {
+                        T *dst = drow + (int64_t)p * g.dp;
+                        T old = 0;
+                        if (g.beta != 0.0f) old = *dst;
+                        T bv = bq;
+                        if (has_bias && bias_p) bv = bias[(int64_t)p * g.bias_stride];
+                        *dst = finish<T>(acc[i][j][r], g.alpha, g.beta, old, has_bias, bv, g.act);
+                    }
+                });
+            });
+        });
+    }
+}
+
+}  // namespace gemm
+}  // namespace agh

@@ -1,10 +1,16 @@
-#include <stdlib.h>
-#include <string.h>
 // Host side of the GEMM entry points: argument checks (the reference's bail!s at
 // src/tensor/linalg.rs:256-279), orientation / loader / tile selection, split-K planning
 // (the job of linalg.rs:306-340) and the launches.  Included once per element type.
 #pragma once
+#include <stdlib.h>
+#include <string.h>
+
+#include <type_traits>
+
 #include "agh_gemm_kernel.h"
+#ifdef AGH_GEMM_WITH_BF16_DIRECT
+#include "agh_gemm_bf16_dl.h"
+#endif
 
 namespace agh {
 namespace gemm {
@@ -44,8 +50,32 @@ int launch_one(const Args &g, int splits) {
     return AGH_OK;
 }
 
+#ifdef AGH_GEMM_WITH_BF16_DIRECT
+template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
+int launch_one_dl(const Args &g, int splits) {
+    auto kern = gemm_bf16_dl_kernel<BP, BQ, WGP, WGQ, LP, LQ>;  // both LDS stages are static
+    dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits);
+    hipLaunchKernelGGL(kern, grid, dim3(WGP * WGQ * 64), 0, stream(), g);
+    AGH_LAUNCH_CHECK("gemm (direct-to-LDS) kernel launch");
+    return AGH_OK;
+}
+#endif
+
 template <typename T, int BP, int BQ, int WGP, int WGQ, bool SCALAR_OK>
-int launch_loaders(const Args &g, int splits, int lp, int lq) {
+int launch_loaders(const Args &g, int splits, int lp, int lq, bool direct) {
+#ifdef AGH_GEMM_WITH_BF16_DIRECT
+    if constexpr (std::is_same<T, uint16_t>::value && !SCALAR_OK) {
+        if (direct) {
+            switch (lp * 3 + lq) {
+                case LD_K * 3 + LD_K: return launch_one_dl<BP, BQ, WGP, WGQ, LD_K, LD_K>(g, splits);
+                case LD_K * 3 + LD_R: return launch_one_dl<BP, BQ, WGP, WGQ, LD_K, LD_R>(g, splits);
+                case LD_R * 3 + LD_K: return launch_one_dl<BP, BQ, WGP, WGQ, LD_R, LD_K>(g, splits);
+                case LD_R * 3 + LD_R: return launch_one_dl<BP, BQ, WGP, WGQ, LD_R, LD_R>(g, splits);
+                default: break;
+            }
+        }
+    }
+#endif
     switch (lp * 3 + lq) {
         case LD_K * 3 + LD_K: return launch_one<T, BP, BQ, WGP, WGQ, LD_K, LD_K>(g, splits);
         case LD_K * 3 + LD_R: return launch_one<T, BP, BQ, WGP, WGQ, LD_K, LD_R>(g, splits);
@@ -67,15 +97,15 @@ int launch_loaders(const Args &g, int splits, int lp, int lq) {
 }
 
 template <typename T>
-int launch_cfg(int cfg, const Args &g, int splits, int lp, int lq) {
+int launch_cfg(int cfg, const Args &g, int splits, int lp, int lq, bool direct) {
     switch (cfg) {
-        case 0: return launch_loaders<T, 256, 256, 2, 2, false>(g, splits, lp, lq);
-        case 1: return launch_loaders<T, 128, 256, 2, 2, false>(g, splits, lp, lq);
-        case 2: return launch_loaders<T, 256, 128, 2, 2, false>(g, splits, lp, lq);
-        case 3: return launch_loaders<T, 128, 128, 2, 2, false>(g, splits, lp, lq);
-        case 4: return launch_loaders<T, 64, 64, 2, 2, true>(g, splits, lp, lq);
-        case 5: return launch_loaders<T, 32, 128, 1, 4, true>(g, splits, lp, lq);
-        case 6: return launch_loaders<T, 128, 32, 4, 1, true>(g, splits, lp, lq);
+        case 0: return launch_loaders<T, 256, 256, 2, 2, false>(g, splits, lp, lq, direct);
+        case 1: return launch_loaders<T, 128, 256, 2, 2, false>(g, splits, lp, lq, direct);
+        case 2: return launch_loaders<T, 256, 128, 2, 2, false>(g, splits, lp, lq, direct);
+        case 3: return launch_loaders<T, 128, 128, 2, 2, false>(g, splits, lp, lq, direct);
+        case 4: return launch_loaders<T, 64, 64, 2, 2, true>(g, splits, lp, lq, false);
+        case 5: return launch_loaders<T, 32, 128, 1, 4, true>(g, splits, lp, lq, false);
+        case 6: return launch_loaders<T, 128, 32, 4, 1, true>(g, splits, lp, lq, false);
         default: return fail(AGH_EINVAL, "gemm: bad tile config %d", cfg);
     }
 }
@@ -190,13 +220,17 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     splits = ktiles > 0 ? (ktiles + tiles_per_split - 1) / tiles_per_split : 1;
     g.k_per_split = tiles_per_split * BK;
 
+    // bf16 with both operands vector-loadable and k a multiple of the 64-wide k-tile takes the
+    // direct-to-LDS kernel (AGH_GEMM_DIRECT=0 forces the register-staged one)
+    const bool direct = sizeof(T) == 2 && !any_scalar && g.K > 0 && g.K % 64 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0;
+
     if (splits > 1) {
         void *ws = nullptr;
         const size_t bytes = (size_t)splits * g.NQ * g.NPpad * sizeof(float);
         if (int rc = workspace(bytes, &ws)) return rc;
         g.ws = (float *)ws;
         g.store_mode = ST_SPLITK;
-        if (int rc = launch_cfg<T>(best, g, splits, lp, lq)) return rc;
+        if (int rc = launch_cfg<T>(best, g, splits, lp, lq, direct)) return rc;
         const size_t total = (size_t)g.NQ * g.NP;
         const size_t blocks = (total + 255) / 256;
         if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: output too large for split-K", name);
@@ -205,7 +239,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         return AGH_OK;
     }
     g.store_mode = vec_store ? ST_VEC : ST_SCALAR;
-    return launch_cfg<T>(best, g, 1, lp, lq);
+    return launch_cfg<T>(best, g, 1, lp, lq, direct);
 }
 
 }  // namespace gemm
