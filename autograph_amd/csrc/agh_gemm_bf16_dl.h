@@ -170,83 +170,100 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
         static_for<TQ>([&](auto jc) { acc[decltype(ic)::value][decltype(jc)::value] = (f32x16)(0.0f); });
     });
 
-    auto issue_loads = [&](unsigned char *stage) {
-        const uint32_t sp = __builtin_amdgcn_readfirstlane(lds_address(stage) + wave * DlP::NL * 1024);
-        const uint32_t sq = __builtin_amdgcn_readfirstlane(lds_address(stage) + P_BYTES + wave * DlQ::NL * 1024);
-#pragma unroll
-        for (int i = 0; i < DlP::NL; ++i) {
-            direct_load16(gp[i], sp + i * 1024);
-            gp[i] += stepP;
-        }
-#pragma unroll
-        for (int i = 0; i < DlQ::NL; ++i) {
-            direct_load16(gq[i], sq + i * 1024);
-            gq[i] += stepQ;
+    // ---- direct loads: NLT per wave per k-tile (P's first, then Q's), issued one at a time ----
+    constexpr int NLP = DlP::NL, NLQ = DlQ::NL, NLT = NLP + NLQ;
+    // `adv_p` / `adv_q` is the k-tile step, or 0 once the pointer is at the last k-tile (so a
+    // load issued past the end re-reads the last tile into a free stage instead of leaving the
+    // matrix; keeping the loads unconditional keeps the MFMA stream free of branches)
+    auto issue_load = [&](uint32_t stage_addr, auto lc, int64_t adv_p, int64_t adv_q) {
+        constexpr int l = decltype(lc)::value;
+        if constexpr (l < NLP) {
+            direct_load16(gp[l], stage_addr + (wave * NLP + l) * 1024);
+            gp[l] += adv_p;
+        } else {
+            direct_load16(gq[l - NLP], stage_addr + P_BYTES + (wave * NLQ + (l - NLP)) * 1024);
+            gq[l - NLP] += adv_q;
         }
     };
 
+    // ---- fragment reads: TP + TQ units per substep, in the order the MFMAs first need them ----
     // two fragment sets, named separately so every register index is a compile-time constant
     uint4 pfa[TP], qfa[TQ], pfb[TP], qfb[TQ];
-    auto read_frags = [&](uint4 (&pf)[TP], uint4 (&qf)[TQ], const unsigned char *stage, auto sc) {
-        constexpr int s = decltype(sc)::value;
-        const unsigned char *sp = stage;
-        const unsigned char *sq = stage + P_BYTES;
-        static_for<TP>([&](auto ic) { pf[decltype(ic)::value] = FrP::read(sp, fp[decltype(ic)::value], s); });
-        static_for<TQ>([&](auto jc) { qf[decltype(jc)::value] = FrQ::read(sq, fq[decltype(jc)::value], s); });
+    constexpr int NU = TP + TQ;
+    auto read_unit = [&](uint4 (&pf)[TP], uint4 (&qf)[TQ], const unsigned char *stage, auto sc, auto uc) {
+        constexpr int s = decltype(sc)::value, u = decltype(uc)::value;
+        // unit order: P0, Q0, Q1, ..., Q(TQ-1), P1, ..., P(TP-1)
+        if constexpr (u == 0) pf[0] = FrP::read(stage, fp[0], s);
+        else if constexpr (u <= TQ) qf[u - 1] = FrQ::read(stage + P_BYTES, fq[u - 1], s);
+        else pf[u - TQ] = FrP::read(stage, fp[u - TQ], s);
     };
-    auto mma = [&](const uint4 (&pf)[TP], const uint4 (&qf)[TQ]) {
-        static_for<TP>([&](auto ic) {
-            static_for<TQ>([&](auto jc) {
-                constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
-                Mma<T>::run(acc[i][j], pf[i], qf[j]);
+
+    // ---- one phase: TP*TQ MFMAs on fragment set X; after MFMA number n the phase issues read
+    // unit n of fragment set Y (if READ) and its share of the direct loads
+    // [L0, L1), spread evenly over the MFMAs.  sched_barrier(0) after each MFMA pins this interleaving: the matrix pipe is
+    // handed a new MFMA every 32 cycles while LDS reads and global loads trickle out between.
+    constexpr int NM = TP * TQ;
+    auto phase = [&](const uint4 (&xp)[TP], const uint4 (&xq)[TQ], uint4 (&yp)[TP], uint4 (&yq)[TQ], auto readc,
+                     const unsigned char *rstage, auto sc, uint32_t lstage_addr, auto l0c, auto l1c, int64_t adv_p,
+                     int64_t adv_q) {
+        constexpr bool READ = decltype(readc)::value;
+        constexpr int L0 = decltype(l0c)::value, L1 = decltype(l1c)::value, NLD = L1 - L0;
+        static_for<NM>([&](auto nc) {
+            constexpr int n = decltype(nc)::value, i = n / TQ, j = n % TQ;
+            Mma<T>::run(acc[i][j], xp[i], xq[j]);
+            if constexpr (READ && n < NU) read_unit(yp, yq, rstage, sc, nc);
+            // loads [n*NLD/NM, (n+1)*NLD/NM) of this phase's share go out after MFMA n
+            constexpr int LA = n * NLD / NM, LB = (n + 1) * NLD / NM;
+            static_for<LB - LA>([&](auto tc) {
+                issue_load(lstage_addr, std::integral_constant<int, L0 + LA + decltype(tc)::value>{}, adv_p, adv_q);
             });
+            __builtin_amdgcn_sched_barrier(0);
         });
     };
     using S0 = std::integral_constant<int, 0>;
     using S1 = std::integral_constant<int, 1>;
     using S2 = std::integral_constant<int, 2>;
     using S3 = std::integral_constant<int, 3>;
+    using Yes = std::true_type;
+    using No = std::false_type;
+    using L_0 = std::integral_constant<int, 0>;
+    using L_T = std::integral_constant<int, NLT>;
 
-    // One k-tile: multiply the tile in `cur` while the next one streams into `nxt`.
-    auto step = [&](unsigned char *cur, unsigned char *nxt, bool more) {
-        // sched_barrier(0) pins the phase order: each batch of LDS reads is issued one MFMA
-        // batch (16 MFMAs, ~512 cycles) before its first use
-        if (more) issue_loads(nxt);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(pfb, qfb, cur, S1{});
-        __builtin_amdgcn_sched_barrier(0);
-        mma(pfa, qfa);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(pfa, qfa, cur, S2{});
-        __builtin_amdgcn_sched_barrier(0);
-        mma(pfb, qfb);
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(pfb, qfb, cur, S3{});
-        __builtin_amdgcn_sched_barrier(0);
-        mma(pfa, qfa);
-        __builtin_amdgcn_sched_barrier(0);
-        // every wave has issued its last reads of `cur`; the next tile must have landed
+    // One k-tile.  On entry: tile kt is visible in `cur`, its substep-0 fragments are in set A,
+    // and the loads of tile kt+1 into `nxt` are in flight (issued during the previous tile's
+    // last phase).  The barrier sits between phase 2 and phase 3: by then every wave has issued
+    // (and waited for) its last reads of `cur`, so `cur` can be refilled with tile kt+2 while
+    // phase 3 multiplies out of registers.  `adv` says whether a tile kt+3 exists.
+    auto step = [&](unsigned char *cur, unsigned char *nxt, bool adv) {
+        phase(pfa, qfa, pfb, qfb, Yes{}, cur, S1{}, 0u, L_0{}, L_0{}, 0, 0);
+        phase(pfb, qfb, pfa, qfa, Yes{}, cur, S2{}, 0u, L_0{}, L_0{}, 0, 0);
+        phase(pfa, qfa, pfb, qfb, Yes{}, cur, S3{}, 0u, L_0{}, L_0{}, 0, 0);
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (more) read_frags(pfa, qfa, nxt, S0{});  // first fragments of the next tile, under the last MFMAs
         __builtin_amdgcn_sched_barrier(0);
-        mma(pfb, qfb);
-        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t cur_addr = __builtin_amdgcn_readfirstlane(lds_address(cur));
+        phase(pfb, qfb, pfa, qfa, Yes{}, nxt, S0{}, cur_addr, L_0{}, L_T{}, adv ? stepP : 0, adv ? stepQ : 0);
     };
 
     if (KT > 0) {
-        issue_loads(stage0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const uint32_t a0 = __builtin_amdgcn_readfirstlane(lds_address(stage0));
+        const uint32_t a1 = __builtin_amdgcn_readfirstlane(lds_address(stage1));
+        // tile 0 -> stage0, tile min(1, KT-1) -> stage1
+        static_for<NLT>([&](auto lc) { issue_load(a0, lc, KT > 1 ? stepP : 0, KT > 1 ? stepQ : 0); });
+        static_for<NLT>([&](auto lc) { issue_load(a1, lc, KT > 2 ? stepP : 0, KT > 2 ? stepQ : 0); });
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLT) : "memory");  // tile 0 has landed
         __syncthreads();
-        read_frags(pfa, qfa, stage0, S0{});
+        static_for<NU>([&](auto uc) { read_unit(pfa, qfa, stage0, S0{}, uc); });
     }
     int kt = 0;
     for (; kt + 2 <= KT; kt += 2) {
-        step(stage0, stage1, true);
-        step(stage1, stage0, kt + 2 < KT);
+        step(stage0, stage1, kt + 3 < KT);
+        step(stage1, stage0, kt + 4 < KT);
     }
     if (kt < KT) step(stage0, stage1, false);
+    // the last phase may have re-issued loads into a free stage: let them land before LDS is reused
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ------------------------------------------------------------ epilogue ----
     const uint32_t lrow = lane & 31, lg = lane >> 5;

@@ -174,6 +174,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     g.bias_stride = bias_stride;
     g.act = act;
     g.NPpad = (g.NP + 3) & ~3;
+    g.dbg = env_int("AGH_GEMM_DBG", 0);
 
     int lp = k > 0 ? pick_loader<T>(g.P, g.ps, g.pk, g.NP, g.K) : LD_S;
     int lq = k > 0 ? pick_loader<T>(g.Q, g.qs, g.qk, g.NQ, g.K) : LD_S;

@@ -66,6 +66,7 @@ struct Args {
     float alpha, beta;
     int bias_on_p, has_bias, act;
     int store_mode;
+    int dbg;  // timing experiments only (AGH_GEMM_DBG): 1 = skip global loads, 2 = skip LDS fragment reads, 4 = skip MFMAs
 };
 
 template <typename T> struct Geo;
