@@ -240,6 +240,11 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         return AGH_OK;
     }
     g.store_mode = vec_store ? ST_VEC : ST_SCALAR;
+    // the direct-to-LDS kernel can transpose its output tile through LDS and store full 16-byte
+    // chunks when nothing has to be read back from C
+    if (direct && best <= 3 && vec_store && beta == 0.0f && g.NP % 8 == 0 && (g.dq % 8 == 0 || g.NQ == 1) &&
+        aligned(C, 16))
+        g.store_mode = ST_STAGED;
     return launch_cfg<T>(best, g, 1, lp, lq, direct);
 }
 

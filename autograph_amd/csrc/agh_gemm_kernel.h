@@ -51,7 +51,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 enum { LD_K = 0, LD_R = 1, LD_S = 2 };
-enum { ST_SCALAR = 0, ST_VEC = 1, ST_SPLITK = 2 };
+enum { ST_SCALAR = 0, ST_VEC = 1, ST_SPLITK = 2, ST_STAGED = 3 };  // ST_STAGED: direct-to-LDS bf16 kernel only
 
 struct Args {
     const void *P;
@@ -79,12 +79,19 @@ __device__ __forceinline__ uint32_t lds_off(uint32_t r, uint32_t c) { return r *
 // ---- epilogue arithmetic in the order the reference's separate ops round ----
 template <typename T>
 __device__ __forceinline__ T finish(float acc, float alpha, float beta, T cold, bool has_bias, T bias, int act) {
-    float v = alpha * acc;
-    if (beta != 0.0f) v = v + beta * Elem<T>::to_f32(cold);
-    T r = Elem<T>::from_f32(v);
-    if (has_bias) r = Elem<T>::from_f32(Elem<T>::to_f32(bias) + Elem<T>::to_f32(r));
-    if (act == AGH_ACT_RELU) r = (Elem<T>::to_f32(r) >= 0.0f) ? r : Elem<T>::zero();
-    return r;
+    // selects only: a branch per output element would dominate the epilogue
+    const float v0 = alpha * acc;
+    const float v1 = v0 + beta * Elem<T>::to_f32(cold);
+    T r = Elem<T>::from_f32(beta != 0.0f ? v1 : v0);  // beta == 0 never uses C (and keeps the sign of a zero)
+    const T rb = Elem<T>::from_f32(Elem<T>::to_f32(bias) + Elem<T>::to_f32(r));
+    r = has_bias ? rb : r;
+    const bool neg = !(Elem<T>::to_f32(r) >= 0.0f);
+    return (act == AGH_ACT_RELU && neg) ? Elem<T>::zero() : r;
+}
+// alpha only (no C, no bias, no activation): the plain `dot` epilogue
+template <typename T>
+__device__ __forceinline__ T finish_plain(float acc, float alpha) {
+    return Elem<T>::from_f32(alpha * acc);
 }
 
 // ---- global -> register loaders (one operand tile of BR rows x 8 chunks) ----

@@ -62,17 +62,19 @@ struct FastDiv {
 };
 
 // ---- bf16 <-> f32 exactly as the `half` crate does it (the reference's bf16 type) ----
+// (written with selects, not branches: these sit in GEMM epilogues and per-element loops)
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
-    uint32_t x = (uint32_t)h << 16;
-    if ((h & 0x7FFFu) > 0x7F80u) x |= 0x00400000u;  // NaN: set the quiet bit
-    return __uint_as_float(x);
+    const uint32_t x = (uint32_t)h << 16;
+    const bool nan = (h & 0x7FFFu) > 0x7F80u;
+    return __uint_as_float(nan ? (x | 0x00400000u) : x);  // NaN: set the quiet bit
 }
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-    uint32_t x = __float_as_uint(f);
-    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
-    // round to nearest even: up iff the round bit is set and (sticky or lsb) is set
-    uint32_t up = ((x & 0x00008000u) != 0 && (x & 0x00017FFFu) != 0) ? 1u : 0u;
-    return (uint16_t)((x >> 16) + up);
+    const uint32_t x = __float_as_uint(f);
+    // round to nearest even on bit 16: adding 0x7FFF + lsb carries exactly when the discarded
+    // half is above 0x8000, or equal to it with an odd kept part
+    const uint32_t rne = (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;
+    const bool nan = (x & 0x7FFFFFFFu) > 0x7F800000u;
+    return (uint16_t)(nan ? ((x >> 16) | 0x0040u) : rne);
 }
 
 template <typename T> struct Elem;
