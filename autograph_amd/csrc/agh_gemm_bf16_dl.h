@@ -148,7 +148,7 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     const int split = blockIdx.y;
     const int kbeg = split * g.k_per_split;
     const int kend = min(g.K, kbeg + g.k_per_split);
-    const int KT = (g.dbg & 16) ? 0 : (kend > kbeg ? (kend - kbeg) / BK : 0);
+    const int KT = kend > kbeg ? (kend - kbeg) / BK : 0;
 
     // global source pointers of this lane's direct loads, advanced by one k-tile per iteration
     int64_t offp[DlP::NL], offq[DlQ::NL];
@@ -272,11 +272,9 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
     T *D = (T *)g.D;
     const T *bias = (const T *)g.bias;
-    const int mode = (g.dbg & 8) ? 99 : g.store_mode;
+    const int mode = g.store_mode;
     const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;
-    if (mode == 99) {
-        if (acc[0][0][0] == 12345.678f) D[0] = 1;  // timing experiment: no stores
-    } else if (mode == ST_STAGED) {
+    if (mode == ST_STAGED) {
         // beta == 0, D rows 16-byte aligned, NP a multiple of 8.  A lane holds 4 consecutive p of
         // ONE q row, and the 32 lanes of a half-wave hold 32 different q rows, so storing straight
         // from the accumulators writes 8 bytes into each of 64 different cache lines per
@@ -288,51 +286,59 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
         constexpr int NST = 32 / RPI;                  // store instructions per pass
         static_assert(4 * 32 * EPITCH <= STAGE_BYTES, "epilogue staging must fit in one LDS stage");
         unsigned char *region = stage0 + wave * 32 * EPITCH;
-        const bool plain = !has_bias && g.act == AGH_ACT_NONE;
         const int pwb = p0 + wp * TP * 32, qwb = q0 + wq * TQ * 32;
-        static_for<TQ>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const int q = qwb + j * 32 + (int)lrow;
-            T bq = 0;
-            if (q < g.NQ && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
-            static_for<TP>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<4>([&](auto bc) {
-                    constexpr int blk = decltype(bc)::value;
-                    const int pl = i * 32 + blk * 8 + (int)lg * 4;  // p inside the wave tile
-                    T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
-                    if (has_bias && bias_p) {
-                        const int p = min(pwb + pl, g.NP - 4);
-                        b0 = bias[(int64_t)(p + 0) * g.bias_stride];
-                        b1 = bias[(int64_t)(p + 1) * g.bias_stride];
-                        b2 = bias[(int64_t)(p + 2) * g.bias_stride];
-                        b3 = bias[(int64_t)(p + 3) * g.bias_stride];
-                    }
-                    T o0, o1, o2, o3;
-                    if (plain) {
-                        o0 = finish_plain<T>(acc[i][j][blk * 4 + 0], g.alpha);
-                        o1 = finish_plain<T>(acc[i][j][blk * 4 + 1], g.alpha);
-                        o2 = finish_plain<T>(acc[i][j][blk * 4 + 2], g.alpha);
-                        o3 = finish_plain<T>(acc[i][j][blk * 4 + 3], g.alpha);
-                    } else {
-                        o0 = finish<T>(acc[i][j][blk * 4 + 0], g.alpha, 0.0f, (T)0, has_bias, b0, g.act);
-                        o1 = finish<T>(acc[i][j][blk * 4 + 1], g.alpha, 0.0f, (T)0, has_bias, b1, g.act);
-                        o2 = finish<T>(acc[i][j][blk * 4 + 2], g.alpha, 0.0f, (T)0, has_bias, b2, g.act);
-                        o3 = finish<T>(acc[i][j][blk * 4 + 3], g.alpha, 0.0f, (T)0, has_bias, b3, g.act);
-                    }
-                    *(uint2 *)(region + lrow * EPITCH + pl * 2) =
-                        make_uint2((uint32_t)o0 | ((uint32_t)o1 << 16), (uint32_t)o2 | ((uint32_t)o3 << 16));
+        // two fully separate instantiations (plain `dot` / bias+activation) so that the plain one
+        // carries no bias or activation state through its unrolled body
+        auto staged = [&](auto plainc) {
+            constexpr bool PLAIN = decltype(plainc)::value;
+            static_for<TQ>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                T bq = 0;
+                if constexpr (!PLAIN) {
+                    const int q = qwb + j * 32 + (int)lrow;
+                    if (q < g.NQ && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
+                }
+                static_for<TP>([&](auto ic) {
+                    constexpr int i = decltype(ic)::value;
+                    static_for<4>([&](auto bc) {
+                        constexpr int blk = decltype(bc)::value;
+                        const int pl = i * 32 + blk * 8 + (int)lg * 4;  // p inside the wave tile
+                        T o0, o1, o2, o3;
+                        if constexpr (PLAIN) {
+                            o0 = finish_plain<T>(acc[i][j][blk * 4 + 0], g.alpha);
+                            o1 = finish_plain<T>(acc[i][j][blk * 4 + 1], g.alpha);
+                            o2 = finish_plain<T>(acc[i][j][blk * 4 + 2], g.alpha);
+                            o3 = finish_plain<T>(acc[i][j][blk * 4 + 3], g.alpha);
+                        } else {
+                            T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
+                            if (has_bias && bias_p) {
+                                const int p = min(pwb + pl, g.NP - 4);
+                                b0 = bias[(int64_t)(p + 0) * g.bias_stride];
+                                b1 = bias[(int64_t)(p + 1) * g.bias_stride];
+                                b2 = bias[(int64_t)(p + 2) * g.bias_stride];
+                                b3 = bias[(int64_t)(p + 3) * g.bias_stride];
+                            }
+                            o0 = finish<T>(acc[i][j][blk * 4 + 0], g.alpha, 0.0f, (T)0, has_bias, b0, g.act);
+                            o1 = finish<T>(acc[i][j][blk * 4 + 1], g.alpha, 0.0f, (T)0, has_bias, b1, g.act);
+                            o2 = finish<T>(acc[i][j][blk * 4 + 2], g.alpha, 0.0f, (T)0, has_bias, b2, g.act);
+                            o3 = finish<T>(acc[i][j][blk * 4 + 3], g.alpha, 0.0f, (T)0, has_bias, b3, g.act);
+                        }
+                        *(uint2 *)(region + lrow * EPITCH + pl * 2) =
+                            make_uint2((uint32_t)o0 | ((uint32_t)o1 << 16), (uint32_t)o2 | ((uint32_t)o3 << 16));
+                    });
+                });
+                // same wave, LDS executes in order: the reads below see the writes above
+                static_for<NST>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    const int row = r * RPI + lane / CPRW, chunk = lane % CPRW;
+                    const uint4 v = *(const uint4 *)(region + row * EPITCH + chunk * 16);
+                    const int qq = qwb + j * 32 + row, pp = pwb + chunk * 8;
+                    if (qq < g.NQ && pp < g.NP) *(uint4 *)(D + (int64_t)qq * g.dq + pp) = v;
                 });
             });
-            // same wave, LDS executes in order: the reads below see the writes above
-            static_for<NST>([&](auto rc) {
-                constexpr int r = decltype(rc)::value;
-                const int row = r * RPI + lane / CPRW, chunk = lane % CPRW;
-                const uint4 v = *(const uint4 *)(region + row * EPITCH + chunk * 16);
-                const int qq = qwb + j * 32 + row, pp = pwb + chunk * 8;
-                if (qq < g.NQ && pp < g.NP && (!(g.dbg & 32) || v.x == 0x12345678u)) *(uint4 *)(D + (int64_t)qq * g.dq + pp) = v;
-            });
-        });
+        };
+        if (!has_bias && g.act == AGH_ACT_NONE) staged(std::true_type{});
+        else staged(std::false_type{});
     } else if (mode == ST_SPLITK) {
         static_for<TQ>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
