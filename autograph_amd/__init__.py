@@ -4,6 +4,16 @@ The package is a thin host layer over libautograph_hip.so; importing it fails lo
 the library has not been built.
 """
 from ._ffi import LIB_PATH, AghError, lib  # noqa: F401
+from .layer import (  # noqa: F401
+    Conv2,
+    Dense,
+    Flatten,
+    LeNet5,
+    MaxPool2,
+    Relu,
+    conv2_direct_forward,
+    conv2_im2col_forward,
+)
 from .tensor import (  # noqa: F401
     BF16,
     F32,

@@ -21,6 +21,8 @@ ptr = C.c_void_p
 f32 = C.c_float
 
 _GEMM = [i64, i64, i64, f32, ptr, i64, i64, i64, ptr, i64, i64, i64, f32, ptr, i64, i64, i64]
+_GEMM_B = [i64, i64, i64, i64, f32, ptr, i64, i64, i64, i64, ptr, i64, i64, i64, i64, f32, ptr, i64, i64, i64, i64,
+           ptr, i64, i64, C.c_int]
 _CONV = [ptr, ptr] + [i64] * 12
 _POOL = [ptr, ptr] + [i64] * 7
 
@@ -34,6 +36,13 @@ SIGNATURES = {
     "agh_memcpy_h2d": ([ptr, ptr, C.c_size_t], C.c_int),
     "agh_memcpy_d2h": ([ptr, ptr, C.c_size_t], C.c_int),
     "agh_memcpy_d2d": ([ptr, ptr, C.c_size_t], C.c_int),
+    "agh_memcpy_d2h_async": ([ptr, ptr, C.c_size_t], C.c_int),
+    "agh_host_alloc": ([C.POINTER(ptr), C.c_size_t], C.c_int),
+    "agh_host_free": ([ptr], C.c_int),
+    "agh_graph_begin": ([], C.c_int),
+    "agh_graph_end": ([C.POINTER(ptr)], C.c_int),
+    "agh_graph_launch": ([ptr], C.c_int),
+    "agh_graph_destroy": ([ptr], C.c_int),
     "agh_memset": ([ptr, C.c_int, C.c_size_t], C.c_int),
     "agh_sync": ([], C.c_int),
     "agh_stream": ([], ptr),
@@ -45,10 +54,14 @@ SIGNATURES = {
     "agh_gemm_bf16": (_GEMM, C.c_int),
     "agh_gemm_f32_bias_act": (_GEMM + [ptr, i64, i64, C.c_int], C.c_int),
     "agh_gemm_bf16_bias_act": (_GEMM + [ptr, i64, i64, C.c_int], C.c_int),
+    "agh_gemm_f32_batched": (_GEMM_B, C.c_int),
+    "agh_gemm_bf16_batched": (_GEMM_B, C.c_int),
     "agh_im2col_conv2_f32": (_CONV, C.c_int),
     "agh_im2col_conv2_bf16": (_CONV, C.c_int),
     "agh_col2im_conv2_f32": (_CONV, C.c_int),
     "agh_col2im_conv2_bf16": (_CONV, C.c_int),
+    "agh_conv2_direct_f32": ([ptr, ptr, ptr, ptr] + [i64] * 13 + [C.c_int, C.c_int], C.c_int),
+    "agh_conv2_direct_bf16": ([ptr, ptr, ptr, ptr] + [i64] * 13 + [C.c_int, C.c_int], C.c_int),
     "agh_max_pool2_f32": (_POOL, C.c_int),
     "agh_max_pool2_bf16": (_POOL, C.c_int),
     "agh_max_pool2_backward_f32": (_POOL, C.c_int),

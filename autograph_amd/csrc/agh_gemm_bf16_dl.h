@@ -157,9 +157,11 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     const int64_t stepP = (int64_t)BK * g.pk * 2, stepQ = (int64_t)BK * g.qk * 2;
     const unsigned char *gp[DlP::NL], *gq[DlQ::NL];
 #pragma unroll
-    for (int i = 0; i < DlP::NL; ++i) gp[i] = (const unsigned char *)g.P + offp[i] + (int64_t)kbeg * g.pk * 2;
+    for (int i = 0; i < DlP::NL; ++i)
+        gp[i] = (const unsigned char *)g.P + offp[i] + ((int64_t)kbeg * g.pk + (int64_t)blockIdx.z * g.batch_p) * 2;
 #pragma unroll
-    for (int i = 0; i < DlQ::NL; ++i) gq[i] = (const unsigned char *)g.Q + offq[i] + (int64_t)kbeg * g.qk * 2;
+    for (int i = 0; i < DlQ::NL; ++i)
+        gq[i] = (const unsigned char *)g.Q + offq[i] + ((int64_t)kbeg * g.qk + (int64_t)blockIdx.z * g.batch_q) * 2;
 
     uint32_t fp[TP], fq[TQ];
     FrP::offsets(fp, wp * TP * 32, lane);
@@ -270,7 +272,7 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     // ------------------------------------------------------------ epilogue ----
     const uint32_t lrow = lane & 31, lg = lane >> 5;
     const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
-    T *D = (T *)g.D;
+    T *D = (T *)g.D + (int64_t)blockIdx.z * g.batch_d;
     const T *bias = (const T *)g.bias;
     const int mode = g.store_mode;
     const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;

@@ -44,7 +44,7 @@ int launch_one(const Args &g, int splits) {
             AGH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_done = true;
     }
-    dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits);
+    dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits, (unsigned)g.batch);
     hipLaunchKernelGGL(kern, grid, dim3(WGP * WGQ * 64), smem, stream(), g);
     AGH_LAUNCH_CHECK("gemm kernel launch");
     return AGH_OK;
@@ -54,7 +54,7 @@ int launch_one(const Args &g, int splits) {
 template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
 int launch_one_dl(const Args &g, int splits) {
     auto kern = gemm_bf16_dl_kernel<BP, BQ, WGP, WGQ, LP, LQ>;  // both LDS stages are static
-    dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits);
+    dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits, (unsigned)g.batch);
     hipLaunchKernelGGL(kern, grid, dim3(WGP * WGQ * 64), 0, stream(), g);
     AGH_LAUNCH_CHECK("gemm (direct-to-LDS) kernel launch");
     return AGH_OK;
@@ -132,9 +132,11 @@ template <typename T>
 int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, const void *a, int64_t off_a,
                int64_t rsa, int64_t csa, const void *b, int64_t off_b, int64_t rsb, int64_t csb, float beta, void *c,
                int64_t off_c, int64_t rsc, int64_t csc, const void *bias, int64_t off_bias, int64_t bias_stride,
-               int act) {
+               int act, int64_t batch = 1, int64_t batch_a = 0, int64_t batch_b = 0, int64_t batch_c = 0) {
     AGH_API_ENTER();
-    if (m < 0 || k < 0 || n < 0) return fail(AGH_EINVAL, "%s: negative dimension", name);
+    if (m < 0 || k < 0 || n < 0 || batch < 0) return fail(AGH_EINVAL, "%s: negative dimension", name);
+    if (batch > 65535) return fail(AGH_ERANGE, "%s: batch count above 65535", name);
+    if (batch == 0) return AGH_OK;
     const int64_t lim = ((int64_t)1 << 31) - 512;
     if (m > lim || k > lim || n > lim) return fail(AGH_ERANGE, "%s: dimension does not fit 31 bits", name);
     if (act != AGH_ACT_NONE && act != AGH_ACT_RELU) return fail(AGH_EINVAL, "%s: unknown activation %d", name, act);
@@ -159,13 +161,17 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         g.Q = A; g.qs = rsa; g.qk = csa; g.NQ = (int)m;
         g.dp = csc; g.dq = rsc;
         g.bias_on_p = 1;
+        g.batch_p = batch_b; g.batch_q = batch_a;
     } else {
         g.P = A; g.ps = rsa; g.pk = csa; g.NP = (int)m;
         g.Q = B; g.qs = csb; g.qk = rsb; g.NQ = (int)n;
         g.dp = rsc; g.dq = csc;
         g.bias_on_p = 0;
+        g.batch_p = batch_a; g.batch_q = batch_b;
     }
     g.D = C;
+    g.batch = (int)batch;
+    g.batch_d = batch_c;
     g.K = (int)k;
     g.alpha = alpha;
     g.beta = beta;
@@ -174,12 +180,15 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     g.bias_stride = bias_stride;
     g.act = act;
     g.NPpad = (g.NP + 3) & ~3;
-    g.dbg = env_int("AGH_GEMM_DBG", 0);
 
     int lp = k > 0 ? pick_loader<T>(g.P, g.ps, g.pk, g.NP, g.K) : LD_S;
     int lq = k > 0 ? pick_loader<T>(g.Q, g.qs, g.qk, g.NQ, g.K) : LD_S;
+    // every matrix of a batch must satisfy the same alignment as the first
+    const bool batch_aligned = batch == 1 || (g.batch_p % EPC == 0 && g.batch_q % EPC == 0);
+    if (!batch_aligned) lp = lq = LD_S;
     const bool any_scalar = (lp == LD_S || lq == LD_S);
-    const bool vec_store = g.dp == 1 && g.NP % 4 == 0 && (g.dq % 4 == 0 || g.NQ == 1) && aligned(C, 4 * sizeof(T));
+    const bool vec_store = g.dp == 1 && g.NP % 4 == 0 && (g.dq % 4 == 0 || g.NQ == 1) && aligned(C, 4 * sizeof(T)) &&
+                           (batch == 1 || g.batch_d % 4 == 0);
 
     // ---- tile shape: minimise (rounds of workgroups) x (tile area) / efficiency ----
     const int cus = compute_units() > 0 ? compute_units() : 256;
@@ -188,7 +197,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     for (int i = 0; i < kNumCfgs; ++i) {
         const TileCfg &t = kCfgs[i];
         if (any_scalar && !t.scalar_ok) continue;
-        const int64_t tiles = (int64_t)((g.NP + t.bp - 1) / t.bp) * ((g.NQ + t.bq - 1) / t.bq);
+        const int64_t tiles = (int64_t)((g.NP + t.bp - 1) / t.bp) * ((g.NQ + t.bq - 1) / t.bq) * batch;
         if (tiles > 0x7FFFFFFF) continue;
         // a CU works through ceil(tiles / CUs) tiles; co-resident workgroups share its MFMA rate
         const int64_t rounds = (tiles + cus - 1) / cus;
@@ -203,17 +212,17 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     g.tiles_q = (g.NQ + t.bq - 1) / t.bq;
 
     // ---- split-K when the tile grid cannot fill the chip and k is long ----
-    const int64_t tiles = (int64_t)g.tiles_p * g.tiles_q;
+    const int64_t tiles = (int64_t)g.tiles_p * g.tiles_q * batch;
     const int64_t slots = (int64_t)cus;
     int splits = 1;
     const int ktiles = (g.K + BK - 1) / BK;
-    if (tiles * 2 <= slots && ktiles >= 8) {
+    if (tiles * 2 <= slots && ktiles >= 8 && batch == 1) {
         int64_t s = slots / tiles;
         if (s > ktiles / 4) s = ktiles / 4;
         if (s > 64) s = 64;
         if (s > 1) splits = (int)s;
     }
-    splits = env_int("AGH_GEMM_SPLITS", splits);
+    if (batch == 1) splits = env_int("AGH_GEMM_SPLITS", splits);
     if (splits < 1) splits = 1;
     if (splits > ktiles && ktiles > 0) splits = ktiles;
     if (ktiles == 0) splits = 1;
@@ -243,7 +252,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     // the direct-to-LDS kernel can transpose its output tile through LDS and store full 16-byte
     // chunks when nothing has to be read back from C
     if (direct && best <= 3 && vec_store && beta == 0.0f && g.NP % 8 == 0 && (g.dq % 8 == 0 || g.NQ == 1) &&
-        aligned(C, 16))
+        aligned(C, 16) && (batch == 1 || g.batch_d % 8 == 0))
         g.store_mode = ST_STAGED;
     return launch_cfg<T>(best, g, 1, lp, lq, direct);
 }

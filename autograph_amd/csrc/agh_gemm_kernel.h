@@ -60,13 +60,13 @@ struct Args {
     const void *bias;
     float *ws;  // split-K partials [splits][NQ][NPpad]
     int64_t ps, pk, qs, qk, dp, dq, bias_stride;
-    int NP, NQ, K, NPpad;
+    int64_t batch_p, batch_q, batch_d;  // element strides between consecutive matrices (grid.z = batch)
+    int NP, NQ, K, NPpad, batch;
     int tiles_p, tiles_q;
     int k_per_split;  // multiple of the k-tile
     float alpha, beta;
     int bias_on_p, has_bias, act;
     int store_mode;
-    int dbg;  // timing experiments only (AGH_GEMM_DBG): 1 = skip global loads, 2 = skip LDS fragment reads, 4 = skip MFMAs
 };
 
 template <typename T> struct Geo;
@@ -285,8 +285,8 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     const int kend = min(g.K, kbeg + g.k_per_split);
     const int KT = kend > kbeg ? (kend - kbeg + BK - 1) / BK : 0;
 
-    const T *P = (const T *)g.P;
-    const T *Q = (const T *)g.Q;
+    const T *P = (const T *)g.P + (int64_t)blockIdx.z * g.batch_p;
+    const T *Q = (const T *)g.Q + (int64_t)blockIdx.z * g.batch_q;
 
     f32x16 acc[TP][TQ];
 #pragma unroll
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     // One loop nest per store mode, each small enough to unroll fully: the accumulators must
     // only ever be indexed by compile-time constants or they would be demoted to scratch.
     const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
-    T *D = (T *)g.D;
+    T *D = (T *)g.D + (int64_t)blockIdx.z * g.batch_d;
     const T *bias = (const T *)g.bias;
     const int mode = g.store_mode;
     const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;

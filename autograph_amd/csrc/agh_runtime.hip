@@ -147,6 +147,65 @@ int agh_memcpy_d2d(void *dst, const void *src, size_t bytes) {
     return AGH_OK;
 }
 
+int agh_memcpy_d2h_async(void *dst, const void *src, size_t bytes) {
+    AGH_API_ENTER();
+    if (bytes == 0) return AGH_OK;
+    if (!dst || !src) return fail(AGH_ENULL, "agh_memcpy_d2h_async: null pointer");
+    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+    return AGH_OK;
+}
+
+int agh_host_alloc(void **ptr, size_t bytes) {
+    AGH_API_ENTER();
+    if (!ptr) return fail(AGH_ENULL, "agh_host_alloc: null out pointer");
+    *ptr = nullptr;
+    AGH_HIP(hipHostMalloc(ptr, bytes ? bytes : 64, hipHostMallocDefault));
+    return AGH_OK;
+}
+
+int agh_host_free(void *ptr) {
+    AGH_API_ENTER();
+    if (!ptr) return AGH_OK;
+    AGH_HIP(hipStreamSynchronize(g_stream));
+    AGH_HIP(hipHostFree(ptr));
+    return AGH_OK;
+}
+
+int agh_graph_begin(void) {
+    AGH_API_ENTER();
+    AGH_HIP(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal));
+    return AGH_OK;
+}
+
+int agh_graph_end(void **graph_exec) {
+    AGH_API_ENTER();
+    if (!graph_exec) return fail(AGH_ENULL, "agh_graph_end: null out pointer");
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    AGH_HIP(hipStreamEndCapture(g_stream, &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    hipGraphDestroy(graph);
+    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    *graph_exec = (void *)exec;
+    return AGH_OK;
+}
+
+int agh_graph_launch(void *graph_exec) {
+    AGH_API_ENTER();
+    if (!graph_exec) return fail(AGH_ENULL, "agh_graph_launch: null graph");
+    AGH_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, g_stream));
+    return AGH_OK;
+}
+
+int agh_graph_destroy(void *graph_exec) {
+    AGH_API_ENTER();
+    if (!graph_exec) return AGH_OK;
+    AGH_HIP(hipStreamSynchronize(g_stream));
+    AGH_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    return AGH_OK;
+}
+
 int agh_sync(void) {
     AGH_API_ENTER();
     AGH_HIP(hipStreamSynchronize(g_stream));

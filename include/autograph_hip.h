@@ -66,10 +66,26 @@ int agh_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int agh_memcpy_d2d(void *dst, const void *src, size_t bytes);
 /* Tensor::zeros / fill for byte patterns (src/tensor.rs:1394-1416). */
 int agh_memset(void *dst, int byte_value, size_t bytes);
+/* Same copy without the wait (for use inside a captured graph, or when the caller syncs). */
+int agh_memcpy_d2h_async(void *dst, const void *src, size_t bytes);
+/* Pinned host memory for transfers that must not stage through a bounce buffer. */
+int agh_host_alloc(void **ptr, size_t bytes);
+int agh_host_free(void *ptr);
 /* device.wait() (src/tensor/linalg.rs:549). */
 int agh_sync(void);
 /* The hipStream_t all work is enqueued on (for callers that record their own events). */
 void *agh_stream(void);
+
+/* Launch-bound sequences (a LeNet5 forward pass is a dozen tiny kernels) can be recorded once
+ * and replayed as one hipGraph: between agh_graph_begin and agh_graph_end every launch entry
+ * point and agh_memcpy_d2h_async is captured instead of executed.  No entry point that
+ * allocates, frees or waits (agh_malloc, agh_free, agh_sync, agh_memcpy_d2h, a first split-K
+ * GEMM that has to grow the workspace) may be called while capturing: run the sequence once
+ * eagerly first.  The reference has no counterpart (krnl dispatches kernel by kernel). */
+int agh_graph_begin(void);
+int agh_graph_end(void **graph_exec);
+int agh_graph_launch(void *graph_exec);
+int agh_graph_destroy(void *graph_exec);
 
 /* Timing helpers: hipEvent pairs recorded on the library's stream. */
 int agh_event_create(void **event);
@@ -115,6 +131,23 @@ int agh_gemm_bf16_bias_act(int64_t m, int64_t k, int64_t n, float alpha,
                            float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc,
                            const void *bias, int64_t off_bias, int64_t bias_stride, int act);
 
+/* A batch of `batch` independent GEMMs in one launch; matrix i of each operand starts
+ * batch_stride_* elements after matrix i-1 (0 = shared by the whole batch), bias/act as in
+ * the fused entry points (bias may be null, act AGH_ACT_NONE).  This is how the conv2_im2col
+ * chain (src/learn/neural_network/layer.rs:968-1004) writes its result straight in NCHW
+ * layout: per image, C is the [oh*ow, oc] product seen column-major (rsc = 1, csc = oh*ow),
+ * which removes the reference's `permuted_axes([0,3,1,2]).to_standard_layout()` copy. */
+int agh_gemm_f32_batched(int64_t batch, int64_t m, int64_t k, int64_t n, float alpha,
+                         const void *a, int64_t off_a, int64_t rsa, int64_t csa, int64_t batch_stride_a,
+                         const void *b, int64_t off_b, int64_t rsb, int64_t csb, int64_t batch_stride_b,
+                         float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc, int64_t batch_stride_c,
+                         const void *bias, int64_t off_bias, int64_t bias_stride, int act);
+int agh_gemm_bf16_batched(int64_t batch, int64_t m, int64_t k, int64_t n, float alpha,
+                          const void *a, int64_t off_a, int64_t rsa, int64_t csa, int64_t batch_stride_a,
+                          const void *b, int64_t off_b, int64_t rsb, int64_t csb, int64_t batch_stride_b,
+                          float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc, int64_t batch_stride_c,
+                          const void *bias, int64_t off_bias, int64_t bias_stride, int act);
+
 /* ------------------------------------------------------------ im2col / col2im ---- */
 
 /* Im2ColConv2 device branch (src/tensor/ops.rs:842-880; semantics from the host impl
@@ -140,6 +173,24 @@ int agh_col2im_conv2_f32(const void *x, void *y, int64_t bs, int64_t c, int64_t 
 int agh_col2im_conv2_bf16(const void *x, void *y, int64_t bs, int64_t c, int64_t ih, int64_t iw,
                           int64_t fh, int64_t fw, int64_t ph, int64_t pw,
                           int64_t sh, int64_t sw, int64_t dh, int64_t dw);
+
+/* ---------------------------------------------------------- direct convolution ---- */
+
+/* Conv2 forward without a materialised patch matrix, for layers whose input image and filter
+ * bank fit in LDS (returns AGH_ERANGE otherwise: use im2col + gemm).  Same result as the
+ * conv2_im2col chain (src/learn/neural_network/layer.rs:950-1005) up to f32 summation order;
+ * the reference's host has the analogous conv_direct path (layer/conv_direct.rs:23-83).
+ * x: [bs,ic,ih,iw], w: [oc,ic,fh,fw], bias: null or [oc] (conv2's add_assign, layer.rs:944-946),
+ * act: the Relu layer that follows (layer.rs:1254-1267), pool2x2 != 0: also the MaxPool2 with
+ * filter [2,2] and stride [2,2] that follows (layer.rs:1193-1216) with its first-strict-max rule.
+ * y: [bs,oc,oh,ow], or [bs,oc,oh/2,ow/2] with the pool.  Rounding order as the separate
+ * layers: T(conv) -> T(bias + .) -> relu -> pool. */
+int agh_conv2_direct_f32(const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic,
+                         int64_t ih, int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw,
+                         int64_t sh, int64_t sw, int64_t dh, int64_t dw, int act, int pool2x2);
+int agh_conv2_direct_bf16(const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic,
+                          int64_t ih, int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw,
+                          int64_t sh, int64_t sw, int64_t dh, int64_t dw, int act, int pool2x2);
 
 /* ---------------------------------------------------------------- max pool ---- */
 

@@ -1,0 +1,190 @@
+"""Layer-level parity on the GPU: Conv2 (im2col chain and direct kernel), fused ReLU/MaxPool2,
+Dense, and the LeNet5 forward pass of the reference's benchmark, against the CPU oracle.
+
+Mirrors conv2_im2col_<T>_<opts> (tests/integration_tests.rs:986-993, body :1182-1251), which
+checks the chain against the naive 7-deep loop on x, w = (1..=10).cycle() data.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from refgrid import BATCH_IN_OUT, conv_options, input_shapes
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ag():
+    import autograph_amd as ag
+    ag.Device(0)
+    return ag
+
+
+def to_dtype(x, dtype):
+    return orc.f32_to_bf16(x) if dtype == "bf16" else np.ascontiguousarray(x, dtype=np.float32)
+
+
+def as_f32(x):
+    return orc.bf16_to_f32(x) if x.dtype == np.uint16 else x
+
+
+def cyc10(shape):
+    return ((np.arange(int(np.prod(shape))) % 10) + 1).astype(np.float32).reshape(shape)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("alg", ["im2col", "direct"])
+def test_conv2_reference_grid(ag, dtype, alg):
+    """Whole filter/padding/stride/dilation grid x (batch, inputs, outputs) list; exact-integer data.
+    f32 must be exact (all sums < 2^24); bf16 must be the correctly rounded exact sum."""
+    n = 0
+    for f, p, s, d in conv_options():
+        for ih, iw in list(input_shapes(f, p, s, d))[::3]:
+            for bs, ic, oc in BATCH_IN_OUT:
+                x = to_dtype(cyc10((bs, ic, ih, iw)), dtype)
+                w = to_dtype(cyc10((oc, ic) + f), dtype)
+                want = orc.conv2_naive_f64(as_f32(x), as_f32(w), p, s, d)
+                fn = ag.conv2_im2col_forward if alg == "im2col" else ag.conv2_direct_forward
+                y = fn(ag.Tensor.from_array(x), ag.Tensor.from_array(w), padding=p, stride=s, dilation=d).into_array()
+                assert y.shape == want.shape
+                if dtype == "f32":
+                    assert np.array_equal(y.astype(np.float64), want), (alg, bs, ic, oc, ih, iw, f, p, s, d)
+                else:
+                    # f32 accumulation of these integers is exact, so the result is the single RNE
+                    # rounding of the exact sum (the reference compares two bf16 computations with
+                    # epsilon = fh*fw, :1239-1243; this is the tighter statement)
+                    assert np.array_equal(y, orc.f32_to_bf16(want.astype(np.float32))), (alg, bs, ic, oc, ih, iw, f, p, s, d)
+                n += 1
+    assert n > 500
+
+
+CONV_SEEDED = [
+    # bs, ic, ih, iw, oc, filter, padding, stride, dilation
+    (100, 1, 28, 28, 6, (5, 5), (0, 0), (1, 1), (1, 1)),    # LeNet5 conv1
+    (100, 6, 12, 12, 16, (5, 5), (0, 0), (1, 1), (1, 1)),   # LeNet5 conv2
+    (8, 16, 20, 20, 32, (3, 3), (1, 1), (1, 1), (1, 1)),
+    (3, 5, 17, 23, 7, (3, 5), (2, 1), (2, 3), (2, 1)),
+    (4, 64, 14, 14, 128, (3, 3), (1, 1), (1, 1), (1, 1)),   # config-3 shaped, small batch
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("case", CONV_SEEDED)
+def test_conv2_seeded_both_algorithms(ag, dtype, case):
+    bs, ic, ih, iw, oc, f, p, s, d = case
+    rng = np.random.default_rng(21)
+    x = to_dtype(rng.standard_normal((bs, ic, ih, iw)), dtype)
+    w = to_dtype(rng.standard_normal((oc, ic) + f) * np.sqrt(2.0 / (ic * f[0] * f[1])), dtype)
+    b = to_dtype(rng.standard_normal(oc) * 0.1, dtype)
+    want = orc.conv2_naive_f64(as_f32(x), as_f32(w), p, s, d)
+    scale = orc.conv2_naive_f64(np.abs(as_f32(x)), np.abs(as_f32(w)), p, s, d)
+    k = ic * f[0] * f[1]
+    tx, tw, tb = ag.Tensor.from_array(x), ag.Tensor.from_array(w), ag.Tensor.from_array(b)
+    for alg in ("im2col", "direct"):
+        fn = ag.conv2_im2col_forward if alg == "im2col" else ag.conv2_direct_forward
+        try:
+            y = fn(tx, tw, padding=p, stride=s, dilation=d).into_array()
+        except ag.AghError as e:
+            assert alg == "direct" and e.code == -4  # does not fit in LDS: documented fallback
+            continue
+        got = as_f32(y).astype(np.float64)
+        if dtype == "f32":
+            assert np.all(np.abs(got - want) <= 1e-5 * np.sqrt(k) * scale + 1e-30), alg
+        else:
+            ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0**-126))) - 7)
+            assert np.all(np.abs(got - want) <= ulp + 1e-2 * np.abs(want) + 8 * np.sqrt(k) * 2.0**-24 * scale), alg
+        # bias + relu epilogue: equals the separate ops applied to this very conv result, bit for bit
+        yb = fn(tx, tw, padding=p, stride=s, dilation=d, bias=tb, relu=True).into_array()
+        n, c, h, wd = y.shape
+        flat = np.ascontiguousarray(y.transpose(0, 2, 3, 1).reshape(-1, c))
+        ref = orc.relu(orc.bias_add_rows(flat, b)).reshape(n, h, wd, c).transpose(0, 3, 1, 2)
+        assert np.array_equal(yb, ref), alg
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_conv2_direct_fused_relu_pool(ag, dtype):
+    """conv -> Relu -> MaxPool2(2x2) in one launch equals the three layers applied to the conv result."""
+    rng = np.random.default_rng(22)
+    for (bs, ic, ih, iw, oc, f) in [(100, 1, 28, 28, 6, (5, 5)), (100, 6, 12, 12, 16, (5, 5)), (5, 3, 11, 9, 10, (3, 3))]:
+        x = to_dtype(rng.uniform(0, 1, (bs, ic, ih, iw)), dtype)
+        w = to_dtype(rng.uniform(-1, 1, (oc, ic) + f) * np.sqrt(2.0 / (ic * f[0] * f[1])), dtype)
+        tx, tw = ag.Tensor.from_array(x), ag.Tensor.from_array(w)
+        conv = ag.conv2_direct_forward(tx, tw).into_array()
+        fused = ag.conv2_direct_forward(tx, tw, relu=True, pool2x2=True).into_array()
+        assert np.array_equal(fused, orc.max_pool2(orc.relu(conv), (2, 2)))
+
+
+def he(rng, shape, fan_in):  # Uniform(-a, a), a = sqrt(2/fan_in): layer.rs:345-349, :463-467
+    a = np.sqrt(2.0 / fan_in)
+    return rng.uniform(-a, a, shape).astype(np.float32)
+
+
+def lenet_params(rng):
+    return [he(rng, (6, 1, 5, 5), 25), he(rng, (16, 6, 5, 5), 150), he(rng, (256, 128), 256), he(rng, (128, 84), 128),
+            he(rng, (84, 10), 84), he(rng, (10,), 84)]
+
+
+def oracle_lenet_bf16(x, params):
+    """The reference's DEVICE numerics for bf16 (f32 accumulate, one rounding per op), layer by layer."""
+    w1, w2, wd1, wd2, wd3, b3 = params
+
+    def conv(h, w):
+        bs, ic, ih, iw = h.shape
+        oc, _, fh, fw = w.shape
+        cols = orc.im2col_conv2(h, (fh, fw))
+        out = orc.gemm_bf16_f32acc(cols, w.reshape(oc, -1).T)
+        oh, ow = ih - fh + 1, iw - fw + 1
+        return np.ascontiguousarray(out.reshape(bs, oh, ow, oc).transpose(0, 3, 1, 2))
+
+    h = orc.max_pool2(orc.relu(conv(x, w1)), (2, 2))
+    h = orc.max_pool2(orc.relu(conv(h, w2)), (2, 2)).reshape(x.shape[0], 256)
+    h = orc.relu(orc.gemm_bf16_f32acc(h, wd1))
+    h = orc.relu(orc.gemm_bf16_f32acc(h, wd2))
+    return orc.bias_add_rows(orc.gemm_bf16_f32acc(h, wd3), b3)
+
+
+@pytest.mark.parametrize("bs", [1, 100, 1000])
+def test_lenet5_forward_f32(ag, bs):
+    rng = np.random.default_rng(23)
+    params = lenet_params(rng)
+    x = rng.uniform(0, 1, (bs, 1, 28, 28)).astype(np.float32)
+    want = orc.lenet5_forward_f32(x, *params)
+    model = ag.LeNet5.from_arrays(*params)
+    tx = ag.Tensor.from_array(x)
+    tol = 2e-4 * max(1.0, np.abs(want).max())  # six chained f32 layers, k up to 256
+    for name, out in (("im2col", model.forward(tx, algorithm="im2col")), ("direct", model.forward(tx, algorithm="direct")),
+                      ("fused", model.forward_fused(tx))):
+        got = out.into_array()
+        assert got.shape == (bs, 10)
+        assert np.abs(got - want).max() <= tol, (name, np.abs(got - want).max())
+    # graph-captured inference: several replays, each checked, with host work between them
+    host = C.c_void_p()
+    ag._ffi.check(ag.lib.agh_host_alloc(C.byref(host), bs * 10 * 4))
+    logits = model.capture(tx, host.value)
+    eager = model.forward_fused(tx).into_array()
+    for i in range(4):
+        ag._ffi.check(ag.lib.agh_memset(logits._ptr(), 0xFF, bs * 10 * 4))
+        model.replay()
+        ag._ffi.check(ag.lib.agh_sync())
+        pinned = np.ctypeslib.as_array(C.cast(host.value, C.POINTER(C.c_float)), shape=(bs, 10)).copy()
+        assert np.array_equal(pinned, eager), i
+        assert np.array_equal(logits.into_array(), eager), i
+    del model
+    ag._ffi.check(ag.lib.agh_host_free(host))
+
+
+@pytest.mark.parametrize("bs", [1, 100])
+def test_lenet5_forward_bf16(ag, bs):
+    rng = np.random.default_rng(24)
+    params = [orc.f32_to_bf16(p) for p in lenet_params(rng)]
+    x = orc.f32_to_bf16(rng.uniform(0, 1, (bs, 1, 28, 28)).astype(np.float32))
+    want = orc.bf16_to_f32(oracle_lenet_bf16(x, params)).astype(np.float64)
+    model = ag.LeNet5.from_arrays(*params)
+    tx = ag.Tensor.from_array(x)
+    for name, out in (("im2col", model.forward(tx, algorithm="im2col")), ("fused", model.forward_fused(tx))):
+        got = orc.bf16_to_f32(out.into_array()).astype(np.float64)
+        # every layer may differ from the oracle by one bf16 rounding; six layers compound
+        assert np.abs(got - want).max() <= 0.05 * max(1.0, np.abs(want).max()), (name, np.abs(got - want).max())
+        assert np.mean(np.abs(got - want)) <= 0.01 * max(1.0, np.abs(want).max()), name
