@@ -124,6 +124,342 @@ __global__ __launch_bounds__(256) void conv2_direct_kernel(const T *__restrict__
     }
 }
 
+// ---- row-tiled variant for stride 1, dilation 1 (any padding) ----
+//
+// A work item computes WT = 8 consecutive output pixels of one output row - or, with the pool
+// fused, of a PAIR of rows, i.e. four whole pool windows - for OCT output channels.  The staged
+// image is zero-padded in LDS, so the inner loop has no bounds checks: per (channel, input row)
+// it reads WT + FW - 1 input values once (three 16-byte LDS reads) and the FW x OCT filter values
+// of the filter row(s) that input row meets (uniform addresses, LDS broadcasts), then does up to
+// 2 * FW * WT * OCT FMAs out of registers - about 12 FMAs per LDS read instead of 3.
+struct RowTileParams {
+    int bs, ic, ih, iw, oc, oh, ow, fh, ph, pw;
+    int act, has_bias;
+    int imgs, ngroups, ocpad;
+    int ihp, pitch;       // padded rows staged per channel, LDS row pitch (floats, multiple of 4)
+    int nwb;              // WT-wide blocks per output row
+    int nrows;            // output rows (or row pairs with the pool) per image
+    int yh, yw;
+    int items_per_img;
+    FastDiv div_items, div_rowsxwb, div_nwb, div_ocpad, div_pitch, div_ihp;
+};
+
+template <typename T, int FW, int OCT, bool POOL>
+__global__ __launch_bounds__(256) void conv2_rowtile_kernel(const T *__restrict__ x, const T *__restrict__ w,
+                                                             const T *__restrict__ bias, T *__restrict__ y,
+                                                             RowTileParams p) {
+    constexpr int WT = 8, NR = POOL ? 2 : 1, XW = WT + FW - 1, XV = (XW + 3) / 4;
+    extern __shared__ __align__(16) float smem_f[];
+    const int taps = p.ic * p.fh * FW;
+    float *ws = smem_f;                                         // [ic][fh][FW][ocpad]
+    float *xs = smem_f + (((size_t)taps * p.ocpad + 3) & ~(size_t)3);  // [imgs][ic][ihp][pitch], zero padded
+    const int ch_sz = p.ihp * p.pitch, img_sz = p.ic * ch_sz;
+    const int b0 = blockIdx.x * p.imgs;
+    const int nimg = min(p.imgs, p.bs - b0);
+
+    for (int e = threadIdx.x; e < taps * p.ocpad; e += blockDim.x) {
+        uint32_t tap, o;
+        p.div_ocpad.divmod((uint32_t)e, tap, o);
+        ws[e] = (int)o < p.oc ? Elem<T>::to_f32(w[(size_t)o * taps + tap]) : 0.0f;
+    }
+    for (int e = threadIdx.x; e < nimg * img_sz; e += blockDim.x) {
+        uint32_t r1, col, r2, row;  // r2 = img * ic + channel
+        p.div_pitch.divmod((uint32_t)e, r1, col);
+        p.div_ihp.divmod(r1, r2, row);
+        const int hi = (int)row - p.ph, wi = (int)col - p.pw;
+        float v = 0.0f;
+        if (hi >= 0 && hi < p.ih && wi >= 0 && wi < p.iw)
+            v = Elem<T>::to_f32(x[((size_t)b0 * p.ic + r2) * p.ih * p.iw + (size_t)hi * p.iw + wi]);
+        xs[e] = v;
+    }
+    __syncthreads();
+
+    const int total = nimg * p.items_per_img;
+    for (int item = threadIdx.x; item < total; item += blockDim.x) {
+        uint32_t img, r0, grp, r1, row, wb;
+        p.div_items.divmod((uint32_t)item, img, r0);
+        p.div_rowsxwb.divmod(r0, grp, r1);
+        p.div_nwb.divmod(r1, row, wb);
+        const int ho0 = POOL ? 2 * (int)row : (int)row;  // first output row of this item
+        const float *xi = xs + (size_t)img * img_sz + ho0 * p.pitch + wb * WT;
+        const float *wg = ws + grp * OCT;
+
+        float acc[NR][WT][OCT];
+#pragma unroll
+        for (int a = 0; a < NR; ++a)
+#pragma unroll
+            for (int t = 0; t < WT; ++t)
+#pragma unroll
+                for (int o = 0; o < OCT; ++o) acc[a][t][o] = 0.0f;
+
+        for (int ci = 0; ci < p.ic; ++ci) {
+            const float *xc = xi + ci * ch_sz;
+            const float *wc = wg + (size_t)ci * p.fh * FW * p.ocpad;
+            // input row r (relative to ho0) meets filter row r of output row 0 and r-1 of output row 1
+            for (int r = 0; r < p.fh + NR - 1; ++r) {
+                float xin[XV * 4];
+#pragma unroll
+                for (int v = 0; v < XV; ++v) {
+                    const float4 q = *(const float4 *)(xc + r * p.pitch + 4 * v);
+                    xin[4 * v + 0] = q.x; xin[4 * v + 1] = q.y; xin[4 * v + 2] = q.z; xin[4 * v + 3] = q.w;
+                }
+#pragma unroll
+                for (int a = 0; a < NR; ++a) {
+                    const int fi = r - a;
+                    if (fi >= 0 && fi < p.fh) {
+                        const float *wr = wc + fi * FW * p.ocpad;
+#pragma unroll
+                        for (int fj = 0; fj < FW; ++fj) {
+                            float wv[OCT];
+#pragma unroll
+                            for (int o = 0; o < OCT; ++o) wv[o] = wr[fj * p.ocpad + o];
+#pragma unroll
+                            for (int t = 0; t < WT; ++t)
+#pragma unroll
+                                for (int o = 0; o < OCT; ++o)
+                                    acc[a][t][o] = __builtin_fmaf(xin[t + fj], wv[o], acc[a][t][o]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < OCT; ++o) {
+            const int oc = grp * OCT + o;
+            const bool live = oc < p.oc;
+            const T bv = (p.has_bias && live) ? bias[oc] : Elem<T>::zero();
+            T *yp = y + (((size_t)(b0 + img) * p.oc + (live ? oc : 0)) * p.yh + row) * p.yw;
+            if (POOL) {
+#pragma unroll
+                for (int j = 0; j < WT / 2; ++j) {
+                    // window in row-major order: (0,2j) (0,2j+1) (1,2j) (1,2j+1); first strict maximum wins
+                    T m = round_bias_relu<T>(acc[0][2 * j][o], p.has_bias != 0, bv, p.act);
+                    float mf = Elem<T>::to_f32(m);
+                    const T v1 = round_bias_relu<T>(acc[0][2 * j + 1][o], p.has_bias != 0, bv, p.act);
+                    const T v2 = round_bias_relu<T>(acc[NR - 1][2 * j][o], p.has_bias != 0, bv, p.act);
+                    const T v3 = round_bias_relu<T>(acc[NR - 1][2 * j + 1][o], p.has_bias != 0, bv, p.act);
+                    float f = Elem<T>::to_f32(v1);
+                    if (f > mf) { m = v1; mf = f; }
+                    f = Elem<T>::to_f32(v2);
+                    if (f > mf) { m = v2; mf = f; }
+                    f = Elem<T>::to_f32(v3);
+                    if (f > mf) { m = v3; mf = f; }
+                    const int px = wb * (WT / 2) + j;
+                    if (live && px < p.yw) yp[px] = m;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < WT; ++t) {
+                    const int px = wb * WT + t;
+                    if (live && px < p.yw) yp[px] = round_bias_relu<T>(acc[0][t][o], p.has_bias != 0, bv, p.act);
+                }
+            }
+        }
+    }
+}
+
+// ---- LeNet5 inference in one launch ----
+//
+// The model of the reference's benchmark (benches/neural-network-benches/src/
+// autograph_backend.rs:88-162): conv 1->6 5x5, relu, pool 2x2, conv 6->16 5x5, relu, pool 2x2,
+// flatten, dense 256->128, relu, dense 128->84, relu, dense 84->10 + bias.  At batch 1000 the
+// whole forward pass is 0.57 GFLOP; run layer by layer it is bound by launch latency and by
+// round trips of tiny activations through HBM.  Here a workgroup takes IMGS images through all
+// twelve layers with every activation in LDS: the two conv+relu+pool stages use the same
+// row-tiled inner loop as conv2_rowtile_kernel, the Dense stages are LDS-broadcast dot products
+// against weights read (coalesced) from L2.  Activations are rounded to T after every layer,
+// exactly where the layer-by-layer path rounds, so both paths agree per layer up to f32
+// summation order.
+template <int FW, int OCT, int WT>
+__device__ __forceinline__ void rowpair_conv(const float *xi, int ch_sz, int pitch, int ic, int fh, const float *wg,
+                                             int ocpad, float (&acc)[2][WT][OCT]) {
+    constexpr int XW = WT + FW - 1, XV = (XW + 3) / 4;
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int t = 0; t < WT; ++t)
+#pragma unroll
+            for (int o = 0; o < OCT; ++o) acc[a][t][o] = 0.0f;
+    for (int ci = 0; ci < ic; ++ci) {
+        const float *xc = xi + ci * ch_sz;
+        const float *wc = wg + (size_t)ci * fh * FW * ocpad;
+        for (int r = 0; r < fh + 1; ++r) {
+            float xin[XV * 4];
+#pragma unroll
+            for (int v = 0; v < XV; ++v) {
+                const float4 q = *(const float4 *)(xc + r * pitch + 4 * v);
+                xin[4 * v + 0] = q.x; xin[4 * v + 1] = q.y; xin[4 * v + 2] = q.z; xin[4 * v + 3] = q.w;
+            }
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const int fi = r - a;
+                if (fi >= 0 && fi < fh) {
+                    const float *wr = wc + fi * FW * ocpad;
+#pragma unroll
+                    for (int fj = 0; fj < FW; ++fj) {
+                        float wv[OCT];
+#pragma unroll
+                        for (int o = 0; o < OCT; ++o) wv[o] = wr[fj * ocpad + o];
+#pragma unroll
+                        for (int t = 0; t < WT; ++t)
+#pragma unroll
+                            for (int o = 0; o < OCT; ++o) acc[a][t][o] = __builtin_fmaf(xin[t + fj], wv[o], acc[a][t][o]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// relu + first-strict-maximum pooling of window j of a row pair, rounding to T first
+template <typename T, int OCT, int WT>
+__device__ __forceinline__ float relu_pool_window(const float (&acc)[2][WT][OCT], int j, int o) {
+    const T zero = Elem<T>::zero();
+    T m = round_bias_relu<T>(acc[0][2 * j][o], false, zero, AGH_ACT_RELU);
+    float mf = Elem<T>::to_f32(m);
+    const T v1 = round_bias_relu<T>(acc[0][2 * j + 1][o], false, zero, AGH_ACT_RELU);
+    const T v2 = round_bias_relu<T>(acc[1][2 * j][o], false, zero, AGH_ACT_RELU);
+    const T v3 = round_bias_relu<T>(acc[1][2 * j + 1][o], false, zero, AGH_ACT_RELU);
+    float f = Elem<T>::to_f32(v1);
+    if (f > mf) mf = f;
+    f = Elem<T>::to_f32(v2);
+    if (f > mf) mf = f;
+    f = Elem<T>::to_f32(v3);
+    if (f > mf) mf = f;
+    return mf;  // activations stay in LDS as f32 copies of the T values
+}
+
+template <typename T>
+__global__ __launch_bounds__(512) void lenet5_forward_kernel(const T *__restrict__ x, const T *__restrict__ w1,
+                                                              const T *__restrict__ w2, const T *__restrict__ wd1,
+                                                              const T *__restrict__ wd2, const T *__restrict__ wd3,
+                                                              const T *__restrict__ b3, T *__restrict__ out, int bs) {
+    constexpr int IMGS = 4;
+    __shared__ __align__(16) float xs[IMGS * 28 * 28];     // input images, pitch 28
+    __shared__ __align__(16) float w1s[25 * 6];            // [tap][oc]
+    __shared__ __align__(16) float p1[IMGS * 6 * 12 * 12]; // after conv1 + relu + pool
+    __shared__ __align__(16) float w2s[150 * 16];          // [ci][fi][fj][oc]
+    __shared__ __align__(16) float p2[IMGS * 256];         // after conv2 + relu + pool, flattened [c][h][w]
+    __shared__ __align__(16) float d1[IMGS * 128];
+    __shared__ __align__(16) float d2[IMGS * 84];
+    __shared__ __align__(16) float parts[16 * IMGS * 128];  // dense1 partial sums
+    constexpr int NT = 512;  // 8 waves: two per SIMD, so one can wait on LDS while the other multiplies
+    const int tid = threadIdx.x;
+    const int b0 = blockIdx.x * IMGS;
+    const int nimg = min(IMGS, bs - b0);
+
+    for (int e = tid; e < 150; e += NT) { const int tap = e / 6, o = e - tap * 6; w1s[e] = Elem<T>::to_f32(w1[o * 25 + tap]); }
+    for (int e = tid; e < 2400; e += NT) { const int tap = e >> 4, o = e & 15; w2s[e] = Elem<T>::to_f32(w2[o * 150 + tap]); }
+    for (int e = tid; e < IMGS * 784; e += NT) xs[e] = e < nimg * 784 ? Elem<T>::to_f32(x[(size_t)b0 * 784 + e]) : 0.0f;
+    // dense1 weights of this thread (see the dense1 stage below), requested now, used much later
+    float4 wreg[16];
+    {
+        const int cg = tid & 31, kg = tid >> 5;
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            const T *src = wd1 + (size_t)(kg * 16 + kk) * 128 + cg * 4;
+            if constexpr (sizeof(T) == 4) {
+                wreg[kk] = *(const float4 *)src;
+            } else {
+                const uint2 raw = *(const uint2 *)src;
+                wreg[kk] = make_float4(bf16_to_f32((uint16_t)(raw.x & 0xFFFF)), bf16_to_f32((uint16_t)(raw.x >> 16)),
+                                       bf16_to_f32((uint16_t)(raw.y & 0xFFFF)), bf16_to_f32((uint16_t)(raw.y >> 16)));
+            }
+        }
+    }
+    __syncthreads();
+
+    // conv1 (1->6, 5x5) + relu + pool: items = img x 3 channel pairs x 12 row pairs x 3 column blocks of 8
+    if (tid < IMGS * 108) {
+        const int img = tid / 108, r0 = tid - img * 108;
+        const int grp = r0 / 36, r1 = r0 - grp * 36;
+        const int row = r1 / 3, wb = r1 - row * 3;
+        float acc[2][8][2];
+        rowpair_conv<5, 2, 8>(xs + img * 784 + 2 * row * 28 + wb * 8, 784, 28, 1, 5, w1s + grp * 2, 6, acc);
+#pragma unroll
+        for (int o = 0; o < 2; ++o)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                p1[((img * 6 + grp * 2 + o) * 12 + row) * 12 + wb * 4 + j] = relu_pool_window<T, 2, 8>(acc, j, o);
+    }
+    __syncthreads();
+
+    // conv2 (6->16, 5x5) + relu + pool: items = img x 16 channels x 4 row pairs x 2 column blocks of 4
+    {
+        const int img = tid >> 7, r0 = tid & 127;
+        const int oc = r0 >> 3, row = (r0 >> 1) & 3, wb = r0 & 1;
+        float acc[2][4][1];
+        rowpair_conv<5, 1, 4>(p1 + img * 864 + 2 * row * 12 + wb * 4, 144, 12, 6, 5, w2s + oc, 16, acc);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) p2[img * 256 + (oc * 4 + row) * 4 + wb * 2 + j] = relu_pool_window<T, 1, 4>(acc, j, 0);
+    }
+    __syncthreads();
+
+    // dense1 256 -> 128 + relu.  Thread (cg, kg) owns the weights W1[16kg .. 16kg+15][4cg .. 4cg+3]; they
+    // were fetched into registers at the top of the kernel (16 coalesced 16-byte loads per thread, in
+    // flight during both convolution stages).  Each thread forms its 4 columns x 4 images partial sums
+    // over its 16 k, the 16 k-groups are then added through LDS in a fixed order.
+    {
+        const int cg = tid & 31, kg = tid >> 5;
+        float part[IMGS][4];
+#pragma unroll
+        for (int r = 0; r < IMGS; ++r)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) part[r][c] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < 16; kk += 4) {
+            float4 xv[IMGS];
+#pragma unroll
+            for (int r = 0; r < IMGS; ++r) xv[r] = *(const float4 *)(p2 + r * 256 + kg * 16 + kk);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const float4 wv = wreg[kk + u];
+#pragma unroll
+                for (int r = 0; r < IMGS; ++r) {
+                    const float xk = u == 0 ? xv[r].x : u == 1 ? xv[r].y : u == 2 ? xv[r].z : xv[r].w;
+                    part[r][0] = __builtin_fmaf(xk, wv.x, part[r][0]);
+                    part[r][1] = __builtin_fmaf(xk, wv.y, part[r][1]);
+                    part[r][2] = __builtin_fmaf(xk, wv.z, part[r][2]);
+                    part[r][3] = __builtin_fmaf(xk, wv.w, part[r][3]);
+                }
+            }
+        }
+        // xs and p1 are free by now: the [kg][img][128] partials (16*4*128 floats = 32 KB) do not fit xs
+        // alone, so they go to a buffer of their own
+#pragma unroll
+        for (int r = 0; r < IMGS; ++r)
+            *(float4 *)(parts + (kg * IMGS + r) * 128 + cg * 4) = make_float4(part[r][0], part[r][1], part[r][2], part[r][3]);
+    }
+    __syncthreads();
+    {
+        const int o = tid;  // IMGS * 128 == NT
+        float a = 0.0f;
+#pragma unroll
+        for (int kg = 0; kg < 16; ++kg) a += parts[kg * IMGS * 128 + o];
+        d1[o] = Elem<T>::to_f32(round_bias_relu<T>(a, false, Elem<T>::zero(), AGH_ACT_RELU));
+    }
+    __syncthreads();
+    // dense2 128 -> 84 + relu (weights straight from L2, 32 loads in flight per thread)
+    if (tid < IMGS * 84) {
+        const int r = tid / 84, c = tid - r * 84;
+        float a = 0.0f;
+        const float *xr = d1 + r * 128;
+#pragma unroll 32
+        for (int k = 0; k < 128; ++k) a = __builtin_fmaf(xr[k], Elem<T>::to_f32(wd2[k * 84 + c]), a);
+        d2[tid] = Elem<T>::to_f32(round_bias_relu<T>(a, false, Elem<T>::zero(), AGH_ACT_RELU));
+    }
+    __syncthreads();
+    // dense3 84 -> 10 + bias
+    if (tid < IMGS * 10) {
+        const int r = tid / 10, c = tid - r * 10;
+        float a = 0.0f;
+        const float *xr = d2 + r * 84;
+#pragma unroll 28
+        for (int k = 0; k < 84; ++k) a = __builtin_fmaf(xr[k], Elem<T>::to_f32(wd3[k * 10 + c]), a);
+        if (r < nimg) out[(size_t)(b0 + r) * 10 + c] = round_bias_relu<T>(a, true, b3[c], AGH_ACT_NONE);
+    }
+}
+
 template <typename T, bool POOL>
 int launch_oct(int oct, dim3 grid, dim3 block, size_t smem, const T *x, const T *w, const T *bias, T *y,
                const ConvParams &p) {
@@ -156,6 +492,69 @@ int conv2_direct_entry(const char *name, const void *x, const void *w, const voi
     if (pool2x2 && (oh < 2 || ow < 2)) return fail(AGH_EINVAL, "%s: output smaller than the 2x2 pool window", name);
     if (bs == 0) return AGH_OK;
     if (!x || !w || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+
+    // stride 1, dilation 1, filter width 3 or 5: row-tiled kernel
+    if (sh == 1 && sw == 1 && dh == 1 && dw == 1 && (fw == 3 || fw == 5)) {
+        RowTileParams q;
+        q.bs = bs; q.ic = ic; q.ih = ih; q.iw = iw; q.oc = oc; q.oh = oh; q.ow = ow; q.fh = fh; q.ph = ph; q.pw = pw;
+        q.act = act; q.has_bias = bias != nullptr;
+        // two output channels per work item unless that leaves fewer than ~4 waves per CU in flight
+        const int64_t cus0 = compute_units() > 0 ? compute_units() : 256;
+        const int64_t rows0 = pool2x2 ? oh / 2 : oh, wbs0 = (ow + 7) / 8;
+        const int oct = (oc <= 1 || bs * rows0 * wbs0 * ((oc + 1) / 2) < cus0 * 4 * 64) ? 1 : 2;
+        q.ngroups = (oc + oct - 1) / oct;
+        q.ocpad = q.ngroups * oct;
+        q.nwb = (ow + 7) / 8;
+        q.ihp = ih + 2 * ph;
+        int64_t pitch = iw + 2 * pw;
+        if (pitch < q.nwb * 8 + fw - 1) pitch = q.nwb * 8 + fw - 1;
+        // whole 16-byte reads of WT + FW - 1 floats starting at a multiple of 8
+        const int64_t xw4 = ((8 + fw - 1 + 3) / 4) * 4;
+        if (pitch < (q.nwb - 1) * 8 + xw4) pitch = (q.nwb - 1) * 8 + xw4;
+        q.pitch = (int)((pitch + 3) & ~(int64_t)3);
+        q.yh = pool2x2 ? oh / 2 : oh;
+        q.yw = pool2x2 ? ow / 2 : ow;
+        q.nrows = q.yh;
+        const int64_t items = (int64_t)q.nrows * q.nwb * q.ngroups;
+        const int64_t taps = ic * fh * fw;
+        const int64_t w_bytes = ((taps * q.ocpad + 3) & ~(int64_t)3) * 4, img_bytes = (int64_t)ic * q.ihp * q.pitch * 4;
+        constexpr int64_t kLds = 64 * 1024;
+        if (w_bytes + img_bytes <= kLds && items <= ((int64_t)1 << 24)) {
+            const int64_t cus = compute_units() > 0 ? compute_units() : 256;
+            int64_t imgs = items >= 256 ? 1 : 256 / items;
+            while (imgs > 1 && w_bytes + imgs * img_bytes > kLds) --imgs;
+            while (imgs > 1 && (bs + imgs - 1) / imgs < cus) --imgs;
+            if (imgs > bs) imgs = bs;
+            q.imgs = (int)imgs;
+            q.items_per_img = (int)items;
+            q.div_items = FastDiv((uint32_t)items);
+            q.div_rowsxwb = FastDiv((uint32_t)(q.nrows * q.nwb));
+            q.div_nwb = FastDiv((uint32_t)q.nwb);
+            q.div_ocpad = FastDiv((uint32_t)q.ocpad);
+            q.div_pitch = FastDiv((uint32_t)q.pitch);
+            q.div_ihp = FastDiv((uint32_t)q.ihp);
+            const int64_t work = imgs * items;
+            const int threads = work >= 256 ? 256 : (int)((work + 63) / 64 * 64);
+            const int64_t blocks = (bs + imgs - 1) / imgs;
+            if (blocks > 0x7FFFFFFF) return fail(AGH_ERANGE, "%s: too many workgroups", name);
+            const size_t smem = (size_t)(w_bytes + imgs * img_bytes);
+            const dim3 grid((unsigned)blocks), block(threads);
+            const T *xp = (const T *)x, *wp = (const T *)w, *bp = (const T *)bias;
+            T *yp = (T *)y;
+#define AGH_RT(FWV, OCTV, POOLV) \
+    hipLaunchKernelGGL((conv2_rowtile_kernel<T, FWV, OCTV, POOLV>), grid, block, smem, stream(), xp, wp, bp, yp, q)
+            if (fw == 3) {
+                if (oct == 1) { if (pool2x2) AGH_RT(3, 1, true); else AGH_RT(3, 1, false); }
+                else { if (pool2x2) AGH_RT(3, 2, true); else AGH_RT(3, 2, false); }
+            } else {
+                if (oct == 1) { if (pool2x2) AGH_RT(5, 1, true); else AGH_RT(5, 1, false); }
+                else { if (pool2x2) AGH_RT(5, 2, true); else AGH_RT(5, 2, false); }
+            }
+#undef AGH_RT
+            AGH_LAUNCH_CHECK(name);
+            return AGH_OK;
+        }
+    }
 
     ConvParams p;
     p.bs = bs; p.ic = ic; p.ih = ih; p.iw = iw; p.oc = oc; p.oh = oh; p.ow = ow;
@@ -218,6 +617,31 @@ int agh_conv2_direct_bf16(const void *x, const void *w, const void *bias, void *
                           int64_t sw, int64_t dh, int64_t dw, int act, int pool2x2) {
     return conv2_direct_entry<uint16_t>("agh_conv2_direct_bf16", x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, sh,
                                         sw, dh, dw, act, pool2x2);
+}
+
+int agh_lenet5_forward_f32(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                           const void *wd3, const void *b3, void *logits, int64_t bs) {
+    AGH_API_ENTER();
+    if (bs < 0 || bs > ((int64_t)1 << 30)) return fail(AGH_EINVAL, "agh_lenet5_forward_f32: bad batch size");
+    if (bs == 0) return AGH_OK;
+    if (!x || !w1 || !w2 || !wd1 || !wd2 || !wd3 || !b3 || !logits) return fail(AGH_ENULL, "agh_lenet5_forward_f32: null buffer");
+    hipLaunchKernelGGL(lenet5_forward_kernel<float>, dim3((unsigned)((bs + 3) / 4)), dim3(512), 0, stream(),
+                       (const float *)x, (const float *)w1, (const float *)w2, (const float *)wd1, (const float *)wd2,
+                       (const float *)wd3, (const float *)b3, (float *)logits, (int)bs);
+    AGH_LAUNCH_CHECK("agh_lenet5_forward_f32");
+    return AGH_OK;
+}
+int agh_lenet5_forward_bf16(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                            const void *wd3, const void *b3, void *logits, int64_t bs) {
+    AGH_API_ENTER();
+    if (bs < 0 || bs > ((int64_t)1 << 30)) return fail(AGH_EINVAL, "agh_lenet5_forward_bf16: bad batch size");
+    if (bs == 0) return AGH_OK;
+    if (!x || !w1 || !w2 || !wd1 || !wd2 || !wd3 || !b3 || !logits) return fail(AGH_ENULL, "agh_lenet5_forward_bf16: null buffer");
+    hipLaunchKernelGGL(lenet5_forward_kernel<uint16_t>, dim3((unsigned)((bs + 3) / 4)), dim3(512), 0, stream(),
+                       (const uint16_t *)x, (const uint16_t *)w1, (const uint16_t *)w2, (const uint16_t *)wd1,
+                       (const uint16_t *)wd2, (const uint16_t *)wd3, (const uint16_t *)b3, (uint16_t *)logits, (int)bs);
+    AGH_LAUNCH_CHECK("agh_lenet5_forward_bf16");
+    return AGH_OK;
 }
 
 }  // extern "C"

@@ -216,7 +216,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     const int64_t slots = (int64_t)cus;
     int splits = 1;
     const int ktiles = (g.K + BK - 1) / BK;
-    if (tiles * 2 <= slots && ktiles >= 8 && batch == 1) {
+    if (tiles * 2 <= slots && ktiles >= 32 && batch == 1) {
         int64_t s = slots / tiles;
         if (s > ktiles / 4) s = ktiles / 4;
         if (s > 64) s = 64;

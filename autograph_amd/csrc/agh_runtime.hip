@@ -67,6 +67,10 @@ int agh_init(int device_index) {
     if (device_index < 0 || device_index >= count)
         return fail(AGH_EINVAL, "agh_init: device index %d out of range (found %d devices)", device_index, count);
     AGH_HIP(hipSetDevice(device_index));
+    // latency matters for launch-bound work (a LeNet5 inference is tens of microseconds): spin, do not
+    // sleep, in synchronising calls.  Best effort: the flag cannot change once the device is active.
+    (void)hipSetDeviceFlags(hipDeviceScheduleSpin);
+    (void)hipGetLastError();
     hipDeviceProp_t prop;
     AGH_HIP(hipGetDeviceProperties(&prop, device_index));
     g_cus = prop.multiProcessorCount;
@@ -185,7 +189,7 @@ int agh_graph_end(void **graph_exec) {
     AGH_HIP(hipStreamEndCapture(g_stream, &graph));
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    hipGraphDestroy(graph);
+    (void)hipGraphDestroy(graph);
     if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
     *graph_exec = (void *)exec;
     return AGH_OK;

@@ -139,6 +139,23 @@ class LeNet5:
         h = self.dense2.forward(h, relu=True)
         return self.dense3.forward(h)
 
+    def forward_single_launch(self, x, out_ptr=None):
+        """The whole forward pass as ONE kernel (agh_lenet5_forward_*), activations in LDS.  With
+        `out_ptr` (device memory or pinned host memory) the logits go there; else a new tensor."""
+        x = x.as_standard_layout()
+        bs = x.shape[0]
+        if x.shape[1:] != (1, 28, 28):
+            raise AghError(-1, f"LeNet5 expects [bs,1,28,28] inputs, got {x.shape}")
+        out = None
+        if out_ptr is None:
+            out = Tensor.uninit((bs, 10), x.dtype)
+            out_ptr = out._ptr()
+        ws = [self.conv1.weight, self.conv2.weight, self.dense1.weight, self.dense2.weight, self.dense3.weight,
+              self.dense3.bias]
+        check(getattr(lib, f"agh_lenet5_forward_{x.dtype}")(x._data_ptr(), *[w.as_standard_layout()._data_ptr() for w in ws],
+                                                           out_ptr, bs))
+        return out
+
     # -- graph-captured inference on fixed buffers --
     def capture(self, x, host_out_ptr=None):
         """Record `forward_fused` on `x` (and, if given, the device->host copy of the logits into a

@@ -68,8 +68,8 @@ def rand_bf16(orc, rng, shape, std=0.02):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib", action="store_true",
@@ -190,6 +190,74 @@ def main():
             run(f"max_pool2_backward_{dt}_b256x64x56x56", lambda: ag._ffi.check(fn_pb(dx._ptr(), py._ptr(), bs * ci, hw, hw, 2, 2, 2, 2)),
                 es * (2 * nx + ny), "GB/s", PEAK_HBM_GBS)
             del x, wt, cols, dx, py
+
+    # ---------------- LeNet5 f32 inference, batch 1000 (BASELINE configs[0]) ----------------
+    lenet = None
+    if not args.no_extras:
+        try:
+            bsl = 1000
+            xl = rng.uniform(0, 1, (bsl, 1, 28, 28)).astype(np.float32)
+
+            def he(shape, fan_in):  # Uniform(-a, a), a = sqrt(2 / fan_in)
+                a_ = np.sqrt(2.0 / fan_in)
+                return rng.uniform(-a_, a_, shape).astype(np.float32)
+
+            params = [he((6, 1, 5, 5), 25), he((16, 6, 5, 5), 150), he((256, 128), 256), he((128, 84), 128),
+                      he((84, 10), 84), he((10,), 84)]
+            model = ag.LeNet5.from_arrays(*params)
+            txl = ag.Tensor.from_array(xl)
+            host = C.c_void_p()
+            ag._ffi.check(ag.lib.agh_host_alloc(C.byref(host), bsl * 10 * 4))
+            host2 = C.c_void_p()
+            ag._ffi.check(ag.lib.agh_host_alloc(C.byref(host2), bsl * 10 * 4))
+            model.capture(txl, host2.value)  # layered forward (5 launches) + D2H of the logits, as one graph
+
+            def wall(fn, nwarm=100, nrep=1000):
+                for _ in range(nwarm):
+                    fn()
+                t0 = time.perf_counter()
+                for _ in range(nrep):
+                    fn()
+                return (time.perf_counter() - t0) * 1e3 / nrep
+
+            def infer():  # whole network in one launch, logits written straight into pinned host memory
+                model.forward_single_launch(txl, host.value)
+                ag._ffi.check(ag.lib.agh_sync())  # logits are on the host when this returns
+
+            def infer_graph():
+                model.replay()
+                ag._ffi.check(ag.lib.agh_sync())
+
+            gpu_ms = wall(infer)
+            got = np.ctypeslib.as_array(C.cast(host.value, C.POINTER(C.c_float)), shape=(bsl, 10)).copy()
+            graph_ms = wall(infer_graph, 50, 300)
+            _, kernel_ms = timer.time(lambda: model.forward_single_launch(txl, host.value), 50, 20)
+            # layer-by-layer path (12 launches, im2col + gemm convolutions), eager
+            _, layered_ms = timer.time(lambda: model.forward(txl, algorithm="im2col"), 20, 5)
+            lenet = {"gpu_ms": round(gpu_ms, 4), "gpu_kernel_ms": round(kernel_ms, 4), "gpu_graph_5_launches_ms": round(graph_ms, 4),
+                     "gpu_layered_im2col_ms": round(layered_ms, 4),
+                     "what": "gpu_ms: one launch of the whole-network kernel (input resident in HBM, [1000,10] logits written "
+                             "into pinned host memory), wall clock per inference including the host-side wait; "
+                             "gpu_kernel_ms: the same launch between HIP events; gpu_graph_5_launches_ms: graph replay of "
+                             "conv+relu+pool x2 and 3 Dense GEMMs plus D2H"}
+            if not args.no_cpu:
+                thr = orc.max_threads()
+                want = orc.lenet5_forward_f32(xl, *params, direct=True)
+                t0 = time.perf_counter()
+                ncpu = 20
+                for _ in range(ncpu):
+                    orc.lenet5_forward_f32(xl, *params, direct=True)
+                cpu_ms = (time.perf_counter() - t0) * 1e3 / ncpu
+                lenet.update({"cpu_ms": round(cpu_ms, 3), "cpu_threads": thr, "speedup": round(cpu_ms / gpu_ms, 1),
+                              "max_abs_diff_vs_cpu": float(np.abs(got - want).max()),
+                              "cpu_what": "oracle port of the host path: direct f32 convolutions over the batch on all "
+                                          "cores (as conv_direct), blocked sgemm on <=4 threads for Dense"})
+            extras["lenet5_f32_infer_b1000"] = lenet
+            log("lenet5 f32 b=1000:", lenet)
+            del model
+        except Exception as e:
+            extras["lenet5_f32_infer_b1000"] = {"error": str(e)}
+            log("lenet5: FAILED", e)
 
     # ---------------- CPU baseline: the oracle's restatement of the host path ----------------
     cpu = None

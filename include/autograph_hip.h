@@ -192,6 +192,18 @@ int agh_conv2_direct_bf16(const void *x, const void *w, const void *bias, void *
                           int64_t ih, int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw,
                           int64_t sh, int64_t sw, int64_t dh, int64_t dw, int act, int pool2x2);
 
+/* The LeNet5 of the reference's benchmark (benches/neural-network-benches/src/
+ * autograph_backend.rs:88-162) as ONE launch: conv 1->6 5x5, relu, pool 2x2, conv 6->16 5x5, relu,
+ * pool 2x2, flatten, dense 256->128, relu, dense 128->84, relu, dense 84->10 + bias, with all
+ * activations in LDS and rounded to T after every layer like the layer-by-layer path.
+ * x: [bs,1,28,28], w1: [6,1,5,5], w2: [16,6,5,5], wd1: [256,128], wd2: [128,84], wd3: [84,10]
+ * (Dense weights are [inputs, outputs], layer.rs:482-486), b3: [10], logits: [bs,10] - a device
+ * buffer, or pinned host memory from agh_host_alloc so the result needs no separate copy. */
+int agh_lenet5_forward_f32(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                           const void *wd3, const void *b3, void *logits, int64_t bs);
+int agh_lenet5_forward_bf16(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                            const void *wd3, const void *b3, void *logits, int64_t bs);
+
 /* ---------------------------------------------------------------- max pool ---- */
 
 /* MaxPool2 device branch (src/tensor/ops.rs:1117-1133; rule from the host impl

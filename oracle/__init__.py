@@ -67,6 +67,8 @@ _sig("orc_gemm_bf16_hostfold", _g + _v + _v + [_p])
 _sig("orc_gemm_f32_host", _g + [C.c_float] + _v + _v + [C.c_float] + _v + [C.c_int])
 _sig("orc_conv2_naive_f64", [_p, _p, _p] + [_i64] * 13)
 _sig("orc_lenet5_forward_f32", [_p, _i64, _p, _p, _p, _p, _p, _p, _p, C.c_int])
+_sig("orc_lenet5_forward_f32_alg", [_p, _i64, _p, _p, _p, _p, _p, _p, _p, C.c_int, C.c_int])
+_sig("orc_conv2_direct_f32", [_p, _p, _p] + [_i64] * 7)
 _sig("orc_max_threads", [], C.c_int)
 
 
@@ -256,11 +258,23 @@ def conv2_naive_f64(x, w, padding=(0, 0), stride=(1, 1), dilation=(1, 1)):
     return y
 
 
-def lenet5_forward_f32(x, w1, w2, wd1, wd2, wd3, b3, threads=None):
-    """Weights: w1 [6,1,5,5], w2 [16,6,5,5], wd* [in,out] (Dense layout, layer.rs:482-486), b3 [10]."""
+def conv2_direct_f32(x, w):
+    """Host f32 direct convolution, default options (stride 1, no padding, no dilation)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    bs, ic, ih, iw = x.shape
+    oc, _, fh, fw = w.shape
+    y = np.empty((bs, oc, ih - fh + 1, iw - fw + 1), dtype=np.float32)
+    _lib.orc_conv2_direct_f32(_ptr(x), _ptr(w), _ptr(y), bs, ic, ih, iw, oc, fh, fw)
+    return y
+
+
+def lenet5_forward_f32(x, w1, w2, wd1, wd2, wd3, b3, threads=None, direct=False):
+    """Weights: w1 [6,1,5,5], w2 [16,6,5,5], wd* [in,out] (Dense layout, layer.rs:482-486), b3 [10].
+    direct=True runs the convolutions as the reference host does for f32 (conv_direct)."""
     arrs = [np.ascontiguousarray(a, dtype=np.float32) for a in (x, w1, w2, wd1, wd2, wd3, b3)]
     bs = arrs[0].shape[0]
     out = np.empty((bs, 10), dtype=np.float32)
-    _lib.orc_lenet5_forward_f32(_ptr(arrs[0]), bs, *[_ptr(a) for a in arrs[1:]], _ptr(out),
-                                threads or min(4, max_threads()))
+    _lib.orc_lenet5_forward_f32_alg(_ptr(arrs[0]), bs, *[_ptr(a) for a in arrs[1:]], _ptr(out),
+                                    threads or min(4, max_threads()), 1 if direct else 0)
     return out

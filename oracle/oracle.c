@@ -480,18 +480,61 @@ static void conv_im2col_f32(const float *x, const float *w, float *y, i64 bs, i6
     free(out);
 }
 
+/* Host f32 Conv2 for default options as the reference runs it: a direct convolution
+ * (layer.rs:936-943 -> layer/conv_direct.rs:23-83, :760-946), images dealt to threads
+ * (rayon broadcast over the batch), SIMD along the output row.  Restated as an axpy of one
+ * filter tap over one output plane at a time; summation order is (ic, fi, fj) like
+ * conv_direct's, FMA contraction allowed as with its `mul_add` under +fma. */
+__attribute__((optimize("fp-contract=fast")))
+void orc_conv2_direct_f32(const float *x, const float *w, float *y, i64 bs, i64 ic, i64 ih, i64 iw, i64 oc, i64 fh,
+                          i64 fw) {
+    const i64 oh = ih - fh + 1, ow = iw - fw + 1;
+#pragma omp parallel for schedule(static, 1)
+    for (i64 b = 0; b < bs; ++b)
+        for (i64 o = 0; o < oc; ++o) {
+            float *yp = y + (b * oc + o) * oh * ow;
+            for (i64 i = 0; i < oh * ow; ++i) yp[i] = 0.0f;
+            for (i64 c = 0; c < ic; ++c) {
+                const float *xp = x + (b * ic + c) * ih * iw;
+                for (i64 fi = 0; fi < fh; ++fi)
+                    for (i64 fj = 0; fj < fw; ++fj) {
+                        const float wv = w[((o * ic + c) * fh + fi) * fw + fj];
+                        for (i64 ho = 0; ho < oh; ++ho) {
+                            const float *xr = xp + (ho + fi) * iw + fj;
+                            float *yr = yp + ho * ow;
+                            for (i64 wo = 0; wo < ow; ++wo) yr[wo] += wv * xr[wo];
+                        }
+                    }
+            }
+        }
+}
+
+/* direct != 0: convolutions through orc_conv2_direct_f32 (what the reference host does for f32);
+ * direct == 0: through im2col + sgemm (what conv2_im2col does). */
+void orc_lenet5_forward_f32_alg(const float *x, i64 bs, const float *w1, const float *w2, const float *wd1,
+                                const float *wd2, const float *wd3, const float *b3, float *logits, int threads,
+                                int direct);
+
 void orc_lenet5_forward_f32(const float *x, i64 bs, const float *w1, const float *w2, const float *wd1,
                             const float *wd2, const float *wd3, const float *b3, float *logits, int threads) {
+    orc_lenet5_forward_f32_alg(x, bs, w1, w2, wd1, wd2, wd3, b3, logits, threads, 0);
+}
+
+void orc_lenet5_forward_f32_alg(const float *x, i64 bs, const float *w1, const float *w2, const float *wd1,
+                                const float *wd2, const float *wd3, const float *b3, float *logits, int threads,
+                                int direct) {
     float *c1 = (float *)malloc(sizeof(float) * bs * 6 * 24 * 24);
     float *p1 = (float *)malloc(sizeof(float) * bs * 6 * 12 * 12);
     float *c2 = (float *)malloc(sizeof(float) * bs * 16 * 8 * 8);
     float *p2 = (float *)malloc(sizeof(float) * bs * 16 * 4 * 4);
     float *d1 = (float *)malloc(sizeof(float) * bs * 128);
     float *d2 = (float *)malloc(sizeof(float) * bs * 84);
-    conv_im2col_f32(x, w1, c1, bs, 1, 28, 28, 6, 5, 5, threads);
+    if (direct) orc_conv2_direct_f32(x, w1, c1, bs, 1, 28, 28, 6, 5, 5);
+    else conv_im2col_f32(x, w1, c1, bs, 1, 28, 28, 6, 5, 5, threads);
     orc_relu_f32(c1, c1, bs * 6 * 24 * 24);
     orc_max_pool2_f32(c1, p1, bs * 6, 24, 24, 2, 2, 2, 2);
-    conv_im2col_f32(p1, w2, c2, bs, 6, 12, 12, 16, 5, 5, threads);
+    if (direct) orc_conv2_direct_f32(p1, w2, c2, bs, 6, 12, 12, 16, 5, 5);
+    else conv_im2col_f32(p1, w2, c2, bs, 6, 12, 12, 16, 5, 5, threads);
     orc_relu_f32(c2, c2, bs * 16 * 8 * 8);
     orc_max_pool2_f32(c2, p2, bs * 16, 8, 8, 2, 2, 2, 2);
     orc_gemm_f32_host(bs, 256, 128, 1.0f, p2, 0, 256, 1, wd1, 0, 128, 1, 0.0f, d1, 0, 128, 1, threads);

@@ -155,7 +155,7 @@ def test_lenet5_forward_f32(ag, bs):
     tx = ag.Tensor.from_array(x)
     tol = 2e-4 * max(1.0, np.abs(want).max())  # six chained f32 layers, k up to 256
     for name, out in (("im2col", model.forward(tx, algorithm="im2col")), ("direct", model.forward(tx, algorithm="direct")),
-                      ("fused", model.forward_fused(tx))):
+                      ("fused", model.forward_fused(tx)), ("single", model.forward_single_launch(tx))):
         got = out.into_array()
         assert got.shape == (bs, 10)
         assert np.abs(got - want).max() <= tol, (name, np.abs(got - want).max())
@@ -171,6 +171,14 @@ def test_lenet5_forward_f32(ag, bs):
         pinned = np.ctypeslib.as_array(C.cast(host.value, C.POINTER(C.c_float)), shape=(bs, 10)).copy()
         assert np.array_equal(pinned, eager), i
         assert np.array_equal(logits.into_array(), eager), i
+    # single-launch kernel writing straight into pinned host memory
+    single = model.forward_single_launch(tx).into_array()
+    for i in range(3):
+        C.memset(host.value, 0xFF, bs * 10 * 4)
+        model.forward_single_launch(tx, host.value)
+        ag._ffi.check(ag.lib.agh_sync())
+        pinned = np.ctypeslib.as_array(C.cast(host.value, C.POINTER(C.c_float)), shape=(bs, 10)).copy()
+        assert np.array_equal(pinned, single), i
     del model
     ag._ffi.check(ag.lib.agh_host_free(host))
 
@@ -183,7 +191,8 @@ def test_lenet5_forward_bf16(ag, bs):
     want = orc.bf16_to_f32(oracle_lenet_bf16(x, params)).astype(np.float64)
     model = ag.LeNet5.from_arrays(*params)
     tx = ag.Tensor.from_array(x)
-    for name, out in (("im2col", model.forward(tx, algorithm="im2col")), ("fused", model.forward_fused(tx))):
+    for name, out in (("im2col", model.forward(tx, algorithm="im2col")), ("fused", model.forward_fused(tx)),
+                      ("single", model.forward_single_launch(tx))):
         got = orc.bf16_to_f32(out.into_array()).astype(np.float64)
         # every layer may differ from the oracle by one bf16 rounding; six layers compound
         assert np.abs(got - want).max() <= 0.05 * max(1.0, np.abs(want).max()), (name, np.abs(got - want).max())

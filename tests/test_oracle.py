@@ -374,3 +374,15 @@ def test_lenet5_forward_vs_torch():
     h = F.relu(h @ t(wd2).double())
     want = (h @ t(wd3).double() + t(b3).double()).numpy()
     assert np.max(np.abs(got - want)) < 1e-4 * max(1.0, np.max(np.abs(want)))
+    got_direct = orc.lenet5_forward_f32(x, w1, w2, wd1, wd2, wd3, b3, direct=True)
+    assert np.max(np.abs(got_direct - want)) < 1e-4 * max(1.0, np.max(np.abs(want)))
+
+
+def test_conv2_direct_host_vs_torch():
+    rng = np.random.default_rng(9)
+    for (bs, ic, ih, iw, oc, f) in [(3, 1, 28, 28, 6, (5, 5)), (2, 6, 12, 12, 16, (5, 5)), (1, 3, 9, 7, 4, (3, 2))]:
+        x = rng.standard_normal((bs, ic, ih, iw)).astype(np.float32)
+        w = rng.standard_normal((oc, ic) + f).astype(np.float32)
+        want = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double()).numpy()
+        got = orc.conv2_direct_f32(x, w)
+        assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(ic * f[0] * f[1]) * np.max(np.abs(want))
