@@ -43,6 +43,8 @@ __global__ __launch_bounds__(kThreads) void fill_bytes_kernel(uint8_t *dst, uint
 // when the chunk is all channels the workgroup writes ONE contiguous block of
 // ow * c*fh*fw elements with 16-byte stores; the input is read once per (ho, fi) pair and
 // re-reads across neighbouring ho hit L2.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 struct Im2colParams {
     int bs, c, ih, iw, oh, ow;
     int fh, fw, ph, pw, sh, sw, dh, dw;
@@ -50,73 +52,161 @@ struct Im2colParams {
     int nchunk;    // ceil(c / cc)
     int span;      // input columns a row of patches touches: (ow-1)*sw + (fw-1)*dw + 1
     int span_pad;  // LDS row pitch (elements)
+    int nslot;     // 16-byte pieces per image row (vector staging)
+    int npad;      // padding cells per staged row: pw on the left, the rest right of the image
     int ktot;      // c*fh*fw
-    FastDiv div_l, div_ff, div_fw, div_nchunk, div_oh;
+    FastDiv div_l, div_ff, div_fw, div_nchunk, div_oh, div_span, div_fh, div_nslot, div_npad;
 };
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool VSTAGE>
 __global__ __launch_bounds__(kThreads) void im2col_lds_kernel(const T *__restrict__ x, T *__restrict__ y,
                                                                Im2colParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    // layout: int tab[Lmax rounded to 4] | T tile[cc*fh*span_pad]
+    // layout: int tab[L rounded to 4] | T tile[cc*fh*span_pad]
     uint32_t bid = blockIdx.x;
     uint32_t t0, chunk, b, ho;
     p.div_nchunk.divmod(bid, t0, chunk);
     p.div_oh.divmod(t0, b, ho);
     const int c0 = chunk * p.cc;
-    const int ccur = p.cc;  // cc divides c
     const int ff = p.fh * p.fw;
-    const int L = ccur * ff;             // columns this workgroup writes per patch row
-    const int Lmax = p.cc * ff;
+    const int L = p.cc * ff;  // columns this workgroup writes per patch row (cc divides c)
     int *tab = (int *)smem_raw;
-    T *tile = (T *)(smem_raw + (size_t)((Lmax + 3) & ~3) * sizeof(int));
+    T *tile = (T *)(smem_raw + (size_t)((L + 3) & ~3) * sizeof(int));
 
-    // column j = (cl, fi, fj)  ->  LDS offset of its element for wo = 0
+    // Column j = (cl, fi, fj) -> LDS offset of its element for wo = 0.  With vector stores, lane l of a
+    // wave later reads the VEC offsets of its 16-byte group jv with one table read and fetches the VEC
+    // elements one per LDS instruction; were every lane to fetch element u of its group in instruction u,
+    // the lanes of a half-wave would hit every fourth LDS bank only.  So the group's entries are kept
+    // rotated by (l / 8) % 4 dwords: in instruction u the four 8-lane blocks of a half-wave fetch
+    // elements u, u+1, u+2, u+3 (dwords) of their groups, which covers all 32 banks when the row pitch
+    // makes consecutive columns fall in consecutive banks.  The rotation is undone in registers.
     for (int j = threadIdx.x; j < L; j += kThreads) {
         uint32_t cl, r, fi, fj;
         p.div_ff.divmod(j, cl, r);
         p.div_fw.divmod(r, fi, fj);
-        tab[j] = (cl * p.fh + fi) * p.span_pad + fj * p.dw;
+        int slot = j;
+        if constexpr (VEC > 1) {
+            const int jv = j / VEC, u = j % VEC;
+            const int rot = ((jv >> 3) & 3) * (VEC / 4);
+            slot = jv * VEC + ((u - rot + VEC) % VEC);
+        }
+        tab[slot] = (cl * p.fh + fi) * p.span_pad + fj * p.dw;
     }
-    // stage rows: one wave per (channel, fi) row, lanes along the row
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwave = kThreads >> 6;
-    const int nrows = ccur * p.fh;
-    for (int r = wave; r < nrows; r += nwave) {
-        int cl = r / p.fh, fi = r - cl * p.fh;
-        int hidx = -p.ph + fi * p.dh + p.sh * (int)ho;
-        bool hok = hidx >= 0 && hidx < p.ih;
-        const T *src = x + (((size_t)b * p.c + c0 + cl) * p.ih + (hok ? hidx : 0)) * (size_t)p.iw;
-        T *dst = tile + (size_t)r * p.span_pad;
-        for (int j = lane; j < p.span; j += 64) {
-            int widx = j - p.pw;
-            T v = 0;
-            if (hok && widx >= 0 && widx < p.iw) v = src[widx];
-            dst[j] = v;
+    // Stage rows.  The staged space is flattened over the workgroup and walked in batches of SU items
+    // per thread: all SU global loads are issued before the first LDS store, so a thread pays the
+    // memory latency once per batch and not once per item.
+    const uint32_t nrows = (uint32_t)(p.cc * p.fh);
+    if constexpr (VSTAGE) {
+        // Items are 16-byte pieces of the image rows (iw is a whole number of them); the padding cells
+        // left and right of the image are zeroed separately.
+        constexpr int SV = 16 / (int)sizeof(T), SU = 4;
+        const uint32_t nitem = nrows * (uint32_t)p.nslot;
+        for (uint32_t s0 = threadIdx.x; s0 < nitem; s0 += kThreads * SU) {
+            union { u32x4 q; T e[SV]; } v[SU];
+            uint32_t dsto[SU];
+#pragma unroll
+            for (int u = 0; u < SU; ++u) {
+                const uint32_t s = s0 + u * kThreads;
+                uint32_t r, sl, cl, fi;
+                p.div_nslot.divmod(s, r, sl);
+                p.div_fh.divmod(r, cl, fi);
+                const int hidx = -p.ph + (int)fi * p.dh + p.sh * (int)ho;
+                const bool ok = s < nitem && hidx >= 0 && hidx < p.ih;
+                v[u].q = u32x4{0, 0, 0, 0};
+                if (ok) v[u].q = *(const u32x4 *)(x + (((size_t)b * p.c + c0 + cl) * p.ih + hidx) * (size_t)p.iw + sl * SV);
+                dsto[u] = s < nitem ? r * p.span_pad + p.pw + sl * SV : 0xFFFFFFFFu;
+            }
+#pragma unroll
+            for (int u = 0; u < SU; ++u)
+                if (dsto[u] != 0xFFFFFFFFu) {
+#pragma unroll
+                    for (int k = 0; k < SV; ++k) tile[dsto[u] + k] = v[u].e[k];
+                }
+        }
+        const uint32_t npad = nrows * (uint32_t)p.npad;
+        for (uint32_t s = threadIdx.x; s < npad; s += kThreads) {
+            uint32_t r, k;
+            p.div_npad.divmod(s, r, k);
+            tile[r * p.span_pad + ((int)k < p.pw ? k : p.iw + k)] = 0;
+        }
+    } else {
+        const uint32_t nstage = nrows * (uint32_t)p.span;
+        constexpr int SU = 8;
+        for (uint32_t s0 = threadIdx.x; s0 < nstage; s0 += kThreads * SU) {
+            T v[SU];
+            uint32_t dsto[SU];
+#pragma unroll
+            for (int u = 0; u < SU; ++u) {
+                const uint32_t s = s0 + u * kThreads;
+                uint32_t r, j, cl, fi;
+                p.div_span.divmod(s, r, j);
+                p.div_fh.divmod(r, cl, fi);
+                const int hidx = -p.ph + (int)fi * p.dh + p.sh * (int)ho;
+                const int widx = (int)j - p.pw;
+                const bool ok = s < nstage && hidx >= 0 && hidx < p.ih && widx >= 0 && widx < p.iw;
+                v[u] = 0;
+                if (ok) v[u] = x[(((size_t)b * p.c + c0 + cl) * p.ih + hidx) * (size_t)p.iw + widx];
+                dsto[u] = s < nstage ? r * p.span_pad + j : 0xFFFFFFFFu;
+            }
+#pragma unroll
+            for (int u = 0; u < SU; ++u)
+                if (dsto[u] != 0xFFFFFFFFu) tile[dsto[u]] = v[u];
         }
     }
     __syncthreads();
 
     const size_t row0 = ((size_t)b * p.oh + ho) * p.ow;  // first patch row of this workgroup
     T *ybase = y + row0 * p.ktot + (size_t)c0 * ff;
-    const uint32_t total = (uint32_t)p.ow * L;
-    if (VEC > 1) {
-        // every patch-row segment starts 16-byte aligned and has a length that is a multiple of VEC
-        for (uint32_t e = threadIdx.x * VEC; e < total; e += kThreads * VEC) {
-            uint32_t wo, j;
-            p.div_l.divmod(e, wo, j);
-            const int base = wo * p.sw;
-            __align__(16) T vals[VEC];
+    if constexpr (VEC > 1) {
+        // Every patch-row segment starts 16-byte aligned and holds a multiple of VEC elements.  A wave
+        // takes WO_U patch rows at a time (wave-uniform, so the row base lives in scalar registers) and
+        // its lanes walk the 16-byte groups of the segment: one table read serves WO_U stores, and the
+        // per-lane arithmetic is the add of the patch's column base to each table offset plus the
+        // un-rotation of the four dwords.
+        constexpr int WO_U = 2, nwave = kThreads >> 6;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+        const bool rot1 = (lane & 8) != 0, rot2 = (lane & 16) != 0;
+        const int LV = L / VEC;
+        for (int wg = wave * WO_U; wg < p.ow; wg += nwave * WO_U) {
+            for (int jv = lane; jv < LV; jv += 64) {
+                int4 offs[VEC / 4];
 #pragma unroll
-            for (int u = 0; u < VEC; u += 4) {
-                int4 o = *(const int4 *)(tab + j + u);
-                vals[u + 0] = tile[o.x + base];
-                vals[u + 1] = tile[o.y + base];
-                vals[u + 2] = tile[o.z + base];
-                vals[u + 3] = tile[o.w + base];
+                for (int u = 0; u < VEC / 4; ++u) offs[u] = *(const int4 *)(tab + jv * VEC + 4 * u);
+                uint32_t d[WO_U][4];
+#pragma unroll
+                for (int w = 0; w < WO_U; ++w) {
+                    const int base = min(wg + w, p.ow - 1) * p.sw;  // clamped: a duplicate row, not stored
+                    T t[VEC];
+#pragma unroll
+                    for (int u = 0; u < VEC / 4; ++u) {
+                        t[4 * u + 0] = tile[offs[u].x + base];
+                        t[4 * u + 1] = tile[offs[u].y + base];
+                        t[4 * u + 2] = tile[offs[u].z + base];
+                        t[4 * u + 3] = tile[offs[u].w + base];
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if constexpr (sizeof(T) == 4) d[w][k] = (uint32_t)t[k];
+                        else d[w][k] = (uint32_t)t[2 * k] | ((uint32_t)t[2 * k + 1] << 16);
+                    }
+                }
+#pragma unroll
+                for (int w = 0; w < WO_U; ++w) {
+                    uint32_t r[4];
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) r[m] = rot1 ? d[w][(m + 3) & 3] : d[w][m];
+                    u32x4 o;
+                    o.x = rot2 ? r[2] : r[0];
+                    o.y = rot2 ? r[3] : r[1];
+                    o.z = rot2 ? r[0] : r[2];
+                    o.w = rot2 ? r[1] : r[3];
+                    if (wg + w < p.ow)
+                        __builtin_nontemporal_store(o, (u32x4 *)(ybase + (size_t)(wg + w) * p.ktot + jv * VEC));
+                }
             }
-            *(uint4 *)(ybase + (size_t)wo * p.ktot + j) = *(const uint4 *)vals;
         }
     } else {
+        const uint32_t total = (uint32_t)p.ow * L;
         for (uint32_t e = threadIdx.x; e < total; e += kThreads) {
             uint32_t wo, j;
             p.div_l.divmod(e, wo, j);
@@ -171,9 +261,18 @@ int im2col_launch(const char *name, const void *x, void *y, int64_t bs, int64_t 
     p.fh = fh; p.fw = fw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
     p.ktot = c * fh * fw;
     const int64_t span = (ow - 1) * sw + (fw - 1) * dw + 1;
-    const int64_t span_pad = span | 1;  // odd pitch spreads the rows over the LDS banks
     const int ff = fh * fw;
     constexpr int VEC = 16 / sizeof(T);
+    // Vector staging copies whole 16-byte pieces of the image rows: needs rows that are a whole number
+    // of pieces and start on 16 bytes.
+    const bool vstage = iw % VEC == 0 && ((uintptr_t)x & 15) == 0;
+    // LDS row pitch: at least the columns a patch row touches (and the whole padded image row for
+    // vector staging), and congruent to fw modulo the 32 LDS banks (128 bytes), so that column
+    // (cl, fi, fj) of a patch sits fw*(cl*fh+fi)+fj banks after column 0: consecutive patch columns
+    // fall in consecutive banks, which the rotated table of the kernel relies on.
+    constexpr int64_t kBankElems = 128 / sizeof(T);
+    int64_t span_pad = std::max<int64_t>(span, vstage ? pw + iw : 0);
+    span_pad += ((fw - span_pad) % kBankElems + kBankElems) % kBankElems;
     constexpr int64_t kLdsBudget = 48 * 1024;
     auto lds_bytes = [&](int64_t cc) {
         return (int64_t)((cc * ff + 3) & ~3) * 4 + cc * fh * span_pad * (int64_t)sizeof(T);
@@ -204,20 +303,27 @@ int im2col_launch(const char *name, const void *x, void *y, int64_t bs, int64_t 
     p.nchunk = c / cc;
     p.span = span;
     p.span_pad = span_pad;
+    p.nslot = iw / VEC;
+    p.npad = pw + std::max<int64_t>(0, span - pw - iw);
     p.div_l = FastDiv((uint32_t)(cc * ff));
     p.div_ff = FastDiv((uint32_t)ff);
     p.div_fw = FastDiv((uint32_t)fw);
     p.div_nchunk = FastDiv((uint32_t)p.nchunk);
     p.div_oh = FastDiv((uint32_t)oh);
+    p.div_fh = FastDiv((uint32_t)fh);
+    p.div_span = FastDiv((uint32_t)span);
+    p.div_nslot = FastDiv((uint32_t)std::max(1, p.nslot));
+    p.div_npad = FastDiv((uint32_t)std::max(1, p.npad));
     const int64_t nblocks = bs * oh * p.nchunk;
     if (nblocks > 0x7FFFFFFFll) return fail(AGH_ERANGE, "%s: too many workgroups", name);
     const size_t smem = (size_t)lds_bytes(cc);
-    if (vec)
-        hipLaunchKernelGGL((im2col_lds_kernel<T, VEC>), dim3((unsigned)nblocks), dim3(kThreads), smem, stream(),
-                           (const T *)x, (T *)y, p);
-    else
-        hipLaunchKernelGGL((im2col_lds_kernel<T, 1>), dim3((unsigned)nblocks), dim3(kThreads), smem, stream(),
-                           (const T *)x, (T *)y, p);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)nblocks), dim3(kThreads), smem, stream(), (const T *)x, (T *)y, p);
+    };
+    if (vec && vstage) launch(im2col_lds_kernel<T, VEC, true>);
+    else if (vec) launch(im2col_lds_kernel<T, VEC, false>);
+    else if (vstage) launch(im2col_lds_kernel<T, 1, true>);
+    else launch(im2col_lds_kernel<T, 1, false>);
     AGH_LAUNCH_CHECK(name);
     return AGH_OK;
 }
