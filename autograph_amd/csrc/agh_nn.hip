@@ -375,6 +375,331 @@ __global__ __launch_bounds__(kThreads) void col2im_gather_kernel(const T *__rest
     y[e] = acc;
 }
 
+// Streaming form, used whenever its tiles fit in LDS.  One workgroup owns a band of image rows of
+// one image and a chunk of cc channels and walks the patch rows hi that touch the band in ascending
+// order.  Per step it copies the cc*fh*fw-wide segments of the gw patches of that patch row into LDS
+// with coalesced 4-byte loads (requested one step ahead, held in registers meanwhile), then every
+// thread adds, for the pixel columns (channel, wy) it owns, the entries that fall on them: taps fj
+// descending = patch column wi ascending.  Sums live in an LDS ring of (fh-1)*dh+1 image rows per
+// column; a row is final once the walk has passed its last patch row, and is then written out and
+// its ring slot cleared.  Each patch entry is read from HBM exactly once (plus the fh-1 patch rows
+// that two neighbouring bands both need), and the order of the adds per pixel is the host's.
+struct Col2imRingParams {
+    int c, gh, gw, ih, iw;  // patch grid gh x gw, image ih x iw
+    int fh, fw, ph, pw, sh, sw, dh, dw;
+    int ktot, cc, nchunk, nband, band_rows;
+    int ngroup;  // images * bands
+    int rows;    // patch rows per step (unit-stride kernel)
+    int lw;     // 32-bit words per patch segment (cc*fh*fw elements)
+    int pitch;  // LDS pitch of a staged segment (elements); an odd number of words
+    int rh;     // ring rows
+    FastDiv div_nchunk, div_nband, div_iw, div_lw, div_sw, div_rh;
+};
+
+constexpr int kCol2imPrefetch = 32;  // 32-bit words a thread holds for the next step
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void col2im_ring_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                                Col2imRingParams p) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    constexpr int PF = kCol2imPrefetch;
+    constexpr int EPW = 4 / (int)sizeof(T);  // elements per 32-bit word
+    const int tid = threadIdx.x;
+    const int ncol = p.cc * p.iw;
+    uint32_t *ring = (uint32_t *)smem_raw;  // [rh][ncol], one 32-bit slot per running sum
+    T *stage = (T *)(ring + p.rh * ncol);   // [gw][pitch]
+    uint32_t *stage32 = (uint32_t *)stage;
+    uint32_t t0, band, chunk, b;
+    p.div_nband.divmod(blockIdx.x, t0, band);
+    p.div_nchunk.divmod(t0, b, chunk);
+    const int c0 = chunk * p.cc, ff = p.fh * p.fw;
+    const int hy0 = band * p.band_rows, hy1 = min(p.ih, hy0 + p.band_rows);
+    // patch rows whose window [hi*sh - ph, hi*sh - ph + (fh-1)*dh] meets [hy0, hy1)
+    const int lo_num = hy0 + p.ph - (p.fh - 1) * p.dh;
+    const int hi_lo = lo_num <= 0 ? 0 : (lo_num + p.sh - 1) / p.sh;
+    const int hi_hi = min(p.gh - 1, (hy1 - 1 + p.ph) / p.sh);
+
+    for (int i = tid; i < p.rh * ncol; i += kThreads) ring[i] = 0;
+
+    const uint32_t nwords = (uint32_t)p.gw * p.lw;
+    const int ktotw = p.ktot / EPW, pitchw = p.pitch / EPW;
+    uint32_t reg[PF];
+    auto prefetch = [&](int hi) {
+        const uint32_t *src = (const uint32_t *)(x + ((size_t)b * p.gh + hi) * p.gw * p.ktot + (size_t)c0 * ff);
+#pragma unroll
+        for (int i = 0; i < PF; ++i) {
+            const uint32_t e = tid + i * kThreads;
+            uint32_t wi, k;
+            p.div_lw.divmod(e, wi, k);
+            reg[i] = 0;
+            if (e < nwords) reg[i] = __builtin_nontemporal_load(src + (size_t)wi * ktotw + k);
+        }
+    };
+    auto slot_to = [](uint32_t v) -> T {
+        if constexpr (sizeof(T) == 4) return __uint_as_float(v);
+        else return (T)v;
+    };
+    auto to_slot = [](T v) -> uint32_t {
+        if constexpr (sizeof(T) == 4) return __float_as_uint(v);
+        else return (uint32_t)v;
+    };
+
+    if (hi_lo <= hi_hi) prefetch(hi_lo);
+    int next_flush = hy0;
+    for (int hi = hi_lo; hi <= hi_hi; ++hi) {
+        __syncthreads();  // the previous step's reads of the stage (and the clearing of the ring) are done
+#pragma unroll
+        for (int i = 0; i < PF; ++i) {
+            const uint32_t e = tid + i * kThreads;
+            uint32_t wi, k;
+            p.div_lw.divmod(e, wi, k);
+            if (e < nwords) stage32[wi * pitchw + k] = reg[i];
+        }
+        __syncthreads();
+        if (hi < hi_hi) prefetch(hi + 1);
+        const int start = hi * p.sh - p.ph;
+        const int fend = hi == hi_hi ? hy1 : min(hy1, start + p.sh);
+        for (int col = tid; col < ncol; col += kThreads) {
+            uint32_t cl, wy;
+            p.div_iw.divmod((uint32_t)col, cl, wy);
+            const T *sc = stage + cl * ff;
+            for (int fi = 0; fi < p.fh; ++fi) {
+                const int hy = start + fi * p.dh;
+                if (hy < hy0 || hy >= hy1) continue;
+                const int slot = (int)(hy - p.div_rh.div((uint32_t)hy) * p.rh) * ncol + col;
+                T acc = slot_to(ring[slot]);
+                for (int fj = p.fw - 1; fj >= 0; --fj) {
+                    const int tw = (int)wy + p.pw - fj * p.dw;
+                    if (tw < 0) continue;
+                    uint32_t wi, rw;
+                    p.div_sw.divmod((uint32_t)tw, wi, rw);
+                    if (rw != 0 || wi >= (uint32_t)p.gw) continue;
+                    const T v = sc[wi * p.pitch + fi * p.fw + fj];
+                    acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(v));
+                }
+                ring[slot] = to_slot(acc);
+            }
+            // rows no later patch row reaches: write them out; rows outside the window got nothing
+            T *yc = y + (((size_t)b * p.c + c0 + cl) * p.ih) * (size_t)p.iw + wy;
+            for (int hy = next_flush; hy < fend; ++hy) {
+                T val = Elem<T>::zero();
+                if (hy >= start && hy < start + p.rh) {
+                    const int slot = (int)(hy - p.div_rh.div((uint32_t)hy) * p.rh) * ncol + col;
+                    val = slot_to(ring[slot]);
+                    ring[slot] = 0;
+                }
+                yc[(size_t)hy * p.iw] = val;
+            }
+        }
+        next_flush = max(next_flush, fend);
+    }
+    // band rows no patch row touches at all
+    for (int col = tid; col < ncol; col += kThreads) {
+        uint32_t cl, wy;
+        p.div_iw.divmod((uint32_t)col, cl, wy);
+        T *yc = y + (((size_t)b * p.c + c0 + cl) * p.ih) * (size_t)p.iw + wy;
+        for (int hy = next_flush; hy < hy1; ++hy) yc[(size_t)hy * p.iw] = Elem<T>::zero();
+    }
+}
+
+// Unit stride and dilation, square filter known at compile time: the streaming form with everything
+// the general kernel computes per tap hoisted or folded.  The stage carries FW-1-pw all-zero segments
+// on either side, so a tap never has to ask whether its patch column exists (adding +0 to a running
+// sum changes nothing: a sum that starts at +0 can never be -0).  The F running sums of a pixel
+// column sit in registers and move down one place per step, the finished one leaving for memory.
+// Per thread and step: eight 16-byte loads, the stage write, and per owned pixel column F*F LDS
+// reads and adds.
+// Workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its own; the chunks of one
+// (image, band) share cache lines where their segments meet, so they are given ids 8 apart: same
+// XCD, dispatched together.
+template <typename T, int F>
+__global__ __launch_bounds__(kThreads) void col2im_ring_unit_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                                     Col2imRingParams p) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    constexpr int PFV = kCol2imPrefetch / 4;  // 16-byte vectors a thread holds for the next step
+    constexpr int EPW = 4 / (int)sizeof(T);
+    constexpr int NCOL = 4;                   // pixel columns per thread (cc*iw <= NCOL*kThreads)
+    const int tid = threadIdx.x;
+    const int ncol = p.cc * p.iw;
+    const int padl = max(0, F - 1 - p.pw);
+    T *stage = (T *)smem_raw;                 // [gw + 2*padl][pitch]
+    uint32_t *stage32 = (uint32_t *)stage;
+    uint32_t slot8, chunk, b, band;
+    p.div_nchunk.divmod(blockIdx.x >> 3, slot8, chunk);
+    const uint32_t group = slot8 * 8 + (blockIdx.x & 7);  // (image, band) pair
+    if (group >= (uint32_t)p.ngroup) return;
+    p.div_nband.divmod(group, b, band);
+    constexpr int ff = F * F;
+    const int c0 = chunk * p.cc;
+    const int hy0 = band * p.band_rows, hy1 = min(p.ih, hy0 + p.band_rows);
+    const int hi_lo = max(0, hy0 + p.ph - (F - 1));
+    const int hi_hi = min(p.gh - 1, hy1 - 1 + p.ph);
+    const int ktotw = p.ktot / EPW, pitchw = p.pitch / EPW;
+
+    for (int r = 0; r < p.rows; ++r)
+        for (int i = tid; i < padl * pitchw; i += kThreads) {
+            stage32[r * (p.gw + 2 * padl) * pitchw + i] = 0;
+            stage32[(r * (p.gw + 2 * padl) + p.gw + padl) * pitchw + i] = 0;
+        }
+
+    // launch-constant per-thread offsets.  A step takes `rows` patch rows; vector slot i of a thread
+    // belongs to patch row i / per_row of the step (wave-uniform), so its base pointer is a scalar.
+    const int lv = p.lw / 4;
+    const uint32_t nvec = (uint32_t)p.gw * lv;
+    const int per_row = (nvec + kThreads - 1) / kThreads, rows = p.rows;
+    const int nseg = p.gw + 2 * padl;
+    uint32_t src_off[PFV], dst_off[PFV];
+#pragma unroll
+    for (int i = 0; i < PFV; ++i) {
+        const int r = i / per_row;
+        const uint32_t e = tid + (i - r * per_row) * kThreads;
+        uint32_t wi, kv;
+        p.div_lw.divmod(e, wi, kv);  // divides by lv for this kernel
+        src_off[i] = (e < nvec && r < rows) ? wi * ktotw + kv * 4 : 0xFFFFFFFFu;
+        dst_off[i] = (r * nseg + wi + padl) * pitchw + kv * 4;
+    }
+    int tap_base[NCOL];
+    T *ycol[NCOL];
+    T acc[NCOL][F];
+#pragma unroll
+    for (int j = 0; j < NCOL; ++j) {
+        const int col = tid + j * kThreads;
+        uint32_t cl, wy;
+        p.div_iw.divmod((uint32_t)min(col, ncol - 1), cl, wy);
+        // element offset of tap fj = 0 of filter row 0; tap (fi, fj) is at + fi*F - fj*(pitch-1)
+        tap_base[j] = ((int)wy + p.pw + padl) * p.pitch + (int)cl * ff;
+        ycol[j] = y + (((size_t)b * p.c + c0 + cl) * p.ih) * (size_t)p.iw + wy;
+#pragma unroll
+        for (int fi = 0; fi < F; ++fi) acc[j][fi] = Elem<T>::zero();
+    }
+    const int tap_step = p.pitch - 1;
+
+    u32x4 reg[PFV];
+    auto prefetch = [&](int hi) {
+#pragma unroll
+        for (int i = 0; i < PFV; ++i) {
+            const int r = i / per_row;
+            // rows past the last one re-read it (never used): keeps the loads unconditional per row
+            const int hr = min(hi + r, hi_hi);
+            const uint32_t *src = (const uint32_t *)(x + ((size_t)b * p.gh + hr) * p.gw * p.ktot + (size_t)c0 * ff);
+            if (src_off[i] != 0xFFFFFFFFu) reg[i] = __builtin_nontemporal_load((const u32x4 *)(src + src_off[i]));
+        }
+    };
+
+    if (hi_lo <= hi_hi) prefetch(hi_lo);
+    for (int hi0 = hi_lo; hi0 <= hi_hi; hi0 += rows) {
+        __syncthreads();  // the previous step's reads of the stage are done
+#pragma unroll
+        for (int i = 0; i < PFV; ++i)
+            if (src_off[i] != 0xFFFFFFFFu) {
+                stage32[dst_off[i] + 0] = reg[i].x;
+                stage32[dst_off[i] + 1] = reg[i].y;
+                stage32[dst_off[i] + 2] = reg[i].z;
+                stage32[dst_off[i] + 3] = reg[i].w;
+            }
+        __syncthreads();
+        if (hi0 + rows <= hi_hi) prefetch(hi0 + rows);
+        for (int r = 0; r < rows && hi0 + r <= hi_hi; ++r) {
+            // acc[j][fi] is the running sum of image row start + fi
+            const int hi = hi0 + r;
+            const int start = hi - p.ph;
+            const bool last = hi == hi_hi;
+            const T *st = stage + r * nseg * p.pitch;
+#pragma unroll
+            for (int j = 0; j < NCOL; ++j) {
+                const int col = tid + j * kThreads;
+                if (col < ncol) {
+#pragma unroll
+                    for (int fi = 0; fi < F; ++fi) {
+                        const int hy = start + fi;
+                        if (hy >= hy0 && hy < hy1) {  // wave-uniform
+#pragma unroll
+                            for (int fj = F - 1; fj >= 0; --fj) {
+                                const T v = st[tap_base[j] - fj * tap_step + fi * F];
+                                acc[j][fi] = Elem<T>::from_f32(Elem<T>::to_f32(acc[j][fi]) + Elem<T>::to_f32(v));
+                            }
+                        }
+                    }
+                    // row `start` gets nothing from later patch rows; after the last patch row all rows are final
+                    if (start >= hy0 && start < hy1) ycol[j][(size_t)start * p.iw] = acc[j][0];
+                    if (last) {
+#pragma unroll
+                        for (int fi = 1; fi < F; ++fi)
+                            if (start + fi >= hy0 && start + fi < hy1) ycol[j][(size_t)(start + fi) * p.iw] = acc[j][fi];
+                    }
+#pragma unroll
+                    for (int fi = 0; fi + 1 < F; ++fi) acc[j][fi] = acc[j][fi + 1];
+                    acc[j][F - 1] = Elem<T>::zero();
+                }
+            }
+        }
+    }
+}
+
+// Picks the chunk/band split of the streaming kernel; false when the geometry does not fit.
+template <typename T>
+bool col2im_ring_plan(Col2imRingParams &p, size_t &smem, int64_t &nblocks, bool unit, const void *x, int64_t bs, int64_t c,
+                      int64_t gh, int64_t gw, int64_t ih, int64_t iw, int64_t fh, int64_t fw, int64_t ph, int64_t pw,
+                      int64_t sh, int64_t sw, int64_t dh, int64_t dw) {
+    constexpr int64_t es = sizeof(T), epw = 4 / es;
+    const int64_t ff = fh * fw, ktot = c * ff;
+    if (((uintptr_t)x & 3) != 0 || ktot % epw != 0) return false;
+    // the unit-stride kernel loads 16-byte vectors and carries zero segments around the stage
+    if (unit && (((uintptr_t)x & 15) != 0 || (ktot * es) % 16 != 0)) return false;
+    const int64_t segs = unit ? gw + 2 * std::max<int64_t>(0, fw - 1 - pw) : gw;
+    const int64_t rh = (fh - 1) * dh + 1;
+    constexpr int64_t kLdsBudget = 48 * 1024;
+    int64_t cc = 0, lds = 0, pitch = 0, nrows = 1;
+    for (int64_t d = c; d >= 1; --d) {
+        if (c % d != 0 || (d * ff) % epw != 0) continue;
+        if (unit && ((d * ff * es) % 16 != 0 || d * iw > 4 * kThreads)) continue;
+        const int64_t lw = d * ff / epw;
+        if (gw * lw > (int64_t)kThreads * kCol2imPrefetch) continue;
+        const int64_t pitchw = lw | 1;  // odd: threads of a wave walk patches, i.e. whole pitches
+        int64_t need = rh * d * iw * 4 + segs * pitchw * 4;
+        if (unit) {
+            // as many patch rows per step as the prefetch registers and 40 KB of LDS hold
+            const int64_t per_row = (gw * (lw / 4) + kThreads - 1) / kThreads;
+            nrows = std::max<int64_t>(1, std::min<int64_t>({(int64_t)(kCol2imPrefetch / 4) / per_row, gh,
+                                                             (40 * 1024) / (segs * pitchw * 4)}));
+            need = nrows * segs * pitchw * 4;
+        }
+        if (need > kLdsBudget) continue;
+        cc = d; lds = need; pitch = pitchw * epw;
+        break;
+    }
+    if (cc == 0) return false;
+    const int64_t nchunk = c / cc;
+    const int64_t cus = compute_units() > 0 ? compute_units() : 256;
+    const int64_t resident = cus * std::min<int64_t>(unit ? 4 : 2, (160 * 1024) / lds);  // registers allow 4 / 2
+    // bands: more of them fill the chip, fewer of them re-read fewer boundary patch rows
+    int64_t best_nb = 1, best_cost = -1;
+    for (int64_t nb = 1; nb <= std::min<int64_t>(ih, 32); ++nb) {
+        const int64_t rows = (ih + nb - 1) / nb;
+        if ((ih + rows - 1) / rows != nb) continue;  // would leave an empty band
+        const int64_t steps = ((rows + (fh - 1) * dh) / sh + nrows) / nrows;
+        const int64_t waves = (bs * nchunk * nb + resident - 1) / resident;
+        const int64_t cost = waves * (steps + 2);
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_nb = nb; }
+    }
+    nblocks = unit ? ((bs * best_nb + 7) / 8) * 8 * nchunk : bs * nchunk * best_nb;
+    p.ngroup = bs * best_nb;
+    p.rows = nrows;
+    if (nblocks > 0x7FFFFFFFll) return false;
+    p.c = c; p.gh = gh; p.gw = gw; p.ih = ih; p.iw = iw;
+    p.fh = fh; p.fw = fw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+    p.ktot = ktot; p.cc = cc; p.nchunk = nchunk; p.nband = best_nb; p.band_rows = (ih + best_nb - 1) / best_nb;
+    p.lw = cc * ff / epw; p.pitch = pitch; p.rh = rh;
+    p.div_nchunk = FastDiv((uint32_t)nchunk);
+    p.div_nband = FastDiv((uint32_t)best_nb);
+    p.div_iw = FastDiv((uint32_t)iw);
+    p.div_lw = FastDiv((uint32_t)(unit ? p.lw / 4 : p.lw));
+    p.div_sw = FastDiv((uint32_t)sw);
+    p.div_rh = FastDiv((uint32_t)rh);
+    smem = (size_t)lds;
+    return true;
+}
+
 template <typename T>
 int col2im_launch(const char *name, const void *x, void *y, int64_t bs, int64_t c, int64_t ih, int64_t iw,
                   int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t sh, int64_t sw, int64_t dh, int64_t dw) {
@@ -393,6 +718,32 @@ int col2im_launch(const char *name, const void *x, void *y, int64_t bs, int64_t 
     Col2imParams p;
     p.bs = bs; p.c = c; p.ih = ih; p.iw = iw; p.oh = oh; p.ow = ow;
     p.fh = fh; p.fw = fw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+    {
+        Col2imRingParams rp;
+        size_t smem = 0;
+        int64_t nblocks = 0;
+        const bool unit_geom = sh == 1 && sw == 1 && dh == 1 && dw == 1 && fh == fw &&
+                               (fh == 1 || fh == 2 || fh == 3 || fh == 5 || fh == 7);
+        auto launch = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3((unsigned)nblocks), dim3(kThreads), smem, stream(), (const T *)x, (T *)y, rp);
+        };
+        if (unit_geom && col2im_ring_plan<T>(rp, smem, nblocks, true, x, bs, c, ih, iw, oh, ow, fh, fw, ph, pw, sh, sw, dh, dw)) {
+            switch (fh) {
+                case 1: launch(col2im_ring_unit_kernel<T, 1>); break;
+                case 2: launch(col2im_ring_unit_kernel<T, 2>); break;
+                case 3: launch(col2im_ring_unit_kernel<T, 3>); break;
+                case 5: launch(col2im_ring_unit_kernel<T, 5>); break;
+                default: launch(col2im_ring_unit_kernel<T, 7>); break;
+            }
+            AGH_LAUNCH_CHECK(name);
+            return AGH_OK;
+        }
+        if (col2im_ring_plan<T>(rp, smem, nblocks, false, x, bs, c, ih, iw, oh, ow, fh, fw, ph, pw, sh, sw, dh, dw)) {
+            launch(col2im_ring_kernel<T>);
+            AGH_LAUNCH_CHECK(name);
+            return AGH_OK;
+        }
+    }
     p.ktot = c * fh * fw;
     p.div_ow = FastDiv((uint32_t)ow);
     p.div_oh = FastDiv((uint32_t)oh);
