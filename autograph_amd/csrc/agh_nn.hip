@@ -9,6 +9,7 @@ using namespace agh;
 namespace {
 
 constexpr int kThreads = 256;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 inline int64_t conv_out(int64_t i, int64_t f, int64_t p, int64_t s, int64_t d) {
     return (i + 2 * p - d * (f - 1) - 1) / s + 1;
@@ -27,9 +28,9 @@ __global__ __launch_bounds__(kThreads) void fill_bytes_kernel(uint8_t *dst, uint
     size_t tail = bytes - head - body * 16;
     size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     size_t stride = (size_t)gridDim.x * blockDim.x;
-    uint4 v = make_uint4(pattern, pattern, pattern, pattern);
-    uint4 *mid = (uint4 *)(dst + head);
-    for (size_t i = tid; i < body; i += stride) mid[i] = v;
+    const u32x4 v = {pattern, pattern, pattern, pattern};
+    uint8_t *mid = dst + head;
+    for (size_t i = tid; i < body; i += stride) __builtin_nontemporal_store(v, (u32x4 *)mid + i);
     if (tid < head) dst[tid] = (uint8_t)pattern;
     if (tid < tail) dst[head + body * 16 + tid] = (uint8_t)pattern;
 }
@@ -43,8 +44,6 @@ __global__ __launch_bounds__(kThreads) void fill_bytes_kernel(uint8_t *dst, uint
 // when the chunk is all channels the workgroup writes ONE contiguous block of
 // ow * c*fh*fw elements with 16-byte stores; the input is read once per (ho, fi) pair and
 // re-reads across neighbouring ho hit L2.
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
 struct Im2colParams {
     int bs, c, ih, iw, oh, ow;
     int fh, fw, ph, pw, sh, sw, dh, dw;
@@ -816,6 +815,105 @@ __global__ __launch_bounds__(kThreads) void max_pool2_backward_kernel(T *__restr
         }
 }
 
+// 2x2 windows, stride 2, rows a multiple of 8 elements: one thread takes four neighbouring windows of
+// an output row, i.e. 8 input elements from each of two rows, with 16-byte accesses.  Same visiting
+// order inside a window as the general kernel: (0,0), (0,1), (1,0), (1,1), strictly-greater wins.
+template <typename T>
+struct Row8 {
+    T e[8];
+};
+template <typename T>
+__device__ __forceinline__ Row8<T> load_row8(const T *p) {
+    Row8<T> r;
+    if constexpr (sizeof(T) == 4) {
+        *(u32x4 *)&r.e[0] = __builtin_nontemporal_load((const u32x4 *)p);
+        *(u32x4 *)&r.e[4] = __builtin_nontemporal_load((const u32x4 *)p + 1);
+    } else {
+        *(u32x4 *)&r.e[0] = __builtin_nontemporal_load((const u32x4 *)p);
+    }
+    return r;
+}
+template <typename T>
+__device__ __forceinline__ void store_row8(T *p, const Row8<T> &r) {
+    if constexpr (sizeof(T) == 4) {
+        *((u32x4 *)p) = *(const u32x4 *)&r.e[0];
+        *((u32x4 *)p + 1) = *(const u32x4 *)&r.e[4];
+    } else {
+        *((u32x4 *)p) = *(const u32x4 *)&r.e[0];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void max_pool2_2x2_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                                  PoolParams p, size_t groups) {
+    const size_t g = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (g >= groups) return;
+    const uint32_t gpr = (uint32_t)p.ow >> 2;  // groups per output row
+    const size_t orow = g / gpr;               // plane * oh + ho
+    const uint32_t gi = (uint32_t)(g - orow * gpr);
+    const size_t plane = orow / p.oh;
+    const uint32_t ho = (uint32_t)(orow - plane * p.oh);
+    const T *src = x + (plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)gi * 8;
+    const Row8<T> r0 = load_row8(src), r1 = load_row8(src + p.iw);
+    __align__(16) T out[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        T m = r0.e[2 * k];
+        float mf = Elem<T>::to_f32(m);
+        const T c[3] = {r0.e[2 * k + 1], r1.e[2 * k], r1.e[2 * k + 1]};
+#pragma unroll
+        for (int q = 0; q < 3; ++q) {
+            const float vf = Elem<T>::to_f32(c[q]);
+            if (vf > mf) { m = c[q]; mf = vf; }
+        }
+        out[k] = m;
+    }
+    T *dst = y + orow * p.ow + (size_t)gi * 4;
+    if constexpr (sizeof(T) == 4) *(u32x4 *)dst = *(const u32x4 *)out;
+    else *(uint2 *)dst = *(const uint2 *)out;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void max_pool2_backward_2x2_kernel(T *__restrict__ dx, const T *__restrict__ dy,
+                                                                           PoolParams p, size_t groups) {
+    const size_t g = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (g >= groups) return;
+    const uint32_t gpr = (uint32_t)p.ow >> 2;
+    const size_t orow = g / gpr;
+    const uint32_t gi = (uint32_t)(g - orow * gpr);
+    const size_t plane = orow / p.oh;
+    const uint32_t ho = (uint32_t)(orow - plane * p.oh);
+    T *win = dx + (plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)gi * 8;
+    Row8<T> r0 = load_row8(win), r1 = load_row8(win + p.iw);
+    __align__(16) T gy[4];
+    const T *gsrc = dy + orow * p.ow + (size_t)gi * 4;
+    if constexpr (sizeof(T) == 4) *(u32x4 *)gy = *(const u32x4 *)gsrc;
+    else *(uint2 *)gy = *(const uint2 *)gsrc;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float mf = Elem<T>::to_f32(r0.e[2 * k]);
+        int am = 0;
+        const T c[3] = {r0.e[2 * k + 1], r1.e[2 * k], r1.e[2 * k + 1]};
+#pragma unroll
+        for (int q = 0; q < 3; ++q) {
+            const float vf = Elem<T>::to_f32(c[q]);
+            if (vf > mf) { mf = vf; am = q + 1; }
+        }
+        // `0 + dy` in T, as the host's `+=` on the zeroed cell computes it
+        const T gv = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(gy[k]));
+        r0.e[2 * k] = am == 0 ? gv : Elem<T>::zero();
+        r0.e[2 * k + 1] = am == 1 ? gv : Elem<T>::zero();
+        r1.e[2 * k] = am == 2 ? gv : Elem<T>::zero();
+        r1.e[2 * k + 1] = am == 3 ? gv : Elem<T>::zero();
+    }
+    store_row8(win, r0);
+    store_row8(win + p.iw, r1);
+}
+
+inline bool pool_2x2_fast(const PoolParams &p, const void *a, const void *b) {
+    return p.h == 2 && p.w == 2 && p.sh == 2 && p.sw == 2 && p.iw % 8 == 0 && (((uintptr_t)a | (uintptr_t)b) & 15) == 0;
+}
+
 // Overlapping windows: the host visits windows of a plane one after another and each sees
 // what the previous ones wrote, so a plane is walked by a single thread.
 template <typename T>
@@ -868,6 +966,13 @@ int max_pool2_launch(const char *name, const void *x, void *y, int64_t bc, int64
     if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
     size_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
+    if (pool_2x2_fast(p, x, y)) {
+        const size_t groups = total / 4;
+        hipLaunchKernelGGL(max_pool2_2x2_kernel<T>, dim3((unsigned)((groups + kThreads - 1) / kThreads)), dim3(kThreads),
+                           0, stream(), (const T *)x, (T *)y, p, groups);
+        AGH_LAUNCH_CHECK(name);
+        return AGH_OK;
+    }
     hipLaunchKernelGGL(max_pool2_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(), (const T *)x,
                        (T *)y, p, total);
     AGH_LAUNCH_CHECK(name);
@@ -883,7 +988,11 @@ int max_pool2_backward_launch(const char *name, void *dx, const void *dy, int64_
     const size_t total = (size_t)bc * p.oh * p.ow;
     if (total == 0) return AGH_OK;
     if (!dx || !dy) return fail(AGH_ENULL, "%s: null buffer", name);
-    if (sh >= h && sw >= w) {
+    if (pool_2x2_fast(p, dx, dy) && total / 4 <= 0x7FFFFFFFull * kThreads) {
+        const size_t groups = total / 4;
+        hipLaunchKernelGGL(max_pool2_backward_2x2_kernel<T>, dim3((unsigned)((groups + kThreads - 1) / kThreads)),
+                           dim3(kThreads), 0, stream(), (T *)dx, (const T *)dy, p, groups);
+    } else if (sh >= h && sw >= w) {
         size_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
         hipLaunchKernelGGL(max_pool2_backward_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(),
