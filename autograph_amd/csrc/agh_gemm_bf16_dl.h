@@ -293,47 +293,73 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
         // carries no bias or activation state through its unrolled body
         auto staged = [&](auto plainc) {
             constexpr bool PLAIN = decltype(plainc)::value;
+            // A bias along p (C's unit-stride axis) is added after the transposition, where a lane
+            // holds 8 consecutive p of a row and needs the same 8 bias values for every row it stores:
+            // they are loaded once.  (bias and activation act on the already rounded product, so the
+            // result is the same as applying them before staging.)
+            const int chunk = lane % CPRW;
+            T bp[8];
+            if constexpr (!PLAIN) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    bp[e] = 0;
+                    if (has_bias && bias_p) bp[e] = bias[(int64_t)min(pwb + chunk * 8 + e, g.NP - 1) * g.bias_stride];
+                }
+            }
+            const bool post_bias = has_bias && bias_p, relu = g.act == AGH_ACT_RELU;
             static_for<TQ>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 T bq = 0;
+                bool pre_bias = false;
                 if constexpr (!PLAIN) {
                     const int q = qwb + j * 32 + (int)lrow;
-                    if (q < g.NQ && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
+                    pre_bias = has_bias && !bias_p;
+                    if (q < g.NQ && pre_bias) bq = bias[(int64_t)q * g.bias_stride];
                 }
                 static_for<TP>([&](auto ic) {
                     constexpr int i = decltype(ic)::value;
                     static_for<4>([&](auto bc) {
                         constexpr int blk = decltype(bc)::value;
                         const int pl = i * 32 + blk * 8 + (int)lg * 4;  // p inside the wave tile
-                        T o0, o1, o2, o3;
-                        if constexpr (PLAIN) {
-                            o0 = finish_plain<T>(acc[i][j][blk * 4 + 0], g.alpha);
-                            o1 = finish_plain<T>(acc[i][j][blk * 4 + 1], g.alpha);
-                            o2 = finish_plain<T>(acc[i][j][blk * 4 + 2], g.alpha);
-                            o3 = finish_plain<T>(acc[i][j][blk * 4 + 3], g.alpha);
-                        } else {
-                            T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
-                            if (has_bias && bias_p) {
-                                const int p = min(pwb + pl, g.NP - 4);
-                                b0 = bias[(int64_t)(p + 0) * g.bias_stride];
-                                b1 = bias[(int64_t)(p + 1) * g.bias_stride];
-                                b2 = bias[(int64_t)(p + 2) * g.bias_stride];
-                                b3 = bias[(int64_t)(p + 3) * g.bias_stride];
+                        T o[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] = finish_plain<T>(acc[i][j][blk * 4 + e], g.alpha);
+                        if constexpr (!PLAIN) {
+                            if (pre_bias) {  // wave-uniform
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    o[e] = Elem<T>::from_f32(Elem<T>::to_f32(bq) + Elem<T>::to_f32(o[e]));
                             }
-                            o0 = finish<T>(acc[i][j][blk * 4 + 0], g.alpha, 0.0f, (T)0, has_bias, b0, g.act);
-                            o1 = finish<T>(acc[i][j][blk * 4 + 1], g.alpha, 0.0f, (T)0, has_bias, b1, g.act);
-                            o2 = finish<T>(acc[i][j][blk * 4 + 2], g.alpha, 0.0f, (T)0, has_bias, b2, g.act);
-                            o3 = finish<T>(acc[i][j][blk * 4 + 3], g.alpha, 0.0f, (T)0, has_bias, b3, g.act);
                         }
                         *(uint2 *)(region + lrow * EPITCH + pl * 2) =
-                            make_uint2((uint32_t)o0 | ((uint32_t)o1 << 16), (uint32_t)o2 | ((uint32_t)o3 << 16));
+                            make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
                     });
                 });
                 // same wave, LDS executes in order: the reads below see the writes above
                 static_for<NST>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
-                    const int row = r * RPI + lane / CPRW, chunk = lane % CPRW;
-                    const uint4 v = *(const uint4 *)(region + row * EPITCH + chunk * 16);
+                    const int row = r * RPI + lane / CPRW;
+                    uint4 v = *(const uint4 *)(region + row * EPITCH + chunk * 16);
+                    if constexpr (!PLAIN) {
+                        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                        if (post_bias) {  // wave-uniform
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const T lo = Elem<T>::from_f32(Elem<T>::to_f32(bp[2 * e]) + Elem<T>::to_f32((T)(w[e] & 0xFFFFu)));
+                                const T hi = Elem<T>::from_f32(Elem<T>::to_f32(bp[2 * e + 1]) + Elem<T>::to_f32((T)(w[e] >> 16)));
+                                w[e] = (uint32_t)lo | ((uint32_t)hi << 16);
+                            }
+                        }
+                        if (relu) {  // wave-uniform; keeps x when x >= 0 (so -0 stays, NaN goes to 0)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const bool klo = __uint_as_float(w[e] << 16) >= 0.0f;
+                                const bool khi = __uint_as_float(w[e] & 0xFFFF0000u) >= 0.0f;
+                                w[e] = (klo ? (w[e] & 0xFFFFu) : 0u) | (khi ? (w[e] & 0xFFFF0000u) : 0u);
+                            }
+                        }
+                        v = make_uint4(w[0], w[1], w[2], w[3]);
+                    }
                     const int qq = qwb + j * 32 + row, pp = pwb + chunk * 8;
                     if (qq < g.NQ && pp < g.NP) *(uint4 *)(D + (int64_t)qq * g.dq + pp) = v;
                 });
