@@ -121,7 +121,9 @@ struct FragRead {
     }
 };
 
-template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
+// STAGED: the kernel is only launched with store_mode == ST_STAGED (the common case); the other
+// epilogues are compiled out, which keeps their register demand from spilling accumulators.
+template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ, bool STAGED>
 __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     typedef uint16_t T;
     constexpr int NW = WGP * WGQ;
@@ -274,7 +276,7 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
     T *D = (T *)g.D + (int64_t)blockIdx.z * g.batch_d;
     const T *bias = (const T *)g.bias;
-    const int mode = g.store_mode;
+    const int mode = STAGED ? (int)ST_STAGED : g.store_mode;
     const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;
     if (mode == ST_STAGED) {
         // beta == 0, D rows 16-byte aligned, NP a multiple of 8.  A lane holds 4 consecutive p of

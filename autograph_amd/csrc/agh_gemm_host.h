@@ -8,9 +8,6 @@
 #include <type_traits>
 
 #include "agh_gemm_kernel.h"
-#ifdef AGH_GEMM_WITH_BF16_DIRECT
-#include "agh_gemm_bf16_dl.h"
-#endif
 
 namespace agh {
 namespace gemm {
@@ -51,14 +48,10 @@ int launch_one(const Args &g, int splits) {
 }
 
 #ifdef AGH_GEMM_WITH_BF16_DIRECT
+// direct-to-LDS bf16 kernels: defined and explicitly instantiated in agh_gemm_bf16_dl_<tile>.hip
+// (one translation unit per tile shape, so they compile in parallel)
 template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
-int launch_one_dl(const Args &g, int splits) {
-    auto kern = gemm_bf16_dl_kernel<BP, BQ, WGP, WGQ, LP, LQ>;  // both LDS stages are static
-    dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits, (unsigned)g.batch);
-    hipLaunchKernelGGL(kern, grid, dim3(WGP * WGQ * 64), 0, stream(), g);
-    AGH_LAUNCH_CHECK("gemm (direct-to-LDS) kernel launch");
-    return AGH_OK;
-}
+int launch_one_dl(const Args &g, int splits);
 #endif
 
 template <typename T, int BP, int BQ, int WGP, int WGQ, bool SCALAR_OK>
