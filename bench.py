@@ -22,7 +22,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3     # MI355X f32 matrix
 PEAK_HBM_GBS = 8000.0
-TRAFFIC_BYTES_BF16_8192 = 1.796e9  # profiles/gemm_bf16_8192_hbm_counters.md
+TRAFFIC_BYTES_BF16_8192 = 1.750e9  # FETCH_SIZE + WRITE_SIZE per launch, from the counter summary kept under profiles/
 
 
 def log(*a):
@@ -99,7 +99,7 @@ def main():
     flop = 2.0 * n * n * n
     value = flop / (wall_ms * 1e-3) / 1e12
     achieved = flop / (dev_ms * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "kernel": "gemm_kernel<bf16,256x256> (v_mfma_f32_32x32x16_bf16)",
+    roofline = {"bound": "mfma", "kernel": "gemm_bf16_dl_kernel<256,256,2,2,1,0,true> (v_mfma_f32_32x32x16_bf16, direct-to-LDS loads)",
                 "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/
@@ -235,11 +235,12 @@ def main():
             # layer-by-layer path (12 launches, im2col + gemm convolutions), eager
             _, layered_ms = timer.time(lambda: model.forward(txl, algorithm="im2col"), 20, 5)
             lenet = {"gpu_ms": round(gpu_ms, 4), "gpu_kernel_ms": round(kernel_ms, 4), "gpu_graph_5_launches_ms": round(graph_ms, 4),
-                     "gpu_layered_im2col_ms": round(layered_ms, 4),
+                     "gpu_layered_im2col_eager_ms": round(layered_ms, 4),
                      "what": "gpu_ms: one launch of the whole-network kernel (input resident in HBM, [1000,10] logits written "
                              "into pinned host memory), wall clock per inference including the host-side wait; "
                              "gpu_kernel_ms: the same launch between HIP events; gpu_graph_5_launches_ms: graph replay of "
-                             "conv+relu+pool x2 and 3 Dense GEMMs plus D2H"}
+                             "conv+relu+pool x2 and 3 Dense GEMMs plus D2H; gpu_layered_im2col_eager_ms: the 12-launch "
+                             "layer-by-layer path, each layer allocating its output"}
             if not args.no_cpu:
                 thr = orc.max_threads()
                 want = orc.lenet5_forward_f32(xl, *params, direct=True)
@@ -263,7 +264,7 @@ def main():
     cpu = None
     if not args.no_cpu:
         t0 = time.perf_counter()
-        s = 768  # bounded sample of the same workload: scalar bf16 fold is O(mnk) on one thread
+        s = 1024  # bounded sample of the same workload: scalar bf16 fold is O(mnk) on one thread, ~11 s
         ha, hb = rand_bf16(orc, rng, (s, s)), rand_bf16(orc, rng, (s, s))
         t1 = time.perf_counter()
         orc.gemm_bf16_hostfold(ha, hb)
