@@ -9,8 +9,10 @@ from .layer import (  # noqa: F401
     Dense,
     Flatten,
     LeNet5,
+    LeNet5Trainer,
     MaxPool2,
     Relu,
+    SGD,
     conv2_direct_forward,
     conv2_im2col_forward,
 )

@@ -72,6 +72,18 @@ SIGNATURES = {
     "agh_relu_bf16": ([ptr, ptr, i64], C.c_int),
     "agh_relu_backward_f32": ([ptr, ptr, ptr, i64], C.c_int),
     "agh_relu_backward_bf16": ([ptr, ptr, ptr, i64], C.c_int),
+    "agh_assign_f32": ([ptr] + [i64] * 5 + [ptr] + [i64] * 9, C.c_int),
+    "agh_assign_bf16": ([ptr] + [i64] * 5 + [ptr] + [i64] * 9, C.c_int),
+    "agh_scaled_add_f32": ([ptr, f32, ptr, i64], C.c_int),
+    "agh_scaled_add_bf16": ([ptr, f32, ptr, i64], C.c_int),
+    "agh_sgd_momentum_f32": ([ptr, ptr, f32, f32, ptr, i64], C.c_int),
+    "agh_sgd_momentum_bf16": ([ptr, ptr, f32, f32, ptr, i64], C.c_int),
+    "agh_sum_axis0_f32": ([ptr, ptr, i64, i64], C.c_int),
+    "agh_sum_axis0_bf16": ([ptr, ptr, i64, i64], C.c_int),
+    "agh_cross_entropy_loss_f32": ([ptr, ptr, i64, i64, ptr], C.c_int),
+    "agh_cross_entropy_loss_bf16": ([ptr, ptr, i64, i64, ptr], C.c_int),
+    "agh_cross_entropy_backward_f32": ([ptr, ptr, f32, ptr, i64, i64], C.c_int),
+    "agh_cross_entropy_backward_bf16": ([ptr, ptr, f32, ptr, i64, i64], C.c_int),
 }
 
 for _name, (_args, _res) in SIGNATURES.items():

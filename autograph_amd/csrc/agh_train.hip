@@ -1,0 +1,274 @@
+// Kernels around the contraction path that a training step needs: strided copy (`assign`),
+// `scaled_add`, SGD with momentum, the axis-0 sum behind the bias gradient, and cross-entropy
+// loss / gradient.  All follow the reference's HOST arithmetic: every operation the host performs
+// in the element type is rounded to the element type here too, sums run in the host's order.
+#include "agh_internal.h"
+
+using namespace agh;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+unsigned grid_for(size_t n) {
+    size_t blocks = (n + kThreads - 1) / kThreads;
+    size_t cap = (size_t)compute_units() * 32;
+    if (cap == 0) cap = 8192;
+    return (unsigned)(blocks < cap ? blocks : cap);
+}
+
+// ---------------------------------------------------------------- assign ----
+struct AssignParams {
+    int64_t sx[4], sy[4];
+    FastDiv div1, div2, div3;  // by d1*d2*d3, d2*d3, d3
+    uint32_t d23, d3;
+};
+
+// One thread per element, index space walked with the last dimension fastest, so a destination in
+// standard layout is written with consecutive lanes on consecutive elements.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void assign_kernel(const T *__restrict__ x, T *__restrict__ y, AssignParams p,
+                                                           uint32_t total) {
+    for (uint32_t e = blockIdx.x * kThreads + threadIdx.x; e < total; e += gridDim.x * kThreads) {
+        uint32_t i0, r0, i1, r1, i2, i3;
+        p.div1.divmod(e, i0, r0);
+        p.div2.divmod(r0, i1, r1);
+        p.div3.divmod(r1, i2, i3);
+        const int64_t ix = i0 * p.sx[0] + i1 * p.sx[1] + i2 * p.sx[2] + i3 * p.sx[3];
+        const int64_t iy = i0 * p.sy[0] + i1 * p.sy[1] + i2 * p.sy[2] + i3 * p.sy[3];
+        y[iy] = x[ix];
+    }
+}
+
+template <typename T>
+int assign_launch(const char *name, const void *x, int64_t off_x, const int64_t (&sx)[4], void *y, int64_t off_y,
+                  const int64_t (&sy)[4], const int64_t (&d)[4]) {
+    AGH_API_ENTER();
+    int64_t total = 1;
+    for (int i = 0; i < 4; ++i) {
+        if (d[i] < 0) return fail(AGH_EINVAL, "%s: negative dimension", name);
+        if (d[i] > ((int64_t)1 << 30)) return fail(AGH_ERANGE, "%s: dimension too large", name);
+        total *= d[i];
+        if (total > ((int64_t)1 << 31) - 1) return fail(AGH_ERANGE, "%s: more than 2^31-1 elements", name);
+    }
+    if (total == 0) return AGH_OK;
+    if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+    AssignParams p;
+    for (int i = 0; i < 4; ++i) { p.sx[i] = sx[i]; p.sy[i] = sy[i]; }
+    p.div1 = FastDiv((uint32_t)(d[1] * d[2] * d[3]));
+    p.div2 = FastDiv((uint32_t)(d[2] * d[3]));
+    p.div3 = FastDiv((uint32_t)d[3]);
+    hipLaunchKernelGGL(assign_kernel<T>, dim3(grid_for((size_t)total)), dim3(kThreads), 0, stream(),
+                       (const T *)x + off_x, (T *)y + off_y, p, (uint32_t)total);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+// ------------------------------------------------------------ scaled_add ----
+template <typename T>
+__global__ __launch_bounds__(kThreads) void scaled_add_kernel(T *__restrict__ y, float alpha, const T *__restrict__ x, size_t n) {
+    const float a = Elem<T>::to_f32(Elem<T>::from_f32(alpha));  // alpha is cast to the element type first
+    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads) {
+        const T prod = Elem<T>::from_f32(a * Elem<T>::to_f32(x[i]));
+        y[i] = Elem<T>::from_f32(Elem<T>::to_f32(prod) + Elem<T>::to_f32(y[i]));
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void sgd_momentum_kernel(T *__restrict__ w, const T *__restrict__ dw, float lr, float m,
+                                                                 T *__restrict__ v, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads) {
+        const float mv = m * Elem<T>::to_f32(v[i]);
+        const float vn = mv + Elem<T>::to_f32(dw[i]);
+        const float step = lr * vn;
+        v[i] = Elem<T>::from_f32(vn);
+        w[i] = Elem<T>::from_f32(Elem<T>::to_f32(w[i]) - step);
+    }
+}
+
+// ------------------------------------------------------------- sum axis 0 ----
+// One thread per column, rows added one at a time in the element type, starting from zero.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void sum_axis0_kernel(const T *__restrict__ x, T *__restrict__ y, int64_t rows, int64_t cols) {
+    const int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (j >= cols) return;
+    T acc = Elem<T>::zero();
+    for (int64_t i = 0; i < rows; ++i) acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(x[i * cols + j]));
+    y[j] = acc;
+}
+
+// ---------------------------------------------------------- cross entropy ----
+template <typename T>
+__device__ __forceinline__ void row_max_sum(const T *row, int classes, float &m, float &s) {
+    m = Elem<T>::to_f32(row[0]);
+    for (int j = 0; j < classes; ++j) m = fmaxf(m, Elem<T>::to_f32(row[j]));
+    s = 0.0f;
+    for (int j = 0; j < classes; ++j) s += expf(Elem<T>::to_f32(row[j]) - m);
+}
+
+// A single workgroup: rows are evaluated 256 at a time, then one thread adds the 256 row losses to
+// the running total in row order, which is the order of the host's loop.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void cross_entropy_loss_kernel(const T *__restrict__ x, const uint8_t *__restrict__ t,
+                                                                       int64_t bs, int classes, float *__restrict__ out) {
+    __shared__ float part[kThreads];
+    float total = 0.0f;
+    for (int64_t base = 0; base < bs; base += kThreads) {
+        const int64_t r = base + threadIdx.x;
+        float l = 0.0f;
+        if (r < bs) {
+            const T *row = x + r * classes;
+            float m, s;
+            row_max_sum(row, classes, m, s);
+            l = logf(s) - (Elem<T>::to_f32(row[t[r]]) - m);
+        }
+        part[threadIdx.x] = l;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const int cnt = (int)min((int64_t)kThreads, bs - base);
+            for (int i = 0; i < cnt; ++i) total += part[i];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *out = total;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void cross_entropy_backward_kernel(const T *__restrict__ x, const uint8_t *__restrict__ t,
+                                                                           float dy, T *__restrict__ dx, int64_t bs, int classes) {
+    const int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (r >= bs) return;
+    const T *row = x + r * classes;
+    float m, s;
+    row_max_sum(row, classes, m, s);
+    const int tr = t[r];
+    for (int j = 0; j < classes; ++j) {
+        const float p = expf(Elem<T>::to_f32(row[j]) - m) / s;
+        const float diff = p - (j == tr ? 1.0f : 0.0f);
+        dx[r * classes + j] = Elem<T>::from_f32(dy * diff);
+    }
+}
+
+template <typename T>
+int scaled_add_launch(const char *name, void *y, float alpha, const void *x, int64_t n) {
+    AGH_API_ENTER();
+    if (n < 0) return fail(AGH_EINVAL, "%s: negative length", name);
+    if (n == 0) return AGH_OK;
+    if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+    hipLaunchKernelGGL(scaled_add_kernel<T>, dim3(grid_for((size_t)n)), dim3(kThreads), 0, stream(), (T *)y,
+                       alpha, (const T *)x, (size_t)n);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+template <typename T>
+int sgd_momentum_launch(const char *name, void *w, const void *dw, float lr, float m, void *v, int64_t n) {
+    AGH_API_ENTER();
+    if (n < 0) return fail(AGH_EINVAL, "%s: negative length", name);
+    if (n == 0) return AGH_OK;
+    if (!w || !dw || !v) return fail(AGH_ENULL, "%s: null buffer", name);
+    hipLaunchKernelGGL(sgd_momentum_kernel<T>, dim3(grid_for((size_t)n)), dim3(kThreads), 0, stream(), (T *)w,
+                       (const T *)dw, lr, m, (T *)v, (size_t)n);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+template <typename T>
+int sum_axis0_launch(const char *name, const void *x, void *y, int64_t rows, int64_t cols) {
+    AGH_API_ENTER();
+    if (rows < 0 || cols < 0) return fail(AGH_EINVAL, "%s: negative shape", name);
+    if (cols == 0) return AGH_OK;
+    if (!y || (!x && rows > 0)) return fail(AGH_ENULL, "%s: null buffer", name);
+    const int64_t blocks = (cols + kThreads - 1) / kThreads;
+    if (blocks > 0x7FFFFFFFll) return fail(AGH_ERANGE, "%s: too many columns", name);
+    hipLaunchKernelGGL(sum_axis0_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(), (const T *)x, (T *)y,
+                       rows, cols);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+int ce_check(const char *name, const void *x, const void *t, int64_t bs, int64_t classes) {
+    if (bs < 0 || classes < 1) return fail(AGH_EINVAL, "%s: invalid shape", name);
+    if (classes > 256) return fail(AGH_ERANGE, "%s: targets are u8, at most 256 classes", name);
+    if (bs > 0 && (!x || !t)) return fail(AGH_ENULL, "%s: null buffer", name);
+    return AGH_OK;
+}
+
+template <typename T>
+int ce_loss_launch(const char *name, const void *x, const void *t, int64_t bs, int64_t classes, float *loss) {
+    AGH_API_ENTER();
+    if (int rc = ce_check(name, x, t, bs, classes)) return rc;
+    if (!loss) return fail(AGH_ENULL, "%s: null output", name);
+    hipLaunchKernelGGL(cross_entropy_loss_kernel<T>, dim3(1), dim3(kThreads), 0, stream(), (const T *)x,
+                       (const uint8_t *)t, bs, (int)classes, loss);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+template <typename T>
+int ce_backward_launch(const char *name, const void *x, const void *t, float dy, void *dx, int64_t bs, int64_t classes) {
+    AGH_API_ENTER();
+    if (int rc = ce_check(name, x, t, bs, classes)) return rc;
+    if (bs == 0) return AGH_OK;
+    if (!dx) return fail(AGH_ENULL, "%s: null output", name);
+    const int64_t blocks = (bs + kThreads - 1) / kThreads;
+    if (blocks > 0x7FFFFFFFll) return fail(AGH_ERANGE, "%s: batch too large", name);
+    // `dy /= batch_size` first, in f32, as the host does
+    hipLaunchKernelGGL(cross_entropy_backward_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(),
+                       (const T *)x, (const uint8_t *)t, dy / (float)bs, (T *)dx, bs, (int)classes);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+}  // namespace
+
+#define AGH_ASSIGN_ARGS                                                                                              \
+    const void *x, int64_t off_x, int64_t sx0, int64_t sx1, int64_t sx2, int64_t sx3, void *y, int64_t off_y,      \
+        int64_t sy0, int64_t sy1, int64_t sy2, int64_t sy3, int64_t d0, int64_t d1, int64_t d2, int64_t d3
+
+extern "C" {
+
+int agh_assign_f32(AGH_ASSIGN_ARGS) {
+    const int64_t sx[4] = {sx0, sx1, sx2, sx3}, sy[4] = {sy0, sy1, sy2, sy3}, d[4] = {d0, d1, d2, d3};
+    return assign_launch<uint32_t>("agh_assign_f32", x, off_x, sx, y, off_y, sy, d);
+}
+int agh_assign_bf16(AGH_ASSIGN_ARGS) {
+    const int64_t sx[4] = {sx0, sx1, sx2, sx3}, sy[4] = {sy0, sy1, sy2, sy3}, d[4] = {d0, d1, d2, d3};
+    return assign_launch<uint16_t>("agh_assign_bf16", x, off_x, sx, y, off_y, sy, d);
+}
+
+int agh_scaled_add_f32(void *y, float alpha, const void *x, int64_t n) {
+    return scaled_add_launch<float>("agh_scaled_add_f32", y, alpha, x, n);
+}
+int agh_scaled_add_bf16(void *y, float alpha, const void *x, int64_t n) {
+    return scaled_add_launch<uint16_t>("agh_scaled_add_bf16", y, alpha, x, n);
+}
+
+int agh_sgd_momentum_f32(void *w, const void *dw, float learning_rate, float momentum, void *velocity, int64_t n) {
+    return sgd_momentum_launch<float>("agh_sgd_momentum_f32", w, dw, learning_rate, momentum, velocity, n);
+}
+int agh_sgd_momentum_bf16(void *w, const void *dw, float learning_rate, float momentum, void *velocity, int64_t n) {
+    return sgd_momentum_launch<uint16_t>("agh_sgd_momentum_bf16", w, dw, learning_rate, momentum, velocity, n);
+}
+
+int agh_sum_axis0_f32(const void *x, void *y, int64_t rows, int64_t cols) {
+    return sum_axis0_launch<float>("agh_sum_axis0_f32", x, y, rows, cols);
+}
+int agh_sum_axis0_bf16(const void *x, void *y, int64_t rows, int64_t cols) {
+    return sum_axis0_launch<uint16_t>("agh_sum_axis0_bf16", x, y, rows, cols);
+}
+
+int agh_cross_entropy_loss_f32(const void *x, const void *target_u8, int64_t bs, int64_t classes, float *loss) {
+    return ce_loss_launch<float>("agh_cross_entropy_loss_f32", x, target_u8, bs, classes, loss);
+}
+int agh_cross_entropy_loss_bf16(const void *x, const void *target_u8, int64_t bs, int64_t classes, float *loss) {
+    return ce_loss_launch<uint16_t>("agh_cross_entropy_loss_bf16", x, target_u8, bs, classes, loss);
+}
+int agh_cross_entropy_backward_f32(const void *x, const void *target_u8, float dy, void *dx, int64_t bs, int64_t classes) {
+    return ce_backward_launch<float>("agh_cross_entropy_backward_f32", x, target_u8, dy, dx, bs, classes);
+}
+int agh_cross_entropy_backward_bf16(const void *x, const void *target_u8, float dy, void *dx, int64_t bs, int64_t classes) {
+    return ce_backward_launch<uint16_t>("agh_cross_entropy_backward_bf16", x, target_u8, dy, dx, bs, classes);
+}
+
+}  // extern "C"

@@ -1,14 +1,14 @@
 """Host-side mirror of the reference's layer structs for the hot path:
 `Conv2`, `Dense`, `MaxPool2`, `Relu`, `Flatten` with `forward` (src/learn/neural_network/layer.rs),
 and the LeNet5 model of the reference's benchmark (benches/neural-network-benches/src/
-autograph_backend.rs:88-162).  Inference only: parameters are plain tensors.
+autograph_backend.rs:88-162), plus one training step of it (`LeNet5Trainer`, `SGD`).
 """
 import ctypes as C
 
 import numpy as np
 
 from ._ffi import AghError, check, lib
-from .tensor import Im2ColConv2Options, MaxPool2Options, Tensor, _ITEMSIZE
+from .tensor import Im2ColConv2Options, MaxPool2Options, Tensor, _ITEMSIZE, gemm
 
 
 def conv2_im2col_forward(x, weight, padding=(0, 0), stride=(1, 1), dilation=(1, 1), bias=None, relu=False):
@@ -202,3 +202,168 @@ class LeNet5:
                 lib.agh_graph_destroy(g)
             except Exception:
                 pass
+
+
+class SGD:
+    """`SGD` (optimizer.rs:389-427): plain `scaled_add(-learning_rate)` or, with momentum, the f32
+    velocity update of optimizer.rs:509-512."""
+
+    def __init__(self, momentum=None):
+        self.momentum = momentum
+
+    def update(self, learning_rate, value, grad, velocity=None):
+        if self.momentum is None:
+            check(getattr(lib, f"agh_scaled_add_{value.dtype}")(value._data_ptr(), -learning_rate, grad._data_ptr(), len(value)))
+        else:
+            check(getattr(lib, f"agh_sgd_momentum_{value.dtype}")(value._data_ptr(), grad._data_ptr(), learning_rate,
+                                                                  self.momentum, velocity._data_ptr(), len(value)))
+
+
+class LeNet5Trainer:
+    """One training step of the benchmark's LeNet5 (autograph_backend.rs:70-86): forward, summed
+    cross-entropy loss, backward through the edges the reference's autograd builds (conv:
+    layer.rs:950-1005, dot: autograd.rs:607-627, bias: :571-599 and :490-542, relu: layer.rs:1253-1267,
+    pool: layer.rs:1193-1216, flatten / permute: autograd.rs:384-445), and the SGD update.
+
+    Every buffer is allocated here, once; `step` only launches kernels, so it can be captured into
+    a graph (`capture`) and replayed.  Gradients stay available in `grads` after a step."""
+
+    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None):
+        self.model, self.bs, self.lr = model, batch_size, learning_rate
+        self.opt = optimizer if optimizer is not None else SGD()
+        bs, dt = batch_size, model.conv1.weight.dtype
+        self.dt = dt
+        u = lambda *shape: Tensor.uninit(shape, dt)  # noqa: E731
+        self.cols1, self.c1, self.r1, self.p1 = u(bs * 576, 25), u(bs, 6, 24, 24), u(bs, 6, 24, 24), u(bs, 6, 12, 12)
+        self.cols2, self.c2, self.r2, self.p2 = u(bs * 64, 150), u(bs, 16, 8, 8), u(bs, 16, 8, 8), u(bs, 16, 4, 4)
+        self.d1, self.a1, self.d2, self.a2, self.logits = u(bs, 128), u(bs, 128), u(bs, 84), u(bs, 84), u(bs, 10)
+        self.g_logits, self.g_a2, self.g_d2 = u(bs, 10), u(bs, 84), u(bs, 84)
+        self.g_a1, self.g_d1, self.g_f = u(bs, 128), u(bs, 128), u(bs, 256)
+        self.g_r2, self.g_c2, self.gm2, self.gcols2 = u(bs, 16, 8, 8), u(bs, 16, 8, 8), u(bs * 64, 16), u(bs * 64, 150)
+        self.g_p1, self.g_r1, self.g_c1, self.gm1 = u(bs, 6, 12, 12), u(bs, 6, 24, 24), u(bs, 6, 24, 24), u(bs * 576, 6)
+        m = model
+        self.params = [m.conv1.weight, m.conv2.weight, m.dense1.weight, m.dense2.weight, m.dense3.weight, m.dense3.bias]
+        self.grads = [Tensor.uninit(p.shape, dt) for p in self.params]
+        self.velocities = [Tensor.zeros(p.shape, dt) for p in self.params] if self.opt.momentum is not None else [None] * 6
+        host = C.c_void_p()
+        check(lib.agh_host_alloc(C.byref(host), 4))
+        self._loss_host = host
+        self._graph = None
+
+    def __del__(self):
+        try:
+            if getattr(self, "_graph", None):
+                lib.agh_graph_destroy(self._graph)
+            if getattr(self, "_loss_host", None):
+                lib.agh_host_free(self._loss_host)
+        except Exception:
+            pass
+
+    # raw launches on preallocated tensors
+    def _fn(self, stem):
+        return getattr(lib, f"{stem}_{self.dt}")
+
+    def _conv_forward(self, x, weight, cols, y):
+        bs, ic, ih, iw = x.shape
+        oc, _, fh, fw = weight.shape
+        oh, ow = ih - fh + 1, iw - fw + 1
+        check(self._fn("agh_im2col_conv2")(x._data_ptr(), cols._ptr(), bs, ic, ih, iw, fh, fw, 0, 0, 1, 1, 1, 1))
+        L, K = oh * ow, ic * fh * fw
+        wm = weight.into_shape((oc, K))
+        check(getattr(lib, f"agh_gemm_{self.dt}_batched")(
+            bs, L, K, oc, 1.0, cols._ptr(), 0, K, 1, L * K, wm._ptr(), wm.offset, 1, K, 0,
+            0.0, y._ptr(), 0, 1, L, oc * L, None, 0, 0, 0))
+
+    def _pool(self, x, y):
+        bs, c, ih, iw = x.shape
+        check(self._fn("agh_max_pool2")(x._data_ptr(), y._ptr(), bs * c, ih, iw, 2, 2, 2, 2))
+
+    def _pool_backward(self, x, dy, dx):
+        """dx <- x, then the in-place backward (layer.rs:1203-1211)."""
+        bs, c, ih, iw = x.shape
+        check(lib.agh_memcpy_d2d(dx._ptr(), x._data_ptr(), len(x) * _ITEMSIZE[self.dt]))
+        check(self._fn("agh_max_pool2_backward")(dx._ptr(), dy._data_ptr(), bs * c, ih, iw, 2, 2, 2, 2))
+
+    def _relu(self, x, y):
+        check(self._fn("agh_relu")(x._data_ptr(), y._ptr(), len(x)))
+
+    def _relu_backward(self, x, dy, dx):
+        check(self._fn("agh_relu_backward")(x._data_ptr(), dy._data_ptr(), dx._ptr(), len(x)))
+
+    def _nhwc_matrix(self, g, out):
+        """[bs, c, h, w] gradient -> standard-layout [bs*h*w, c] matrix (autograd.rs:429-445)."""
+        v = g.permuted_axes([0, 2, 3, 1])
+        check(self._fn("agh_assign")(v._ptr(), v.offset, *v.strides, out._ptr(), 0, *_std4(v.shape), *v.shape))
+
+    def step(self, x, target):
+        """x: [bs,1,28,28] tensor, target: device `Buffer` of bs u8 labels.  The loss lands in pinned
+        host memory (`loss()` after a sync)."""
+        bs = self.bs
+        w1, w2, wd1, wd2, wd3, b3 = self.params
+        dw1, dw2, dwd1, dwd2, dwd3, db3 = self.grads
+        # forward
+        self._conv_forward(x, w1, self.cols1, self.c1)
+        self._relu(self.c1, self.r1)
+        self._pool(self.r1, self.p1)
+        self._conv_forward(self.p1, w2, self.cols2, self.c2)
+        self._relu(self.c2, self.r2)
+        self._pool(self.r2, self.p2)
+        f = self.p2.into_shape((bs, 256))
+        gemm(1.0, f, wd1, 0.0, self.d1)
+        self._relu(self.d1, self.a1)
+        gemm(1.0, self.a1, wd2, 0.0, self.d2)
+        self._relu(self.d2, self.a2)
+        gemm(1.0, self.a2, wd3, 0.0, self.logits, bias=b3)
+        check(self._fn("agh_cross_entropy_loss")(self.logits._ptr(), target.ptr, bs, 10, self._loss_host))
+        # backward
+        check(self._fn("agh_cross_entropy_backward")(self.logits._ptr(), target.ptr, 1.0, self.g_logits._ptr(), bs, 10))
+        check(self._fn("agh_sum_axis0")(self.g_logits._ptr(), db3._ptr(), bs, 10))
+        gemm(1.0, self.a2.t(), self.g_logits, 0.0, dwd3)
+        gemm(1.0, self.g_logits, wd3.t(), 0.0, self.g_a2)
+        self._relu_backward(self.d2, self.g_a2, self.g_d2)
+        gemm(1.0, self.a1.t(), self.g_d2, 0.0, dwd2)
+        gemm(1.0, self.g_d2, wd2.t(), 0.0, self.g_a1)
+        self._relu_backward(self.d1, self.g_a1, self.g_d1)
+        gemm(1.0, f.t(), self.g_d1, 0.0, dwd1)
+        gemm(1.0, self.g_d1, wd1.t(), 0.0, self.g_f)
+        self._pool_backward(self.r2, self.g_f.into_shape((bs, 16, 4, 4)), self.g_r2)
+        self._relu_backward(self.c2, self.g_r2, self.g_c2)
+        self._nhwc_matrix(self.g_c2, self.gm2)
+        gemm(1.0, self.gm2.t(), self.cols2, 0.0, dw2.into_shape((16, 150)))
+        gemm(1.0, self.gm2, w2.into_shape((16, 150)), 0.0, self.gcols2)
+        check(self._fn("agh_col2im_conv2")(self.gcols2._ptr(), self.g_p1._ptr(), bs, 6, 8, 8, 5, 5, 0, 0, 1, 1, 1, 1))
+        self._pool_backward(self.r1, self.g_p1, self.g_r1)
+        self._relu_backward(self.c1, self.g_r1, self.g_c1)
+        self._nhwc_matrix(self.g_c1, self.gm1)
+        gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
+        # update
+        for p, g, v in zip(self.params, self.grads, self.velocities):
+            self.opt.update(self.lr, p, g, v)
+
+    def loss(self):
+        """The last step's loss; call after `agh_sync`."""
+        return float(C.cast(self._loss_host, C.POINTER(C.c_float))[0])
+
+    def capture(self, x, target):
+        """Run one step eagerly (allocates the split-K workspace), then record a step into a graph.
+        NOTE: both the eager step and the capture pass update the parameters."""
+        self.step(x, target)
+        check(lib.agh_sync())
+        check(lib.agh_graph_begin())
+        try:
+            self.step(x, target)
+        finally:
+            g = C.c_void_p()
+            check(lib.agh_graph_end(C.byref(g)))
+        self._graph = g
+
+    def replay(self):
+        check(lib.agh_graph_launch(self._graph))
+
+
+def _std4(shape):
+    strides, acc = [], 1
+    for d in reversed(shape):
+        strides.append(acc)
+        acc *= d
+    return tuple(reversed(strides))

@@ -262,10 +262,76 @@ class Tensor:
         return out
 
     def as_standard_layout(self):
+        """`as_standard_layout` (src/tensor.rs): self if already contiguous, else a strided copy."""
         if self.is_standard_layout():
             return self
-        raise AghError(-1, "as_standard_layout: strided copy kernels are not part of this build; "
-                           "pass a standard-layout tensor")
+        return self.to_standard_layout()
+
+    def to_standard_layout(self):
+        """Strided copy into a fresh standard-layout tensor (`assign`, src/tensor/ops.rs:257-318)."""
+        if self.ndim > 4:
+            raise AghError(-1, "to_standard_layout: more than 4 dimensions")
+        out = Tensor.uninit(self.shape, self.dtype)
+        pad = 4 - self.ndim
+        dims = [1] * pad + list(self.shape)
+        sx = [0] * pad + list(self.strides)
+        sy = [0] * pad + list(out.strides)
+        check(self._fn("agh_assign")(self._ptr(), self.offset, *sx, out._ptr(), 0, *sy, *dims))
+        return out
+
+    def broadcast(self, shape):
+        """View with stride 0 along broadcast axes (ndarray `broadcast`)."""
+        shape = tuple(shape)
+        pad = len(shape) - self.ndim
+        if pad < 0:
+            return None
+        strides = [0] * pad
+        for d, s, want in zip(self.shape, self.strides, shape[pad:]):
+            if d == want:
+                strides.append(s)
+            elif d == 1:
+                strides.append(0)
+            else:
+                return None
+        return Tensor(self.buffer, shape, strides, self.offset, self.dtype)
+
+    # -- scaled_add / sum_axis / cross entropy (src/tensor/ops.rs:257-318, reduce.rs:59-113, learn/criterion.rs) --
+    def scaled_add(self, alpha, rhs):
+        """In place: self = alpha * rhs + self, each operation rounded to the element type."""
+        if self.dtype != rhs.dtype or self.shape != rhs.shape:
+            raise AghError(-1, f"scaled_add: {self.dtype}{self.shape} vs {rhs.dtype}{rhs.shape}")
+        if not self.is_standard_layout():
+            raise AghError(-1, "scaled_add: destination must be in standard layout")
+        x = rhs.as_standard_layout()
+        check(self._fn("agh_scaled_add")(self._data_ptr(), alpha, x._data_ptr(), len(self)))
+
+    def sum_axis0(self):
+        x = self.as_standard_layout()
+        rows, cols = x.shape
+        y = Tensor.uninit((cols,), self.dtype)
+        check(self._fn("agh_sum_axis0")(x._data_ptr(), y._ptr(), rows, cols))
+        return y
+
+    def cross_entropy_loss(self, target, out_ptr=None):
+        """Sum of the per-row losses (f32).  `target`: u8 class indices on the device (a `Buffer`).
+        With `out_ptr` (device or pinned host memory) nothing is copied back and None is returned."""
+        x = self.as_standard_layout()
+        bs, classes = x.shape
+        if out_ptr is not None:
+            check(self._fn("agh_cross_entropy_loss")(x._data_ptr(), target.ptr, bs, classes, out_ptr))
+            return None
+        tmp = Buffer(4)
+        check(self._fn("agh_cross_entropy_loss")(x._data_ptr(), target.ptr, bs, classes, tmp.ptr))
+        out = np.empty(1, dtype=np.float32)
+        check(lib.agh_memcpy_d2h(out.ctypes.data, tmp.ptr, 4))
+        return float(out[0])
+
+    def cross_entropy_loss_backward(self, target, dy=1.0):
+        x = self.as_standard_layout()
+        bs, classes = x.shape
+        dx = Tensor.uninit(x.shape, x.dtype)
+        check(self._fn("agh_cross_entropy_backward")(x._data_ptr(), target.ptr, dy, dx._ptr(), bs, classes))
+        return dx
 
 
 def gemm(alpha, a, b, beta, c, bias=None, relu=False):

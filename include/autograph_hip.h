@@ -235,6 +235,49 @@ int agh_relu_bf16(const void *x, void *y, int64_t n);
 int agh_relu_backward_f32(const void *x, const void *dy, void *dx, int64_t n);
 int agh_relu_backward_bf16(const void *x, const void *dy, void *dx, int64_t n);
 
+/* ---- around the contraction path: what a training step needs besides the ops above ----
+ * All follow the HOST arithmetic of the reference: every operation the host performs in the
+ * element type is rounded to the element type, sums run in the host's order. */
+
+/* `assign` with BinaryOp::Identity and alpha = 1: strided copy of up to 4 dimensions between views
+ * of the same element type (src/tensor/ops.rs:257-318; device kernels assign{2,4}_<X>_<Y> :1353-1438).
+ * This is `into_standard_layout` / `to_standard_layout_shared` (the NHWC<->NCHW copies of
+ * layer.rs:1000-1004 and autograd.rs:396-445) and the broadcast of a bias.  Index space d0..d3 (pad
+ * with 1), element strides signed, a stride 0 on x broadcasts. */
+int agh_assign_f32(const void *x, int64_t off_x, int64_t sx0, int64_t sx1, int64_t sx2, int64_t sx3,
+                   void *y, int64_t off_y, int64_t sy0, int64_t sy1, int64_t sy2, int64_t sy3,
+                   int64_t d0, int64_t d1, int64_t d2, int64_t d3);
+int agh_assign_bf16(const void *x, int64_t off_x, int64_t sx0, int64_t sx1, int64_t sx2, int64_t sx3,
+                    void *y, int64_t off_y, int64_t sy0, int64_t sy1, int64_t sy2, int64_t sy3,
+                    int64_t d0, int64_t d1, int64_t d2, int64_t d3);
+
+/* `scaled_add`: y = alpha * x + y on contiguous buffers, product and sum each one operation in the
+ * element type; alpha is cast to the element type first (src/tensor/ops.rs:294-296; plain SGD is
+ * scaled_add(-learning_rate), optimizer.rs:419-424). */
+int agh_scaled_add_f32(void *y, float alpha, const void *x, int64_t n);
+int agh_scaled_add_bf16(void *y, float alpha, const void *x, int64_t n);
+
+/* SGD with momentum: in f32, v = momentum*v + dw; w -= learning_rate*v; both cast back
+ * (optimizer.rs:430-465, kernel :509-512). */
+int agh_sgd_momentum_f32(void *w, const void *dw, float learning_rate, float momentum, void *velocity, int64_t n);
+int agh_sgd_momentum_bf16(void *w, const void *dw, float learning_rate, float momentum, void *velocity, int64_t n);
+
+/* Sum over axis 0 of a row-major [rows, cols] array into y[cols]: zero, then one add in the element
+ * type per row, rows ascending (src/tensor/reduce.rs:59-62 on the host; the bias gradient,
+ * autograd.rs:490-542). */
+int agh_sum_axis0_f32(const void *x, void *y, int64_t rows, int64_t cols);
+int agh_sum_axis0_bf16(const void *x, void *y, int64_t rows, int64_t cols);
+
+/* Cross-entropy loss summed over the batch, f32 arithmetic, rows in order
+ * (src/learn/criterion.rs:205-226); targets are u8 class indices.  `loss` is one float in device
+ * memory or in memory from agh_host_alloc. */
+int agh_cross_entropy_loss_f32(const void *x, const void *target_u8, int64_t bs, int64_t classes, float *loss);
+int agh_cross_entropy_loss_bf16(const void *x, const void *target_u8, int64_t bs, int64_t classes, float *loss);
+/* Its gradient: dx = T((dy / bs) * (softmax(x) - onehot(t))), f32 arithmetic
+ * (src/learn/neural_network/criterion.rs:79-103). */
+int agh_cross_entropy_backward_f32(const void *x, const void *target_u8, float dy, void *dx, int64_t bs, int64_t classes);
+int agh_cross_entropy_backward_bf16(const void *x, const void *target_u8, float dy, void *dx, int64_t bs, int64_t classes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -70,6 +70,17 @@ _sig("orc_lenet5_forward_f32", [_p, _i64, _p, _p, _p, _p, _p, _p, _p, C.c_int])
 _sig("orc_lenet5_forward_f32_alg", [_p, _i64, _p, _p, _p, _p, _p, _p, _p, C.c_int, C.c_int])
 _sig("orc_conv2_direct_f32", [_p, _p, _p] + [_i64] * 7)
 _sig("orc_max_threads", [], C.c_int)
+_sig("orc_assign4", [_p, _i64, _p, _p, _i64, _p, _p, _i64])
+_sig("orc_scaled_add_f32", [_p, C.c_float, _p, _i64])
+_sig("orc_scaled_add_bf16", [_p, C.c_float, _p, _i64])
+_sig("orc_sgd_momentum_f32", [_p, _p, C.c_float, C.c_float, _p, _i64])
+_sig("orc_sgd_momentum_bf16", [_p, _p, C.c_float, C.c_float, _p, _i64])
+_sig("orc_sum_axis0_f32", [_p, _p, _i64, _i64])
+_sig("orc_sum_axis0_bf16", [_p, _p, _i64, _i64])
+_sig("orc_cross_entropy_loss_f32", [_p, _p, _i64, _i64], C.c_float)
+_sig("orc_cross_entropy_loss_bf16", [_p, _p, _i64, _i64], C.c_float)
+_sig("orc_cross_entropy_backward_f32", [_p, _p, C.c_float, _p, _i64, _i64])
+_sig("orc_cross_entropy_backward_bf16", [_p, _p, C.c_float, _p, _i64, _i64])
 
 
 def max_threads():
@@ -278,3 +289,123 @@ def lenet5_forward_f32(x, w1, w2, wd1, wd2, wd3, b3, threads=None, direct=False)
     _lib.orc_lenet5_forward_f32_alg(_ptr(arrs[0]), bs, *[_ptr(a) for a in arrs[1:]], _ptr(out),
                                     threads or min(4, max_threads()), 1 if direct else 0)
     return out
+
+
+# ------------------------------------------------------------- training tail ----
+def to_standard_layout(a):
+    """Strided copy (<= 4-D) of any numpy view into a fresh C-contiguous array, through orc_assign4."""
+    assert a.ndim <= 4
+    es = a.itemsize
+    base = a if a.base is None else a.base
+    while base.base is not None:
+        base = base.base
+    base = np.asarray(base)
+    off = (a.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // es
+    pad = 4 - a.ndim
+    dims = (C.c_int64 * 4)(*([1] * pad + list(a.shape)))
+    sx = (C.c_int64 * 4)(*([0] * pad + [st // es for st in a.strides]))
+    out = np.empty(a.shape, dtype=a.dtype)
+    sy = (C.c_int64 * 4)(*([0] * pad + [st // es for st in out.strides]))
+    _lib.orc_assign4(_ptr(base), off, sx, _ptr(out), 0, sy, dims, es)
+    return out
+
+
+def scaled_add(y, alpha, x):
+    """y + alpha * x with the product and the sum each rounded to the element type; returns a new array."""
+    y = np.array(y, order="C", copy=True)
+    x = np.ascontiguousarray(x)
+    assert x.shape == y.shape and x.dtype == y.dtype
+    (_lib.orc_scaled_add_bf16 if _is_bf16(y) else _lib.orc_scaled_add_f32)(_ptr(y), float(alpha), _ptr(x), y.size)
+    return y
+
+
+def sgd_momentum(w, dw, lr, momentum, v):
+    """Returns (w', v')."""
+    w, v = np.array(w, order="C", copy=True), np.array(v, order="C", copy=True)
+    dw = np.ascontiguousarray(dw)
+    (_lib.orc_sgd_momentum_bf16 if _is_bf16(w) else _lib.orc_sgd_momentum_f32)(_ptr(w), _ptr(dw), float(lr), float(momentum), _ptr(v), w.size)
+    return w, v
+
+
+def sum_axis0(x):
+    x = np.ascontiguousarray(x)
+    rows, cols = x.shape
+    y = np.empty(cols, dtype=x.dtype)
+    (_lib.orc_sum_axis0_bf16 if _is_bf16(x) else _lib.orc_sum_axis0_f32)(_ptr(x), _ptr(y), rows, cols)
+    return y
+
+
+def cross_entropy_loss(x, t):
+    x, t = np.ascontiguousarray(x), np.ascontiguousarray(t, dtype=np.uint8)
+    bs, classes = x.shape
+    return float((_lib.orc_cross_entropy_loss_bf16 if _is_bf16(x) else _lib.orc_cross_entropy_loss_f32)(_ptr(x), _ptr(t), bs, classes))
+
+
+def cross_entropy_backward(x, t, dy=1.0):
+    x, t = np.ascontiguousarray(x), np.ascontiguousarray(t, dtype=np.uint8)
+    bs, classes = x.shape
+    dx = np.empty_like(x)
+    (_lib.orc_cross_entropy_backward_bf16 if _is_bf16(x) else _lib.orc_cross_entropy_backward_f32)(_ptr(x), _ptr(t), float(dy), _ptr(dx), bs, classes)
+    return dx
+
+
+def lenet5_train_step(x, t, params, lr=0.01, momentum=None, velocities=None):
+    """One training step of the benchmark's LeNet5 (benches/neural-network-benches/src/autograph_backend.rs:70-86,
+    layers :88-162) chained from the host ops above in the order the autograd edges run them
+    (layer.rs:950-1005 conv, autograd.rs:607-627 dot, :571-599 bias, layer.rs:1253-1267 relu, :1193-1216 pool).
+    GEMMs use f32 accumulation with one rounding (the numerics the tolerance is stated against).
+    params = [w1, w2, wd1, wd2, wd3, b3]; returns (loss, new_params, grads, new_velocities)."""
+    w1, w2, wd1, wd2, wd3, b3 = params
+    bf = _is_bf16(w1)
+    mm = gemm_bf16_f32acc if bf else (lambda a, b: gemm_f64acc(a, b).astype(np.float32))
+    bs = x.shape[0]
+
+    def conv_fwd(h, w):
+        oc, ic, fh, fw = w.shape
+        cols = im2col_conv2(h, (fh, fw))
+        oh, ow = h.shape[2] - fh + 1, h.shape[3] - fw + 1
+        ym = mm(cols, w.reshape(oc, -1).T)
+        y = to_standard_layout(ym.reshape(bs, oh, ow, oc).transpose(0, 3, 1, 2))
+        return cols, y
+
+    cols1, c1 = conv_fwd(x, w1)
+    r1 = relu(c1)
+    p1 = max_pool2(r1, (2, 2))
+    cols2, c2 = conv_fwd(p1, w2)
+    r2 = relu(c2)
+    p2 = max_pool2(r2, (2, 2))
+    f = p2.reshape(bs, 256)
+    d1 = mm(f, wd1)
+    a1 = relu(d1)
+    d2 = mm(a1, wd2)
+    a2 = relu(d2)
+    logits = bias_add_rows(mm(a2, wd3), b3)
+    loss = cross_entropy_loss(logits, t)
+
+    g = cross_entropy_backward(logits, t, 1.0)
+    db3 = sum_axis0(g)
+    dwd3 = mm(a2.T, g)
+    g = relu_backward(d2, mm(g, wd3.T))
+    dwd2 = mm(a1.T, g)
+    g = relu_backward(d1, mm(g, wd2.T))
+    dwd1 = mm(f.T, g)
+    g = mm(g, wd1.T).reshape(bs, 16, 4, 4)
+    g = relu_backward(c2, max_pool2_backward(r2, g, (2, 2)))
+    gm = to_standard_layout(g.transpose(0, 2, 3, 1)).reshape(bs * 64, 16)
+    dw2 = mm(gm.T, cols2).reshape(w2.shape)
+    g = col2im_conv2(mm(gm, w2.reshape(16, 150)), (8, 8), (5, 5))
+    g = relu_backward(c1, max_pool2_backward(r1, g, (2, 2)))
+    gm = to_standard_layout(g.transpose(0, 2, 3, 1)).reshape(bs * 576, 6)
+    dw1 = mm(gm.T, cols1).reshape(w1.shape)
+
+    grads = [dw1, dw2, dwd1, dwd2, dwd3, db3]
+    if momentum is None:
+        alpha = -lr
+        new_params = [scaled_add(p, alpha, gr) for p, gr in zip(params, grads)]
+        new_v = None
+    else:
+        if velocities is None:
+            velocities = [np.zeros_like(p) for p in params]
+        pairs = [sgd_momentum(p, gr, lr, momentum, v) for p, gr, v in zip(params, grads, velocities)]
+        new_params, new_v = [a for a, _ in pairs], [b for _, b in pairs]
+    return loss, new_params, grads, new_v

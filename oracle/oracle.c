@@ -546,6 +546,128 @@ void orc_lenet5_forward_f32_alg(const float *x, i64 bs, const float *w1, const f
     free(c1); free(p1); free(c2); free(p2); free(d1); free(d2);
 }
 
+/* ------------------------------------------------- training tail (host) ---- */
+
+/* Strided copy of up to 4 dims, same element type: `assign` with BinaryOp::Identity, alpha = 1
+ * (src/tensor/ops.rs:257-318): y[i] = x[i] over the index space `d`, element strides sx / sy
+ * (a stride 0 on x is a broadcast).  es = element size in bytes. */
+void orc_assign4(const void *x, i64 off_x, const i64 *sx, void *y, i64 off_y, const i64 *sy, const i64 *d, i64 es) {
+    const unsigned char *xb = (const unsigned char *)x;
+    unsigned char *yb = (unsigned char *)y;
+    for (i64 i0 = 0; i0 < d[0]; ++i0)
+        for (i64 i1 = 0; i1 < d[1]; ++i1)
+            for (i64 i2 = 0; i2 < d[2]; ++i2)
+                for (i64 i3 = 0; i3 < d[3]; ++i3) {
+                    const i64 ix = off_x + i0 * sx[0] + i1 * sx[1] + i2 * sx[2] + i3 * sx[3];
+                    const i64 iy = off_y + i0 * sy[0] + i1 * sy[1] + i2 * sy[2] + i3 * sy[3];
+                    memcpy(yb + iy * es, xb + ix * es, (size_t)es);
+                }
+}
+
+/* scaled_add: y = alpha * x + y with BinaryOp::Add (src/tensor/ops.rs:294-296 `op.eval(alpha * x, y)`):
+ * the product and the sum are each one operation in T.  alpha is given in T's precision already
+ * (optimizer.rs:420-423 casts -learning_rate to the parameter type first). */
+void orc_scaled_add_f32(float *y, float alpha, const float *x, i64 n) {
+    for (i64 i = 0; i < n; ++i) {
+        volatile float prod = alpha * x[i];
+        y[i] = prod + y[i];
+    }
+}
+void orc_scaled_add_bf16(bf16_t *y, float alpha, const bf16_t *x, i64 n) {
+    const bf16_t a = f32_to_bf16(alpha);
+    for (i64 i = 0; i < n; ++i) y[i] = bf16_add(bf16_mul(a, x[i]), y[i]);
+}
+
+/* SGD with momentum (optimizer.rs:430-465, kernel :509-512): in f32, v = m*v + dw; w -= lr*v; then
+ * both cast back to T. */
+void orc_sgd_momentum_f32(float *w, const float *dw, float lr, float m, float *v, i64 n) {
+    for (i64 i = 0; i < n; ++i) {
+        volatile float mv = m * v[i];
+        const float vn = mv + dw[i];
+        volatile float step = lr * vn;
+        v[i] = vn;
+        w[i] = w[i] - step;
+    }
+}
+void orc_sgd_momentum_bf16(bf16_t *w, const bf16_t *dw, float lr, float m, bf16_t *v, i64 n) {
+    for (i64 i = 0; i < n; ++i) {
+        volatile float mv = m * bf16_to_f32(v[i]);
+        const float vn = mv + bf16_to_f32(dw[i]);
+        volatile float step = lr * vn;
+        v[i] = f32_to_bf16(vn);
+        w[i] = f32_to_bf16(bf16_to_f32(w[i]) - step);
+    }
+}
+
+/* Sum over axis 0 of a row-major [rows, cols] array, as ndarray's sum_axis does it when the axis is
+ * not the one with the smallest stride (reduce.rs:59-62 -> ndarray `res = res + &subview` per row):
+ * zeros, then one add in T per row, rows ascending.  This is the bias gradient (autograd.rs:490-542). */
+void orc_sum_axis0_f32(const float *x, float *y, i64 rows, i64 cols) {
+    for (i64 j = 0; j < cols; ++j) y[j] = 0.0f;
+    for (i64 i = 0; i < rows; ++i)
+        for (i64 j = 0; j < cols; ++j) y[j] = y[j] + x[i * cols + j];
+}
+void orc_sum_axis0_bf16(const bf16_t *x, bf16_t *y, i64 rows, i64 cols) {
+    for (i64 j = 0; j < cols; ++j) y[j] = 0;
+    for (i64 i = 0; i < rows; ++i)
+        for (i64 j = 0; j < cols; ++j) y[j] = bf16_add(y[j], x[i * cols + j]);
+}
+
+/* cross_entropy_loss_host (src/learn/criterion.rs:205-226): per row, m = max in f32, s = sum of
+ * exp(x - m) in f32 in element order, loss += ln(s) - (x[t] - m), rows in order, all f32. */
+static float ce_loss_rows(const float *row_f32, i64 classes, i64 t) {
+    float m = row_f32[0];
+    for (i64 j = 0; j < classes; ++j) m = fmaxf(m, row_f32[j]);
+    float s = 0.0f;
+    for (i64 j = 0; j < classes; ++j) s += expf(row_f32[j] - m);
+    return logf(s) - (row_f32[t] - m);
+}
+float orc_cross_entropy_loss_f32(const float *x, const uint8_t *t, i64 bs, i64 classes) {
+    float y = 0.0f;
+    for (i64 i = 0; i < bs; ++i) y += ce_loss_rows(x + i * classes, classes, t[i]);
+    return y;
+}
+float orc_cross_entropy_loss_bf16(const bf16_t *x, const uint8_t *t, i64 bs, i64 classes) {
+    float y = 0.0f;
+    float *row = (float *)malloc((size_t)classes * sizeof(float));
+    for (i64 i = 0; i < bs; ++i) {
+        for (i64 j = 0; j < classes; ++j) row[j] = bf16_to_f32(x[i * classes + j]);
+        y += ce_loss_rows(row, classes, t[i]);
+    }
+    free(row);
+    return y;
+}
+
+/* cross_entropy_loss_backward host branch (src/learn/neural_network/criterion.rs:79-103):
+ * dy /= bs; dx = T(dy * (exp(x - m) / s - [j == t])) with f32 arithmetic. */
+static void ce_backward_row(const float *row, float *out, i64 classes, i64 t, float dy) {
+    float m = row[0];
+    for (i64 j = 0; j < classes; ++j) m = fmaxf(m, row[j]);
+    float s = 0.0f;
+    for (i64 j = 0; j < classes; ++j) s += expf(row[j] - m);
+    for (i64 j = 0; j < classes; ++j) {
+        const float onehot = (j == t) ? 1.0f : 0.0f;
+        volatile float p = expf(row[j] - m) / s;
+        volatile float diff = p - onehot;
+        out[j] = dy * diff;
+    }
+}
+void orc_cross_entropy_backward_f32(const float *x, const uint8_t *t, float dy, float *dx, i64 bs, i64 classes) {
+    dy /= (float)bs;
+    for (i64 i = 0; i < bs; ++i) ce_backward_row(x + i * classes, dx + i * classes, classes, t[i], dy);
+}
+void orc_cross_entropy_backward_bf16(const bf16_t *x, const uint8_t *t, float dy, bf16_t *dx, i64 bs, i64 classes) {
+    dy /= (float)bs;
+    float *row = (float *)malloc((size_t)classes * 2 * sizeof(float));
+    float *out = row + classes;
+    for (i64 i = 0; i < bs; ++i) {
+        for (i64 j = 0; j < classes; ++j) row[j] = bf16_to_f32(x[i * classes + j]);
+        ce_backward_row(row, out, classes, t[i], dy);
+        for (i64 j = 0; j < classes; ++j) dx[i * classes + j] = f32_to_bf16(out[j]);
+    }
+    free(row);
+}
+
 int orc_max_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

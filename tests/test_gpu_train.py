@@ -1,0 +1,171 @@
+"""GPU parity of the kernels a training step adds around the contraction path (strided copy,
+scaled_add, SGD, axis-0 sum, cross-entropy) and of one whole LeNet5 training step
+(benches/neural-network-benches/src/autograph_backend.rs:70-86) against the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ag():
+    import autograph_amd as ag
+    ag.Device(0)
+    return ag
+
+
+def to_dtype(x, dtype):
+    return orc.f32_to_bf16(x) if dtype == "bf16" else np.ascontiguousarray(x, dtype=np.float32)
+
+
+def as_f32(x):
+    return orc.bf16_to_f32(x) if x.dtype == np.uint16 else x
+
+
+def labels(ag, t):
+    buf = ag.Buffer(t.size)
+    ag._ffi.check(ag.lib.agh_memcpy_h2d(buf.ptr, t.ctypes.data, t.size))
+    ag._ffi.check(ag.lib.agh_sync())
+    return buf
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_assign_strided_views(ag, dtype):
+    rng = np.random.default_rng(41)
+    base = to_dtype(rng.standard_normal((5, 6, 7, 8)), dtype)
+    t = ag.Tensor.from_array(base)
+    for axes in [(0, 2, 3, 1), (0, 3, 1, 2), (3, 2, 1, 0), (1, 0, 3, 2)]:
+        got = t.permuted_axes(axes).to_standard_layout().into_array()
+        assert np.array_equal(got, np.ascontiguousarray(base.transpose(axes)))
+    m = ag.Tensor.from_array(base.reshape(30, 56))
+    assert np.array_equal(m.t().to_standard_layout().into_array(), np.ascontiguousarray(base.reshape(30, 56).T))
+    assert np.array_equal(m.slice_rows(None, None, -2).to_standard_layout().into_array(), base.reshape(30, 56)[::-2])
+    v = ag.Tensor.from_array(base[0, 0, 0])  # [8] broadcast over rows
+    assert np.array_equal(v.broadcast((4, 8)).to_standard_layout().into_array(), np.broadcast_to(base[0, 0, 0], (4, 8)))
+    # the conv backward's NCHW -> NHWC copy at LeNet5 size
+    g = to_dtype(rng.standard_normal((100, 16, 8, 8)), dtype)
+    got = ag.Tensor.from_array(g).permuted_axes((0, 2, 3, 1)).to_standard_layout().into_array()
+    assert np.array_equal(got, orc.to_standard_layout(g.transpose(0, 2, 3, 1)))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_scaled_add_sgd_sum_axis0_bit_exact(ag, dtype):
+    rng = np.random.default_rng(42)
+    for n in (1, 255, 46920, 300001):
+        y, x, v = (to_dtype(rng.standard_normal(n), dtype) for _ in range(3))
+        ty = ag.Tensor.from_array(y)
+        ty.scaled_add(-0.01, ag.Tensor.from_array(x))
+        assert np.array_equal(ty.into_array(), orc.scaled_add(y, -0.01, x))
+        tw, tv = ag.Tensor.from_array(y), ag.Tensor.from_array(v)
+        ag.SGD(momentum=0.9).update(0.01, tw, ag.Tensor.from_array(x), tv)
+        w2, v2 = orc.sgd_momentum(y, x, 0.01, 0.9, v)
+        assert np.array_equal(tw.into_array(), w2) and np.array_equal(tv.into_array(), v2)
+    for rows, cols in [(100, 10), (1, 7), (1000, 300), (257, 1)]:
+        a = to_dtype(rng.standard_normal((rows, cols)) * 4, dtype)
+        assert np.array_equal(ag.Tensor.from_array(a).sum_axis0().into_array(), orc.sum_axis0(a))
+    a = to_dtype(np.array([[256.0, 1.0]] + [[1.0, 1.0]] * 64), dtype)
+    assert np.array_equal(ag.Tensor.from_array(a).sum_axis0().into_array(), orc.sum_axis0(a))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_cross_entropy(ag, dtype):
+    rng = np.random.default_rng(43)
+    for bs, classes in [(100, 10), (7, 3), (1000, 10), (513, 256)]:
+        x = to_dtype(rng.standard_normal((bs, classes)) * 3, dtype)
+        t = rng.integers(0, classes, bs).astype(np.uint8)
+        tx, tt = ag.Tensor.from_array(x), labels(ag, t)
+        want = orc.cross_entropy_loss(x, t)
+        got = tx.cross_entropy_loss(tt)
+        assert abs(got - want) <= 2e-6 * bs + 1e-6 * abs(want), (got, want)  # expf / logf differ by an ulp or two
+        g = tx.cross_entropy_loss_backward(tt).into_array()
+        wg = orc.cross_entropy_backward(x, t)
+        if dtype == "f32":
+            assert np.all(np.abs(g - wg) <= 4e-6 * np.abs(wg) + 1e-9)
+        else:
+            gf, wf = as_f32(g).astype(np.float64), as_f32(wg).astype(np.float64)
+            assert np.all(np.abs(gf - wf) <= 2.0**-7 * np.abs(wf))  # at most one bf16 step apart
+            assert np.mean(g != wg) < 0.01
+    x = to_dtype(np.array([[1000.0, 999.0, -1000.0]]), dtype)
+    tt = labels(ag, np.array([1], dtype=np.uint8))
+    assert abs(ag.Tensor.from_array(x).cross_entropy_loss(tt) - orc.cross_entropy_loss(x, np.array([1], dtype=np.uint8))) < 1e-5
+
+
+def he(rng, shape, fan_in):
+    a = np.sqrt(2.0 / fan_in)
+    return rng.uniform(-a, a, shape).astype(np.float32)
+
+
+def lenet_params(rng):
+    return [he(rng, (6, 1, 5, 5), 25), he(rng, (16, 6, 5, 5), 150), he(rng, (256, 128), 256), he(rng, (128, 84), 128),
+            he(rng, (84, 10), 84), he(rng, (10,), 84)]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("momentum", [None, 0.01])
+def test_lenet5_train_step(ag, dtype, momentum):
+    rng = np.random.default_rng(44)
+    params = [to_dtype(p, dtype) for p in lenet_params(rng)]
+    bs = 100
+    x = to_dtype(rng.uniform(0, 1, (bs, 1, 28, 28)), dtype)
+    t = rng.integers(0, 10, bs).astype(np.uint8)
+    want_loss, want_params, want_grads, want_v = orc.lenet5_train_step(x, t, params, lr=0.01, momentum=momentum)
+
+    model = ag.LeNet5.from_arrays(*params)
+    trainer = ag.LeNet5Trainer(model, bs, learning_rate=0.01, optimizer=ag.SGD(momentum))
+    tx, tt = ag.Tensor.from_array(x), labels(ag, t)
+    trainer.step(tx, tt)
+    ag._ffi.check(ag.lib.agh_sync())
+    assert abs(trainer.loss() - want_loss) <= (1e-5 if dtype == "f32" else 1e-2) * abs(want_loss)
+    for name, g, w in zip(("dw1", "dw2", "dwd1", "dwd2", "dwd3", "db3"), trainer.grads, want_grads):
+        gf, wf = as_f32(g.into_array()).astype(np.float64), as_f32(w).astype(np.float64)
+        scale = np.abs(wf).max()
+        if dtype == "f32":
+            # f32 sums in another order (k up to 57600 for dw1): 1e-5 * sqrt(k) of the scale
+            assert np.abs(gf - wf).max() <= 3e-3 * scale, name
+        else:
+            # bf16: every GEMM may differ from the oracle's by one rounding, and a flipped relu / pool
+            # decision moves single entries; the bulk has to agree
+            assert np.abs(gf - wf).max() <= 0.1 * scale, name
+            assert np.abs(gf - wf).mean() <= 0.01 * scale, name
+    for name, p, w, old in zip(("w1", "w2", "wd1", "wd2", "wd3", "b3"), trainer.params, want_params, params):
+        pf, wf, of = (as_f32(a).astype(np.float64) for a in (p.into_array(), w, old))
+        step = np.abs(wf - of).max()
+        assert np.abs(pf - wf).max() <= (3e-3 if dtype == "f32" else 0.1) * step + (0 if dtype == "f32" else 2.0**-8 * np.abs(wf).max()), name
+    # the update itself is exact: applying the oracle's update to the GPU's own gradients gives the GPU's parameters
+    for p, old, g, v in zip(trainer.params, params, trainer.grads, trainer.velocities):
+        ga = g.into_array()
+        if momentum is None:
+            assert np.array_equal(p.into_array(), orc.scaled_add(old, -0.01, ga))
+        else:
+            w2, v2 = orc.sgd_momentum(old, ga, 0.01, momentum, np.zeros_like(old))
+            assert np.array_equal(p.into_array(), w2) and np.array_equal(v.into_array(), v2)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_lenet5_train_graph_replay_equals_eager(ag, dtype):
+    rng = np.random.default_rng(45)
+    params = [to_dtype(p, dtype) for p in lenet_params(rng)]
+    bs = 100
+    x = to_dtype(rng.uniform(0, 1, (bs, 1, 28, 28)), dtype)
+    t = rng.integers(0, 10, bs).astype(np.uint8)
+    tx, tt = ag.Tensor.from_array(x), labels(ag, t)
+    eager = ag.LeNet5Trainer(ag.LeNet5.from_arrays(*params), bs, optimizer=ag.SGD(0.01))
+    graph = ag.LeNet5Trainer(ag.LeNet5.from_arrays(*params), bs, optimizer=ag.SGD(0.01))
+    graph.capture(tx, tt)  # two steps: one eager, one while recording... recording does not execute
+    losses = []
+    for i in range(3):
+        eager.step(tx, tt)
+        ag._ffi.check(ag.lib.agh_sync())
+        losses.append(eager.loss())
+    # capture() ran ONE real step (work recorded during capture is not executed); two replays follow
+    for i in range(2):
+        graph.replay()
+        ag._ffi.check(ag.lib.agh_sync())
+        assert graph.loss() == losses[i + 1], i
+    for a, b in zip(eager.params, graph.params):
+        assert np.array_equal(a.into_array(), b.into_array())
+    assert losses[2] < losses[0]  # three steps on the same batch lower its loss

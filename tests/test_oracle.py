@@ -386,3 +386,146 @@ def test_conv2_direct_host_vs_torch():
         want = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double()).numpy()
         got = orc.conv2_direct_f32(x, w)
         assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(ic * f[0] * f[1]) * np.max(np.abs(want))
+
+
+# ------------------------------------------------------------ training tail ----
+def tbf(x):
+    """numpy uint16 bf16 bits -> torch.bfloat16 tensor."""
+    return torch.from_numpy(np.ascontiguousarray(x).view(np.int16)).view(torch.bfloat16)
+
+
+def tbits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def test_assign4_strided_views_vs_numpy():
+    rng = np.random.default_rng(31)
+    base = rng.integers(0, 2**16, (5, 6, 7, 8)).astype(np.uint16)
+    views = [base.transpose(0, 2, 3, 1), base.transpose(3, 2, 1, 0), base[::2, ::-1, 1:6, ::3], base[:, 2],
+             base[1, :, 3], np.broadcast_to(base[0, 0, 0], (4, 8)), base.astype(np.float32).transpose(0, 3, 1, 2)]
+    for v in views:
+        got = orc.to_standard_layout(v)
+        assert got.flags["C_CONTIGUOUS"] and np.array_equal(got, np.ascontiguousarray(v))
+
+
+def test_scaled_add_vs_torch_per_op_rounding():
+    """bf16: the product and the sum round separately (torch.bfloat16 elementwise ops do exactly that)."""
+    rng = np.random.default_rng(32)
+    y = orc.f32_to_bf16(rng.standard_normal(5000).astype(np.float32))
+    x = orc.f32_to_bf16(rng.standard_normal(5000).astype(np.float32) * 3)
+    alpha = -0.01
+    a_t = torch.tensor(alpha, dtype=torch.float32).to(torch.bfloat16)
+    want = tbits(a_t * tbf(x) + tbf(y))
+    assert np.array_equal(orc.scaled_add(y, alpha, x), want)
+    # a fused multiply-add would differ somewhere on this much data: the check can tell the two apart
+    fused = orc.f32_to_bf16(orc.bf16_to_f32(y) + float(a_t) * orc.bf16_to_f32(x))
+    assert not np.array_equal(fused, want)
+    yf, xf = rng.standard_normal(1000).astype(np.float32), rng.standard_normal(1000).astype(np.float32)
+    assert np.array_equal(orc.scaled_add(yf, 0.3, xf), (np.float32(0.3) * xf) + yf)
+
+
+def test_sgd_momentum_vs_closed_form():
+    rng = np.random.default_rng(33)
+    w, dw, v = (rng.standard_normal(3000).astype(np.float32) for _ in range(3))
+    lr, m = np.float32(0.01), np.float32(0.9)
+    vn = m * v + dw
+    w2, v2 = orc.sgd_momentum(w, dw, lr, m, v)
+    assert np.array_equal(v2, vn) and np.array_equal(w2, w - lr * vn)
+    wb, dwb, vb = orc.f32_to_bf16(w), orc.f32_to_bf16(dw), orc.f32_to_bf16(v)
+    vnf = m * orc.bf16_to_f32(vb) + orc.bf16_to_f32(dwb)
+    w2, v2 = orc.sgd_momentum(wb, dwb, lr, m, vb)
+    # the weight uses the UNrounded new velocity (optimizer.rs:509-512 runs in f32, casts at the end)
+    assert np.array_equal(v2, bf16_bits_torch(vnf)) and np.array_equal(w2, bf16_bits_torch(orc.bf16_to_f32(wb) - lr * vnf))
+
+
+def test_sum_axis0_is_sequential_in_element_type():
+    # 256 + 1 + 1 + ... in bf16 stays 256 when added one by one (ulp(256) = 2); any pairwise order gives more
+    x = orc.f32_to_bf16(np.array([[256.0, 1.0]] + [[1.0, 1.0]] * 64, dtype=np.float32))
+    assert orc.bf16_to_f32(orc.sum_axis0(x)).tolist() == [256.0, 65.0]
+    rng = np.random.default_rng(34)
+    xb = orc.f32_to_bf16(rng.standard_normal((100, 10)).astype(np.float32))
+    acc = torch.zeros(10, dtype=torch.bfloat16)
+    for row in tbf(xb):
+        acc = acc + row
+    assert np.array_equal(orc.sum_axis0(xb), tbits(acc))
+    xf = rng.standard_normal((50, 7)).astype(np.float32)
+    want = np.zeros(7, dtype=np.float32)
+    for row in xf:
+        want = want + row
+    assert np.array_equal(orc.sum_axis0(xf), want)
+
+
+def test_cross_entropy_vs_torch():
+    rng = np.random.default_rng(35)
+    for bs, classes in [(100, 10), (7, 3), (1, 5)]:
+        x = (rng.standard_normal((bs, classes)) * 3).astype(np.float32)
+        t = rng.integers(0, classes, bs).astype(np.uint8)
+        xt = torch.from_numpy(x).double().requires_grad_(True)
+        loss = F.cross_entropy(xt, torch.from_numpy(t).long(), reduction="sum")
+        (loss / bs).backward()
+        assert abs(orc.cross_entropy_loss(x, t) - loss.item()) <= 2e-6 * max(1.0, abs(loss.item()))
+        assert np.allclose(orc.cross_entropy_backward(x, t), xt.grad.numpy(), rtol=1e-5, atol=1e-8)
+        xb = orc.f32_to_bf16(x)
+        xbt = torch.from_numpy(orc.bf16_to_f32(xb)).double().requires_grad_(True)
+        lossb = F.cross_entropy(xbt, torch.from_numpy(t).long(), reduction="sum")
+        (lossb / bs).backward()
+        assert abs(orc.cross_entropy_loss(xb, t) - lossb.item()) <= 2e-6 * max(1.0, abs(lossb.item()))
+        gb = orc.bf16_to_f32(orc.cross_entropy_backward(xb, t)).astype(np.float64)
+        assert np.all(np.abs(gb - xbt.grad.numpy()) <= 2.0**-8 * np.abs(xbt.grad.numpy()) + 1e-12)
+    # huge logits: the max is subtracted before exp
+    x = np.array([[1000.0, 999.0, -1000.0]], dtype=np.float32)
+    assert abs(orc.cross_entropy_loss(x, np.array([1], dtype=np.uint8)) - (np.log1p(np.exp(-1.0)) + 1.0)) < 1e-6
+
+
+def lenet_params_np(rng):
+    def he(shape, fan_in):
+        a = np.sqrt(2.0 / fan_in)
+        return rng.uniform(-a, a, shape).astype(np.float32)
+    return [he((6, 1, 5, 5), 25), he((16, 6, 5, 5), 150), he((256, 128), 256), he((128, 84), 128), he((84, 10), 84), he((10,), 84)]
+
+
+def torch_lenet_grads(x, t, params):
+    p = [torch.from_numpy(a).double().requires_grad_(True) for a in params]
+    h = F.max_pool2d(F.relu(F.conv2d(torch.from_numpy(x).double(), p[0])), 2)
+    h = F.max_pool2d(F.relu(F.conv2d(h, p[1])), 2).reshape(x.shape[0], 256)
+    logits = F.relu(F.relu(h @ p[2]) @ p[3]) @ p[4] + p[5]
+    loss = F.cross_entropy(logits, torch.from_numpy(t).long(), reduction="sum")
+    (loss / x.shape[0]).backward()
+    return loss.item(), [a.grad.numpy() for a in p]
+
+
+def test_lenet5_train_step_f32_vs_torch_autograd():
+    """Pins the whole backward chain (transposes, col2im geometry, pool/relu masks, bias sum, update sign)."""
+    rng = np.random.default_rng(36)
+    params = lenet_params_np(rng)
+    x = rng.uniform(0, 1, (20, 1, 28, 28)).astype(np.float32)
+    t = rng.integers(0, 10, 20).astype(np.uint8)
+    loss, new_params, grads, _ = orc.lenet5_train_step(x, t, params, lr=0.01)
+    want_loss, want_grads = torch_lenet_grads(x, t, params)
+    assert abs(loss - want_loss) <= 1e-5 * abs(want_loss)
+    for g, w, p, pn in zip(grads, want_grads, params, new_params):
+        assert g.shape == w.shape
+        assert np.abs(g - w).max() <= 2e-5 * max(1e-3, np.abs(w).max())
+        assert np.array_equal(pn, (np.float32(-0.01) * g) + p)
+    # momentum variant: first step from zero velocity
+    _, p_m, _, v_m = orc.lenet5_train_step(x, t, params, lr=0.01, momentum=0.01)
+    for g, p, pn, v in zip(grads, params, p_m, v_m):
+        assert np.array_equal(v, g) and np.array_equal(pn, p - np.float32(0.01) * g)
+
+
+def test_lenet5_train_step_bf16_close_to_f64_grads():
+    rng = np.random.default_rng(37)
+    params = [orc.f32_to_bf16(p) for p in lenet_params_np(rng)]
+    x = orc.f32_to_bf16(rng.uniform(0, 1, (20, 1, 28, 28)).astype(np.float32))
+    t = rng.integers(0, 10, 20).astype(np.uint8)
+    loss, new_params, grads, _ = orc.lenet5_train_step(x, t, params, lr=0.01)
+    want_loss, want_grads = torch_lenet_grads(orc.bf16_to_f32(x), t, [orc.bf16_to_f32(p) for p in params])
+    assert abs(loss - want_loss) <= 2e-2 * abs(want_loss)
+    for g, w in zip(grads, want_grads):
+        gf = orc.bf16_to_f32(g).astype(np.float64)
+        # bf16 activations and gradients round at every layer (and flip a few relu/pool decisions):
+        # up to about a tenth of the largest entry on single elements, far less on average
+        assert np.abs(gf - w).max() <= 0.12 * np.abs(w).max()
+        assert np.abs(gf - w).mean() <= 0.02 * np.abs(w).max()
+    for p, pn, g in zip(params, new_params, grads):
+        assert np.array_equal(pn, orc.scaled_add(p, -0.01, g))
