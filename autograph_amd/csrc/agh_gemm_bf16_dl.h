@@ -229,7 +229,6 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     using S2 = std::integral_constant<int, 2>;
     using S3 = std::integral_constant<int, 3>;
     using Yes = std::true_type;
-    using No = std::false_type;
     using L_0 = std::integral_constant<int, 0>;
     using L_T = std::integral_constant<int, NLT>;
 

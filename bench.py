@@ -265,6 +265,68 @@ def main():
             extras["lenet5_f32_infer_b1000"] = {"error": str(e)}
             log("lenet5: FAILED", e)
 
+    # ---------------- LeNet5 training step, batch 100 (BASELINE configs[4]) ----------------
+    if not args.no_extras:
+        for dt in ("bf16", "f32"):
+            key = f"lenet5_{dt}_train_b100"
+            try:
+                bst = 100
+                conv = (lambda a: orc.f32_to_bf16(a)) if dt == "bf16" else (lambda a: a)
+                xt = conv(rng.uniform(0, 1, (bst, 1, 28, 28)).astype(np.float32))
+                tt = rng.integers(0, 10, bst).astype(np.uint8)
+
+                def he2(shape, fan_in):
+                    a_ = np.sqrt(2.0 / fan_in)
+                    return conv(rng.uniform(-a_, a_, shape).astype(np.float32))
+
+                tparams = [he2((6, 1, 5, 5), 25), he2((16, 6, 5, 5), 150), he2((256, 128), 256), he2((128, 84), 128),
+                           he2((84, 10), 84), he2((10,), 84)]
+                trainer = ag.LeNet5Trainer(ag.LeNet5.from_arrays(*tparams), bst, learning_rate=0.01, optimizer=ag.SGD(0.01))
+                txx = ag.Tensor.from_array(xt)
+                tbuf = ag.Buffer(bst)
+                ag._ffi.check(ag.lib.agh_memcpy_h2d(tbuf.ptr, tt.ctypes.data, bst))
+                trainer.capture(txx, tbuf)
+
+                def train_graph():
+                    trainer.replay()
+                    ag._ffi.check(ag.lib.agh_sync())  # the loss is in host memory when this returns
+
+                def train_eager():
+                    trainer.step(txx, tbuf)
+                    ag._ffi.check(ag.lib.agh_sync())
+
+                for _ in range(20):
+                    train_graph()
+                t0 = time.perf_counter()
+                for _ in range(200):
+                    train_graph()
+                g_ms = (time.perf_counter() - t0) * 1e3 / 200
+                for _ in range(5):
+                    train_eager()
+                t0 = time.perf_counter()
+                for _ in range(50):
+                    train_eager()
+                e_ms = (time.perf_counter() - t0) * 1e3 / 50
+                rec = {"gpu_ms": round(g_ms, 4), "gpu_eager_ms": round(e_ms, 4), "last_loss": round(trainer.loss(), 4),
+                       "what": "forward + summed cross-entropy + backward + SGD(momentum 0.01) update, 45 launches; gpu_ms: "
+                               "graph replay, wall clock per step including the host-side wait for the loss; "
+                               "gpu_eager_ms: the same launches issued one by one from the host"}
+                if not args.no_cpu:
+                    orc.lenet5_train_step(xt, tt, tparams, lr=0.01, momentum=0.01)
+                    t0 = time.perf_counter()
+                    for _ in range(10):
+                        orc.lenet5_train_step(xt, tt, tparams, lr=0.01, momentum=0.01)
+                    c_ms = (time.perf_counter() - t0) * 1e3 / 10
+                    rec.update({"cpu_ms": round(c_ms, 3), "speedup": round(c_ms / g_ms, 1),
+                                "cpu_what": "oracle port of the host ops chained in Python; its bf16 GEMMs accumulate in f32 "
+                                            "(the host's per-operation-rounded fold would be slower still)"})
+                extras[key] = rec
+                log(f"lenet5 {dt} train b=100:", rec)
+                del trainer
+            except Exception as e:
+                extras[key] = {"error": str(e)}
+                log(f"lenet5 {dt} train: FAILED", e)
+
     # ---------------- CPU baseline: the oracle's restatement of the host path ----------------
     cpu = None
     if not args.no_cpu:
