@@ -53,6 +53,8 @@ struct Im2colParams {
     int span_pad;  // LDS row pitch (elements)
     int nslot;     // 16-byte pieces per image row (vector staging)
     int npad;      // padding cells per staged row: pw on the left, the rest right of the image
+    int nblocks;   // workgroups with work
+    int per_xcd;   // ceil(nblocks / 8)
     int ktot;      // c*fh*fw
     FastDiv div_l, div_ff, div_fw, div_nchunk, div_oh, div_span, div_fh, div_nslot, div_npad;
 };
@@ -62,7 +64,11 @@ __global__ __launch_bounds__(kThreads) void im2col_lds_kernel(const T *__restric
                                                                Im2colParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     // layout: int tab[L rounded to 4] | T tile[cc*fh*span_pad]
-    uint32_t bid = blockIdx.x;
+    // Workgroup ids are dealt round-robin to the 8 XCDs, each with an L2 of its own.  Neighbouring
+    // output rows of an image stage the same input rows, so every XCD is given a contiguous run of
+    // (image, output row) pairs: the re-reads then hit its L2 instead of going out to memory again.
+    const uint32_t bid = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (bid >= (uint32_t)p.nblocks) return;
     uint32_t t0, chunk, b, ho;
     p.div_nchunk.divmod(bid, t0, chunk);
     p.div_oh.divmod(t0, b, ho);
@@ -314,10 +320,12 @@ int im2col_launch(const char *name, const void *x, void *y, int64_t bs, int64_t 
     p.div_nslot = FastDiv((uint32_t)std::max(1, p.nslot));
     p.div_npad = FastDiv((uint32_t)std::max(1, p.npad));
     const int64_t nblocks = bs * oh * p.nchunk;
-    if (nblocks > 0x7FFFFFFFll) return fail(AGH_ERANGE, "%s: too many workgroups", name);
+    if (nblocks > 0x7FFFFFF0ll) return fail(AGH_ERANGE, "%s: too many workgroups", name);
     const size_t smem = (size_t)lds_bytes(cc);
+    p.nblocks = (int)nblocks;
+    p.per_xcd = (int)((nblocks + 7) / 8);
     auto launch = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, dim3((unsigned)nblocks), dim3(kThreads), smem, stream(), (const T *)x, (T *)y, p);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(p.per_xcd * 8)), dim3(kThreads), smem, stream(), (const T *)x, (T *)y, p);
     };
     if (vec && vstage) launch(im2col_lds_kernel<T, VEC, true>);
     else if (vec) launch(im2col_lds_kernel<T, VEC, false>);

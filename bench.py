@@ -71,11 +71,15 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
+    ap.add_argument("--sections", default="kernels,lenet,train",
+                    help="which extras to run: kernels (other GEMMs, im2col/col2im/pool), lenet (inference), "
+                         "train (training step); the last two replay captured graphs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib", action="store_true",
                     help="also run a plain elementwise pass of known size (agh_relu_f32 over 2^28 floats: 1 GiB read, "
                          "1 GiB written) so HBM byte counters of a profiler run can be scaled against it")
     args = ap.parse_args()
+    sections = set(args.sections.split(","))
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); nothing here runs across GPUs")
 
@@ -118,7 +122,7 @@ def main():
         log(f"calibration pass: {ms:.3f} ms  {8.0 * ncal / ms / 1e6:.0f} GB/s")
         del cx, cy
 
-    if not args.no_extras:
+    if not args.no_extras and "kernels" in sections:
         ks, kw = max(3, args.steps // 4), 2
 
         def run(name, fn, work, unit, peak, steps=ks):
@@ -198,7 +202,7 @@ def main():
 
     # ---------------- LeNet5 f32 inference, batch 1000 (BASELINE configs[0]) ----------------
     lenet = None
-    if not args.no_extras:
+    if not args.no_extras and "lenet" in sections:
         try:
             bsl = 1000
             xl = rng.uniform(0, 1, (bsl, 1, 28, 28)).astype(np.float32)
@@ -266,7 +270,7 @@ def main():
             log("lenet5: FAILED", e)
 
     # ---------------- LeNet5 training step, batch 100 (BASELINE configs[4]) ----------------
-    if not args.no_extras:
+    if not args.no_extras and "train" in sections:
         for dt in ("bf16", "f32"):
             key = f"lenet5_{dt}_train_b100"
             try:
