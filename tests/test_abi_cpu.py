@@ -43,3 +43,16 @@ def test_option_shape_formulas():
     c = Col2ImConv2Options(shape=(5, 6), filter=(3, 5), padding=(1, 0), stride=(2, 1), dilation=(1, 2))
     assert c.output_shape() == (orc.col2im_out(5, 3, 1, 2, 1), orc.col2im_out(6, 5, 0, 1, 2))
     assert MaxPool2Options((2, 3), (2, 2)).output_shape((9, 8)) == (orc.pool_out(9, 2, 2), orc.pool_out(8, 3, 2))
+
+
+def test_rust_sys_crate_declares_the_header():
+    """rust/autograph-hip-sys/src/lib.rs (source only, no Rust toolchain here) must declare every entry
+    point of the header with the same number of arguments."""
+    text = open(os.path.join(ROOT, "include", "autograph_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    c_decls = {n: (0 if a.strip() in ("", "void") else a.count(",") + 1)
+               for n, a in re.findall(r"\b(agh_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text)}
+    rs = open(os.path.join(ROOT, "rust", "autograph-hip-sys", "src", "lib.rs")).read()
+    rs_decls = {n: (0 if not a.strip() else a.count(",") + 1) for n, a in re.findall(r"pub fn (agh_[a-z0-9_]+)\(([^)]*)\)", rs)}
+    assert rs_decls == c_decls
+    assert sorted(c_decls) == header_symbols()
