@@ -116,6 +116,50 @@ def test_conv2_direct_fused_relu_pool(ag, dtype):
         assert np.array_equal(fused, orc.max_pool2(orc.relu(conv), (2, 2)))
 
 
+CONV_MFMA = [
+    # bs, ic, ih, iw, oc, filter, padding: shapes the implicit-GEMM (matrix core) convolution takes
+    (2, 64, 56, 56, 128, (3, 3), (1, 1)),    # config-3 layer, small batch
+    (3, 16, 24, 24, 64, (5, 5), (0, 0)),     # one 16-channel step per tap, partial last tile (400 positions)
+    (2, 32, 16, 16, 192, (3, 3), (1, 1)),    # two output-channel tiles, the second half empty
+    (1, 128, 8, 32, 64, (1, 1), (0, 0)),     # 1x1, staged tile exactly 64 KB
+    (2, 16, 20, 16, 64, (3, 5), (1, 2)),     # rectangular filter, unequal padding, odd step count (15)
+]
+
+
+@pytest.mark.parametrize("case", CONV_MFMA)
+def test_conv2_direct_bf16_matrix_core_path(ag, case):
+    bs, ic, ih, iw, oc, f, p = case
+    rng = np.random.default_rng(25)
+    x = orc.f32_to_bf16(rng.standard_normal((bs, ic, ih, iw)).astype(np.float32))
+    w = orc.f32_to_bf16((rng.standard_normal((oc, ic) + f) * np.sqrt(2.0 / (ic * f[0] * f[1]))).astype(np.float32))
+    b = orc.f32_to_bf16((rng.standard_normal(oc) * 0.1).astype(np.float32))
+    tx, tw, tb = ag.Tensor.from_array(x), ag.Tensor.from_array(w), ag.Tensor.from_array(b)
+    y = ag.conv2_direct_forward(tx, tw, padding=p).into_array()
+    want = orc.conv2_naive_f64(orc.bf16_to_f32(x), orc.bf16_to_f32(w), p, (1, 1), (1, 1))
+    scale = orc.conv2_naive_f64(np.abs(orc.bf16_to_f32(x)), np.abs(orc.bf16_to_f32(w)), p, (1, 1), (1, 1))
+    assert y.shape == want.shape
+    k = ic * f[0] * f[1]
+    got = orc.bf16_to_f32(y).astype(np.float64)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0**-126))) - 7)
+    assert np.all(np.abs(got - want) <= ulp + 1e-2 * np.abs(want) + 8 * np.sqrt(k) * 2.0**-24 * scale)
+    # and against the im2col + GEMM chain: same f32 sums in another order, so at most one bf16 step apart
+    chain = orc.bf16_to_f32(ag.conv2_im2col_forward(tx, tw, padding=p).into_array()).astype(np.float64)
+    assert np.all(np.abs(got - chain) <= 2 * ulp + 16 * np.sqrt(k) * 2.0**-24 * scale)
+    assert np.mean(got != chain) < 0.2
+    # bias + relu epilogue: equals the separate ops applied to this very conv result, bit for bit
+    yb = ag.conv2_direct_forward(tx, tw, padding=p, bias=tb, relu=True).into_array()
+    n, c, h, wd = y.shape
+    flat = np.ascontiguousarray(y.transpose(0, 2, 3, 1).reshape(-1, c))
+    ref = orc.relu(orc.bias_add_rows(flat, b)).reshape(n, h, wd, c).transpose(0, 3, 1, 2)
+    assert np.array_equal(yb, ref)
+    # exact-integer data: every sum is exact in f32, so the result is the single RNE rounding of it
+    xi = orc.f32_to_bf16(((np.arange(x.size) % 10) + 1).astype(np.float32).reshape(x.shape))
+    wi = orc.f32_to_bf16(((np.arange(w.size) % 7) - 3).astype(np.float32).reshape(w.shape))
+    yi = ag.conv2_direct_forward(ag.Tensor.from_array(xi), ag.Tensor.from_array(wi), padding=p).into_array()
+    exact = orc.conv2_naive_f64(orc.bf16_to_f32(xi), orc.bf16_to_f32(wi), p, (1, 1), (1, 1))
+    assert np.array_equal(yi, orc.f32_to_bf16(exact.astype(np.float32)))
+
+
 def he(rng, shape, fan_in):  # Uniform(-a, a), a = sqrt(2/fan_in): layer.rs:345-349, :463-467
     a = np.sqrt(2.0 / fan_in)
     return rng.uniform(-a, a, shape).astype(np.float32)
