@@ -72,14 +72,21 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
     const bool nan = (h & 0x7FFFu) > 0x7F80u;
     return __uint_as_float(nan ? (x | 0x00400000u) : x);  // NaN: set the quiet bit
 }
-__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-    const uint32_t x = __float_as_uint(f);
-    // round to nearest even on bit 16: adding 0x7FFF + lsb carries exactly when the discarded
-    // half is above 0x8000, or equal to it with an odd kept part
-    const uint32_t rne = (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;
-    const bool nan = (x & 0x7FFFFFFFu) > 0x7F800000u;
-    return (uint16_t)(nan ? ((x >> 16) | 0x0040u) : rne);
+// f32 -> bf16, round to nearest even, NaN -> (x >> 16) | 0x40.  gfx950 has this as an instruction
+// (v_cvt_pk_bf16_f32, which the conversion below compiles to); it agrees with the `half` crate's
+// rule on every f32 whose low half is one of 0, 1, 0x4000, 0x7FFF, 0x8000, 0x8001, 0xC000, 0xFFFF
+// for all 65536 high halves (ties, NaNs with any payload, infinities, subnormals): checked on the device.
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+// two at once: low half = a, high half = b
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float a, float b) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t in = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(in, bf16x2_t));
 }
+// widening without the NaN quieting of bf16_to_f32: for values that go straight into an addition
+// (which quiets a signalling NaN itself) or that this library has just rounded (already quiet)
+__device__ __forceinline__ float bf16_raw_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
 template <typename T> struct Elem;
 template <> struct Elem<float> {
