@@ -9,6 +9,8 @@
 // what im2col + GEMM move; bias and ReLU are applied in the epilogue in the order the separate
 // layers round.  Sums are f32 in k order (tap, channel), one rounding at the end, so results agree
 // with the im2col chain within its bf16 tolerance, not bit for bit.
+#include <type_traits>
+
 #include "agh_internal.h"
 
 using namespace agh;
@@ -29,6 +31,7 @@ struct ConvMfmaParams {
     int npos, tiles_per_img, oc_tiles;
     int lcols;     // staged columns: iw + 2*pw
     int nch_mask;  // ic/8 - 1 (16-byte chunks per pixel, a power of two)
+    int kshift;    // log2(pixels per 256 bytes): the swizzle key of pixel q is (q >> kshift) & nch_mask
     int K;         // fh*fw*ic
     FastDiv div_ow, div_tiles, div_octiles, div_vec;
 };
@@ -67,6 +70,9 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
     const int pix_bytes = p.ic * 2;
 
     // ---- stage the input rows: items = (row, channel pair, 8-column vector) ----
+    // The 16-byte channel chunks of pixel q are stored at chunk ^ key(q), key(q) = (q >> kshift) & nch_mask:
+    // the lanes of a ds_read_b128 of the k loop address 16 consecutive pixels and the same chunk, and this
+    // puts those 16 reads on 16 different 16-byte columns of the 256-byte LDS row.
     {
         const int nvec = p.iw >> 3, npair = p.ic >> 1;
         const uint32_t items = (uint32_t)lrows * npair * nvec;
@@ -74,7 +80,7 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
         constexpr int SB = 4;
         for (uint32_t it0 = tid; it0 < items; it0 += kThreads * SB) {
             uint4 r0[SB], r1[SB];
-            int base[SB], col0[SB], cpart[SB];
+            int base[SB], pix0[SB], cpart[SB];
 #pragma unroll
             for (int u = 0; u < SB; ++u) {
                 const uint32_t it = it0 + u * kThreads;
@@ -91,8 +97,8 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
                     r1[u] = *(const uint4 *)(src + (size_t)p.ih * p.iw);
                 }
                 const int c = 2 * (int)c2;
-                col0[u] = p.pw + (int)v * 8;
-                base[u] = it < items ? ((int)lr * p.lcols + col0[u]) * pix_bytes + (c & 7) * 2 : -1;
+                pix0[u] = (int)lr * p.lcols + p.pw + (int)v * 8;
+                base[u] = it < items ? pix0[u] * pix_bytes + (c & 7) * 2 : -1;
                 cpart[u] = c >> 3;
             }
 #pragma unroll
@@ -102,7 +108,7 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t a = (lo[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu, bb = (hi2[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
-                    const int addr = base[u] + j * pix_bytes + ((cpart[u] ^ ((col0[u] + j) & p.nch_mask)) << 4);
+                    const int addr = base[u] + j * pix_bytes + ((cpart[u] ^ (((pix0[u] + j) >> p.kshift) & p.nch_mask)) << 4);
                     *(uint32_t *)(lds + addr) = a | (bb << 16);
                 }
             }
@@ -148,49 +154,89 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
     // ---- k loop: taps outer, 16 channels per step, operands of step s+1 requested before the MFMAs of step s ----
     const int ncc = p.ic >> 4;
     int fi = 0, fj = 0, cc = 0;  // position of the NEXT step to load
-    int abase[4], akey[4];          // byte address of the lane's pixel for tap (0,0); swizzle key of the current fj, << 4
+    int abase[4], akey[4];          // byte address of the lane's pixel for tap (0,0); swizzle key of the current tap, << 4
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
         abase[mt] = apix[mt] * pix_bytes;
-        akey[mt] = (acol[mt] & p.nch_mask) << 4;
+        akey[mt] = ((apix[mt] >> p.kshift) & p.nch_mask) << 4;
     }
     const int kg16 = kg << 4;
-    auto load_step = [&](uint4(&a)[4], uint4(&bq)[2]) {
-        const int tapbytes = (fi * p.lcols + fj) * pix_bytes;  // scalar
-        const int chunk16 = kg16 + (cc << 5);
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) a[mt] = *(const uint4 *)(lds + abase[mt] + tapbytes + (chunk16 ^ akey[mt]));
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-            bq[nt] = *(const uint4 *)brow[nt];
-            brow[nt] += 64 * 8;
-        }
+    // A fragments: next step's LDS reads are issued before this step's MFMAs.  B fragments come from L2
+    // (several hundred cycles away), so they are requested three steps ahead into a ring of four
+    // register sets.  The main loop takes four steps per trip so every register index is static, and
+    // it contains no branch around a load: a load that would run past the last step re-reads a valid
+    // location instead (with conditional loads the compiler can no longer count outstanding loads and
+    // waits for all of them before every MFMA group, which serialises the L2 latency into each step).
+    int tapbytes_next = 0, chunk16_next = kg16;  // of the step the next load_a_part calls will fetch
+    auto prepare_a = [&](int s) {  // scalar / per-lane state for fetching step s's A fragments
+        tapbytes_next = s < nsteps ? (fi * p.lcols + fj) * pix_bytes : 0;
+        chunk16_next = kg16 + ((s < nsteps ? cc : 0) << 5);
+    };
+    auto load_a_part = [&](uint4(&a)[4], auto mtc) {
+        constexpr int mt = decltype(mtc)::value;
+        a[mt] = *(const uint4 *)(lds + abase[mt] + tapbytes_next + (chunk16_next ^ akey[mt]));
+    };
+    auto advance_a = [&]() {
         if (++cc == ncc) {
             cc = 0;
             if (++fj == p.fw) { fj = 0; ++fi; }
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt) akey[mt] = ((acol[mt] + fj) & p.nch_mask) << 4;
+            for (int mt = 0; mt < 4; ++mt) akey[mt] = (((apix[mt] + fi * p.lcols + fj) >> p.kshift) & p.nch_mask) << 4;
         }
     };
-    auto mma_step = [&](const uint4(&a)[4], const uint4(&bq)[2]) {
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
-                acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[mt]),
-                                                                      __builtin_bit_cast(bf16x8_t, bq[nt]), acc[mt][nt], 0, 0, 0);
+    auto load_b_part = [&](uint4(&bq)[2], int s, auto ntc) {
+        constexpr int nt = decltype(ntc)::value;
+        bq[nt] = *(const uint4 *)(brow[nt] + (size_t)min(s, nsteps - 1) * (64 * 8));
+    };
+    auto mma = [&](const uint4(&a)[4], const uint4(&bq)[2], auto nc) {
+        constexpr int n = decltype(nc)::value, mt = n >> 1, nt = n & 1;
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[mt]), __builtin_bit_cast(bf16x8_t, bq[nt]),
+                                                              acc[mt][nt], 0, 0, 0);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    using I4 = std::integral_constant<int, 4>;
+    using I5 = std::integral_constant<int, 5>;
+    using I6 = std::integral_constant<int, 6>;
+    using I7 = std::integral_constant<int, 7>;
+    // One step: the eight MFMAs of step s on (a, b), with the fetches of step s+1's A fragments (into an)
+    // and of step s+3's B fragments (into bn) handed out between them, one per MFMA.  sched_barrier pins
+    // the order, so the matrix pipe gets a new MFMA every 32 cycles while the other requests trickle out.
+    // No branch surrounds a load: one that would run past the last step re-reads a valid location (with
+    // conditional loads the compiler can no longer count outstanding loads and waits for all of them).
+    auto step = [&](const uint4(&a)[4], const uint4(&bq)[2], uint4(&an)[4], uint4(&bn)[2], int s) {
+        prepare_a(s + 1);
+        mma(a, bq, I0{}); load_a_part(an, I0{}); __builtin_amdgcn_sched_barrier(0);
+        mma(a, bq, I1{}); load_a_part(an, I1{}); __builtin_amdgcn_sched_barrier(0);
+        mma(a, bq, I2{}); load_a_part(an, I2{}); __builtin_amdgcn_sched_barrier(0);
+        mma(a, bq, I3{}); load_a_part(an, I3{}); __builtin_amdgcn_sched_barrier(0);
+        mma(a, bq, I4{}); load_b_part(bn, s + 3, I0{}); __builtin_amdgcn_sched_barrier(0);
+        mma(a, bq, I5{}); load_b_part(bn, s + 3, I1{}); __builtin_amdgcn_sched_barrier(0);
+        mma(a, bq, I6{}); advance_a(); __builtin_amdgcn_sched_barrier(0);
+        mma(a, bq, I7{}); __builtin_amdgcn_sched_barrier(0);
     };
     if (wave_live) {
-        uint4 a0[4], b0[2], a1[4], b1[2];
-        load_step(a0, b0);
+        uint4 a0[4], a1[4], b0[2], b1[2], b2[2], b3[2];
+        load_b_part(b0, 0, I0{}); load_b_part(b0, 0, I1{});
+        load_b_part(b1, 1, I0{}); load_b_part(b1, 1, I1{});
+        load_b_part(b2, 2, I0{}); load_b_part(b2, 2, I1{});
+        prepare_a(0);
+        load_a_part(a0, I0{}); load_a_part(a0, I1{}); load_a_part(a0, I2{}); load_a_part(a0, I3{});
+        advance_a();
         int s = 0;
-        for (; s + 2 <= nsteps; s += 2) {
-            load_step(a1, b1);
-            mma_step(a0, b0);
-            if (s + 2 < nsteps) load_step(a0, b0);
-            mma_step(a1, b1);
+        for (; s + 4 <= nsteps; s += 4) {
+            step(a0, b0, a1, b3, s);
+            step(a1, b1, a0, b0, s + 1);
+            step(a0, b2, a1, b1, s + 2);
+            step(a1, b3, a0, b2, s + 3);
         }
-        if (s < nsteps) mma_step(a0, b0);
+        // up to three steps left: their B fragments are in b0, b1, b2 and the first one's A fragments in a0
+        const int left = nsteps - s;
+        if (left >= 1) step(a0, b0, a1, b3, s);
+        if (left >= 2) step(a1, b1, a0, b3, s + 1);
+        if (left >= 3) step(a0, b2, a1, b3, s + 2);
     }
     __syncthreads();  // every wave is done with the staged image: LDS becomes the epilogue's transposition space
 
@@ -270,6 +316,7 @@ int conv2_mfma_bf16_try(const char *name, const void *x, const void *w, const vo
     p.act = act; p.has_bias = bias != nullptr;
     p.npos = npos; p.tiles_per_img = tiles; p.oc_tiles = octiles; p.lcols = lcols;
     p.nch_mask = ic / 8 - 1;
+    p.kshift = ic >= 128 ? 0 : (ic == 64 ? 1 : (ic == 32 ? 2 : 3));
     p.K = fh * fw * ic;
     p.div_ow = FastDiv((uint32_t)ow);
     p.div_tiles = FastDiv((uint32_t)tiles);
