@@ -70,9 +70,10 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
     const int pix_bytes = p.ic * 2;
 
     // ---- stage the input rows: items = (row, channel pair, 8-column vector) ----
-    // The 16-byte channel chunks of pixel q are stored at chunk ^ key(q), key(q) = (q >> kshift) & nch_mask:
-    // the lanes of a ds_read_b128 of the k loop address 16 consecutive pixels and the same chunk, and this
-    // puts those 16 reads on 16 different 16-byte columns of the 256-byte LDS row.
+    // The 16-byte channel chunks of pixel q are stored at chunk ^ key(q), key(q) = ((q >> kshift) + (q >> 4)) &
+    // nch_mask.  The lanes of a ds_read_b128 of the k loop address 16 consecutive pixels and the same chunk:
+    // the first term puts those 16 reads on 16 different 16-byte columns of the 256-byte LDS row.  The lanes
+    // of a staging write address pixels 8 apart: the second term spreads those as well.
     {
         const int nvec = p.iw >> 3, npair = p.ic >> 1;
         const uint32_t items = (uint32_t)lrows * npair * nvec;
@@ -108,7 +109,7 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t a = (lo[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu, bb = (hi2[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu;
-                    const int addr = base[u] + j * pix_bytes + ((cpart[u] ^ (((pix0[u] + j) >> p.kshift) & p.nch_mask)) << 4);
+                    const int addr = base[u] + j * pix_bytes + ((cpart[u] ^ ((((pix0[u] + j) >> p.kshift) + ((pix0[u] + j) >> 4)) & p.nch_mask)) << 4);
                     *(uint32_t *)(lds + addr) = a | (bb << 16);
                 }
             }
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
         abase[mt] = apix[mt] * pix_bytes;
-        akey[mt] = ((apix[mt] >> p.kshift) & p.nch_mask) << 4;
+        akey[mt] = (((apix[mt] >> p.kshift) + (apix[mt] >> 4)) & p.nch_mask) << 4;
     }
     const int kg16 = kg << 4;
     // A fragments: next step's LDS reads are issued before this step's MFMAs.  B fragments come from L2
@@ -181,7 +182,10 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
             cc = 0;
             if (++fj == p.fw) { fj = 0; ++fi; }
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt) akey[mt] = (((apix[mt] + fi * p.lcols + fj) >> p.kshift) & p.nch_mask) << 4;
+            for (int mt = 0; mt < 4; ++mt) {
+                const int q = apix[mt] + fi * p.lcols + fj;
+                akey[mt] = (((q >> p.kshift) + (q >> 4)) & p.nch_mask) << 4;
+            }
         }
     };
     auto load_b_part = [&](uint4(&bq)[2], int s, auto ntc) {
@@ -253,20 +257,23 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_bf16_kernel(const uint
             for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
                 for (int blk = 0; blk < 4; ++blk) {
-                    uint16_t o[4];
+                    // two packed conversions give the four rounded values as two dwords
+                    uint32_t w[2] = {f32x2_to_bf16x2(acc[mt][nt][blk * 4 + 0], acc[mt][nt][blk * 4 + 1]),
+                                     f32x2_to_bf16x2(acc[mt][nt][blk * 4 + 2], acc[mt][nt][blk * 4 + 3])};
+                    if (p.has_bias) {  // wave-uniform: bias + rounded product, rounded again
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16(acc[mt][nt][blk * 4 + e]);
-                    if (p.has_bias) {  // wave-uniform
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16(bq + bf16_to_f32(o[e]));
+                        for (int h = 0; h < 2; ++h)
+                            w[h] = f32x2_to_bf16x2(bq + __uint_as_float(w[h] << 16), bq + __uint_as_float(w[h] & 0xFFFF0000u));
                     }
                     if (relu) {  // wave-uniform; keeps x when x >= 0 (so -0 stays, NaN goes to 0)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) o[e] = bf16_to_f32(o[e]) >= 0.0f ? o[e] : (uint16_t)0;
+                        for (int h = 0; h < 2; ++h) {
+                            const bool klo = __uint_as_float(w[h] << 16) >= 0.0f, khi = __uint_as_float(w[h] & 0xFFFF0000u) >= 0.0f;
+                            w[h] = (klo ? (w[h] & 0xFFFFu) : 0u) | (khi ? (w[h] & 0xFFFF0000u) : 0u);
+                        }
                     }
                     const int pl = mt * 32 + blk * 8 + kg * 4;  // position inside the wave's 128
-                    *(uint2 *)(region + l32 * kEpitch + pl * 2) =
-                        make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
+                    *(uint2 *)(region + l32 * kEpitch + pl * 2) = make_uint2(w[0], w[1]);
                 }
             // same wave, LDS executes in order: the reads below see the writes above
 #pragma unroll
