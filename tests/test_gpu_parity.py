@@ -236,6 +236,33 @@ def test_dot_error_behaviour(ag):
     assert ag.lib.agh_max_pool2_f32(None, None, 1, 2, 2, 3, 3, 1, 1) == -1
 
 
+def test_bf16_output_rounding_matches_reference_rule(ag):
+    """The device rounds f32 sums to bf16 with its conversion instruction; the reference's rule is the
+    `half` crate's (round to nearest even, ties included).  A k = 2 product a*1 + b*1 with bf16 a, b
+    builds f32 sums whose discarded half sits on, just above and just below a tie, over every binade."""
+    rng = np.random.default_rng(26)
+    hi = (rng.integers(0x0080, 0x7F00, 8192, dtype=np.uint32) | (rng.integers(0, 2, 8192, dtype=np.uint32) << 15)).astype(np.uint16)
+    hf = orc.bf16_to_f32(hi)
+    ulp = np.float32(2.0) ** (np.floor(np.log2(np.abs(hf))).astype(np.float32) - 7)
+    rows = []
+    for frac in (0.5, -0.5, 0.25, -0.25, 0.75, -0.75, 0.5 + 1 / 64, 0.5 - 1 / 64, -0.5 - 1 / 64, 1 / 128, 0.0):
+        lo = orc.f32_to_bf16((ulp * np.float32(frac)).astype(np.float32))  # an exact power-of-two multiple: itself bf16
+        rows.append(np.stack([hi, lo], axis=1))
+    a = np.concatenate(rows)
+    want = orc.f32_to_bf16(orc.bf16_to_f32(a[:, 0]) + orc.bf16_to_f32(a[:, 1]))
+    ones = orc.f32_to_bf16(np.ones((2, 1), dtype=np.float32))
+    got = ag.Tensor.from_array(a).dot(ag.Tensor.from_array(ones)).into_array()[:, 0]
+    assert np.array_equal(got, want)
+    # the large-tile kernels share the conversion: the same sums as columns of a 256 x 64 x 256 product
+    n = 256
+    big_a = np.zeros((n, 64), dtype=np.uint16)
+    big_a[:, :2] = a[:n]
+    big_b = np.zeros((64, n), dtype=np.uint16)
+    big_b[:2, :] = ones[0, 0]
+    got2 = ag.Tensor.from_array(big_a).dot(ag.Tensor.from_array(big_b)).into_array()
+    assert np.array_equal(got2, np.repeat(want[:n, None], n, axis=1))
+
+
 @pytest.mark.parametrize("dtype,shape", [("f32", (4096, 4096, 4096)), ("bf16", (8192, 8192, 8192)),
                                          ("f32", (8192, 8192, 8192))])
 def test_gemm_full_size_sampled_entries_and_identity(ag, dtype, shape):
