@@ -22,7 +22,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_F32_TFLOPS = 157.3     # MI355X f32 matrix
 PEAK_HBM_GBS = 8000.0
-TRAFFIC_BYTES_BF16_8192 = 1.750e9  # FETCH_SIZE + WRITE_SIZE per launch, from the counter summary kept under profiles/
+TRAFFIC_BYTES_BF16_8192 = 1.747e9  # FETCH_SIZE + WRITE_SIZE per launch, from the counter summary kept under profiles/
 
 
 def log(*a):
