@@ -493,12 +493,10 @@ int conv2_direct_entry(const char *name, const void *x, const void *w, const voi
     if (bs == 0) return AGH_OK;
     if (!x || !w || !y) return fail(AGH_ENULL, "%s: null buffer", name);
 
-    // bf16 with enough channels: implicit GEMM on the matrix cores (returns 1 when the geometry is not its own)
-    if constexpr (sizeof(T) == 2) {
-        if (sh == 1 && sw == 1 && dh == 1 && dw == 1 && !pool2x2) {
-            const int rc = conv2_mfma_bf16_try(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
-            if (rc != 1) return rc;
-        }
+    // enough channels: implicit GEMM on the matrix cores (returns 1 when the geometry is not its own)
+    if (sh == 1 && sw == 1 && dh == 1 && dw == 1 && !pool2x2) {
+        const int rc = conv2_mfma_try<T>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
+        if (rc != 1) return rc;
     }
 
     // stride 1, dilation 1, filter width 3 or 5: row-tiled kernel

@@ -20,10 +20,11 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t e, const char *what);
 // Scratch owned by the library (split-K partials); grows on demand, never shrinks.
 int workspace(size_t bytes, void **ptr);
-// bf16 Conv2 forward as an implicit GEMM (agh_conv_mfma.hip); 1 = geometry not taken, else a status code
-int conv2_mfma_bf16_try(const char *name, const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic,
-                        int64_t ih, int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t oh,
-                        int64_t ow, int act);
+// Conv2 forward as an implicit GEMM (agh_conv_mfma.hip), T = uint16_t (bf16) or float; 1 = geometry not taken,
+// else a status code
+template <typename T>
+int conv2_mfma_try(const char *name, const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic, int64_t ih,
+                   int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t oh, int64_t ow, int act);
 
 #define AGH_API_ENTER()                                           \
     std::lock_guard<std::recursive_mutex> _agh_lock(agh::api_mutex()); \

@@ -123,6 +123,8 @@ CONV_MFMA = [
     (2, 32, 16, 16, 192, (3, 3), (1, 1)),    # two output-channel tiles, the second half empty
     (1, 128, 8, 32, 64, (1, 1), (0, 0)),     # 1x1, staged tile exactly 64 KB
     (2, 16, 20, 16, 64, (3, 5), (1, 2)),     # rectangular filter, unequal padding, odd step count (15)
+    (1, 128, 56, 56, 64, (3, 3), (1, 1)),    # rows of 128 channels exceed half a CU's LDS: two passes of 64 channels
+    (2, 96, 16, 24, 64, (3, 3), (1, 1)),     # channel count not a power of two: three passes of 32
 ]
 
 
@@ -158,6 +160,49 @@ def test_conv2_direct_bf16_matrix_core_path(ag, case):
     yi = ag.conv2_direct_forward(ag.Tensor.from_array(xi), ag.Tensor.from_array(wi), padding=p).into_array()
     exact = orc.conv2_naive_f64(orc.bf16_to_f32(xi), orc.bf16_to_f32(wi), p, (1, 1), (1, 1))
     assert np.array_equal(yi, orc.f32_to_bf16(exact.astype(np.float32)))
+
+
+CONV_MFMA_F32 = [
+    # the f32 variant steps 8 channels at a time
+    (2, 64, 56, 56, 128, (3, 3), (1, 1)),    # config-3 layer, small batch: two passes of 32 channels
+    (3, 8, 24, 24, 64, (5, 5), (0, 0)),      # one 8-channel step per tap, partial last tile (400 positions)
+    (2, 32, 16, 16, 192, (3, 3), (1, 1)),    # two output-channel tiles, the second half empty
+    (1, 128, 8, 32, 64, (1, 1), (0, 0)),     # 1x1
+    (2, 16, 20, 16, 64, (3, 5), (1, 2)),     # rectangular filter, unequal padding, odd step count (30 = 4*7 + 2)
+    (1, 16, 12, 28, 64, (3, 3), (0, 0)),     # width a multiple of 4 only, 260 positions (a 4-position tail tile)
+    (1, 24, 20, 20, 64, (3, 3), (1, 1)),     # three passes of 8 channels
+    (1, 256, 28, 28, 64, (3, 3), (1, 1)),    # four passes of 64 channels
+]
+
+
+@pytest.mark.parametrize("case", CONV_MFMA_F32)
+def test_conv2_direct_f32_matrix_core_path(ag, case):
+    bs, ic, ih, iw, oc, f, p = case
+    rng = np.random.default_rng(26)
+    x = rng.standard_normal((bs, ic, ih, iw)).astype(np.float32)
+    w = (rng.standard_normal((oc, ic) + f) * np.sqrt(2.0 / (ic * f[0] * f[1]))).astype(np.float32)
+    b = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    tx, tw, tb = ag.Tensor.from_array(x), ag.Tensor.from_array(w), ag.Tensor.from_array(b)
+    y = ag.conv2_direct_forward(tx, tw, padding=p).into_array()
+    want = orc.conv2_naive_f64(x, w, p, (1, 1), (1, 1))
+    scale = orc.conv2_naive_f64(np.abs(x), np.abs(w), p, (1, 1), (1, 1))
+    assert y.shape == want.shape
+    k = ic * f[0] * f[1]
+    # f32 products and sums: the GEMM bound, 1e-5 * sqrt(K) relative to the sum of magnitudes
+    assert np.all(np.abs(y.astype(np.float64) - want) <= 1e-5 * np.sqrt(k) * np.maximum(scale, 1e-30))
+    chain = ag.conv2_im2col_forward(tx, tw, padding=p).into_array()
+    assert np.all(np.abs(y.astype(np.float64) - chain) <= 2e-5 * np.sqrt(k) * np.maximum(scale, 1e-30))
+    # bias + relu epilogue: equals the separate ops applied to this very conv result, bit for bit
+    yb = ag.conv2_direct_forward(tx, tw, padding=p, bias=tb, relu=True).into_array()
+    n, c, h, wd = y.shape
+    flat = np.ascontiguousarray(y.transpose(0, 2, 3, 1).reshape(-1, c))
+    ref = orc.relu(orc.bias_add_rows(flat, b)).reshape(n, h, wd, c).transpose(0, 3, 1, 2)
+    assert np.array_equal(yb, ref)
+    # exact-integer data: every product and partial sum is an integer below 2^24, so any order gives the exact result
+    xi = ((np.arange(x.size) % 10) + 1).astype(np.float32).reshape(x.shape)
+    wi = ((np.arange(w.size) % 7) - 3).astype(np.float32).reshape(w.shape)
+    yi = ag.conv2_direct_forward(ag.Tensor.from_array(xi), ag.Tensor.from_array(wi), padding=p).into_array()
+    assert np.array_equal(yi, orc.conv2_naive_f64(xi, wi, p, (1, 1), (1, 1)).astype(np.float32))
 
 
 def he(rng, shape, fan_in):  # Uniform(-a, a), a = sqrt(2/fan_in): layer.rs:345-349, :463-467
