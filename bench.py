@@ -186,19 +186,19 @@ def main():
             run(f"conv_gemm_{dt}_802816x576x128", lambda: ag.gemm(1.0, cols, wt.t(), 0.0, y), 2.0 * bs * hw * hw * 576 * co,
                 "TFLOP/s", PEAK_F32_TFLOPS if dt == "f32" else PEAK_BF16_TFLOPS)
             del y
-            if dt == "bf16":
-                # the same Conv2 forward without the patch matrix: implicit GEMM on the matrix cores, NCHW in, NCHW out
-                w4 = wt.into_shape((co, ci, 3, 3))
-                yc = ag.Tensor.uninit((bs, co, hw, hw), dt)
-                bcv = ag.Tensor.from_array(rand_bf16(orc, rng, (co,), 0.1))
-                fn_d = ag.lib.agh_conv2_direct_bf16
-                run("conv2_forward_fused_bf16_b256_64to128_56x56", lambda: ag._ffi.check(fn_d(
-                    x._ptr(), w4._ptr(), None, yc._ptr(), bs, ci, hw, hw, co, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)),
-                    2.0 * bs * hw * hw * 576 * co, "TFLOP/s", PEAK_BF16_TFLOPS)
-                run("conv2_forward_fused_bf16_bias_relu", lambda: ag._ffi.check(fn_d(
-                    x._ptr(), w4._ptr(), bcv._ptr(), yc._ptr(), bs, ci, hw, hw, co, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0)),
-                    2.0 * bs * hw * hw * 576 * co, "TFLOP/s", PEAK_BF16_TFLOPS)
-                del yc, bcv, w4
+            # the same Conv2 forward without the patch matrix: implicit GEMM on the matrix cores, NCHW in, NCHW out
+            w4 = wt.into_shape((co, ci, 3, 3))
+            yc = ag.Tensor.uninit((bs, co, hw, hw), dt)
+            bcv = ag.Tensor.from_array(rand_bf16(orc, rng, (co,), 0.1) if dt == "bf16" else (rng.standard_normal(co) * 0.1).astype(np.float32))
+            fn_d = getattr(ag.lib, f"agh_conv2_direct_{dt}")
+            peak = PEAK_F32_TFLOPS if dt == "f32" else PEAK_BF16_TFLOPS
+            run(f"conv2_forward_fused_{dt}_b256_64to128_56x56", lambda: ag._ffi.check(fn_d(
+                x._ptr(), w4._ptr(), None, yc._ptr(), bs, ci, hw, hw, co, 3, 3, 1, 1, 1, 1, 1, 1, 0, 0)),
+                2.0 * bs * hw * hw * 576 * co, "TFLOP/s", peak)
+            run(f"conv2_forward_fused_{dt}_bias_relu", lambda: ag._ffi.check(fn_d(
+                x._ptr(), w4._ptr(), bcv._ptr(), yc._ptr(), bs, ci, hw, hw, co, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0)),
+                2.0 * bs * hw * hw * 576 * co, "TFLOP/s", peak)
+            del yc, bcv, w4
             dx = ag.Tensor.uninit((bs, ci, hw, hw), dt)
             run(f"col2im_{dt}_conv3x3_b256", lambda: ag._ffi.check(fn_c(cols._ptr(), dx._ptr(), bs, ci, hw, hw, 3, 3, 1, 1, 1, 1, 1, 1)),
                 bytes_, "GB/s", PEAK_HBM_GBS)

@@ -176,8 +176,10 @@ int agh_col2im_conv2_bf16(const void *x, void *y, int64_t bs, int64_t c, int64_t
 
 /* ---------------------------------------------------------- direct convolution ---- */
 
-/* Conv2 forward without a materialised patch matrix, for layers whose input image and filter
- * bank fit in LDS (returns AGH_ERANGE otherwise: use im2col + gemm).  Same result as the
+/* Conv2 forward without a materialised patch matrix: for layers whose input image and filter
+ * bank fit in LDS, and, on the matrix cores as an implicit GEMM, for unit stride and dilation with
+ * input channels a multiple of 16 (bf16) or 8 (f32), output channels a multiple of 64 and rows of
+ * whole 16-byte vectors (returns AGH_ERANGE otherwise: use im2col + gemm).  Same result as the
  * conv2_im2col chain (src/learn/neural_network/layer.rs:950-1005) up to f32 summation order;
  * the reference's host has the analogous conv_direct path (layer/conv_direct.rs:23-83).
  * x: [bs,ic,ih,iw], w: [oc,ic,fh,fw], bias: null or [oc] (conv2's add_assign, layer.rs:944-946),

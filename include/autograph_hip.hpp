@@ -341,8 +341,9 @@ void gemm(float alpha, const Tensor<T> &a, const Tensor<T> &b, float beta, Tenso
 }
 
 // ---- layers (src/learn/neural_network/layer.rs) ----
-// `Conv2` (layer.rs:844-1047): weight [outputs, inputs, fh, fw]; forward = `conv2_im2col`
-// (layer.rs:950-1005) with the NHWC -> NCHW copy folded into the batched GEMM.
+// `Conv2` (layer.rs:844-1047): weight [outputs, inputs, fh, fw]; forward = `conv2` (layer.rs:930-948):
+// a direct kernel when the geometry has one, else `conv2_im2col` (layer.rs:950-1005) with the
+// NHWC -> NCHW copy folded into the batched GEMM.
 template <typename T> struct Conv2 {
     Tensor<T> weight;
     std::array<int64_t, 2> padding{0, 0}, stride{1, 1}, dilation{1, 1};
@@ -355,9 +356,18 @@ template <typename T> struct Conv2 {
         Im2ColConv2Options o;
         o.filter = {fh, fw}; o.padding = padding; o.stride = stride; o.dilation = dilation;
         const auto out = o.output_shape({ih, iw});
+        Tensor<T> y = Tensor<T>::uninit({bs, oc, out[0], out[1]});
+        // like the reference's host, which takes a direct kernel when it can: the library's direct /
+        // implicit-GEMM kernels first; AGH_ERANGE says the geometry is not theirs, then im2col + GEMM
+        if (input.is_standard_layout() && weight.is_standard_layout()) {
+            const int rc = (kBf16 ? agh_conv2_direct_bf16 : agh_conv2_direct_f32)(
+                input.data_ptr(), weight.data_ptr(), nullptr, y.buffer_ptr(), bs, ic, ih, iw, oc, fh, fw, padding[0], padding[1], stride[0],
+                stride[1], dilation[0], dilation[1], AGH_ACT_NONE, 0);
+            if (rc == AGH_OK) return y;
+            if (rc != AGH_ERANGE) check(rc);
+        }
         const Tensor<T> cols = input.im2col_conv2(o);
         const Tensor<T> wm = weight.into_shape({oc, ic * fh * fw});
-        Tensor<T> y = Tensor<T>::uninit({bs, oc, out[0], out[1]});
         const int64_t L = out[0] * out[1], K = ic * fh * fw;
         check((kBf16 ? agh_gemm_bf16_batched : agh_gemm_f32_batched)(bs, L, K, oc, 1.0f, cols.buffer_ptr(), cols.offset(), K, 1, L * K,
                                                                      wm.buffer_ptr(), wm.offset(), 1, K, 0, 0.0f, y.buffer_ptr(), 0, 1, L,
