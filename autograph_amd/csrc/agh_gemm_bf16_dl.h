@@ -30,6 +30,7 @@ namespace agh {
 namespace gemm {
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint32_t rslot(uint32_t m, uint32_t kr) { return m ^ (kr & 3u) ^ ((m & 1u) << 2); }
 // inverse of rslot in m for a given kr
@@ -362,7 +363,10 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
                         v = make_uint4(w[0], w[1], w[2], w[3]);
                     }
                     const int qq = qwb + j * 32 + row, pp = pwb + chunk * 8;
-                    if (qq < g.NQ && pp < g.NP) *(uint4 *)(D + (int64_t)qq * g.dq + pp) = v;
+                    // streaming store: C is not read again by this launch, and keeping it out of the last-level
+                    // cache leaves that cache to the operand panels, which every tile row / column re-reads
+                    if (qq < g.NQ && pp < g.NP)
+                        __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, (u32x4_t *)(D + (int64_t)qq * g.dq + pp));
                 });
             });
         };

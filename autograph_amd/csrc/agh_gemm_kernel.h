@@ -226,19 +226,30 @@ struct Loader {
     }
 };
 
+// One MFMA group = all the MFMAs that consume one 16-byte fragment pair: a single 32x32x16 for bf16, four
+// 32x32x2 for f32 (PARTS).  `part` lets a caller walk the parts of many accumulators in turn, so that
+// consecutive MFMAs never accumulate into the same registers (a dependent MFMA waits for its predecessor).
 template <typename T> struct Mma;
 template <> struct Mma<uint16_t> {
+    static constexpr int PARTS = 1;
     static __device__ __forceinline__ void run(f32x16 &acc, const uint4 &a, const uint4 &b) {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
                                                       acc, 0, 0, 0);
     }
+    template <int E> static __device__ __forceinline__ void part(f32x16 &acc, const uint4 &a, const uint4 &b) { run(acc, a, b); }
 };
 template <> struct Mma<float> {
+    static constexpr int PARTS = 4;
+    template <int E> static __device__ __forceinline__ void part(f32x16 &acc, const uint4 &a, const uint4 &b) {
+        const uint32_t ae = E == 0 ? a.x : E == 1 ? a.y : E == 2 ? a.z : a.w;
+        const uint32_t be = E == 0 ? b.x : E == 1 ? b.y : E == 2 ? b.z : b.w;
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(ae), __uint_as_float(be), acc, 0, 0, 0);
+    }
     static __device__ __forceinline__ void run(f32x16 &acc, const uint4 &a, const uint4 &b) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), acc, 0, 0, 0);
+        part<0>(acc, a, b);
+        part<1>(acc, a, b);
+        part<2>(acc, a, b);
+        part<3>(acc, a, b);
     }
 };
 
@@ -309,6 +320,39 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     const uint32_t lrow = lane & 31, lg = lane >> 5;
     const uint32_t lane_off = lrow * 128u + ((lg ^ swz(lrow)) << 4);  // tile row bases are multiples of 32
 
+    // Fragment sets A and B alternate between substeps: while the MFMAs of substep s run out of one set,
+    // the LDS reads of substep s+1 fill the other, one read after each of the first TP+TQ MFMA groups.
+    // sched_barrier(0) pins that interleaving (left alone, the scheduler puts every read directly in
+    // front of its first use and the matrix pipe waits out the LDS latency sixteen times per k-tile).
+    constexpr int NU = TP + TQ, NM = TP * TQ;
+    uint4 pfa[TP], qfa[TQ], pfb[TP], qfb[TQ];
+    auto read_unit = [&](uint4(&pf)[TP], uint4(&qf)[TQ], const unsigned char *sp, const unsigned char *sq, int s, auto uc) {
+        constexpr int u = decltype(uc)::value;
+        const uint32_t off = lane_off ^ (uint32_t)(s << 5);
+        // order of first use by the MFMA groups: P0, Q0 .. Q(TQ-1), P1 .. P(TP-1)
+        if constexpr (u == 0) pf[0] = *(const uint4 *)(sp + off);
+        else if constexpr (u <= TQ) qf[u - 1] = *(const uint4 *)(sq + (u - 1) * 32 * 128 + off);
+        else pf[u - TQ] = *(const uint4 *)(sp + (u - TQ) * 32 * 128 + off);
+    };
+    auto phase = [&](const uint4(&xp)[TP], const uint4(&xq)[TQ], uint4(&yp)[TP], uint4(&yq)[TQ], const unsigned char *sp,
+                     const unsigned char *sq, int s) {
+        constexpr int PARTS = Mma<T>::PARTS;
+        static_for<NM * PARTS>([&](auto mc) {  // part-major: consecutive MFMAs write different accumulators
+            constexpr int m = decltype(mc)::value, e = m / NM, n = m % NM, i = n / TQ, j = n % TQ;
+            Mma<T>::template part<e>(acc[i][j], xp[i], xq[j]);
+            if constexpr (m < NU) read_unit(yp, yq, sp, sq, s, mc);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        static_for<(NU > NM * PARTS ? NU - NM * PARTS : 0)>([&](auto rc) {
+            read_unit(yp, yq, sp, sq, s, std::integral_constant<int, NM * PARTS + decltype(rc)::value>{});
+        });
+    };
+    const int wave_p = (wp * TP * 32) * 128, wave_q = BP * 128 + (wq * TQ * 32) * 128;
+    if (KT > 0) static_for<NU>([&](auto uc) { read_unit(pfa, qfa, smem + wave_p, smem + wave_q, 0, uc); });
+
+    // One k-tile: global loads of the next tile go out first; substeps 0-2 multiply while prefetching
+    // fragments; then the next tile is written to the other stage and the barrier publishes it, and the
+    // last substep multiplies out of registers while the first fragments of the next tile are read.
     for (int kt = 0; kt < KT; ++kt) {
         const bool more = kt + 1 < KT;
         if (more) {
@@ -316,27 +360,18 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
             LdP::load(rp, P, g.ps, g.pk, p0, g.NP, k0, kend, tid);
             LdQ::load(rq, Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
         }
-        const unsigned char *sp = smem + (kt & 1) * STAGE_BYTES + (wp * TP * 32) * 128;
-        const unsigned char *sq = smem + (kt & 1) * STAGE_BYTES + BP * 128 + (wq * TQ * 32) * 128;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            uint4 pf[TP], qf[TQ];
-            const uint32_t off = lane_off ^ (uint32_t)(s << 5);
-#pragma unroll
-            for (int i = 0; i < TP; ++i) pf[i] = *(const uint4 *)(sp + i * 32 * 128 + off);
-#pragma unroll
-            for (int j = 0; j < TQ; ++j) qf[j] = *(const uint4 *)(sq + j * 32 * 128 + off);
-#pragma unroll
-            for (int i = 0; i < TP; ++i)
-#pragma unroll
-                for (int j = 0; j < TQ; ++j) Mma<T>::run(acc[i][j], pf[i], qf[j]);
-        }
+        const unsigned char *cur = smem + (kt & 1) * STAGE_BYTES;
+        unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
+        phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 1);
+        phase(pfb, qfb, pfa, qfa, cur + wave_p, cur + wave_q, 2);
+        phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 3);
         if (more) {
-            unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
             LdP::store(rp, nxt, tid);
             LdQ::store(rq, nxt + BP * 128, tid);
         }
         __syncthreads();
+        // after the last tile `nxt` holds stale data: the fragments read from it are never used
+        phase(pfb, qfb, pfa, qfa, nxt + wave_p, nxt + wave_q, 0);
     }
 
     // ------------------------------------------------------------ epilogue ----
