@@ -103,125 +103,124 @@ struct Loader {
     static constexpr int NBLK_TOTAL = 8 * (BR / EPC);      // LD_R: EPC x EPC blocks in the tile
     static constexpr int NBLK = (NBLK_TOTAL + NT - 1) / NT;
 
+    // A tile is moved in NPIECE independent pieces (one 16-byte register, or one EPC x EPC block for LD_R), so
+    // that the kernel can hand them out between MFMAs instead of issuing a burst.
+    static constexpr int NPIECE = MODE == LD_R ? NBLK : NREG;
+    typedef uint4 Regs[NREG > NBLK * EPC ? NREG : NBLK * EPC];
+
     // base: element pointer of the operand; r0: first tile row; NR: rows in the operand;
     // k0: first k of the tile; kend: one past the last valid k.
-    static __device__ __forceinline__ void load(uint4 (&reg)[NREG > NBLK * EPC ? NREG : NBLK * EPC], const T *base,
-                                                int64_t rs, int64_t ks, int r0, int NR, int k0, int kend, int tid) {
+    // LD_K and LD_R pieces are loaded UNCONDITIONALLY from clamped addresses and the k tail is zeroed when the
+    // piece is stored: no branch surrounds a load (behind a branch the compiler can no longer count the loads
+    // in flight and waits for all of them), and nothing touches the loaded value before it is needed.
+    static __device__ __forceinline__ void load(Regs &reg, const T *base, int64_t rs, int64_t ks, int r0, int NR, int k0,
+                                                int kend, int tid) {
+        static_for<NPIECE>([&](auto ic) { load_piece<decltype(ic)::value>(reg, base, rs, ks, r0, NR, k0, kend, tid); });
+    }
+    template <int i>
+    static __device__ __forceinline__ void load_piece(Regs &reg, const T *base, int64_t rs, int64_t ks, int r0, int NR,
+                                                      int k0, int kend, int tid) {
         if constexpr (MODE == LD_K) {
-#pragma unroll
-            for (int i = 0; i < NREG; ++i) {
-                int id = tid + i * NT;
-                int r = id >> 3, c = id & 7;
-                int row = min(r0 + r, NR - 1);
-                int kk = k0 + c * EPC;
-                // branch-free k tail: load a valid chunk, then zero it (K is a multiple of EPC here)
-                const bool ok = kk < kend;
-                if (!ok) kk = kend - EPC;
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (TOTAL % NT == 0 || id < TOTAL) v = *(const uint4 *)(base + (int64_t)row * rs + kk);
-                reg[i] = ok ? v : make_uint4(0, 0, 0, 0);
-            }
+            const int id = min(tid + i * NT, TOTAL - 1);
+            const int r = id >> 3, c = id & 7;
+            const int row = min(r0 + r, NR - 1);
+            const int kk = min(k0 + c * EPC, kend - EPC);  // K is a multiple of EPC here
+            reg[i] = *(const uint4 *)(base + (int64_t)row * rs + kk);
         } else if constexpr (MODE == LD_R) {
+            const int id = min(tid + i * NT, NBLK_TOTAL - 1);
+            const int kb = id & 7, rb = id >> 3;
+            int row = r0 + rb * EPC;
+            if (row >= NR) row = NR - EPC;  // NR is a multiple of EPC on this path
 #pragma unroll
-            for (int i = 0; i < NBLK; ++i) {
-                int id = tid + i * NT;
-                int kb = id & 7, rb = id >> 3;
-                int row = r0 + rb * EPC;
-                if (row >= NR) row = NR - EPC;  // NR is a multiple of EPC on this path
-                bool live = (NBLK_TOTAL % NT == 0 || id < NBLK_TOTAL);
-#pragma unroll
-                for (int e = 0; e < EPC; ++e) {
-                    int kk = k0 + kb * EPC + e;
-                    const bool ok = kk < kend;
-                    if (!ok) kk = kend - 1;
-                    uint4 v = make_uint4(0, 0, 0, 0);
-                    if (live) v = *(const uint4 *)(base + (int64_t)kk * ks + row);
-                    reg[i * EPC + e] = ok ? v : make_uint4(0, 0, 0, 0);
-                }
+            for (int e = 0; e < EPC; ++e) {
+                const int kk = min(k0 + kb * EPC + e, kend - 1);
+                reg[i * EPC + e] = *(const uint4 *)(base + (int64_t)kk * ks + row);
             }
         } else {
+            int id = tid + i * NT;
+            int r = id >> 3, c = id & 7;
+            int row = r0 + r;
+            bool rok = (TOTAL % NT == 0 || id < TOTAL) && row < NR;
+            const T *src = base + (int64_t)row * rs;
+            T tmp[EPC];
 #pragma unroll
-            for (int i = 0; i < NREG; ++i) {
-                int id = tid + i * NT;
-                int r = id >> 3, c = id & 7;
-                int row = r0 + r;
-                bool rok = (TOTAL % NT == 0 || id < TOTAL) && row < NR;
-                const T *src = base + (int64_t)row * rs;
-                T tmp[EPC];
-#pragma unroll
-                for (int e = 0; e < EPC; ++e) {
-                    int kk = k0 + c * EPC + e;
-                    T v = 0;
-                    if (rok && kk < kend) v = src[(int64_t)kk * ks];
-                    tmp[e] = v;
-                }
-                uint4 v;
-                if constexpr (sizeof(T) == 2) {
-                    v.x = (uint32_t)tmp[0] | ((uint32_t)tmp[1] << 16);
-                    v.y = (uint32_t)tmp[2] | ((uint32_t)tmp[3] << 16);
-                    v.z = (uint32_t)tmp[4] | ((uint32_t)tmp[5] << 16);
-                    v.w = (uint32_t)tmp[6] | ((uint32_t)tmp[7] << 16);
-                } else {
-                    v.x = __float_as_uint(tmp[0]);
-                    v.y = __float_as_uint(tmp[1]);
-                    v.z = __float_as_uint(tmp[2]);
-                    v.w = __float_as_uint(tmp[3]);
-                }
-                reg[i] = v;
+            for (int e = 0; e < EPC; ++e) {
+                int kk = k0 + c * EPC + e;
+                T v = 0;
+                if (rok && kk < kend) v = src[(int64_t)kk * ks];
+                tmp[e] = v;
             }
+            uint4 v;
+            if constexpr (sizeof(T) == 2) {
+                v.x = (uint32_t)tmp[0] | ((uint32_t)tmp[1] << 16);
+                v.y = (uint32_t)tmp[2] | ((uint32_t)tmp[3] << 16);
+                v.z = (uint32_t)tmp[4] | ((uint32_t)tmp[5] << 16);
+                v.w = (uint32_t)tmp[6] | ((uint32_t)tmp[7] << 16);
+            } else {
+                v.x = __float_as_uint(tmp[0]);
+                v.y = __float_as_uint(tmp[1]);
+                v.z = __float_as_uint(tmp[2]);
+                v.w = __float_as_uint(tmp[3]);
+            }
+            reg[i] = v;
         }
     }
 
-    // registers -> LDS stage (tile base address `lds`, bytes)
-    static __device__ __forceinline__ void store(const uint4 (&reg)[NREG > NBLK * EPC ? NREG : NBLK * EPC],
-                                                 unsigned char *lds, int tid) {
+    // registers -> LDS stage (tile base address `lds`, bytes); k0 / kend as given to load
+    static __device__ __forceinline__ void store(const Regs &reg, unsigned char *lds, int k0, int kend, int tid) {
+        static_for<NPIECE>([&](auto ic) { store_piece<decltype(ic)::value>(reg, lds, k0, kend, tid); });
+    }
+    template <int i>
+    static __device__ __forceinline__ void store_piece(const Regs &reg, unsigned char *lds, int k0, int kend, int tid) {
         if constexpr (MODE == LD_R) {
+            int id = tid + i * NT;
+            int kb = id & 7, rb = id >> 3;
+            if (!(NBLK_TOTAL % NT == 0 || id < NBLK_TOTAL)) return;
+            uint4 in[EPC];  // in[e] = EPC rows at k = kb*EPC + e
 #pragma unroll
-            for (int i = 0; i < NBLK; ++i) {
-                int id = tid + i * NT;
-                int kb = id & 7, rb = id >> 3;
-                if (!(NBLK_TOTAL % NT == 0 || id < NBLK_TOTAL)) continue;
-                const uint4 *in = &reg[i * EPC];  // in[e] = EPC rows at k = kb*EPC + e
-                if constexpr (sizeof(T) == 4) {
-                    // 4x4 transpose of 32-bit values: pure register renaming
-                    uint4 o0 = make_uint4(in[0].x, in[1].x, in[2].x, in[3].x);
-                    uint4 o1 = make_uint4(in[0].y, in[1].y, in[2].y, in[3].y);
-                    uint4 o2 = make_uint4(in[0].z, in[1].z, in[2].z, in[3].z);
-                    uint4 o3 = make_uint4(in[0].w, in[1].w, in[2].w, in[3].w);
-                    uint32_t r = rb * 4;
-                    *(uint4 *)(lds + lds_off(r + 0, kb)) = o0;
-                    *(uint4 *)(lds + lds_off(r + 1, kb)) = o1;
-                    *(uint4 *)(lds + lds_off(r + 2, kb)) = o2;
-                    *(uint4 *)(lds + lds_off(r + 3, kb)) = o3;
-                } else {
-                    // 8x8 transpose of 16-bit values: one half-word interleave per output word,
-                    // the 32- and 64-bit levels are register renaming
-                    uint32_t w[8][4];
+            for (int e = 0; e < EPC; ++e) {
+                const bool ok = k0 + kb * EPC + e < kend;
+                const uint4 &src = reg[i * EPC + e];
+                in[e] = make_uint4(ok ? src.x : 0u, ok ? src.y : 0u, ok ? src.z : 0u, ok ? src.w : 0u);
+            }
+            if constexpr (sizeof(T) == 4) {
+                // 4x4 transpose of 32-bit values: pure register renaming
+                uint4 o0 = make_uint4(in[0].x, in[1].x, in[2].x, in[3].x);
+                uint4 o1 = make_uint4(in[0].y, in[1].y, in[2].y, in[3].y);
+                uint4 o2 = make_uint4(in[0].z, in[1].z, in[2].z, in[3].z);
+                uint4 o3 = make_uint4(in[0].w, in[1].w, in[2].w, in[3].w);
+                uint32_t r = rb * 4;
+                *(uint4 *)(lds + lds_off(r + 0, kb)) = o0;
+                *(uint4 *)(lds + lds_off(r + 1, kb)) = o1;
+                *(uint4 *)(lds + lds_off(r + 2, kb)) = o2;
+                *(uint4 *)(lds + lds_off(r + 3, kb)) = o3;
+            } else {
+                // 8x8 transpose of 16-bit values: one half-word interleave per output word,
+                // the 32- and 64-bit levels are register renaming
+                uint32_t w[8][4];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const uint4 &s = in[e];
-                        w[e][0] = s.x; w[e][1] = s.y; w[e][2] = s.z; w[e][3] = s.w;
+                for (int e = 0; e < 8; ++e) {
+                    const uint4 &s = in[e];
+                    w[e][0] = s.x; w[e][1] = s.y; w[e][2] = s.z; w[e][3] = s.w;
+                }
+                uint32_t r = rb * 8;
+#pragma unroll
+                for (int rr = 0; rr < 8; ++rr) {
+                    uint32_t o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        uint32_t lo = w[2 * q][rr >> 1], hi = w[2 * q + 1][rr >> 1];
+                        o[q] = (rr & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
                     }
-                    uint32_t r = rb * 8;
-#pragma unroll
-                    for (int rr = 0; rr < 8; ++rr) {
-                        uint32_t o[4];
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            uint32_t lo = w[2 * q][rr >> 1], hi = w[2 * q + 1][rr >> 1];
-                            o[q] = (rr & 1) ? ((lo >> 16) | (hi & 0xFFFF0000u)) : ((lo & 0xFFFFu) | (hi << 16));
-                        }
-                        *(uint4 *)(lds + lds_off(r + rr, kb)) = make_uint4(o[0], o[1], o[2], o[3]);
-                    }
+                    *(uint4 *)(lds + lds_off(r + rr, kb)) = make_uint4(o[0], o[1], o[2], o[3]);
                 }
             }
         } else {
-#pragma unroll
-            for (int i = 0; i < NREG; ++i) {
-                int id = tid + i * NT;
-                int r = id >> 3, c = id & 7;
-                if (TOTAL % NT == 0 || id < TOTAL) *(uint4 *)(lds + lds_off(r, c)) = reg[i];
-            }
+            int id = tid + i * NT;
+            int r = id >> 3, c = id & 7;
+            const bool ok = MODE != LD_K || k0 + c * EPC < kend;
+            const uint4 v = make_uint4(ok ? reg[i].x : 0u, ok ? reg[i].y : 0u, ok ? reg[i].z : 0u, ok ? reg[i].w : 0u);
+            if (TOTAL % NT == 0 || id < TOTAL) *(uint4 *)(lds + lds_off(r, c)) = v;
         }
     }
 };
@@ -311,8 +310,8 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     if (KT > 0) {
         LdP::load(rp, P, g.ps, g.pk, p0, g.NP, kbeg, kend, tid);
         LdQ::load(rq, Q, g.qs, g.qk, q0, g.NQ, kbeg, kend, tid);
-        LdP::store(rp, smem, tid);
-        LdQ::store(rq, smem + BP * 128, tid);
+        LdP::store(rp, smem, kbeg, kend, tid);
+        LdQ::store(rq, smem + BP * 128, kbeg, kend, tid);
     }
     __syncthreads();
 
@@ -334,13 +333,14 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
         else if constexpr (u <= TQ) qf[u - 1] = *(const uint4 *)(sq + (u - 1) * 32 * 128 + off);
         else pf[u - TQ] = *(const uint4 *)(sp + (u - TQ) * 32 * 128 + off);
     };
+    constexpr int PARTS = Mma<T>::PARTS, SLOTS = NM * PARTS;
     auto phase = [&](const uint4(&xp)[TP], const uint4(&xq)[TQ], uint4(&yp)[TP], uint4(&yq)[TQ], const unsigned char *sp,
-                     const unsigned char *sq, int s) {
-        constexpr int PARTS = Mma<T>::PARTS;
-        static_for<NM * PARTS>([&](auto mc) {  // part-major: consecutive MFMAs write different accumulators
+                     const unsigned char *sq, int s, auto &&after) {
+        static_for<SLOTS>([&](auto mc) {  // part-major: consecutive MFMAs write different accumulators
             constexpr int m = decltype(mc)::value, e = m / NM, n = m % NM, i = n / TQ, j = n % TQ;
             Mma<T>::template part<e>(acc[i][j], xp[i], xq[j]);
             if constexpr (m < NU) read_unit(yp, yq, sp, sq, s, mc);
+            after(mc);
             __builtin_amdgcn_sched_barrier(0);
         });
         static_for<(NU > NM * PARTS ? NU - NM * PARTS : 0)>([&](auto rc) {
@@ -350,28 +350,55 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     const int wave_p = (wp * TP * 32) * 128, wave_q = BP * 128 + (wq * TQ * 32) * 128;
     if (KT > 0) static_for<NU>([&](auto uc) { read_unit(pfa, qfa, smem + wave_p, smem + wave_q, 0, uc); });
 
-    // One k-tile: global loads of the next tile go out first; substeps 0-2 multiply while prefetching
-    // fragments; then the next tile is written to the other stage and the barrier publishes it, and the
-    // last substep multiplies out of registers while the first fragments of the next tile are read.
+    // One k-tile.  With vector loaders the pieces of the next tile are requested from global memory one at a
+    // time between the MFMAs of substep 0 and written to the other LDS stage between the MFMAs of substep 2
+    // (a burst of loads fills the memory pipeline's queues, and a wave that cannot issue its load cannot issue
+    // its next MFMA either); past the last tile the same tile is fetched again and never used.  The element
+    // loader keeps its guarded loads together in front of the MFMAs.  Then the barrier publishes that
+    // stage, and the last substep multiplies out of registers while the first fragments of the next tile are read.
+    constexpr bool SPREAD = LP != LD_S && LQ != LD_S;
+    constexpr int NPP = LdP::NPIECE, NPT = LdP::NPIECE + LdQ::NPIECE;
     for (int kt = 0; kt < KT; ++kt) {
         const bool more = kt + 1 < KT;
-        if (more) {
-            const int k0 = kbeg + (kt + 1) * BK;
-            LdP::load(rp, P, g.ps, g.pk, p0, g.NP, k0, kend, tid);
-            LdQ::load(rq, Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
-        }
+        const int k0 = kbeg + (more ? kt + 1 : kt) * BK;
         const unsigned char *cur = smem + (kt & 1) * STAGE_BYTES;
         unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
-        phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 1);
-        phase(pfb, qfb, pfa, qfa, cur + wave_p, cur + wave_q, 2);
-        phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 3);
-        if (more) {
-            LdP::store(rp, nxt, tid);
-            LdQ::store(rq, nxt + BP * 128, tid);
+        if constexpr (!SPREAD) {
+            if (more) {
+                LdP::load(rp, P, g.ps, g.pk, p0, g.NP, k0, kend, tid);
+                LdQ::load(rq, Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
+            }
+        }
+        phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 1, [&](auto mc) {
+            if constexpr (SPREAD) {
+                constexpr int m = decltype(mc)::value, LA = m * NPT / SLOTS, LB = (m + 1) * NPT / SLOTS;
+                static_for<LB - LA>([&](auto tc) {
+                    constexpr int l = LA + decltype(tc)::value;
+                    if constexpr (l < NPP) LdP::template load_piece<l>(rp, P, g.ps, g.pk, p0, g.NP, k0, kend, tid);
+                    else LdQ::template load_piece<l - NPP>(rq, Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
+                });
+            }
+        });
+        phase(pfb, qfb, pfa, qfa, cur + wave_p, cur + wave_q, 2, [](auto) {});
+        phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 3, [&](auto mc) {
+            if constexpr (SPREAD) {
+                constexpr int m = decltype(mc)::value, LA = m * NPT / SLOTS, LB = (m + 1) * NPT / SLOTS;
+                static_for<LB - LA>([&](auto tc) {
+                    constexpr int l = LA + decltype(tc)::value;
+                    if constexpr (l < NPP) LdP::template store_piece<l>(rp, nxt, k0, kend, tid);
+                    else LdQ::template store_piece<l - NPP>(rq, nxt + BP * 128, k0, kend, tid);
+                });
+            }
+        });
+        if constexpr (!SPREAD) {
+            if (more) {
+                LdP::store(rp, nxt, k0, kend, tid);
+                LdQ::store(rq, nxt + BP * 128, k0, kend, tid);
+            }
         }
         __syncthreads();
         // after the last tile `nxt` holds stale data: the fragments read from it are never used
-        phase(pfb, qfb, pfa, qfa, nxt + wave_p, nxt + wave_q, 0);
+        phase(pfb, qfb, pfa, qfa, nxt + wave_p, nxt + wave_q, 0, [](auto) {});
     }
 
     // ------------------------------------------------------------ epilogue ----
