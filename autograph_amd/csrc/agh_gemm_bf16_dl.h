@@ -234,12 +234,17 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     using L_T = std::integral_constant<int, NLT>;
 
     // One k-tile.  On entry: tile kt is visible in `cur`, its substep-0 fragments are in set A,
-    // and the loads of tile kt+1 into `nxt` are in flight (issued during the previous tile's
-    // last phase).  The barrier sits between phase 2 and phase 3: by then every wave has issued
-    // (and waited for) its last reads of `cur`, so `cur` can be refilled with tile kt+2 while
-    // phase 3 multiplies out of registers.  `adv` says whether a tile kt+3 exists.
-    auto step = [&](unsigned char *cur, unsigned char *nxt, bool adv) {
-        phase(pfa, qfa, pfb, qfb, Yes{}, cur, S1{}, 0u, L_0{}, L_0{}, 0, 0);
+    // and the P share of the loads of tile kt+1 into `nxt` is in flight (issued during the previous
+    // tile's last phase); the Q share goes out during phase 0.  Splitting the requests of a tile over
+    // two phases keeps the memory pipeline's queues from filling up: a wave that cannot issue its
+    // load cannot issue its next MFMA either.  The barrier sits between phase 2 and phase 3: by then
+    // every wave has issued (and waited for) its last reads of `cur`, so `cur` can be refilled with
+    // tile kt+2 while phase 3 multiplies out of registers.  `adv0` / `adv` say whether a tile kt+2 /
+    // kt+3 exists.
+    using L_P = std::integral_constant<int, NLP>;
+    auto step = [&](unsigned char *cur, unsigned char *nxt, bool adv0, bool adv) {
+        const uint32_t nxt_addr = __builtin_amdgcn_readfirstlane(lds_address(nxt));
+        phase(pfa, qfa, pfb, qfb, Yes{}, cur, S1{}, nxt_addr, L_P{}, L_T{}, 0, adv0 ? stepQ : 0);
         phase(pfb, qfb, pfa, qfa, Yes{}, cur, S2{}, 0u, L_0{}, L_0{}, 0, 0);
         phase(pfa, qfa, pfb, qfb, Yes{}, cur, S3{}, 0u, L_0{}, L_0{}, 0, 0);
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -247,25 +252,25 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
         asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         const uint32_t cur_addr = __builtin_amdgcn_readfirstlane(lds_address(cur));
-        phase(pfb, qfb, pfa, qfa, Yes{}, nxt, S0{}, cur_addr, L_0{}, L_T{}, adv ? stepP : 0, adv ? stepQ : 0);
+        phase(pfb, qfb, pfa, qfa, Yes{}, nxt, S0{}, cur_addr, L_0{}, L_P{}, adv ? stepP : 0, 0);
     };
 
     if (KT > 0) {
         const uint32_t a0 = __builtin_amdgcn_readfirstlane(lds_address(stage0));
         const uint32_t a1 = __builtin_amdgcn_readfirstlane(lds_address(stage1));
-        // tile 0 -> stage0, tile min(1, KT-1) -> stage1
+        // tile 0 -> stage0, P share of tile min(1, KT-1) -> stage1
         static_for<NLT>([&](auto lc) { issue_load(a0, lc, KT > 1 ? stepP : 0, KT > 1 ? stepQ : 0); });
-        static_for<NLT>([&](auto lc) { issue_load(a1, lc, KT > 2 ? stepP : 0, KT > 2 ? stepQ : 0); });
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLT) : "memory");  // tile 0 has landed
+        static_for<NLP>([&](auto lc) { issue_load(a1, lc, KT > 2 ? stepP : 0, 0); });
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLP) : "memory");  // tile 0 has landed
         __syncthreads();
         static_for<NU>([&](auto uc) { read_unit(pfa, qfa, stage0, S0{}, uc); });
     }
     int kt = 0;
     for (; kt + 2 <= KT; kt += 2) {
-        step(stage0, stage1, kt + 3 < KT);
-        step(stage1, stage0, kt + 4 < KT);
+        step(stage0, stage1, kt + 2 < KT, kt + 3 < KT);
+        step(stage1, stage0, kt + 3 < KT, kt + 4 < KT);
     }
-    if (kt < KT) step(stage0, stage1, false);
+    if (kt < KT) step(stage0, stage1, false, false);
     // the last phase may have re-issued loads into a free stage: let every wave's land before
     // the epilogue reuses LDS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
