@@ -44,6 +44,7 @@ struct ConvMfmaParams {
     int nch_mask;  // 16-byte chunks per staged pixel - 1 (a power of two)
     int kshift;    // log2(pixels per 256 bytes): see the swizzle key below
     int K;         // fh*fw*ic
+    int per_xcd;   // workgroups per XCD when the grid divides by 8, else 0
     FastDiv div_ow, div_tiles, div_octiles, div_vec;
 };
 
@@ -76,7 +77,10 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_kernel(const T *__rest
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & 1, wn = wave >> 1;
     uint32_t t0, oct, b, tile;
-    p.div_octiles.divmod(blockIdx.x, t0, oct);
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a run of consecutive
+    // tiles, so that the input rows two neighbouring position tiles share are fetched from HBM once
+    const uint32_t bid = p.per_xcd ? (blockIdx.x & 7u) * (uint32_t)p.per_xcd + (blockIdx.x >> 3) : blockIdx.x;
+    p.div_octiles.divmod(bid, t0, oct);
     p.div_tiles.divmod(t0, b, tile);
     const int p0 = tile * kTilePos;
     const int plast = min(p0 + kTilePos, p.npos) - 1;
@@ -379,6 +383,7 @@ int conv2_mfma_try(const char *name, const void *x, const void *w, const void *b
     const int64_t pix_bytes = icc * ES;  // pixels per 256 bytes = 256 / pix_bytes (at least 1)
     p.kshift = pix_bytes >= 256 ? 0 : (pix_bytes == 128 ? 1 : (pix_bytes == 64 ? 2 : 3));
     p.K = fh * fw * ic;
+    p.per_xcd = blocks % 8 == 0 ? (int)(blocks / 8) : 0;
     p.div_ow = FastDiv((uint32_t)ow);
     p.div_tiles = FastDiv((uint32_t)tiles);
     p.div_octiles = FastDiv((uint32_t)octiles);

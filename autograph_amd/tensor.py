@@ -136,6 +136,25 @@ class Tensor:
         check(lib.agh_sync())  # `a` may be a temporary
         return t
 
+    # -- serde (src/tensor.rs:1199-1249): the reference's data model, as serde_json writes it --
+    def to_json(self):
+        """Blocking: copies the data to the host (standard layout) and encodes them; see autograph_amd/serde.py."""
+        from . import serde
+        return serde.to_json(self.into_array(), bf16=self.dtype == "bf16")
+
+    @classmethod
+    def from_json(cls, text, dtype=None):
+        """Decodes a tensor the reference (or `to_json`) wrote and uploads it.  `dtype` ("f32" / "bf16"), when
+        given, must match what the text holds, as the typed `Tensor<T, D>` deserialiser's conversion would."""
+        from . import serde
+        array, is_bf16 = serde.from_json(text)
+        if not is_bf16 and array.dtype != np.float32:
+            raise AghError(-1, f"serde: scalar type {serde.scalar_name(array)} has no device tensor here (f32 and bf16 only)")
+        got = "bf16" if is_bf16 else "f32"
+        if dtype is not None and dtype != got:
+            raise AghError(-1, f"Expected {dtype} found {got}")
+        return cls.from_array(array)
+
     def into_array(self):
         """`into_array()`: blocking copy of the whole buffer, then the same strided view."""
         raw = np.empty(self.buffer.nbytes // _ITEMSIZE[self.dtype], dtype=_NPTYPE[self.dtype])

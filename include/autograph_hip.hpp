@@ -416,6 +416,127 @@ template <typename T> struct LeNet5 {
     }
 };
 
+
+// ---- serde (src/tensor.rs:1199-1249) ----
+// The reference's data model `Tensor { dim: (u64, ..), buffer: Buffer(scalar type, len, [u64, ..]) }` as
+// serde_json writes it: {"dim":[..],"buffer":["F32",n,[..]]}.  The u64 items are the buffer's bytes taken
+// eight at a time, each group read as a big-endian integer (pinned by the reference's token test,
+// src/tensor.rs:2236-2277); a last group that is not full is padded with zero bytes.
+namespace serde {
+template <typename T> inline const char *scalar_name() { return std::is_same<T, bf16>::value ? "BF16" : "F32"; }
+
+template <typename T> inline std::string to_json(const Shape &dim, const std::vector<T> &data) {
+    static_assert(std::is_same<T, float>::value || std::is_same<T, bf16>::value, "f32 and bf16 tensors");
+    std::string out = "{\"dim\":[";
+    for (size_t i = 0; i < dim.size(); ++i) out += (i ? "," : "") + std::to_string(dim[i]);
+    out += std::string("],\"buffer\":[\"") + scalar_name<T>() + "\"," + std::to_string(data.size()) + ",[";
+    const unsigned char *raw = reinterpret_cast<const unsigned char *>(data.data());
+    const size_t nbytes = data.size() * sizeof(T);
+    for (size_t b = 0; b < nbytes; b += 8) {
+        uint64_t v = 0;
+        for (size_t j = 0; j < 8; ++j) v = (v << 8) | (b + j < nbytes ? raw[b + j] : 0);
+        out += (b ? "," : "") + std::to_string(v);
+    }
+    return out + "]]}";
+}
+
+// A reader for exactly this shape of document (any JSON whitespace, the two fields in either order).
+class Reader {
+public:
+    explicit Reader(const std::string &s) : s_(s) {}
+    void ws() { while (i_ < s_.size() && (s_[i_] == ' ' || s_[i_] == '\t' || s_[i_] == '\n' || s_[i_] == '\r')) ++i_; }
+    bool peek(char c) { ws(); return i_ < s_.size() && s_[i_] == c; }
+    void expect(char c) { if (!peek(c)) bail(std::string("serde: expected '") + c + "' at offset " + std::to_string(i_)); ++i_; }
+    std::string str() {
+        expect('"');
+        std::string out;
+        while (i_ < s_.size() && s_[i_] != '"') {
+            if (s_[i_] == '\\') bail("serde: escapes do not occur in field or type names");
+            out += s_[i_++];
+        }
+        expect('"');
+        return out;
+    }
+    uint64_t u64() {
+        ws();
+        if (i_ >= s_.size() || s_[i_] < '0' || s_[i_] > '9') bail("serde: expected an unsigned integer at offset " + std::to_string(i_));
+        uint64_t v = 0;
+        while (i_ < s_.size() && s_[i_] >= '0' && s_[i_] <= '9') {
+            const uint64_t d = (uint64_t)(s_[i_++] - '0');
+            if (v > (UINT64_MAX - d) / 10) bail("serde: integer does not fit u64");
+            v = v * 10 + d;
+        }
+        return v;
+    }
+    std::vector<uint64_t> u64_array() {
+        std::vector<uint64_t> out;
+        expect('[');
+        if (peek(']')) { ++i_; return out; }
+        for (;;) {
+            out.push_back(u64());
+            if (peek(',')) { ++i_; continue; }
+            expect(']');
+            return out;
+        }
+    }
+    void end() { ws(); if (i_ != s_.size()) bail("serde: trailing characters"); }
+
+private:
+    const std::string &s_;
+    size_t i_ = 0;
+};
+
+template <typename T> inline void from_json(const std::string &text, Shape &dim, std::vector<T> &data) {
+    Reader r(text);
+    bool have_dim = false, have_buf = false;
+    std::vector<uint64_t> d, items;
+    uint64_t count = 0;
+    r.expect('{');
+    for (;;) {
+        const std::string key = r.str();
+        r.expect(':');
+        if (key == "dim" && !have_dim) {
+            d = r.u64_array();
+            have_dim = true;
+        } else if (key == "buffer" && !have_buf) {
+            r.expect('[');
+            const std::string name = r.str();
+            if (name != scalar_name<T>()) bail(std::string("Expected ") + scalar_name<T>() + " found " + name);
+            r.expect(',');
+            count = r.u64();
+            r.expect(',');
+            items = r.u64_array();
+            r.expect(']');
+            have_buf = true;
+        } else {
+            bail("serde: unknown or repeated field `" + key + "`");
+        }
+        if (r.peek(',')) { r.expect(','); continue; }
+        r.expect('}');
+        break;
+    }
+    r.end();
+    if (!have_dim || !have_buf) bail("serde: missing field");
+    const uint64_t nbytes = count * sizeof(T);
+    if (items.size() != (nbytes + 7) / 8) bail("serde: buffer length does not match its items");
+    uint64_t prod = 1;
+    for (uint64_t x : d) prod *= x;
+    if (prod != count) bail("serde: IncompatibleShape");  // into_shape, src/tensor.rs:1245-1247
+    dim.assign(d.begin(), d.end());
+    data.resize((size_t)count);
+    unsigned char *raw = reinterpret_cast<unsigned char *>(data.data());
+    for (uint64_t b = 0; b < nbytes; ++b) raw[b] = (unsigned char)(items[b / 8] >> (8 * (7 - b % 8)));
+}
+}  // namespace serde
+
+template <typename T> inline std::string to_json(const Tensor<T> &t) { return serde::to_json<T>(t.shape(), t.into_vec()); }
+template <typename T> inline Tensor<T> from_json(const std::string &text) {
+    Shape dim;
+    std::vector<T> data;
+    serde::from_json<T>(text, dim, data);
+    return Tensor<T>::from_vec(dim, data);
+}
+
 }  // namespace agh
 
 #endif  // AUTOGRAPH_HIP_HPP

@@ -57,6 +57,37 @@ static int run_cpu() {
         REQUIRE(e.code() == AGH_ENOINIT);
         REQUIRE(std::string(e.what()).find("agh_init") != std::string::npos);
     }
+    // serde: the documents the Python mirror writes for the same data (known answers), and back
+    {
+        const std::vector<float> f = {1.0f, 2.0f, -0.5f};
+        const std::string jf = serde::to_json<float>({3, 1}, f);
+        REQUIRE(jf == "{\"dim\":[3,1],\"buffer\":[\"F32\",3,[141008071295040,820338753536]]}");
+        const std::vector<bf16> h = {bf16::from_bits(0x3F80), bf16::from_bits(0x4000), bf16::from_bits(0xBF00), bf16::from_bits(0x7FC0),
+                                     bf16::from_bits(0x0001)};
+        const std::string jh = serde::to_json<bf16>({5}, h);
+        REQUIRE(jh == "{\"dim\":[5],\"buffer\":[\"BF16\",5,[9241105235278020735,72057594037927936]]}");
+        Shape dim;
+        std::vector<float> fb;
+        serde::from_json<float>(" { \"buffer\" : [ \"F32\", 3, [141008071295040, 820338753536] ], \"dim\": [3, 1] } ", dim, fb);
+        REQUIRE((dim == Shape{3, 1}) && fb == f);
+        std::vector<bf16> hb;
+        serde::from_json<bf16>(jh, dim, hb);
+        REQUIRE((dim == Shape{5}) && hb.size() == 5 && hb[3].bits == 0x7FC0 && hb[4].bits == 0x0001);
+        const char *bad[] = {"{\"dim\":[3],\"buffer\":[\"BF16\",3,[1,2]]}",         // wrong scalar type for Tensor<f32>
+                             "{\"dim\":[4],\"buffer\":[\"F32\",3,[1,2]]}",          // dim does not hold 3 elements
+                             "{\"dim\":[3],\"buffer\":[\"F32\",3,[1]]}",            // too few items
+                             "{\"dim\":[3],\"buffer\":[\"F32\",3,[1,2]],\"x\":1}",  // unknown field
+                             "{\"dim\":[3]}"};
+        for (const char *b : bad) {
+            bool threw = false;
+            try {
+                serde::from_json<float>(b, dim, fb);
+            } catch (const Error &) {
+                threw = true;
+            }
+            REQUIRE(threw);
+        }
+    }
     std::puts("cpu ok");
     return 0;
 }

@@ -1,0 +1,80 @@
+"""The tensor wire format of the reference (src/tensor.rs:1199-1249), pinned by its own token test
+(src/tensor.rs:2236-2277).  CPU only: the encoding is host logic."""
+import json
+
+import numpy as np
+import pytest
+
+from autograph_amd import serde
+
+
+def test_token_stream_matches_the_reference_test_vector():
+    # tensor_serde: data = [1u32, 2, 3, 4]; the items are the bytes taken 8 at a time, big-endian
+    data = np.array([1, 2, 3, 4], dtype=np.uint32)
+    items = [int.from_bytes(data[:2].tobytes(), "big"), int.from_bytes(data[2:].tobytes(), "big")]
+    assert items == [0x0100000002000000, 0x0300000004000000]  # = u64::to_be of the native-endian pairs
+    want = [("Struct", "Tensor", 2), ("Str", "dim"), ("Tuple", 1), ("U64", 4), ("TupleEnd",), ("Str", "buffer"),
+            ("TupleStruct", "Buffer", 3), ("Str", "U32"), ("U64", 4), ("Seq", 2), ("U64", items[0]), ("U64", items[1]),
+            ("SeqEnd",), ("TupleStructEnd",), ("StructEnd",)]
+    assert serde.to_tokens(data) == want
+
+
+def test_json_is_the_same_data_model():
+    data = np.array([1, 2, 3, 4], dtype=np.uint32)
+    text = serde.to_json(data)
+    assert text == '{"dim":[4],"buffer":["U32",4,[72057594071482368,216172782180892672]]}'
+    back, is_bf16 = serde.from_json(text)
+    assert not is_bf16 and back.dtype == np.uint32 and np.array_equal(back, data)
+
+
+@pytest.mark.parametrize("shape", [(1,), (3,), (2, 3), (6, 1, 5, 5), (84, 10), (0, 4)])
+@pytest.mark.parametrize("kind", ["f32", "bf16"])
+def test_round_trip(shape, kind):
+    rng = np.random.default_rng(3)
+    if kind == "f32":
+        a = rng.standard_normal(shape).astype(np.float32)
+    else:
+        a = rng.integers(0, 1 << 16, shape).astype(np.uint16)
+    text = serde.to_json(a, bf16=kind == "bf16")
+    obj = json.loads(text)
+    assert obj["dim"] == list(shape) and obj["buffer"][0] == ("F32" if kind == "f32" else "BF16")
+    assert obj["buffer"][1] == a.size and len(obj["buffer"][2]) == -(-a.nbytes // 8)
+    back, is_bf16 = serde.from_json(text)
+    assert is_bf16 == (kind == "bf16") and back.shape == tuple(shape) and np.array_equal(back, a)
+    # the token stream carries the same items
+    toks = serde.to_tokens(a, bf16=kind == "bf16")
+    assert [t[1] for t in toks if t[0] == "U64"][a.ndim + 1:] == obj["buffer"][2]
+
+
+def test_rejects_what_the_reference_rejects():
+    good = json.loads(serde.to_json(np.arange(6, dtype=np.float32).reshape(2, 3)))
+    for mutate in (lambda o: o.pop("dim"), lambda o: o.update(extra=1), lambda o: o.__setitem__("dim", [4, 2]),
+                   lambda o: o["buffer"].__setitem__(0, "F31"), lambda o: o["buffer"][2].append(0),
+                   lambda o: o["buffer"].__setitem__(1, 7), lambda o: o["buffer"][2].__setitem__(0, -1),
+                   lambda o: o["buffer"][2].__setitem__(0, 1 << 64)):
+        o = json.loads(json.dumps(good))
+        mutate(o)
+        with pytest.raises(serde.SerdeError):
+            serde.from_json(json.dumps(o))
+    with pytest.raises(serde.SerdeError):
+        serde.from_json("[1, 2")
+
+
+@pytest.mark.gpu
+def test_device_tensor_round_trip():
+    import autograph_amd as ag
+    import oracle as orc
+    ag.Device(0)
+    rng = np.random.default_rng(4)
+    w = rng.standard_normal((16, 6, 5, 5)).astype(np.float32)
+    for arr, dt in ((w, "f32"), (orc.f32_to_bf16(w), "bf16")):
+        t = ag.Tensor.from_array(arr)
+        back = ag.Tensor.from_json(t.to_json(), dtype=dt)
+        assert back.dtype == dt and np.array_equal(back.into_array(), arr)
+        # a transposed view is written in standard layout
+        v = ag.Tensor.from_array(arr.reshape(16, 150)).t()
+        assert np.array_equal(ag.Tensor.from_json(v.to_json()).into_array(), arr.reshape(16, 150).T)
+    with pytest.raises(ag.AghError):
+        ag.Tensor.from_json(ag.Tensor.from_array(w).to_json(), dtype="bf16")
+    with pytest.raises(ag.AghError):
+        ag.Tensor.from_json(serde.to_json(np.arange(4, dtype=np.uint32)))
