@@ -89,7 +89,10 @@ def test_tensor_dot_reference_cases(ag, dtype, n):
 
 
 SHAPES = [(1, 1, 1), (3, 7, 5), (33, 17, 65), (100, 77, 53), (64, 64, 64), (129, 256, 130), (256, 512, 384),
-          (300, 1000, 20), (17, 2048, 9), (1000, 256, 128), (1000, 84, 10), (6400, 150, 16), (100, 25, 6)]
+          (300, 1000, 20), (17, 2048, 9), (1000, 256, 128), (1000, 84, 10), (6400, 150, 16), (100, 25, 6),
+          # k-tile counts 2, 3 and 5 with every dimension a multiple of 8: the direct-to-LDS bf16 kernel's
+          # prologue, odd tail and two-share load order, for all four operand layouts
+          (256, 128, 256), (136, 192, 264), (128, 320, 128)]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
