@@ -499,7 +499,19 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(Args g, int splits) 
     if (e >= total) return;
     const int q = (int)(e / g.NP), p = (int)(e - (size_t)q * g.NP);
     float s = 0.0f;
-    for (int z = 0; z < splits; ++z) s += g.ws[((size_t)z * g.NQ + q) * g.NPpad + p];
+    // eight partials are requested before the first is added (same order of adds): left as a plain loop the
+    // loads issue one per add and the launch is nothing but their latencies in a row
+    const float *wp = g.ws + (size_t)q * g.NPpad + p;
+    const size_t zstride = (size_t)g.NQ * g.NPpad;
+    int z = 0;
+    for (; z + 8 <= splits; z += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = wp[(size_t)(z + u) * zstride];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; z < splits; ++z) s += wp[(size_t)z * zstride];
     T *dst = (T *)g.D + (int64_t)p * g.dp + (int64_t)q * g.dq;
     T old = 0;
     if (g.beta != 0.0f) old = *dst;

@@ -725,7 +725,12 @@ int col2im_launch(const char *name, const void *x, void *y, int64_t bs, int64_t 
     Col2imParams p;
     p.bs = bs; p.c = c; p.ih = ih; p.iw = iw; p.oh = oh; p.ow = ow;
     p.fh = fh; p.fw = fw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
-    {
+    // The streaming (ring) kernels pay off when there is a patch matrix to stream; below a few megabytes one
+    // gathering thread per image pixel finishes sooner.  AGH_COL2IM_RING=1 / 0 forces / forbids the ring form.
+    const int64_t patch_bytes = bs * ih * iw * c * fh * fw * (int64_t)sizeof(T);
+    const char *ring_env = getenv("AGH_COL2IM_RING");
+    const bool use_ring = ring_env ? atoi(ring_env) != 0 : patch_bytes > ((int64_t)4 << 20);
+    if (use_ring) {
         Col2imRingParams rp;
         size_t smem = 0;
         int64_t nblocks = 0;

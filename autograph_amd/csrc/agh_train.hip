@@ -93,7 +93,16 @@ __global__ __launch_bounds__(kThreads) void sum_axis0_kernel(const T *__restrict
     const int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x;
     if (j >= cols) return;
     T acc = Elem<T>::zero();
-    for (int64_t i = 0; i < rows; ++i) acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(x[i * cols + j]));
+    // rows are added one at a time in the element type, in row order; eight are requested before the first add
+    int64_t i = 0;
+    for (; i + 8 <= rows; i += 8) {
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = x[(i + u) * cols + j];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(v[u]));
+    }
+    for (; i < rows; ++i) acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(x[i * cols + j]));
     y[j] = acc;
 }
 

@@ -8,7 +8,7 @@ import ctypes as C
 import numpy as np
 
 from ._ffi import AghError, check, lib
-from .tensor import Im2ColConv2Options, MaxPool2Options, Tensor, _ITEMSIZE, gemm
+from .tensor import Im2ColConv2Options, MaxPool2Options, Tensor, _ITEMSIZE, _std_strides, gemm
 
 
 def conv2_im2col_forward(x, weight, padding=(0, 0), stride=(1, 1), dilation=(1, 1), bias=None, relu=False):
@@ -239,12 +239,36 @@ class LeNet5Trainer:
         self.d1, self.a1, self.d2, self.a2, self.logits = u(bs, 128), u(bs, 128), u(bs, 84), u(bs, 84), u(bs, 10)
         self.g_logits, self.g_a2, self.g_d2 = u(bs, 10), u(bs, 84), u(bs, 84)
         self.g_a1, self.g_d1, self.g_f = u(bs, 128), u(bs, 128), u(bs, 256)
-        self.g_r2, self.g_c2, self.gm2, self.gcols2 = u(bs, 16, 8, 8), u(bs, 16, 8, 8), u(bs * 64, 16), u(bs * 64, 150)
-        self.g_p1, self.g_r1, self.g_c1, self.gm1 = u(bs, 6, 12, 12), u(bs, 6, 24, 24), u(bs, 6, 24, 24), u(bs * 576, 6)
+        # the pooling backward runs in place on the activation it differentiates (its `dx` argument enters
+        # holding x), which nothing reads afterwards: g_r1 / g_r2 are r1 / r2 themselves
+        self.g_r2, self.g_c2, self.gm2, self.gcols2 = self.r2, u(bs, 16, 8, 8), u(bs * 64, 16), u(bs * 64, 150)
+        self.g_p1, self.g_r1, self.g_c1, self.gm1 = u(bs, 6, 12, 12), self.r1, u(bs, 6, 24, 24), u(bs * 576, 6)
+        # Parameters, gradients and velocities each live in ONE buffer (every tensor at a 128-byte aligned
+        # offset, the gaps zero), so the element-wise update of all six parameters is a single launch.  The
+        # model's layers are re-pointed at the views, so model and trainer share storage.
         m = model
-        self.params = [m.conv1.weight, m.conv2.weight, m.dense1.weight, m.dense2.weight, m.dense3.weight, m.dense3.bias]
-        self.grads = [Tensor.uninit(p.shape, dt) for p in self.params]
-        self.velocities = [Tensor.zeros(p.shape, dt) for p in self.params] if self.opt.momentum is not None else [None] * 6
+        old = [m.conv1.weight, m.conv2.weight, m.dense1.weight, m.dense2.weight, m.dense3.weight, m.dense3.bias]
+        offsets, total = [], 0
+        for t in old:
+            offsets.append(total)
+            total += -(-len(t) // 64) * 64
+        self._flat_len = total
+
+        def views(flat):
+            return [Tensor(flat.buffer, t.shape, _std_strides(t.shape), off, dt) for t, off in zip(old, offsets)]
+
+        self._wflat, self._gflat = Tensor.zeros((total,), dt), Tensor.zeros((total,), dt)
+        self.params, self.grads = views(self._wflat), views(self._gflat)
+        for t, v in zip(old, self.params):
+            src = t.as_standard_layout()
+            check(lib.agh_memcpy_d2d(v._data_ptr(), src._data_ptr(), len(t) * _ITEMSIZE[dt]))
+        check(lib.agh_sync())
+        m.conv1.weight, m.conv2.weight, m.dense1.weight, m.dense2.weight, m.dense3.weight, m.dense3.bias = self.params
+        if self.opt.momentum is not None:
+            self._vflat = Tensor.zeros((total,), dt)
+            self.velocities = views(self._vflat)
+        else:
+            self._vflat, self.velocities = None, [None] * 6
         host = C.c_void_p()
         check(lib.agh_host_alloc(C.byref(host), 4))
         self._loss_host = host
@@ -279,9 +303,9 @@ class LeNet5Trainer:
         check(self._fn("agh_max_pool2")(x._data_ptr(), y._ptr(), bs * c, ih, iw, 2, 2, 2, 2))
 
     def _pool_backward(self, x, dy, dx):
-        """dx <- x, then the in-place backward (layer.rs:1203-1211)."""
+        """The in-place backward on a buffer that holds x (layer.rs:1203-1211 copies x first; here `dx` IS x)."""
+        assert dx is x
         bs, c, ih, iw = x.shape
-        check(lib.agh_memcpy_d2d(dx._ptr(), x._data_ptr(), len(x) * _ITEMSIZE[self.dt]))
         check(self._fn("agh_max_pool2_backward")(dx._ptr(), dy._data_ptr(), bs * c, ih, iw, 2, 2, 2, 2))
 
     def _relu(self, x, y):
@@ -317,7 +341,7 @@ class LeNet5Trainer:
         check(self._fn("agh_cross_entropy_loss")(self.logits._ptr(), target.ptr, bs, 10, self._loss_host))
         # backward
         check(self._fn("agh_cross_entropy_backward")(self.logits._ptr(), target.ptr, 1.0, self.g_logits._ptr(), bs, 10))
-        check(self._fn("agh_sum_axis0")(self.g_logits._ptr(), db3._ptr(), bs, 10))
+        check(self._fn("agh_sum_axis0")(self.g_logits._ptr(), db3._data_ptr(), bs, 10))
         gemm(1.0, self.a2.t(), self.g_logits, 0.0, dwd3)
         gemm(1.0, self.g_logits, wd3.t(), 0.0, self.g_a2)
         self._relu_backward(self.d2, self.g_a2, self.g_d2)
@@ -336,9 +360,8 @@ class LeNet5Trainer:
         self._relu_backward(self.c1, self.g_r1, self.g_c1)
         self._nhwc_matrix(self.g_c1, self.gm1)
         gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
-        # update
-        for p, g, v in zip(self.params, self.grads, self.velocities):
-            self.opt.update(self.lr, p, g, v)
+        # update: all parameters at once (element-wise, so one launch over the shared buffers)
+        self.opt.update(self.lr, self._wflat, self._gflat, self._vflat)
 
     def loss(self):
         """The last step's loss; call after `agh_sync`."""

@@ -14,7 +14,7 @@
  *   - matrixmultiply sgemm: only its result up to rounding order is restated
  *     (blocked f32 accumulate); its exact rounding order is "parity unpinned".
  *
- * What pins each function is listed in tests/test_oracle_*.py.
+ * What pins each function is listed in tests/test_oracle.py.
  */
 #include <stdint.h>
 #include <stddef.h>

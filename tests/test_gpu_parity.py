@@ -304,10 +304,14 @@ def test_gemm_full_size_sampled_entries_and_identity(ag, dtype, shape):
 
 
 # ------------------------------------------------------------- im2col / col2im ----
+# col2im has a streaming (ring) form for large patch matrices and a gathering form for small ones; the
+# library picks by size, AGH_COL2IM_RING forces either, and the small reference cases must pass on both
+@pytest.mark.parametrize("ring", ["1", "0"])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-def test_im2col_col2im_reference_grid(ag, dtype):
+def test_im2col_col2im_reference_grid(ag, dtype, ring, monkeypatch):
     """im2col_conv2_<T>_<opts> and col2im_conv2_<T>_<opts> (integration_tests.rs:946-981, :1499-1552):
     ramp inputs over the whole filter/padding/stride/dilation grid; host vs device, bit for bit."""
+    monkeypatch.setenv("AGH_COL2IM_RING", ring)
     count = 0
     for bs, c, ih, iw, f, p, s, d in cases():
         x = to_dtype(np.arange(1, bs * c * ih * iw + 1, dtype=np.float32).reshape(bs, c, ih, iw), dtype)
@@ -336,9 +340,14 @@ IM2COL_SEEDED = [
 ]
 
 
+@pytest.mark.parametrize("ring", ["1", "0", None])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("case", IM2COL_SEEDED)
-def test_im2col_col2im_seeded(ag, dtype, case):
+def test_im2col_col2im_seeded(ag, dtype, case, ring, monkeypatch):
+    if ring is None:
+        monkeypatch.delenv("AGH_COL2IM_RING", raising=False)
+    else:
+        monkeypatch.setenv("AGH_COL2IM_RING", ring)
     bs, c, ih, iw, f, p, s, d = case
     rng = np.random.default_rng(16)
     x = to_dtype(rng.standard_normal((bs, c, ih, iw)), dtype)
