@@ -335,7 +335,7 @@ def main():
                     train_eager()
                 e_ms = (time.perf_counter() - t0) * 1e3 / 50
                 rec = {"gpu_ms": round(g_ms, 4), "gpu_eager_ms": round(e_ms, 4), "last_loss": round(trainer.loss(), 4),
-                       "what": "forward + summed cross-entropy + backward + SGD(momentum 0.01) update, 45 launches; gpu_ms: "
+                       "what": "forward + summed cross-entropy + backward + SGD(momentum 0.01) update, 36 launches; gpu_ms: "
                                "graph replay, wall clock per step including the host-side wait for the loss; "
                                "gpu_eager_ms: the same launches issued one by one from the host"}
                 if not args.no_cpu:
