@@ -185,6 +185,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
 
     // ---- tile shape: minimise (rounds of workgroups) x (tile area) / efficiency ----
     const int cus = compute_units() > 0 ? compute_units() : 256;
+    const bool direct_ok = sizeof(T) == 2 && !any_scalar && g.K > 0 && g.K % 64 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0;
     int best = -1;
     double best_cost = 0;
     for (int i = 0; i < kNumCfgs; ++i) {
@@ -194,7 +195,10 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         if (tiles > 0x7FFFFFFF) continue;
         // a CU works through ceil(tiles / CUs) tiles; co-resident workgroups share its MFMA rate
         const int64_t rounds = (tiles + cus - 1) / cus;
-        const double cost = (double)rounds * t.bp * t.bq / t.eff;
+        // where the direct-to-LDS bf16 kernel applies (the four large tiles), the register-staged small tiles
+        // are a poor second: measured 2x slower at 1024^3 although they put four times as many CUs to work
+        const double eff = (direct_ok && !kCfgs[i].scalar_ok) || !direct_ok ? t.eff : t.eff * 0.4;
+        const double cost = (double)rounds * t.bp * t.bq / eff;
         if (best < 0 || cost < best_cost) { best = i; best_cost = cost; }
     }
     best = env_int("AGH_GEMM_CFG", best);
@@ -225,7 +229,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
 
     // bf16 with both operands vector-loadable and k a multiple of the 64-wide k-tile takes the
     // direct-to-LDS kernel (AGH_GEMM_DIRECT=0 forces the register-staged one)
-    const bool direct = sizeof(T) == 2 && !any_scalar && g.K > 0 && g.K % 64 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0;
+    const bool direct = direct_ok;
 
     if (splits > 1) {
         void *ws = nullptr;
