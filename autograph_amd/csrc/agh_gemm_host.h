@@ -197,7 +197,11 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         const int64_t rounds = (tiles + cus - 1) / cus;
         // where the direct-to-LDS bf16 kernel applies (the four large tiles), the register-staged small tiles
         // are a poor second: measured 2x slower at 1024^3 although they put four times as many CUs to work
-        const double eff = (direct_ok && !kCfgs[i].scalar_ok) || !direct_ok ? t.eff : t.eff * 0.4;
+        double eff = (direct_ok && !kCfgs[i].scalar_ok) || !direct_ok ? t.eff : t.eff * 0.4;
+        // a tile's prologue and epilogue cost about four k-tiles of time when the CU holds one workgroup, next
+        // to nothing when a second workgroup multiplies meanwhile: decides short-k shapes (conv GEMM, k = 576)
+        const double kt = (double)((g.K + BK - 1) / BK);
+        eff *= kt / (kt + (t.wgs_per_cu == 1 ? 4.0 : 0.5));
         const double cost = (double)rounds * t.bp * t.bq / eff;
         if (best < 0 || cost < best_cost) { best = i; best_cost = cost; }
     }
