@@ -362,21 +362,37 @@ __global__ __launch_bounds__(kThreads) void col2im_gather_kernel(const T *__rest
     p.div_c.divmod(plane, b, ci);
     const int ff = p.fh * p.fw;
     const T *xb = x + (size_t)b * p.ih * p.iw * p.ktot + (size_t)ci * ff;
+    // Host order: fi descending (patch row ascending), then fj descending.  Every tap is LOADED, from a clamped
+    // address, and an entry that does not exist contributes +0: the accumulator starts at +0 and a sum that
+    // started at +0 is never -0, so adding +0 changes nothing, exactly like the host's skipped iteration, and
+    // the loads no longer wait for one another behind branches.
     T acc = Elem<T>::zero();
     for (int fi = p.fh - 1; fi >= 0; --fi) {
-        int th = (int)hy + p.ph - fi * p.dh;
-        if (th < 0) continue;
+        const int th = (int)hy + p.ph - fi * p.dh;
         uint32_t hid, rh;
-        p.div_sh.divmod((uint32_t)th, hid, rh);
-        if (rh != 0 || hid >= (uint32_t)p.ih) continue;
-        for (int fj = p.fw - 1; fj >= 0; --fj) {
-            int tw = (int)wy + p.pw - fj * p.dw;
-            if (tw < 0) continue;
-            uint32_t wid, rw;
-            p.div_sw.divmod((uint32_t)tw, wid, rw);
-            if (rw != 0 || wid >= (uint32_t)p.iw) continue;
-            T v = xb[((size_t)hid * p.iw + wid) * p.ktot + fi * p.fw + fj];
-            acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(v));
+        p.div_sh.divmod((uint32_t)max(th, 0), hid, rh);
+        const bool hok = th >= 0 && rh == 0 && hid < (uint32_t)p.ih;
+        const uint32_t hc = min(hid, (uint32_t)p.ih - 1);
+        constexpr int G = 8;  // taps requested together
+        for (int fj0 = p.fw - 1; fj0 >= 0; fj0 -= G) {
+            T v[G];
+            bool ok[G];
+#pragma unroll
+            for (int u = 0; u < G; ++u) {
+                const int fj = fj0 - u;
+                const int fjc = max(fj, 0);
+                const int tw = (int)wy + p.pw - fjc * p.dw;
+                uint32_t wid, rw;
+                p.div_sw.divmod((uint32_t)max(tw, 0), wid, rw);
+                ok[u] = hok && fj >= 0 && tw >= 0 && rw == 0 && wid < (uint32_t)p.iw;
+                const uint32_t wc = min(wid, (uint32_t)p.iw - 1);
+                v[u] = xb[((size_t)hc * p.iw + wc) * p.ktot + fi * p.fw + fjc];
+            }
+#pragma unroll
+            for (int u = 0; u < G; ++u) {
+                const T add = ok[u] ? v[u] : Elem<T>::zero();
+                acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(add));
+            }
         }
     }
     y[e] = acc;

@@ -71,6 +71,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="training section: time eager launches only, no graph capture / replay (rocprofv3 cannot "
+                         "follow the replay of that graph on this image)")
     ap.add_argument("--sections", default="kernels,lenet,train",
                     help="which extras to run: kernels (other GEMMs, im2col/col2im/pool), lenet (inference), "
                          "train (training step); the last two replay captured graphs")
@@ -312,7 +315,8 @@ def main():
                 txx = ag.Tensor.from_array(xt)
                 tbuf = ag.Buffer(bst)
                 ag._ffi.check(ag.lib.agh_memcpy_h2d(tbuf.ptr, tt.ctypes.data, bst))
-                trainer.capture(txx, tbuf)
+                if not args.no_graph:
+                    trainer.capture(txx, tbuf)
 
                 def train_graph():
                     trainer.replay()
@@ -322,18 +326,22 @@ def main():
                     trainer.step(txx, tbuf)
                     ag._ffi.check(ag.lib.agh_sync())
 
-                for _ in range(20):
-                    train_graph()
-                t0 = time.perf_counter()
-                for _ in range(200):
-                    train_graph()
-                g_ms = (time.perf_counter() - t0) * 1e3 / 200
+                g_ms = None
+                if not args.no_graph:
+                    for _ in range(20):
+                        train_graph()
+                    t0 = time.perf_counter()
+                    for _ in range(200):
+                        train_graph()
+                    g_ms = (time.perf_counter() - t0) * 1e3 / 200
                 for _ in range(5):
                     train_eager()
                 t0 = time.perf_counter()
                 for _ in range(50):
                     train_eager()
                 e_ms = (time.perf_counter() - t0) * 1e3 / 50
+                if g_ms is None:
+                    g_ms = e_ms
                 rec = {"gpu_ms": round(g_ms, 4), "gpu_eager_ms": round(e_ms, 4), "last_loss": round(trainer.loss(), 4),
                        "what": "forward + summed cross-entropy + backward + SGD(momentum 0.01) update, 36 launches; gpu_ms: "
                                "graph replay, wall clock per step including the host-side wait for the loss; "
