@@ -25,5 +25,7 @@ from .tensor import (  # noqa: F401
     Im2ColConv2Options,
     MaxPool2Options,
     Tensor,
+    branch,
     gemm,
+    join,
 )

@@ -39,6 +39,9 @@ SIGNATURES = {
     "agh_memcpy_d2h_async": ([ptr, ptr, C.c_size_t], C.c_int),
     "agh_host_alloc": ([C.POINTER(ptr), C.c_size_t], C.c_int),
     "agh_host_free": ([ptr], C.c_int),
+    "agh_branch_begin": ([], C.c_int),
+    "agh_branch_end": ([], C.c_int),
+    "agh_branch_join": ([], C.c_int),
     "agh_graph_begin": ([], C.c_int),
     "agh_graph_end": ([C.POINTER(ptr)], C.c_int),
     "agh_graph_launch": ([ptr], C.c_int),

@@ -13,12 +13,21 @@ static bool g_init = false;
 static int g_device = -1;
 static int g_cus = 0;
 static hipStream_t g_stream = nullptr;
-static void *g_ws = nullptr;
-static size_t g_ws_bytes = 0;
+// A second in-order stream for work the caller declares independent (agh_branch_*).  `g_cur` is the
+// stream entry points launch on: g_stream, or g_side between agh_branch_begin and agh_branch_end.  Each
+// stream has its own workspace (two split-K GEMMs may then run side by side).
+static hipStream_t g_side = nullptr;
+static hipStream_t g_cur = nullptr;
+static bool g_side_dirty = false;  // the branch stream has work the main stream has not waited for
+constexpr int kBranchEvents = 64;
+static hipEvent_t g_events[kBranchEvents];
+static int g_event_next = 0;
+static void *g_ws = nullptr, *g_ws_side = nullptr;
+static size_t g_ws_bytes = 0, g_ws_side_bytes = 0;
 static thread_local char g_err[512] = "";
 
 std::recursive_mutex &api_mutex() { return g_mutex; }
-hipStream_t stream() { return g_stream; }
+hipStream_t stream() { return g_cur; }
 bool initialized() { return g_init; }
 int compute_units() { return g_cus; }
 
@@ -36,18 +45,27 @@ int hip_fail(hipError_t e, const char *what) {
 }
 
 int workspace(size_t bytes, void **ptr) {
-    if (bytes > g_ws_bytes) {
+    const bool side = g_cur == g_side && g_side != nullptr;
+    void *&ws = side ? g_ws_side : g_ws;
+    size_t &have = side ? g_ws_side_bytes : g_ws_bytes;
+    if (bytes > have) {
         // in-order stream: earlier kernels using the old block must finish first
-        AGH_HIP(hipStreamSynchronize(g_stream));
-        if (g_ws) AGH_HIP(hipFree(g_ws));
-        g_ws = nullptr;
-        g_ws_bytes = 0;
+        AGH_HIP(hipStreamSynchronize(g_cur));
+        if (ws) AGH_HIP(hipFree(ws));
+        ws = nullptr;
+        have = 0;
         size_t want = bytes < (size_t)(8u << 20) ? (size_t)(8u << 20) : bytes;
-        AGH_HIP(hipMalloc(&g_ws, want));
-        g_ws_bytes = want;
+        AGH_HIP(hipMalloc(&ws, want));
+        have = want;
     }
-    *ptr = g_ws;
+    *ptr = ws;
     return AGH_OK;
+}
+
+static hipEvent_t next_event() {
+    hipEvent_t e = g_events[g_event_next];
+    g_event_next = (g_event_next + 1) % kBranchEvents;
+    return e;
 }
 
 }  // namespace agh
@@ -75,6 +93,10 @@ int agh_init(int device_index) {
     AGH_HIP(hipGetDeviceProperties(&prop, device_index));
     g_cus = prop.multiProcessorCount;
     AGH_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    AGH_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));  // default priority, like g_stream
+    for (int i = 0; i < kBranchEvents; ++i) AGH_HIP(hipEventCreateWithFlags(&g_events[i], hipEventDisableTiming));
+    g_cur = g_stream;
+    g_side_dirty = false;
     g_device = device_index;
     g_init = true;
     return AGH_OK;
@@ -84,11 +106,15 @@ int agh_shutdown(void) {
     std::lock_guard<std::recursive_mutex> lock(g_mutex);
     if (!g_init) return AGH_OK;
     AGH_HIP(hipStreamSynchronize(g_stream));
+    AGH_HIP(hipStreamSynchronize(g_side));
     if (g_ws) AGH_HIP(hipFree(g_ws));
-    g_ws = nullptr;
-    g_ws_bytes = 0;
+    if (g_ws_side) AGH_HIP(hipFree(g_ws_side));
+    g_ws = g_ws_side = nullptr;
+    g_ws_bytes = g_ws_side_bytes = 0;
+    for (int i = 0; i < kBranchEvents; ++i) (void)hipEventDestroy(g_events[i]);
+    AGH_HIP(hipStreamDestroy(g_side));
     AGH_HIP(hipStreamDestroy(g_stream));
-    g_stream = nullptr;
+    g_stream = g_side = g_cur = nullptr;
     g_init = false;
     g_device = -1;
     return AGH_OK;
@@ -122,6 +148,7 @@ int agh_free(void *ptr) {
     if (!ptr) return AGH_OK;
     // the buffer may still be read by queued kernels
     AGH_HIP(hipStreamSynchronize(g_stream));
+    if (g_side_dirty) AGH_HIP(hipStreamSynchronize(g_side));
     AGH_HIP(hipFree(ptr));
     return AGH_OK;
 }
@@ -186,6 +213,13 @@ int agh_graph_end(void **graph_exec) {
     if (!graph_exec) return fail(AGH_ENULL, "agh_graph_end: null out pointer");
     *graph_exec = nullptr;
     hipGraph_t graph = nullptr;
+    if (g_cur != g_stream) return fail(AGH_EINVAL, "agh_graph_end: still inside a branch");
+    if (g_side_dirty) {  // an arm left open would make the capture invalid
+        hipEvent_t e = next_event();
+        AGH_HIP(hipEventRecord(e, g_side));
+        AGH_HIP(hipStreamWaitEvent(g_stream, e, 0));
+        g_side_dirty = false;
+    }
     AGH_HIP(hipStreamEndCapture(g_stream, &graph));
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
@@ -213,6 +247,39 @@ int agh_graph_destroy(void *graph_exec) {
 int agh_sync(void) {
     AGH_API_ENTER();
     AGH_HIP(hipStreamSynchronize(g_stream));
+    if (g_side_dirty) {
+        AGH_HIP(hipStreamSynchronize(g_side));
+        g_side_dirty = false;
+    }
+    return AGH_OK;
+}
+
+int agh_branch_begin(void) {
+    AGH_API_ENTER();
+    if (g_cur != g_stream) return fail(AGH_EINVAL, "agh_branch_begin: already inside a branch");
+    hipEvent_t e = next_event();
+    AGH_HIP(hipEventRecord(e, g_stream));
+    AGH_HIP(hipStreamWaitEvent(g_side, e, 0));
+    g_cur = g_side;
+    g_side_dirty = true;
+    return AGH_OK;
+}
+
+int agh_branch_end(void) {
+    AGH_API_ENTER();
+    if (g_cur != g_side) return fail(AGH_EINVAL, "agh_branch_end: not inside a branch");
+    g_cur = g_stream;
+    return AGH_OK;
+}
+
+int agh_branch_join(void) {
+    AGH_API_ENTER();
+    if (g_cur != g_stream) return fail(AGH_EINVAL, "agh_branch_join: still inside a branch");
+    if (!g_side_dirty) return AGH_OK;
+    hipEvent_t e = next_event();
+    AGH_HIP(hipEventRecord(e, g_side));
+    AGH_HIP(hipStreamWaitEvent(g_stream, e, 0));
+    g_side_dirty = false;
     return AGH_OK;
 }
 

@@ -3,12 +3,13 @@
 and the LeNet5 model of the reference's benchmark (benches/neural-network-benches/src/
 autograph_backend.rs:88-162), plus one training step of it (`LeNet5Trainer`, `SGD`).
 """
+import contextlib
 import ctypes as C
 
 import numpy as np
 
 from ._ffi import AghError, check, lib
-from .tensor import Im2ColConv2Options, MaxPool2Options, Tensor, _ITEMSIZE, _std_strides, gemm
+from .tensor import Im2ColConv2Options, MaxPool2Options, Tensor, _ITEMSIZE, _std_strides, branch, gemm, join
 
 
 def conv2_im2col_forward(x, weight, padding=(0, 0), stride=(1, 1), dilation=(1, 1), bias=None, relu=False):
@@ -226,10 +227,12 @@ class LeNet5Trainer:
     pool: layer.rs:1193-1216, flatten / permute: autograd.rs:384-445), and the SGD update.
 
     Every buffer is allocated here, once; `step` only launches kernels, so it can be captured into
-    a graph (`capture`) and replayed.  Gradients stay available in `grads` after a step."""
+    a graph (`capture`) and replayed.  Gradients stay available in `grads` after a step.  `overlap`
+    issues the weight gradients beside the input-gradient chain (`branch`); same kernels, same bits."""
 
-    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None):
+    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None, overlap=True):
         self.model, self.bs, self.lr = model, batch_size, learning_rate
+        self._branch = branch if overlap else contextlib.nullcontext
         self.opt = optimizer if optimizer is not None else SGD()
         bs, dt = batch_size, model.conv1.weight.dtype
         self.dt = dt
@@ -339,27 +342,34 @@ class LeNet5Trainer:
         self._relu(self.d2, self.a2)
         gemm(1.0, self.a2, wd3, 0.0, self.logits, bias=b3)
         check(self._fn("agh_cross_entropy_loss")(self.logits._ptr(), target.ptr, bs, 10, self._loss_host))
-        # backward
+        # backward.  The weight gradients of the dense layers and of conv2 feed nothing before the update:
+        # with `overlap` they are issued together, once their operands exist, on the second stream, beside
+        # the rest of the input-gradient chain (one fork and one join).
+        def weight_grads():
+            check(self._fn("agh_sum_axis0")(self.g_logits._ptr(), db3._data_ptr(), bs, 10))
+            gemm(1.0, self.a2.t(), self.g_logits, 0.0, dwd3)
+            gemm(1.0, self.a1.t(), self.g_d2, 0.0, dwd2)
+            gemm(1.0, f.t(), self.g_d1, 0.0, dwd1)
+            gemm(1.0, self.gm2.t(), self.cols2, 0.0, dw2.into_shape((16, 150)))
+
         check(self._fn("agh_cross_entropy_backward")(self.logits._ptr(), target.ptr, 1.0, self.g_logits._ptr(), bs, 10))
-        check(self._fn("agh_sum_axis0")(self.g_logits._ptr(), db3._data_ptr(), bs, 10))
-        gemm(1.0, self.a2.t(), self.g_logits, 0.0, dwd3)
         gemm(1.0, self.g_logits, wd3.t(), 0.0, self.g_a2)
         self._relu_backward(self.d2, self.g_a2, self.g_d2)
-        gemm(1.0, self.a1.t(), self.g_d2, 0.0, dwd2)
         gemm(1.0, self.g_d2, wd2.t(), 0.0, self.g_a1)
         self._relu_backward(self.d1, self.g_a1, self.g_d1)
-        gemm(1.0, f.t(), self.g_d1, 0.0, dwd1)
         gemm(1.0, self.g_d1, wd1.t(), 0.0, self.g_f)
         self._pool_backward(self.r2, self.g_f.into_shape((bs, 16, 4, 4)), self.g_r2)
         self._relu_backward(self.c2, self.g_r2, self.g_c2)
         self._nhwc_matrix(self.g_c2, self.gm2)
-        gemm(1.0, self.gm2.t(), self.cols2, 0.0, dw2.into_shape((16, 150)))
+        with self._branch():
+            weight_grads()
         gemm(1.0, self.gm2, w2.into_shape((16, 150)), 0.0, self.gcols2)
         check(self._fn("agh_col2im_conv2")(self.gcols2._ptr(), self.g_p1._ptr(), bs, 6, 8, 8, 5, 5, 0, 0, 1, 1, 1, 1))
         self._pool_backward(self.r1, self.g_p1, self.g_r1)
         self._relu_backward(self.c1, self.g_r1, self.g_c1)
         self._nhwc_matrix(self.g_c1, self.gm1)
         gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
+        join()
         # update: all parameters at once (element-wise, so one launch over the shared buffers)
         self.opt.update(self.lr, self._wflat, self._gflat, self._vflat)
 

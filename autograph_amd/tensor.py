@@ -7,6 +7,7 @@ point of libautograph_hip.so; nothing is computed on the host.
 
 bf16 tensors travel as numpy ``uint16`` arrays of raw bit patterns.
 """
+import contextlib
 import ctypes as C
 from dataclasses import dataclass, field
 from typing import Tuple
@@ -351,6 +352,23 @@ class Tensor:
         dx = Tensor.uninit(x.shape, x.dtype)
         check(self._fn("agh_cross_entropy_backward")(x._data_ptr(), target.ptr, dy, dx._ptr(), bs, classes))
         return dx
+
+
+@contextlib.contextmanager
+def branch():
+    """Work issued inside the block goes to the library's second stream: it starts after everything
+    issued before the block and runs beside what follows it, until `join()`.  The caller vouches that
+    the two sides write disjoint memory."""
+    check(lib.agh_branch_begin())
+    try:
+        yield
+    finally:
+        check(lib.agh_branch_end())
+
+
+def join():
+    """Later work waits for every `branch()` issued so far."""
+    check(lib.agh_branch_join())
 
 
 def gemm(alpha, a, b, beta, c, bias=None, relu=False):

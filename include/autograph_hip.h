@@ -87,6 +87,19 @@ int agh_graph_end(void **graph_exec);
 int agh_graph_launch(void *graph_exec);
 int agh_graph_destroy(void *graph_exec);
 
+/* Independent work.  Everything issued between agh_branch_begin and agh_branch_end goes to a second
+ * in-order stream: it starts after all work issued before the begin, and runs concurrently with what
+ * the caller issues after the end.  agh_branch_join makes all later work wait for every branch issued
+ * so far; agh_sync waits for both streams.  Several begin/end pairs may precede one join (their work
+ * runs in order among itself).  The CALLER guarantees that a branch and the work issued between its
+ * end and the join touch disjoint outputs (e.g. the weight gradient and the input gradient of one
+ * layer, autograd.rs:607-627: two `dot` calls on the same `output_grad`).  Works under graph capture:
+ * branches become parallel arms of the graph, and a capture must be joined before agh_graph_end.
+ * The reference has no counterpart (krnl has one queue per device). */
+int agh_branch_begin(void);
+int agh_branch_end(void);
+int agh_branch_join(void);
+
 /* Timing helpers: hipEvent pairs recorded on the library's stream. */
 int agh_event_create(void **event);
 int agh_event_destroy(void *event);

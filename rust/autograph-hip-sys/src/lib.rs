@@ -31,6 +31,9 @@ extern "C" {
     pub fn agh_host_free(ptr: *mut c_void) -> c_int;
     pub fn agh_sync() -> c_int;
     pub fn agh_stream() -> *mut c_void;
+    pub fn agh_branch_begin() -> c_int;
+    pub fn agh_branch_end() -> c_int;
+    pub fn agh_branch_join() -> c_int;
     pub fn agh_graph_begin() -> c_int;
     pub fn agh_graph_end(graph_exec: *mut *mut c_void) -> c_int;
     pub fn agh_graph_launch(graph_exec: *mut c_void) -> c_int;

@@ -153,7 +153,8 @@ def test_lenet5_train_graph_replay_equals_eager(ag, dtype):
     x = to_dtype(rng.uniform(0, 1, (bs, 1, 28, 28)), dtype)
     t = rng.integers(0, 10, bs).astype(np.uint8)
     tx, tt = ag.Tensor.from_array(x), labels(ag, t)
-    eager = ag.LeNet5Trainer(ag.LeNet5.from_arrays(*params), bs, optimizer=ag.SGD(0.01))
+    # the eager steps on one stream, the graph with the weight gradients on the second stream
+    eager = ag.LeNet5Trainer(ag.LeNet5.from_arrays(*params), bs, optimizer=ag.SGD(0.01), overlap=False)
     graph = ag.LeNet5Trainer(ag.LeNet5.from_arrays(*params), bs, optimizer=ag.SGD(0.01))
     graph.capture(tx, tt)  # two steps: one eager, one while recording... recording does not execute
     losses = []
@@ -169,3 +170,54 @@ def test_lenet5_train_graph_replay_equals_eager(ag, dtype):
     for a, b in zip(eager.params, graph.params):
         assert np.array_equal(a.into_array(), b.into_array())
     assert losses[2] < losses[0]  # three steps on the same batch lower its loss
+
+
+def test_branch_join_matches_one_stream(ag):
+    """Two products of one left operand (a layer's weight and input gradients, autograd.rs:607-627), the
+    first on the second stream: same bits as in order on one stream, eagerly and in a replayed graph."""
+    rng = np.random.default_rng(46)
+    g = ag.Tensor.from_array(rng.standard_normal((300, 84)).astype(np.float32))
+    a = ag.Tensor.from_array(rng.standard_normal((300, 120)).astype(np.float32))
+    w = ag.Tensor.from_array(rng.standard_normal((120, 84)).astype(np.float32))
+    dw0, da0 = ag.Tensor.zeros((120, 84), "f32"), ag.Tensor.zeros((300, 120), "f32")
+    ag.gemm(1.0, a.t(), g, 0.0, dw0)
+    ag.gemm(1.0, g, w.t(), 0.0, da0)
+    want_dw, want_da = dw0.into_array(), da0.into_array()
+
+    def forked(dw, da):
+        with ag.branch():
+            ag.gemm(1.0, a.t(), g, 0.0, dw)
+        ag.gemm(1.0, g, w.t(), 0.0, da)
+        ag.join()
+
+    dw1, da1 = ag.Tensor.zeros((120, 84), "f32"), ag.Tensor.zeros((300, 120), "f32")
+    forked(dw1, da1)
+    assert np.array_equal(dw1.into_array(), want_dw) and np.array_equal(da1.into_array(), want_da)
+
+    # misuse is an error, and leaves the library usable
+    with pytest.raises(ag.AghError):
+        ag._ffi.check(ag.lib.agh_branch_end())
+    ag._ffi.check(ag.lib.agh_branch_begin())
+    with pytest.raises(ag.AghError):
+        ag._ffi.check(ag.lib.agh_branch_begin())
+    with pytest.raises(ag.AghError):
+        ag._ffi.check(ag.lib.agh_branch_join())
+    ag._ffi.check(ag.lib.agh_branch_end())
+    ag.join()
+
+    dw2, da2 = ag.Tensor.zeros((120, 84), "f32"), ag.Tensor.zeros((300, 120), "f32")
+    ag._ffi.check(ag.lib.agh_sync())
+    ag._ffi.check(ag.lib.agh_graph_begin())
+    try:
+        forked(dw2, da2)
+    finally:
+        graph = C.c_void_p()
+        ag._ffi.check(ag.lib.agh_graph_end(C.byref(graph)))
+    try:
+        zero = np.zeros((120, 84), np.float32)
+        for _ in range(3):
+            ag._ffi.check(ag.lib.agh_memcpy_h2d(dw2._ptr(), zero.ctypes.data, zero.nbytes))
+            ag._ffi.check(ag.lib.agh_graph_launch(graph))
+            assert np.array_equal(dw2.into_array(), want_dw) and np.array_equal(da2.into_array(), want_da)
+    finally:
+        ag._ffi.check(ag.lib.agh_graph_destroy(graph))
