@@ -220,7 +220,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     if (tiles * 2 <= slots && ktiles >= 32 && batch == 1) {
         int64_t s = slots / tiles;
         if (s > ktiles / 4) s = ktiles / 4;
-        if (s > 64) s = 64;
+        if (s > 256) s = 256;
         if (s > 1) splits = (int)s;
     }
     if (batch == 1) splits = env_int("AGH_GEMM_SPLITS", splits);
@@ -243,9 +243,11 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         g.store_mode = ST_SPLITK;
         if (int rc = launch_cfg<T>(best, g, splits, lp, lq, direct)) return rc;
         const size_t total = (size_t)g.NQ * g.NP;
-        const size_t blocks = (total + 255) / 256;
+        int lanes = 1;  // threads per output element: about eight partials each
+        while (lanes < 16 && lanes * 16 <= splits) lanes *= 2;
+        const size_t blocks = (total * lanes + 255) / 256;
         if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: output too large for split-K", name);
-        hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream(), g, splits);
+        hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream(), g, splits, lanes);
         AGH_LAUNCH_CHECK("split-K reduce launch");
         return AGH_OK;
     }

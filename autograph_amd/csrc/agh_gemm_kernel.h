@@ -493,25 +493,31 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
 // Second pass of split-K: sum the partials in split order (deterministic), then the same
 // epilogue as the single-pass kernel.
 template <typename T>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(Args g, int splits) {
-    const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(Args g, int splits, int lanes) {
+    // `lanes` (a power of two, at most 16) neighbouring threads share one output element: lane l adds the
+    // partials l, l + lanes, l + 2*lanes, ... in that order, then the lane sums are combined pairwise.  The
+    // order is fixed by (splits, lanes) alone, so a product is reproducible from run to run.
+    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t total = (size_t)g.NQ * g.NP;
-    if (e >= total) return;
+    const int lane = (int)(t & (size_t)(lanes - 1));
+    size_t e = t / (size_t)lanes;
+    const bool live = e < total;
+    if (!live) e = total - 1;  // whole lane groups stay in step for the exchange below
     const int q = (int)(e / g.NP), p = (int)(e - (size_t)q * g.NP);
     float s = 0.0f;
-    // eight partials are requested before the first is added (same order of adds): left as a plain loop the
-    // loads issue one per add and the launch is nothing but their latencies in a row
+    // eight partials are requested (from clamped addresses) before the first is added: left as a plain loop
+    // the loads issue one per add and the launch is nothing but their latencies in a row
     const float *wp = g.ws + (size_t)q * g.NPpad + p;
     const size_t zstride = (size_t)g.NQ * g.NPpad;
-    int z = 0;
-    for (; z + 8 <= splits; z += 8) {
+    for (int z = lane; z < splits; z += 8 * lanes) {
         float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = wp[(size_t)(z + u) * zstride];
+        for (int u = 0; u < 8; ++u) v[u] = wp[(size_t)min(z + u * lanes, splits - 1) * zstride];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) s += v[u];
+        for (int u = 0; u < 8; ++u) s += z + u * lanes < splits ? v[u] : 0.0f;  // s is never -0: adding +0 is exact
     }
-    for (; z < splits; ++z) s += wp[(size_t)z * zstride];
+    for (int o = lanes >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if (!live || lane != 0) return;
     T *dst = (T *)g.D + (int64_t)p * g.dp + (int64_t)q * g.dq;
     T old = 0;
     if (g.beta != 0.0f) old = *dst;

@@ -179,11 +179,16 @@ def test_split_k_shapes(ag):
     """The weight-gradient shapes of the LeNet5 step (k >> m*n), which the reference splits along k
     (linalg.rs:306-340): dW1 = dY^T * im2col (6 x 57600 x 25), dW2 (16 x 6400 x 150)."""
     rng = np.random.default_rng(13)
-    for (m, k, n) in [(6, 57600, 25), (16, 6400, 150), (64, 16384, 64)]:
+    # the further shapes vary the number of k-groups (8 ... 256, ragged last group) and of threads that share an
+    # output element in the reduction (1 ... 16), and cover an output of several tiles
+    for (m, k, n) in [(6, 57600, 25), (16, 6400, 150), (64, 16384, 64), (5, 1000, 7), (3, 4100, 5), (20, 20001, 30),
+                      (100, 9000, 100)]:
         for dtype in ("f32", "bf16"):
             dy = to_dtype(rng.normal(0, 1, (k, m)), dtype)
             cols = to_dtype(rng.normal(0, 1, (k, n)), dtype)
             out = ag.Tensor.from_array(dy).t().dot(ag.Tensor.from_array(cols)).into_array()
+            again = ag.Tensor.from_array(dy).t().dot(ag.Tensor.from_array(cols)).into_array()
+            assert np.array_equal(out, again), "the reduction order is fixed: same bits on every run"
             if dtype == "f32":
                 assert_f32_gemm_close(out, dy.T, cols)
             else:
