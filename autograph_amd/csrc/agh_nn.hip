@@ -1082,6 +1082,130 @@ int relu_backward_launch(const char *name, const void *x, const void *dy, void *
     return AGH_OK;
 }
 
+
+// ------------------------------------------------------ relu fused with pool ----
+// y = max_pool2(relu(x)) without the intermediate: the same element rule as relu_kernel and the same visiting
+// order as max_pool2_kernel, applied to values that never reach memory.
+template <typename T>
+__device__ __forceinline__ T relu_of(T v) { return Elem<T>::to_f32(v) >= 0.0f ? v : Elem<T>::zero(); }
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void relu_max_pool2_kernel(const T *__restrict__ x, T *__restrict__ y,
+                                                                   PoolParams p, size_t total) {
+    size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    const size_t osz = (size_t)p.oh * p.ow;
+    const size_t plane = e / osz;
+    const uint32_t rem = (uint32_t)(e - plane * osz);
+    uint32_t ho, wo;
+    p.div_ow.divmod(rem, ho, wo);
+    const T *src = x + (plane * p.ih + (size_t)ho * p.sh) * p.iw + (size_t)wo * p.sw;
+    T m = relu_of(src[0]);
+    float mf = Elem<T>::to_f32(m);
+    for (int fi = 0; fi < p.h; ++fi)
+        for (int fj = 0; fj < p.w; ++fj) {
+            T v = relu_of(src[(size_t)fi * p.iw + fj]);
+            float vf = Elem<T>::to_f32(v);
+            if (vf > mf) { m = v; mf = vf; }
+        }
+    y[e] = m;
+}
+
+// dx = relu_backward(x, max_pool2_backward(relu(x), dy)) for windows that do not overlap, one thread per
+// INPUT cell: the cell finds the window that covers it, repeats that window's search for the first strict
+// maximum of relu(x), and takes `0 + dy` if it is that maximum, 0 otherwise; a cell no window covers keeps
+// relu(x), as the in-place pooling backward leaves it.  Then the relu rule of the cell's own x.  dx is
+// [bs, c, ih, iw], or [bs, ih, iw, c] (`nhwc`): the matrix a convolution's weight gradient multiplies.
+struct PoolReluBwdParams {
+    PoolParams p;
+    int c, nhwc;
+    FastDiv div_iw, div_ih, div_c, div_sh, div_sw;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void max_pool2_relu_backward_kernel(const T *__restrict__ x,
+                                                                            const T *__restrict__ dy, T *__restrict__ dx,
+                                                                            PoolReluBwdParams q, size_t total) {
+    size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    const PoolParams &p = q.p;
+    const size_t isz = (size_t)p.ih * p.iw;
+    const uint32_t plane = (uint32_t)(e / isz);  // planes < 2^31 checked on the host
+    const uint32_t rem = (uint32_t)(e - (size_t)plane * isz);
+    uint32_t hy, wx, ho, rh, wo, rw;
+    q.div_iw.divmod(rem, hy, wx);
+    q.div_sh.divmod(hy, ho, rh);
+    q.div_sw.divmod(wx, wo, rw);
+    const T xv = x[e];
+    T g = relu_of(xv);
+    if (rh < (uint32_t)p.h && rw < (uint32_t)p.w && ho < (uint32_t)p.oh && wo < (uint32_t)p.ow) {
+        const T *win = x + ((size_t)plane * p.ih + (size_t)ho * p.sh) * p.iw + (size_t)wo * p.sw;
+        float mf = Elem<T>::to_f32(relu_of(win[0]));
+        int am = 0;
+        for (int fi = 0; fi < p.h; ++fi)
+            for (int fj = 0; fj < p.w; ++fj) {
+                const float vf = Elem<T>::to_f32(relu_of(win[(size_t)fi * p.iw + fj]));
+                if (vf > mf) { mf = vf; am = fi * p.w + fj; }
+            }
+        const T gy = dy[((size_t)plane * p.oh + ho) * p.ow + wo];
+        g = am == (int)(rh * p.w + rw) ? Elem<T>::from_f32(0.0f + Elem<T>::to_f32(gy)) : Elem<T>::zero();
+    }
+    const T out = Elem<T>::to_f32(xv) >= 0.0f ? g : Elem<T>::zero();
+    size_t o = e;
+    if (q.nhwc) {
+        uint32_t b, ci;
+        q.div_c.divmod(plane, b, ci);
+        o = (((size_t)b * p.ih + hy) * p.iw + wx) * q.c + ci;
+    }
+    dx[o] = out;
+}
+
+template <typename T>
+int relu_max_pool2_launch(const char *name, const void *x, void *y, int64_t bc, int64_t ih, int64_t iw, int64_t h,
+                          int64_t w, int64_t sh, int64_t sw) {
+    AGH_API_ENTER();
+    PoolParams p;
+    if (int rc = pool_check(name, bc, ih, iw, h, w, sh, sw, p)) return rc;
+    const size_t total = (size_t)bc * p.oh * p.ow;
+    if (total == 0) return AGH_OK;
+    if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+    size_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
+    hipLaunchKernelGGL(relu_max_pool2_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(), (const T *)x,
+                       (T *)y, p, total);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+template <typename T>
+int max_pool2_relu_backward_launch(const char *name, const void *x, const void *dy, void *dx, int64_t bs, int64_t c,
+                                   int64_t ih, int64_t iw, int64_t h, int64_t w, int64_t sh, int64_t sw, int nhwc) {
+    AGH_API_ENTER();
+    if (bs < 0 || c < 0 || (c > 0 && bs > ((int64_t)1 << 31) / c))
+        return fail(bs < 0 || c < 0 ? AGH_EINVAL : AGH_ERANGE, "%s: invalid batch/channel count", name);
+    PoolReluBwdParams q;
+    if (int rc = pool_check(name, bs * c, ih, iw, h, w, sh, sw, q.p)) return rc;
+    if (sh < h || sw < w)
+        return fail(AGH_EINVAL, "%s: overlapping windows (stride < size) need the separate backward calls", name);
+    const size_t total = (size_t)bs * c * ih * iw;
+    if (total == 0) return AGH_OK;
+    if (!x || !dy || !dx) return fail(AGH_ENULL, "%s: null buffer", name);
+    if (x == dx) return fail(AGH_EINVAL, "%s: dx must not alias x (every cell reads its whole window)", name);
+    q.c = (int)c;
+    q.nhwc = nhwc != 0;
+    q.div_iw = FastDiv((uint32_t)iw);
+    q.div_ih = FastDiv((uint32_t)ih);
+    q.div_c = FastDiv((uint32_t)c);
+    q.div_sh = FastDiv((uint32_t)sh);
+    q.div_sw = FastDiv((uint32_t)sw);
+    size_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
+    hipLaunchKernelGGL(max_pool2_relu_backward_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(),
+                       (const T *)x, (const T *)dy, (T *)dx, q, total);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1131,6 +1255,22 @@ int agh_max_pool2_backward_bf16(void *dx, const void *dy, AGH_POOL_ARGS) {
     return max_pool2_backward_launch<uint16_t>("agh_max_pool2_backward_bf16", dx, dy, AGH_POOL_PASS);
 }
 
+int agh_relu_max_pool2_f32(const void *x, void *y, AGH_POOL_ARGS) {
+    return relu_max_pool2_launch<float>("agh_relu_max_pool2_f32", x, y, AGH_POOL_PASS);
+}
+int agh_relu_max_pool2_bf16(const void *x, void *y, AGH_POOL_ARGS) {
+    return relu_max_pool2_launch<uint16_t>("agh_relu_max_pool2_bf16", x, y, AGH_POOL_PASS);
+}
+int agh_max_pool2_relu_backward_f32(const void *x, const void *dy, void *dx, int64_t bs, int64_t c, int64_t ih,
+                                    int64_t iw, int64_t h, int64_t w, int64_t sh, int64_t sw, int nhwc) {
+    return max_pool2_relu_backward_launch<float>("agh_max_pool2_relu_backward_f32", x, dy, dx, bs, c, ih, iw, h, w, sh,
+                                                 sw, nhwc);
+}
+int agh_max_pool2_relu_backward_bf16(const void *x, const void *dy, void *dx, int64_t bs, int64_t c, int64_t ih,
+                                     int64_t iw, int64_t h, int64_t w, int64_t sh, int64_t sw, int nhwc) {
+    return max_pool2_relu_backward_launch<uint16_t>("agh_max_pool2_relu_backward_bf16", x, dy, dx, bs, c, ih, iw, h, w,
+                                                    sh, sw, nhwc);
+}
 int agh_relu_f32(const void *x, void *y, int64_t n) { return relu_launch<float>("agh_relu_f32", x, y, n); }
 int agh_relu_bf16(const void *x, void *y, int64_t n) { return relu_launch<uint16_t>("agh_relu_bf16", x, y, n); }
 int agh_relu_backward_f32(const void *x, const void *dy, void *dx, int64_t n) {

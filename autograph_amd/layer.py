@@ -237,15 +237,15 @@ class LeNet5Trainer:
         bs, dt = batch_size, model.conv1.weight.dtype
         self.dt = dt
         u = lambda *shape: Tensor.uninit(shape, dt)  # noqa: E731
-        self.cols1, self.c1, self.r1, self.p1 = u(bs * 576, 25), u(bs, 6, 24, 24), u(bs, 6, 24, 24), u(bs, 6, 12, 12)
-        self.cols2, self.c2, self.r2, self.p2 = u(bs * 64, 150), u(bs, 16, 8, 8), u(bs, 16, 8, 8), u(bs, 16, 4, 4)
+        self.cols1, self.c1, self.p1 = u(bs * 576, 25), u(bs, 6, 24, 24), u(bs, 6, 12, 12)
+        self.cols2, self.c2, self.p2 = u(bs * 64, 150), u(bs, 16, 8, 8), u(bs, 16, 4, 4)
         self.d1, self.a1, self.d2, self.a2, self.logits = u(bs, 128), u(bs, 128), u(bs, 84), u(bs, 84), u(bs, 10)
         self.g_logits, self.g_a2, self.g_d2 = u(bs, 10), u(bs, 84), u(bs, 84)
         self.g_a1, self.g_d1, self.g_f = u(bs, 128), u(bs, 128), u(bs, 256)
-        # the pooling backward runs in place on the activation it differentiates (its `dx` argument enters
-        # holding x), which nothing reads afterwards: g_r1 / g_r2 are r1 / r2 themselves
-        self.g_r2, self.g_c2, self.gm2, self.gcols2 = self.r2, u(bs, 16, 8, 8), u(bs * 64, 16), u(bs * 64, 150)
-        self.g_p1, self.g_r1, self.g_c1, self.gm1 = u(bs, 6, 12, 12), self.r1, u(bs, 6, 24, 24), u(bs * 576, 6)
+        # relu(conv) and the NCHW gradient of a convolution's output never exist: relu+pool and their backward
+        # (which writes the [bs*h*w, c] matrix directly) are one launch each
+        self.gm2, self.gcols2 = u(bs * 64, 16), u(bs * 64, 150)
+        self.g_p1, self.gm1 = u(bs, 6, 12, 12), u(bs * 576, 6)
         # Parameters, gradients and velocities each live in ONE buffer (every tensor at a 128-byte aligned
         # offset, the gaps zero), so the element-wise update of all six parameters is a single launch.  The
         # model's layers are re-pointed at the views, so model and trainer share storage.
@@ -301,26 +301,24 @@ class LeNet5Trainer:
             bs, L, K, oc, 1.0, cols._ptr(), 0, K, 1, L * K, wm._ptr(), wm.offset, 1, K, 0,
             0.0, y._ptr(), 0, 1, L, oc * L, None, 0, 0, 0))
 
-    def _pool(self, x, y):
+    def _relu_pool(self, x, y):
+        """Relu then MaxPool2 2x2 (layer.rs:1253-1267, :1193-1216) in one launch; relu(x) is not kept."""
         bs, c, ih, iw = x.shape
-        check(self._fn("agh_max_pool2")(x._data_ptr(), y._ptr(), bs * c, ih, iw, 2, 2, 2, 2))
+        check(self._fn("agh_relu_max_pool2")(x._data_ptr(), y._ptr(), bs * c, ih, iw, 2, 2, 2, 2))
 
-    def _pool_backward(self, x, dy, dx):
-        """The in-place backward on a buffer that holds x (layer.rs:1203-1211 copies x first; here `dx` IS x)."""
-        assert dx is x
+    def _pool_relu_backward(self, x, dy, out):
+        """The backward of that pair from the relu's input x, written as the standard-layout [bs*h*w, c]
+        matrix of the convolution backward (layer.rs:205-220, :1542-1565, autograd.rs:429-445): one launch for
+        the pooling backward, the relu backward and the NHWC copy."""
         bs, c, ih, iw = x.shape
-        check(self._fn("agh_max_pool2_backward")(dx._ptr(), dy._data_ptr(), bs * c, ih, iw, 2, 2, 2, 2))
+        check(self._fn("agh_max_pool2_relu_backward")(x._data_ptr(), dy._data_ptr(), out._ptr(), bs, c, ih, iw,
+                                                      2, 2, 2, 2, 1))
 
     def _relu(self, x, y):
         check(self._fn("agh_relu")(x._data_ptr(), y._ptr(), len(x)))
 
     def _relu_backward(self, x, dy, dx):
         check(self._fn("agh_relu_backward")(x._data_ptr(), dy._data_ptr(), dx._ptr(), len(x)))
-
-    def _nhwc_matrix(self, g, out):
-        """[bs, c, h, w] gradient -> standard-layout [bs*h*w, c] matrix (autograd.rs:429-445)."""
-        v = g.permuted_axes([0, 2, 3, 1])
-        check(self._fn("agh_assign")(v._ptr(), v.offset, *v.strides, out._ptr(), 0, *_std4(v.shape), *v.shape))
 
     def step(self, x, target):
         """x: [bs,1,28,28] tensor, target: device `Buffer` of bs u8 labels.  The loss lands in pinned
@@ -330,11 +328,9 @@ class LeNet5Trainer:
         dw1, dw2, dwd1, dwd2, dwd3, db3 = self.grads
         # forward
         self._conv_forward(x, w1, self.cols1, self.c1)
-        self._relu(self.c1, self.r1)
-        self._pool(self.r1, self.p1)
+        self._relu_pool(self.c1, self.p1)
         self._conv_forward(self.p1, w2, self.cols2, self.c2)
-        self._relu(self.c2, self.r2)
-        self._pool(self.r2, self.p2)
+        self._relu_pool(self.c2, self.p2)
         f = self.p2.into_shape((bs, 256))
         gemm(1.0, f, wd1, 0.0, self.d1)
         self._relu(self.d1, self.a1)
@@ -358,16 +354,12 @@ class LeNet5Trainer:
         gemm(1.0, self.g_d2, wd2.t(), 0.0, self.g_a1)
         self._relu_backward(self.d1, self.g_a1, self.g_d1)
         gemm(1.0, self.g_d1, wd1.t(), 0.0, self.g_f)
-        self._pool_backward(self.r2, self.g_f.into_shape((bs, 16, 4, 4)), self.g_r2)
-        self._relu_backward(self.c2, self.g_r2, self.g_c2)
-        self._nhwc_matrix(self.g_c2, self.gm2)
+        self._pool_relu_backward(self.c2, self.g_f.into_shape((bs, 16, 4, 4)), self.gm2)
         with self._branch():
             weight_grads()
         gemm(1.0, self.gm2, w2.into_shape((16, 150)), 0.0, self.gcols2)
         check(self._fn("agh_col2im_conv2")(self.gcols2._ptr(), self.g_p1._ptr(), bs, 6, 8, 8, 5, 5, 0, 0, 1, 1, 1, 1))
-        self._pool_backward(self.r1, self.g_p1, self.g_r1)
-        self._relu_backward(self.c1, self.g_r1, self.g_c1)
-        self._nhwc_matrix(self.g_c1, self.gm1)
+        self._pool_relu_backward(self.c1, self.g_p1, self.gm1)
         gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
         join()
         # update: all parameters at once (element-wise, so one launch over the shared buffers)
@@ -392,11 +384,3 @@ class LeNet5Trainer:
 
     def replay(self):
         check(lib.agh_graph_launch(self._graph))
-
-
-def _std4(shape):
-    strides, acc = [], 1
-    for d in reversed(shape):
-        strides.append(acc)
-        acc *= d
-    return tuple(reversed(strides))

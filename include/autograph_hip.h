@@ -240,6 +240,25 @@ int agh_max_pool2_backward_f32(void *dx_inout, const void *dy, int64_t bc, int64
 int agh_max_pool2_backward_bf16(void *dx_inout, const void *dy, int64_t bc, int64_t ih, int64_t iw,
                                 int64_t h, int64_t w, int64_t sh, int64_t sw);
 
+/* Relu followed by MaxPool2 in one pass (layer.rs:1253-1267 then :1193-1216, as LeNet5 chains them,
+ * benches/neural-network-benches/src/autograph_backend.rs:114-115, :123-124): y = max_pool2(relu(x)), bit-identical
+ * to agh_relu_* followed by agh_max_pool2_*; relu(x) is not written. */
+int agh_relu_max_pool2_f32(const void *x, void *y, int64_t bc, int64_t ih, int64_t iw,
+                           int64_t h, int64_t w, int64_t sh, int64_t sw);
+int agh_relu_max_pool2_bf16(const void *x, void *y, int64_t bc, int64_t ih, int64_t iw,
+                            int64_t h, int64_t w, int64_t sh, int64_t sw);
+
+/* The backward of that pair in one pass: dx = relu_backward(x, max_pool2_backward(relu(x), dy)), bit-identical
+ * to agh_relu_*, agh_max_pool2_backward_* (in place on relu(x)) and agh_relu_backward_* in a row
+ * (layer.rs:205-220, :1542-1565).  x: [bs, c, ih, iw], the input of the relu; dy: [bs, c, oh, ow]; dx (not
+ * aliasing x): [bs, c, ih, iw], or with nhwc != 0 [bs, ih, iw, c], which is the standard-layout matrix
+ * [bs*ih*iw, c] the convolution backward multiplies (autograd.rs:429-445), so that copy is saved too.
+ * Windows must not overlap (sh >= h, sw >= w), else AGH_EINVAL. */
+int agh_max_pool2_relu_backward_f32(const void *x, const void *dy, void *dx, int64_t bs, int64_t c,
+                                    int64_t ih, int64_t iw, int64_t h, int64_t w, int64_t sh, int64_t sw, int nhwc);
+int agh_max_pool2_relu_backward_bf16(const void *x, const void *dy, void *dx, int64_t bs, int64_t c,
+                                     int64_t ih, int64_t iw, int64_t h, int64_t w, int64_t sh, int64_t sw, int nhwc);
+
 /* -------------------------------------------------------------------- relu ---- */
 
 /* relu / relu_mut (x == y allowed) and relu_backward / relu_backward_mut (dx == dy

@@ -62,6 +62,10 @@ extern "C" {
     pub fn agh_max_pool2_backward_bf16(dx_inout: *mut c_void, dy: *const c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_relu_f32(x: *const c_void, y: *mut c_void, n: i64) -> c_int;
     pub fn agh_relu_bf16(x: *const c_void, y: *mut c_void, n: i64) -> c_int;
+    pub fn agh_relu_max_pool2_f32(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
+    pub fn agh_relu_max_pool2_bf16(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
+    pub fn agh_max_pool2_relu_backward_f32(x: *const c_void, dy: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64, nhwc: c_int) -> c_int;
+    pub fn agh_max_pool2_relu_backward_bf16(x: *const c_void, dy: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64, nhwc: c_int) -> c_int;
     pub fn agh_relu_backward_f32(x: *const c_void, dy: *const c_void, dx: *mut c_void, n: i64) -> c_int;
     pub fn agh_relu_backward_bf16(x: *const c_void, dy: *const c_void, dx: *mut c_void, n: i64) -> c_int;
     pub fn agh_assign_f32(x: *const c_void, off_x: i64, sx0: i64, sx1: i64, sx2: i64, sx3: i64, y: *mut c_void, off_y: i64, sy0: i64, sy1: i64, sy2: i64, sy3: i64, d0: i64, d1: i64, d2: i64, d3: i64) -> c_int;

@@ -449,6 +449,46 @@ def test_max_pool2_special_values(ag):
                               want.view(np.uint32 if dtype == "f32" else np.uint16))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("shape,size,strides", [
+    ((100, 6, 24, 24), (2, 2), (2, 2)), ((100, 16, 8, 8), (2, 2), (2, 2)), ((3, 5, 17, 23), (3, 2), (3, 2)),
+    ((2, 4, 19, 21), (2, 3), (4, 5)), ((1, 1, 4, 4), (2, 2), (2, 2)),
+])
+def test_relu_pool_fused_equals_the_separate_ops(ag, dtype, shape, size, strides):
+    """agh_relu_max_pool2_<T> and agh_max_pool2_relu_backward_<T> against relu -> max_pool2 and
+    max_pool2_backward -> relu_backward of the oracle, bit for bit, including cells no window covers,
+    ties, signed zeros and NaN; the backward in both output layouts."""
+    rng = np.random.default_rng(19)
+    xf = rng.integers(-4, 5, shape).astype(np.float32) * 0.5
+    if shape == (1, 1, 4, 4):
+        nan = np.nan
+        xf = np.array([[[[nan, 3, -1, nan], [-4, 5, -4, -2], [-0.0, 0.0, 0.0, -0.0], [0.0, -0.0, -0.0, 0.0]]]], np.float32)
+    x = to_dtype(xf, dtype)
+    bits = np.uint32 if dtype == "f32" else np.uint16
+    bs, c, ih, iw = shape
+    r = orc.relu(x)
+    want_y = orc.max_pool2(r, size, strides)
+    tx = ag.Tensor.from_array(x)
+    y = ag.Tensor.uninit(want_y.shape, dtype)
+    fwd = getattr(ag.lib, f"agh_relu_max_pool2_{dtype}")
+    ag._ffi.check(fwd(tx._ptr(), y._ptr(), bs * c, ih, iw, *size, *strides))
+    assert np.array_equal(y.into_array().view(bits), want_y.view(bits))
+    dy = to_dtype(rng.standard_normal(want_y.shape), dtype)
+    want_dx = orc.relu_backward(x, orc.max_pool2_backward(r, dy, size, strides))
+    bwd = getattr(ag.lib, f"agh_max_pool2_relu_backward_{dtype}")
+    tdy = ag.Tensor.from_array(dy)
+    for nhwc in (0, 1):
+        dx = ag.Tensor.uninit((bs, ih, iw, c) if nhwc else shape, dtype)
+        ag._ffi.check(bwd(tx._ptr(), tdy._ptr(), dx._ptr(), bs, c, ih, iw, *size, *strides, nhwc))
+        want = np.ascontiguousarray(want_dx.transpose(0, 2, 3, 1)) if nhwc else want_dx
+        assert np.array_equal(dx.into_array().view(bits), want.view(bits)), nhwc
+    # overlapping windows are refused, and so is an output on top of the input
+    with pytest.raises(ag.AghError):
+        ag._ffi.check(bwd(tx._ptr(), tdy._ptr(), dx._ptr(), bs, c, ih, iw, 3, 3, 2, 2, 0))
+    with pytest.raises(ag.AghError):
+        ag._ffi.check(bwd(tx._ptr(), tdy._ptr(), tx._ptr(), bs, c, ih, iw, *size, *strides, 0))
+
+
 # ----------------------------------------------------------------------- relu ----
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_relu_reference_cases(ag, dtype):
