@@ -337,11 +337,12 @@ class LeNet5Trainer:
         gemm(1.0, self.a1, wd2, 0.0, self.d2)
         self._relu(self.d2, self.a2)
         gemm(1.0, self.a2, wd3, 0.0, self.logits, bias=b3)
-        check(self._fn("agh_cross_entropy_loss")(self.logits._ptr(), target.ptr, bs, 10, self._loss_host))
-        # backward.  The weight gradients of the dense layers and of conv2 feed nothing before the update:
+        # backward.  The loss value and the weight gradients of the dense layers and of conv2 feed nothing
+        # before the update:
         # with `overlap` they are issued together, once their operands exist, on the second stream, beside
         # the rest of the input-gradient chain (one fork and one join).
         def weight_grads():
+            check(self._fn("agh_cross_entropy_loss")(self.logits._ptr(), target.ptr, bs, 10, self._loss_host))
             check(self._fn("agh_sum_axis0")(self.g_logits._ptr(), db3._data_ptr(), bs, 10))
             gemm(1.0, self.a2.t(), self.g_logits, 0.0, dwd3)
             gemm(1.0, self.a1.t(), self.g_d2, 0.0, dwd2)
