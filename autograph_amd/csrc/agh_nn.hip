@@ -1160,6 +1160,47 @@ __global__ __launch_bounds__(kThreads) void max_pool2_relu_backward_kernel(const
     dx[o] = out;
 }
 
+// The same for 2x2 windows with stride 2 that tile the image exactly (the case the layer builder defaults to,
+// layer.rs:535-539): one thread per WINDOW, so every cell is covered and the maximum is searched once.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void max_pool2_relu_backward_2x2_kernel(const T *__restrict__ x,
+                                                                                const T *__restrict__ dy,
+                                                                                T *__restrict__ dx, PoolReluBwdParams q,
+                                                                                size_t total) {
+    size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;  // window index = index into dy
+    if (e >= total) return;
+    const PoolParams &p = q.p;
+    const size_t osz = (size_t)p.oh * p.ow;
+    const uint32_t plane = (uint32_t)(e / osz);
+    const uint32_t rem = (uint32_t)(e - (size_t)plane * osz);
+    uint32_t ho, wo;
+    p.div_ow.divmod(rem, ho, wo);
+    const size_t at = ((size_t)plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)wo * 2;
+    const T xv[4] = {x[at], x[at + 1], x[at + p.iw], x[at + p.iw + 1]};
+    const T gy = dy[e];
+    float mf = Elem<T>::to_f32(relu_of(xv[0]));
+    int am = 0;
+#pragma unroll
+    for (int k = 1; k < 4; ++k) {
+        const float vf = Elem<T>::to_f32(relu_of(xv[k]));
+        if (vf > mf) { mf = vf; am = k; }
+    }
+    const T g = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(gy));
+    size_t o = at, ostep = 1, orow = (size_t)p.iw;
+    if (q.nhwc) {
+        uint32_t b, ci;
+        q.div_c.divmod(plane, b, ci);
+        o = (((size_t)b * p.ih + (size_t)ho * 2) * p.iw + (size_t)wo * 2) * q.c + ci;
+        ostep = (size_t)q.c;
+        orow = (size_t)p.iw * q.c;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const T cell = am == k ? g : Elem<T>::zero();
+        dx[o + (k >> 1) * orow + (k & 1) * ostep] = Elem<T>::to_f32(xv[k]) >= 0.0f ? cell : Elem<T>::zero();
+    }
+}
+
 template <typename T>
 int relu_max_pool2_launch(const char *name, const void *x, void *y, int64_t bc, int64_t ih, int64_t iw, int64_t h,
                           int64_t w, int64_t sh, int64_t sw) {
@@ -1198,6 +1239,13 @@ int max_pool2_relu_backward_launch(const char *name, const void *x, const void *
     q.div_c = FastDiv((uint32_t)c);
     q.div_sh = FastDiv((uint32_t)sh);
     q.div_sw = FastDiv((uint32_t)sw);
+    if (h == 2 && w == 2 && sh == 2 && sw == 2 && ih % 2 == 0 && iw % 2 == 0) {
+        const size_t windows = total / 4;
+        hipLaunchKernelGGL(max_pool2_relu_backward_2x2_kernel<T>, dim3((unsigned)((windows + kThreads - 1) / kThreads)),
+                           dim3(kThreads), 0, stream(), (const T *)x, (const T *)dy, (T *)dx, q, windows);
+        AGH_LAUNCH_CHECK(name);
+        return AGH_OK;
+    }
     size_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
     hipLaunchKernelGGL(max_pool2_relu_backward_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(),
