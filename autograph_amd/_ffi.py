@@ -73,6 +73,8 @@ SIGNATURES = {
     "agh_max_pool2_backward_bf16": (_POOL, C.c_int),
     "agh_relu_f32": ([ptr, ptr, i64], C.c_int),
     "agh_relu_bf16": ([ptr, ptr, i64], C.c_int),
+    "agh_conv2_backward_input_f32": ([ptr, ptr, ptr] + [i64] * 13, C.c_int),
+    "agh_conv2_backward_input_bf16": ([ptr, ptr, ptr] + [i64] * 13, C.c_int),
     "agh_relu_max_pool2_f32": ([ptr, ptr] + [i64] * 7, C.c_int),
     "agh_relu_max_pool2_bf16": ([ptr, ptr] + [i64] * 7, C.c_int),
     "agh_max_pool2_relu_backward_f32": ([ptr, ptr, ptr] + [i64] * 8 + [C.c_int], C.c_int),

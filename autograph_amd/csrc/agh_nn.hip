@@ -787,6 +787,120 @@ int col2im_launch(const char *name, const void *x, void *y, int64_t bs, int64_t 
     return AGH_OK;
 }
 
+// ------------------------------------------- conv2 backward w.r.t. the input ----
+// dx = col2im(dy_matrix * W) in one launch, for convolutions whose filter bank fits in LDS (as f32).  One thread
+// owns one image pixel, walks the patch entries that land on it in the host's order like col2im_gather_kernel, and
+// computes each entry where the separate GEMM would have: an f32 dot over the output channels, rounded once to T.
+// The running sum then adds that rounded value in T, so the only difference from GEMM + col2im is the order of
+// the f32 adds inside one dot product.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T *__restrict__ dy, const T *__restrict__ w,
+                                                                         T *__restrict__ y, Col2imParams p, int oc,
+                                                                         size_t total) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    float *wl = (float *)smem_raw;  // [oc][ktot]
+    for (int i = threadIdx.x; i < oc * p.ktot; i += kThreads) wl[i] = Elem<T>::to_f32(w[i]);
+    __syncthreads();
+    size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= total) return;
+    const size_t plane_sz = (size_t)p.oh * p.ow;
+    const uint32_t plane = (uint32_t)(e / plane_sz);
+    const uint32_t rem = (uint32_t)(e - (size_t)plane * plane_sz);
+    uint32_t hy, wy, b, ci;
+    p.div_ow.divmod(rem, hy, wy);
+    p.div_c.divmod(plane, b, ci);
+    const int ff = p.fh * p.fw;
+    constexpr int EPC = 16 / (int)sizeof(T);
+    T acc = Elem<T>::zero();
+    for (int fi = p.fh - 1; fi >= 0; --fi) {
+        const int th = (int)hy + p.ph - fi * p.dh;
+        uint32_t hid, rh;
+        p.div_sh.divmod((uint32_t)max(th, 0), hid, rh);
+        const bool hok = th >= 0 && rh == 0 && hid < (uint32_t)p.ih;
+        const uint32_t hc = min(hid, (uint32_t)p.ih - 1);
+        for (int fj = p.fw - 1; fj >= 0; --fj) {
+            const int tw = (int)wy + p.pw - fj * p.dw;
+            uint32_t wid, rw;
+            p.div_sw.divmod((uint32_t)max(tw, 0), wid, rw);
+            const bool ok = hok && tw >= 0 && rw == 0 && wid < (uint32_t)p.iw;
+            const uint32_t wc = min(wid, (uint32_t)p.iw - 1);
+            // the row is read from a clamped address whether or not the entry exists (it then adds +0)
+            const T *g = dy + (((size_t)b * p.ih + hc) * p.iw + wc) * oc;
+            const float *wt = wl + ci * ff + fi * p.fw + fj;
+            float d = 0.0f;
+            if constexpr (VEC) {
+                for (int o = 0; o < oc; o += EPC) {
+                    const u32x4 v = *(const u32x4 *)(g + o);
+                    if constexpr (sizeof(T) == 4) {
+                        d = fmaf(__uint_as_float(v.x), wt[(o + 0) * p.ktot], d);
+                        d = fmaf(__uint_as_float(v.y), wt[(o + 1) * p.ktot], d);
+                        d = fmaf(__uint_as_float(v.z), wt[(o + 2) * p.ktot], d);
+                        d = fmaf(__uint_as_float(v.w), wt[(o + 3) * p.ktot], d);
+                    } else {
+                        const uint32_t q[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                        for (int h = 0; h < 4; ++h) {
+                            d = fmaf(__uint_as_float(q[h] << 16), wt[(o + 2 * h) * p.ktot], d);
+                            d = fmaf(__uint_as_float(q[h] & 0xFFFF0000u), wt[(o + 2 * h + 1) * p.ktot], d);
+                        }
+                    }
+                }
+            } else {
+                for (int o = 0; o < oc; ++o) d = fmaf(Elem<T>::to_f32(g[o]), wt[o * p.ktot], d);
+            }
+            const T add = ok ? Elem<T>::from_f32(d) : Elem<T>::zero();
+            acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(add));
+        }
+    }
+    y[e] = acc;
+}
+
+template <typename T>
+int conv2_backward_input_launch(const char *name, const void *dy, const void *w, void *dx, int64_t bs, int64_t c,
+                                int64_t ih, int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw,
+                                int64_t sh, int64_t sw, int64_t dh, int64_t dw) {
+    AGH_API_ENTER();
+    if (bs < 0 || c < 0 || ih < 0 || iw < 0 || oc < 0 || fh < 1 || fw < 1 || ph < 0 || pw < 0 || sh < 1 || sw < 1 ||
+        dh < 1 || dw < 1)
+        return fail(AGH_EINVAL, "%s: invalid shape/options", name);
+    if (bs == 0 || c == 0 || ih == 0 || iw == 0) return AGH_OK;
+    const int64_t oh = col2im_out(ih, fh, ph, sh, dh), ow = col2im_out(iw, fw, pw, sw, dw);
+    if (oh < 1 || ow < 1) return fail(AGH_EINVAL, "%s: padding larger than the reconstructed image", name);
+    const int64_t lim = (int64_t)1 << 30;
+    if (bs > lim || c > lim || ih > lim || iw > lim || oh > lim || ow > lim || fh > lim || fw > lim || ph > lim ||
+        pw > lim || sh > lim || sw > lim || dh > lim || dw > lim || oc > lim || c * fh * fw > lim || bs * c > lim ||
+        oh * ow > lim || oh + ph > lim || ow + pw > lim)
+        return fail(AGH_ERANGE, "%s: dimension too large", name);
+    const int64_t ktot = c * fh * fw;
+    if (oc * ktot * 4 > 64 * 1024)
+        return fail(AGH_ERANGE, "%s: filter bank of %lld x %lld does not fit in LDS; use gemm + col2im", name,
+                    (long long)oc, (long long)ktot);
+    if (!dy || !w || !dx) return fail(AGH_ENULL, "%s: null buffer", name);
+    Col2imParams p;
+    p.bs = bs; p.c = c; p.ih = ih; p.iw = iw; p.oh = oh; p.ow = ow;
+    p.fh = fh; p.fw = fw; p.ph = ph; p.pw = pw; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+    p.ktot = (int)ktot;
+    p.div_ow = FastDiv((uint32_t)ow);
+    p.div_oh = FastDiv((uint32_t)oh);
+    p.div_c = FastDiv((uint32_t)c);
+    p.div_sh = FastDiv((uint32_t)sh);
+    p.div_sw = FastDiv((uint32_t)sw);
+    const size_t total = (size_t)bs * c * oh * ow;
+    size_t blocks = (total + kThreads - 1) / kThreads;
+    if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
+    const size_t smem = (size_t)(oc * ktot * 4);
+    constexpr int EPC = 16 / (int)sizeof(T);
+    const bool vec = oc > 0 && oc % EPC == 0 && ((uintptr_t)dy & 15) == 0;
+    if (vec)
+        hipLaunchKernelGGL((conv2_backward_input_kernel<T, true>), dim3((unsigned)blocks), dim3(kThreads), smem, stream(),
+                           (const T *)dy, (const T *)w, (T *)dx, p, (int)oc, total);
+    else
+        hipLaunchKernelGGL((conv2_backward_input_kernel<T, false>), dim3((unsigned)blocks), dim3(kThreads), smem, stream(),
+                           (const T *)dy, (const T *)w, (T *)dx, p, (int)oc, total);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
 // --------------------------------------------------------------- max pool ----
 struct PoolParams {
     int ih, iw, oh, ow, h, w, sh, sw;
@@ -1285,6 +1399,18 @@ int agh_col2im_conv2_f32(const void *x, void *y, AGH_CONV_ARGS) {
 }
 int agh_col2im_conv2_bf16(const void *x, void *y, AGH_CONV_ARGS) {
     return col2im_launch<uint16_t>("agh_col2im_conv2_bf16", x, y, AGH_CONV_PASS);
+}
+int agh_conv2_backward_input_f32(const void *dy, const void *w, void *dx, int64_t bs, int64_t c, int64_t ih, int64_t iw,
+                                 int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t sh, int64_t sw,
+                                 int64_t dh, int64_t dw) {
+    return conv2_backward_input_launch<float>("agh_conv2_backward_input_f32", dy, w, dx, bs, c, ih, iw, oc, fh, fw, ph, pw,
+                                              sh, sw, dh, dw);
+}
+int agh_conv2_backward_input_bf16(const void *dy, const void *w, void *dx, int64_t bs, int64_t c, int64_t ih, int64_t iw,
+                                  int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t sh, int64_t sw,
+                                  int64_t dh, int64_t dw) {
+    return conv2_backward_input_launch<uint16_t>("agh_conv2_backward_input_bf16", dy, w, dx, bs, c, ih, iw, oc, fh, fw, ph,
+                                                 pw, sh, sw, dh, dw);
 }
 
 #define AGH_POOL_ARGS int64_t bc, int64_t ih, int64_t iw, int64_t h, int64_t w, int64_t sh, int64_t sw

@@ -244,7 +244,7 @@ class LeNet5Trainer:
         self.g_a1, self.g_d1, self.g_f = u(bs, 128), u(bs, 128), u(bs, 256)
         # relu(conv) and the NCHW gradient of a convolution's output never exist: relu+pool and their backward
         # (which writes the [bs*h*w, c] matrix directly) are one launch each
-        self.gm2, self.gcols2 = u(bs * 64, 16), u(bs * 64, 150)
+        self.gm2 = u(bs * 64, 16)
         self.g_p1, self.gm1 = u(bs, 6, 12, 12), u(bs * 576, 6)
         # Parameters, gradients and velocities each live in ONE buffer (every tensor at a 128-byte aligned
         # offset, the gaps zero), so the element-wise update of all six parameters is a single launch.  The
@@ -358,8 +358,9 @@ class LeNet5Trainer:
         self._pool_relu_backward(self.c2, self.g_f.into_shape((bs, 16, 4, 4)), self.gm2)
         with self._branch():
             weight_grads()
-        gemm(1.0, self.gm2, w2.into_shape((16, 150)), 0.0, self.gcols2)
-        check(self._fn("agh_col2im_conv2")(self.gcols2._ptr(), self.g_p1._ptr(), bs, 6, 8, 8, 5, 5, 0, 0, 1, 1, 1, 1))
+        # input gradient of conv2: dot with the weight matrix and col2im (layer.rs:976-988) in one launch
+        check(self._fn("agh_conv2_backward_input")(self.gm2._ptr(), w2._data_ptr(), self.g_p1._ptr(), bs, 6, 8, 8, 16,
+                                                   5, 5, 0, 0, 1, 1, 1, 1))
         self._pool_relu_backward(self.c1, self.g_p1, self.gm1)
         gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
         join()

@@ -187,6 +187,21 @@ int agh_col2im_conv2_bf16(const void *x, void *y, int64_t bs, int64_t c, int64_t
                           int64_t fh, int64_t fw, int64_t ph, int64_t pw,
                           int64_t sh, int64_t sw, int64_t dh, int64_t dw);
 
+/* The input-gradient edge of conv2_im2col in one launch: `output_grad.dot(&weight_matrix)?.col2im_conv2(..)`
+ * (src/learn/neural_network/layer.rs:976-988).  dy: the gradient matrix [bs*ih*iw, oc] in standard layout
+ * ((ih, iw) the PATCH GRID, as for col2im), w: the filter bank [oc, c, fh, fw] in standard layout, dx:
+ * [bs, c, oh, ow], fully overwritten.  Every patch entry is an f32 dot over oc rounded once to T, as
+ * agh_gemm_<T> produces it, and the entries are summed like agh_col2im_conv2_<T> (type T, host order): the
+ * result differs from the two separate calls only by the order of the f32 adds inside a dot product.  The
+ * patch matrix [bs*ih*iw, c*fh*fw] is never written.  The filter bank must fit in LDS as f32
+ * (oc*c*fh*fw <= 16384), else AGH_ERANGE: use agh_gemm_<T> + agh_col2im_conv2_<T>. */
+int agh_conv2_backward_input_f32(const void *dy, const void *w, void *dx, int64_t bs, int64_t c,
+                                 int64_t ih, int64_t iw, int64_t oc, int64_t fh, int64_t fw,
+                                 int64_t ph, int64_t pw, int64_t sh, int64_t sw, int64_t dh, int64_t dw);
+int agh_conv2_backward_input_bf16(const void *dy, const void *w, void *dx, int64_t bs, int64_t c,
+                                  int64_t ih, int64_t iw, int64_t oc, int64_t fh, int64_t fw,
+                                  int64_t ph, int64_t pw, int64_t sh, int64_t sw, int64_t dh, int64_t dw);
+
 /* ---------------------------------------------------------- direct convolution ---- */
 
 /* Conv2 forward without a materialised patch matrix: for layers whose input image and filter

@@ -62,6 +62,8 @@ extern "C" {
     pub fn agh_max_pool2_backward_bf16(dx_inout: *mut c_void, dy: *const c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_relu_f32(x: *const c_void, y: *mut c_void, n: i64) -> c_int;
     pub fn agh_relu_bf16(x: *const c_void, y: *mut c_void, n: i64) -> c_int;
+    pub fn agh_conv2_backward_input_f32(dy: *const c_void, w: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
+    pub fn agh_conv2_backward_input_bf16(dy: *const c_void, w: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
     pub fn agh_relu_max_pool2_f32(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_relu_max_pool2_bf16(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_max_pool2_relu_backward_f32(x: *const c_void, dy: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64, nhwc: c_int) -> c_int;

@@ -450,6 +450,49 @@ def test_max_pool2_special_values(ag):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("bs,c,gh,gw,oc,f,p,s,d", [
+    (100, 6, 8, 8, 16, (5, 5), (0, 0), (1, 1), (1, 1)),      # conv2 of LeNet5 (its input gradient)
+    (3, 5, 7, 9, 7, (3, 2), (1, 0), (1, 1), (1, 1)),          # odd channel counts: element loads
+    (2, 4, 6, 5, 8, (3, 3), (1, 1), (2, 2), (1, 1)),          # stride 2: image cells no patch reaches
+    (2, 3, 5, 6, 4, (2, 3), (0, 1), (1, 2), (2, 1)),          # dilation
+])
+def test_conv2_backward_input_fused(ag, dtype, bs, c, gh, gw, oc, f, p, s, d):
+    """agh_conv2_backward_input_<T> = dot with the weight matrix, then col2im (layer.rs:976-988).  On small
+    integers every dot and every sum is exact in f32 and in bf16, so the result must equal the oracle's
+    col2im of the exact product bit for bit (this pins indexing and order); on seeded real data it must be as
+    close to the oracle's chain as the rounding of one dot product allows."""
+    rng = np.random.default_rng(22)
+    fn = getattr(ag.lib, f"agh_conv2_backward_input_{dtype}")
+    k = c * f[0] * f[1]
+    oh = (gh - 1) * s[0] + d[0] * (f[0] - 1) + 1 - 2 * p[0]
+    ow = (gw - 1) * s[1] + d[1] * (f[1] - 1) + 1 - 2 * p[1]
+    for exact in (True, False):
+        if exact:
+            gy = rng.integers(-2, 3, (bs * gh * gw, oc)).astype(np.float32)
+            w = rng.integers(-2, 3, (oc, k)).astype(np.float32)
+        else:
+            gy = rng.standard_normal((bs * gh * gw, oc)).astype(np.float32)
+            w = (rng.standard_normal((oc, k)) * 0.1).astype(np.float32)
+        gyd, wd = to_dtype(gy, dtype), to_dtype(w, dtype)
+        dx = ag.Tensor.uninit((bs, c, oh, ow), dtype)
+        tgy, tw = ag.Tensor.from_array(gyd), ag.Tensor.from_array(wd)
+        ag._ffi.check(fn(tgy._ptr(), tw._ptr(), dx._ptr(), bs, c, gh, gw, oc, *f, *p, *s, *d))
+        got = dx.into_array()
+        cols = orc.gemm_bf16_f32acc(gyd, wd) if dtype == "bf16" else orc.gemm_f64acc(gyd, wd).astype(np.float32)
+        want = orc.col2im_conv2(cols, (gh, gw), f, p, s, d)
+        if exact:
+            assert np.array_equal(got, want)
+        else:
+            # each of the <= fh*fw entries of a pixel may differ by the rounding of one dot product
+            scale = np.abs(as_f32(cols)).max()
+            tol = f[0] * f[1] * scale * (2.0 ** -7 if dtype == "bf16" else 1e-5 * np.sqrt(oc))
+            assert np.abs(as_f32(got).astype(np.float64) - as_f32(want)).max() <= tol
+    big = getattr(ag.lib, f"agh_conv2_backward_input_{dtype}")
+    with pytest.raises(ag.AghError):  # a filter bank that does not fit in LDS is refused, not mis-computed
+        ag._ffi.check(big(dx._ptr(), dx._ptr(), dx._ptr(), 1, 64, 4, 4, 128, 3, 3, 1, 1, 1, 1, 1, 1))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("shape,size,strides", [
     ((100, 6, 24, 24), (2, 2), (2, 2)), ((100, 16, 8, 8), (2, 2), (2, 2)), ((3, 5, 17, 23), (3, 2), (3, 2)),
     ((2, 4, 19, 21), (2, 3), (4, 5)), ((1, 1, 4, 4), (2, 2), (2, 2)),
