@@ -793,13 +793,26 @@ int col2im_launch(const char *name, const void *x, void *y, int64_t bs, int64_t 
 // computes each entry where the separate GEMM would have: an f32 dot over the output channels, rounded once to T.
 // The running sum then adds that rounded value in T, so the only difference from GEMM + col2im is the order of
 // the f32 adds inside one dot product.
-template <typename T, bool VEC>
+template <typename T, bool VEC, bool UNIT, int FW, int OCU>
 __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T *__restrict__ dy, const T *__restrict__ w,
                                                                          T *__restrict__ y, Col2imParams p, int oc,
                                                                          size_t total) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    float *wl = (float *)smem_raw;  // [oc][ktot]
-    for (int i = threadIdx.x; i < oc * p.ktot; i += kThreads) wl[i] = Elem<T>::to_f32(w[i]);
+    float *wl = (float *)smem_raw;  // [ktot][oc]: the output channels of one tap are contiguous
+    // eight elements of w are requested before the first is used: one at a time the staging alone would be
+    // a chain of oc*ktot/256 memory latencies
+    const int nw = oc * p.ktot;
+    for (int i0 = threadIdx.x; i0 < nw; i0 += 8 * kThreads) {
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = w[min(i0 + u * kThreads, nw - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * kThreads;
+            const int o = i / p.ktot, k = i - o * p.ktot;  // coalesced read of w[o][k]
+            if (i < nw) wl[k * oc + o] = Elem<T>::to_f32(v[u]);
+        }
+    }
     __syncthreads();
     size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
     if (e >= total) return;
@@ -811,42 +824,100 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
     p.div_c.divmod(plane, b, ci);
     const int ff = p.fh * p.fw;
     constexpr int EPC = 16 / (int)sizeof(T);
+    const T *gb = dy + (size_t)b * p.ih * p.iw * oc;
     T acc = Elem<T>::zero();
     for (int fi = p.fh - 1; fi >= 0; --fi) {
+        // UNIT: stride 1 in both directions, so every image row / column is a patch row / column (no division)
         const int th = (int)hy + p.ph - fi * p.dh;
-        uint32_t hid, rh;
-        p.div_sh.divmod((uint32_t)max(th, 0), hid, rh);
+        uint32_t hid = (uint32_t)max(th, 0), rh = 0;
+        if constexpr (!UNIT) p.div_sh.divmod((uint32_t)max(th, 0), hid, rh);
         const bool hok = th >= 0 && rh == 0 && hid < (uint32_t)p.ih;
-        const uint32_t hc = min(hid, (uint32_t)p.ih - 1);
+        const T *grow = gb + (size_t)min(hid, (uint32_t)p.ih - 1) * p.iw * oc;
+        const float *wrow = wl + (size_t)(ci * ff + fi * p.fw) * oc;
+        if constexpr (FW > 0 && VEC && UNIT) {
+            // a whole filter row at a time (fw == FW): the FW row vectors of one channel chunk are requested
+            // together, so a pixel waits for fh * oc/EPC loads in a row instead of fh * fw * oc/EPC
+            const T *gp[FW];
+            bool okj[FW];
+            float d[FW];
+#pragma unroll
+            for (int fj = 0; fj < FW; ++fj) {
+                const int tw = (int)wy + p.pw - fj * p.dw;
+                okj[fj] = hok && tw >= 0 && tw < p.iw;
+                gp[fj] = grow + (size_t)min(max(tw, 0), p.iw - 1) * oc;
+                d[fj] = 0.0f;
+            }
+            // OCU channel chunks per trip (oc is a multiple of OCU * EPC): FW * OCU loads in flight
+            for (int o0 = 0; o0 < oc; o0 += OCU * EPC) {
+                u32x4 v[OCU][FW];
+#pragma unroll
+                for (int c = 0; c < OCU; ++c)
+#pragma unroll
+                    for (int fj = 0; fj < FW; ++fj) v[c][fj] = *(const u32x4 *)(gp[fj] + o0 + c * EPC);
+#pragma unroll
+                for (int c = 0; c < OCU; ++c)  // channels ascending inside every dot product
+#pragma unroll
+                    for (int fj = 0; fj < FW; ++fj) {
+                        const float *wt = wrow + fj * oc + o0 + c * EPC;
+                        const float4 w0 = *(const float4 *)wt;
+                        const u32x4 q = v[c][fj];
+                        if constexpr (sizeof(T) == 4) {
+                            d[fj] = fmaf(__uint_as_float(q.x), w0.x, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.y), w0.y, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.z), w0.z, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.w), w0.w, d[fj]);
+                        } else {
+                            const float4 w1 = *(const float4 *)(wt + 4);
+                            d[fj] = fmaf(__uint_as_float(q.x << 16), w0.x, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.x & 0xFFFF0000u), w0.y, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.y << 16), w0.z, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.y & 0xFFFF0000u), w0.w, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.z << 16), w1.x, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.z & 0xFFFF0000u), w1.y, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.w << 16), w1.z, d[fj]);
+                            d[fj] = fmaf(__uint_as_float(q.w & 0xFFFF0000u), w1.w, d[fj]);
+                        }
+                    }
+            }
+#pragma unroll
+            for (int fj = FW - 1; fj >= 0; --fj) {
+                const T add = okj[fj] ? Elem<T>::from_f32(d[fj]) : Elem<T>::zero();
+                acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(add));
+            }
+            continue;
+        }
         for (int fj = p.fw - 1; fj >= 0; --fj) {
             const int tw = (int)wy + p.pw - fj * p.dw;
-            uint32_t wid, rw;
-            p.div_sw.divmod((uint32_t)max(tw, 0), wid, rw);
+            uint32_t wid = (uint32_t)max(tw, 0), rw = 0;
+            if constexpr (!UNIT) p.div_sw.divmod((uint32_t)max(tw, 0), wid, rw);
             const bool ok = hok && tw >= 0 && rw == 0 && wid < (uint32_t)p.iw;
-            const uint32_t wc = min(wid, (uint32_t)p.iw - 1);
             // the row is read from a clamped address whether or not the entry exists (it then adds +0)
-            const T *g = dy + (((size_t)b * p.ih + hc) * p.iw + wc) * oc;
-            const float *wt = wl + ci * ff + fi * p.fw + fj;
+            const T *g = grow + (size_t)min(wid, (uint32_t)p.iw - 1) * oc;
+            const float *wt = wrow + fj * oc;
             float d = 0.0f;
             if constexpr (VEC) {
                 for (int o = 0; o < oc; o += EPC) {
                     const u32x4 v = *(const u32x4 *)(g + o);
+                    const float4 w0 = *(const float4 *)(wt + o);
                     if constexpr (sizeof(T) == 4) {
-                        d = fmaf(__uint_as_float(v.x), wt[(o + 0) * p.ktot], d);
-                        d = fmaf(__uint_as_float(v.y), wt[(o + 1) * p.ktot], d);
-                        d = fmaf(__uint_as_float(v.z), wt[(o + 2) * p.ktot], d);
-                        d = fmaf(__uint_as_float(v.w), wt[(o + 3) * p.ktot], d);
+                        d = fmaf(__uint_as_float(v.x), w0.x, d);
+                        d = fmaf(__uint_as_float(v.y), w0.y, d);
+                        d = fmaf(__uint_as_float(v.z), w0.z, d);
+                        d = fmaf(__uint_as_float(v.w), w0.w, d);
                     } else {
-                        const uint32_t q[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                        for (int h = 0; h < 4; ++h) {
-                            d = fmaf(__uint_as_float(q[h] << 16), wt[(o + 2 * h) * p.ktot], d);
-                            d = fmaf(__uint_as_float(q[h] & 0xFFFF0000u), wt[(o + 2 * h + 1) * p.ktot], d);
-                        }
+                        const float4 w1 = *(const float4 *)(wt + o + 4);
+                        d = fmaf(__uint_as_float(v.x << 16), w0.x, d);
+                        d = fmaf(__uint_as_float(v.x & 0xFFFF0000u), w0.y, d);
+                        d = fmaf(__uint_as_float(v.y << 16), w0.z, d);
+                        d = fmaf(__uint_as_float(v.y & 0xFFFF0000u), w0.w, d);
+                        d = fmaf(__uint_as_float(v.z << 16), w1.x, d);
+                        d = fmaf(__uint_as_float(v.z & 0xFFFF0000u), w1.y, d);
+                        d = fmaf(__uint_as_float(v.w << 16), w1.z, d);
+                        d = fmaf(__uint_as_float(v.w & 0xFFFF0000u), w1.w, d);
                     }
                 }
             } else {
-                for (int o = 0; o < oc; ++o) d = fmaf(Elem<T>::to_f32(g[o]), wt[o * p.ktot], d);
+                for (int o = 0; o < oc; ++o) d = fmaf(Elem<T>::to_f32(g[o]), wt[o], d);
             }
             const T add = ok ? Elem<T>::from_f32(d) : Elem<T>::zero();
             acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(add));
@@ -891,12 +962,25 @@ int conv2_backward_input_launch(const char *name, const void *dy, const void *w,
     const size_t smem = (size_t)(oc * ktot * 4);
     constexpr int EPC = 16 / (int)sizeof(T);
     const bool vec = oc > 0 && oc % EPC == 0 && ((uintptr_t)dy & 15) == 0;
-    if (vec)
-        hipLaunchKernelGGL((conv2_backward_input_kernel<T, true>), dim3((unsigned)blocks), dim3(kThreads), smem, stream(),
-                           (const T *)dy, (const T *)w, (T *)dx, p, (int)oc, total);
-    else
-        hipLaunchKernelGGL((conv2_backward_input_kernel<T, false>), dim3((unsigned)blocks), dim3(kThreads), smem, stream(),
-                           (const T *)dy, (const T *)w, (T *)dx, p, (int)oc, total);
+    const bool unit = sh == 1 && sw == 1;
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), smem, stream(), (const T *)dy, (const T *)w,
+                           (T *)dx, p, (int)oc, total);
+    };
+    const int chunks = vec ? (int)(oc / EPC) : 0;
+    const int ocu = chunks % 4 == 0 ? 4 : chunks % 2 == 0 ? 2 : 1;
+    if (vec && unit && fw == 5) {
+        if (ocu == 4) launch(conv2_backward_input_kernel<T, true, true, 5, 4>);
+        else if (ocu == 2) launch(conv2_backward_input_kernel<T, true, true, 5, 2>);
+        else launch(conv2_backward_input_kernel<T, true, true, 5, 1>);
+    } else if (vec && unit && fw == 3) {
+        if (ocu == 4) launch(conv2_backward_input_kernel<T, true, true, 3, 4>);
+        else if (ocu == 2) launch(conv2_backward_input_kernel<T, true, true, 3, 2>);
+        else launch(conv2_backward_input_kernel<T, true, true, 3, 1>);
+    } else if (vec && unit) launch(conv2_backward_input_kernel<T, true, true, 0, 1>);
+    else if (vec) launch(conv2_backward_input_kernel<T, true, false, 0, 1>);
+    else if (unit) launch(conv2_backward_input_kernel<T, false, true, 0, 1>);
+    else launch(conv2_backward_input_kernel<T, false, false, 0, 1>);
     AGH_LAUNCH_CHECK(name);
     return AGH_OK;
 }

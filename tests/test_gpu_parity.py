@@ -455,6 +455,9 @@ def test_max_pool2_special_values(ag):
     (3, 5, 7, 9, 7, (3, 2), (1, 0), (1, 1), (1, 1)),          # odd channel counts: element loads
     (2, 4, 6, 5, 8, (3, 3), (1, 1), (2, 2), (1, 1)),          # stride 2: image cells no patch reaches
     (2, 3, 5, 6, 4, (2, 3), (0, 1), (1, 2), (2, 1)),          # dilation
+    (2, 4, 6, 5, 8, (3, 3), (1, 1), (1, 1), (1, 1)),          # 3x3, stride 1: a filter row at a time, one chunk
+    (2, 3, 6, 7, 32, (3, 3), (1, 1), (1, 1), (2, 2)),         # the same with four / eight channel chunks, dilated
+    (2, 2, 5, 5, 24, (2, 5), (0, 2), (1, 1), (1, 1)),         # 5 wide, three (f32: six) chunks
 ])
 def test_conv2_backward_input_fused(ag, dtype, bs, c, gh, gw, oc, f, p, s, d):
     """agh_conv2_backward_input_<T> = dot with the weight matrix, then col2im (layer.rs:976-988).  On small
