@@ -2,6 +2,8 @@
 // backward, ReLU, byte fill.  All of them are bounded by HBM traffic, so the work is laid
 // out for coalesced 16-byte stores and single-pass reads; index arithmetic is kept off
 // the critical path with launch-constant multiply-high division.
+#include <type_traits>
+
 #include "agh_internal.h"
 
 using namespace agh;
@@ -793,10 +795,11 @@ int col2im_launch(const char *name, const void *x, void *y, int64_t bs, int64_t 
 // computes each entry where the separate GEMM would have: an f32 dot over the output channels, rounded once to T.
 // The running sum then adds that rounded value in T, so the only difference from GEMM + col2im is the order of
 // the f32 adds inside one dot product.
-template <typename T, bool VEC, bool UNIT, int FW, int OCU>
+template <typename T, bool VEC, bool UNIT, int FW, int OCU, bool LDSG = false>
 __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T *__restrict__ dy, const T *__restrict__ w,
                                                                          T *__restrict__ y, Col2imParams p, int oc,
                                                                          size_t total) {
+    static_assert(!LDSG || (FW > 0 && VEC && UNIT), "the LDS-staged gradient exists for the row-at-a-time form only");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     float *wl = (float *)smem_raw;  // [ktot][oc]: the output channels of one tap are contiguous
     // eight elements of w are requested before the first is used: one at a time the staging alone would be
@@ -813,18 +816,47 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
             if (i < nw) wl[k * oc + o] = Elem<T>::to_f32(v[u]);
         }
     }
+    const size_t plane_sz = (size_t)p.oh * p.ow;
+    // LDSG: an image is at least a workgroup's worth of pixels, so the workgroup's pixels lie in at most two
+    // images, whose gradient matrices [ih*iw][oc] are staged as f32 with a row pitch of oc + 4 (16-byte reads of
+    // neighbouring rows then fall into different banks).  Each row is needed by up to fh*fw pixels: they now
+    // read it from LDS instead of through L1.
+    using S = std::conditional_t<LDSG, float, T>;  // element type the dot products read
+    const int pitch = LDSG ? oc + 4 : oc;
+    float *gl = wl + nw;
+    uint32_t b0 = 0;
+    if constexpr (LDSG) {
+        const size_t e0 = (size_t)blockIdx.x * kThreads, e1 = min(e0 + kThreads, total) - 1;
+        uint32_t c0, c1, b1;
+        p.div_c.divmod((uint32_t)(e0 / plane_sz), b0, c0);
+        p.div_c.divmod((uint32_t)(e1 / plane_sz), b1, c1);
+        const int rows = (int)(b1 - b0 + 1) * p.ih * p.iw, ng = rows * oc;
+        const T *src = dy + (size_t)b0 * p.ih * p.iw * oc;
+        for (int i0 = threadIdx.x; i0 < ng; i0 += 8 * kThreads) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[min(i0 + u * kThreads, ng - 1)];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = i0 + u * kThreads;
+                const int r = i / oc, o = i - r * oc;
+                if (i < ng) gl[r * pitch + o] = Elem<T>::to_f32(v[u]);
+            }
+        }
+    }
     __syncthreads();
     size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
     if (e >= total) return;
-    const size_t plane_sz = (size_t)p.oh * p.ow;
     const uint32_t plane = (uint32_t)(e / plane_sz);
     const uint32_t rem = (uint32_t)(e - (size_t)plane * plane_sz);
     uint32_t hy, wy, b, ci;
     p.div_ow.divmod(rem, hy, wy);
     p.div_c.divmod(plane, b, ci);
     const int ff = p.fh * p.fw;
-    constexpr int EPC = 16 / (int)sizeof(T);
-    const T *gb = dy + (size_t)b * p.ih * p.iw * oc;
+    constexpr int EPC = 16 / (int)sizeof(S);
+    const S *gb;
+    if constexpr (LDSG) gb = gl + (size_t)(b - b0) * p.ih * p.iw * pitch;
+    else gb = dy + (size_t)b * p.ih * p.iw * oc;
     T acc = Elem<T>::zero();
     for (int fi = p.fh - 1; fi >= 0; --fi) {
         // UNIT: stride 1 in both directions, so every image row / column is a patch row / column (no division)
@@ -832,19 +864,19 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
         uint32_t hid = (uint32_t)max(th, 0), rh = 0;
         if constexpr (!UNIT) p.div_sh.divmod((uint32_t)max(th, 0), hid, rh);
         const bool hok = th >= 0 && rh == 0 && hid < (uint32_t)p.ih;
-        const T *grow = gb + (size_t)min(hid, (uint32_t)p.ih - 1) * p.iw * oc;
+        const S *grow = gb + (size_t)min(hid, (uint32_t)p.ih - 1) * p.iw * pitch;
         const float *wrow = wl + (size_t)(ci * ff + fi * p.fw) * oc;
         if constexpr (FW > 0 && VEC && UNIT) {
             // a whole filter row at a time (fw == FW): the FW row vectors of one channel chunk are requested
             // together, so a pixel waits for fh * oc/EPC loads in a row instead of fh * fw * oc/EPC
-            const T *gp[FW];
+            const S *gp[FW];
             bool okj[FW];
             float d[FW];
 #pragma unroll
             for (int fj = 0; fj < FW; ++fj) {
                 const int tw = (int)wy + p.pw - fj * p.dw;
                 okj[fj] = hok && tw >= 0 && tw < p.iw;
-                gp[fj] = grow + (size_t)min(max(tw, 0), p.iw - 1) * oc;
+                gp[fj] = grow + (size_t)min(max(tw, 0), p.iw - 1) * pitch;
                 d[fj] = 0.0f;
             }
             // OCU channel chunks per trip (oc is a multiple of OCU * EPC): FW * OCU loads in flight
@@ -861,7 +893,7 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
                         const float *wt = wrow + fj * oc + o0 + c * EPC;
                         const float4 w0 = *(const float4 *)wt;
                         const u32x4 q = v[c][fj];
-                        if constexpr (sizeof(T) == 4) {
+                        if constexpr (sizeof(S) == 4) {
                             d[fj] = fmaf(__uint_as_float(q.x), w0.x, d[fj]);
                             d[fj] = fmaf(__uint_as_float(q.y), w0.y, d[fj]);
                             d[fj] = fmaf(__uint_as_float(q.z), w0.z, d[fj]);
@@ -892,7 +924,7 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
             if constexpr (!UNIT) p.div_sw.divmod((uint32_t)max(tw, 0), wid, rw);
             const bool ok = hok && tw >= 0 && rw == 0 && wid < (uint32_t)p.iw;
             // the row is read from a clamped address whether or not the entry exists (it then adds +0)
-            const T *g = grow + (size_t)min(wid, (uint32_t)p.iw - 1) * oc;
+            const T *g = (const T *)(const void *)grow + (size_t)min(wid, (uint32_t)p.iw - 1) * oc;  // not with LDSG
             const float *wt = wrow + fj * oc;
             float d = 0.0f;
             if constexpr (VEC) {
@@ -967,6 +999,32 @@ int conv2_backward_input_launch(const char *name, const void *dy, const void *w,
         hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), smem, stream(), (const T *)dy, (const T *)w,
                            (T *)dx, p, (int)oc, total);
     };
+    // f32: the gradient matrices of two images next to the filter bank in LDS, when an image holds at least a
+    // workgroup's worth of pixels (a workgroup then touches at most two images).  Measured at conv2 of LeNet5,
+    // batch 100: 12.3 -> 8.8 us; the bf16 rows are half as long and gain nothing (8.6 -> 9.4 us), so they stay
+    // on the path through L1.
+    const size_t smem_g = smem + (size_t)2 * ih * iw * (oc + 4) * 4;
+    const bool ldsg = sizeof(T) == 4 && vec && unit && (fw == 5 || fw == 3) && c * oh * ow >= kThreads &&
+                      smem_g <= 64 * 1024;
+    if constexpr (sizeof(T) == 4) if (ldsg) {
+        const int ch = (int)(oc / 4);
+        const int u = ch % 4 == 0 ? 4 : ch % 2 == 0 ? 2 : 1;
+        auto launch_g = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), smem_g, stream(), (const T *)dy,
+                               (const T *)w, (T *)dx, p, (int)oc, total);
+        };
+        if (fw == 5) {
+            if (u == 4) launch_g(conv2_backward_input_kernel<T, true, true, 5, 4, true>);
+            else if (u == 2) launch_g(conv2_backward_input_kernel<T, true, true, 5, 2, true>);
+            else launch_g(conv2_backward_input_kernel<T, true, true, 5, 1, true>);
+        } else {
+            if (u == 4) launch_g(conv2_backward_input_kernel<T, true, true, 3, 4, true>);
+            else if (u == 2) launch_g(conv2_backward_input_kernel<T, true, true, 3, 2, true>);
+            else launch_g(conv2_backward_input_kernel<T, true, true, 3, 1, true>);
+        }
+        AGH_LAUNCH_CHECK(name);
+        return AGH_OK;
+    }
     const int chunks = vec ? (int)(oc / EPC) : 0;
     const int ocu = chunks % 4 == 0 ? 4 : chunks % 2 == 0 ? 2 : 1;
     if (vec && unit && fw == 5) {

@@ -458,6 +458,9 @@ def test_max_pool2_special_values(ag):
     (2, 4, 6, 5, 8, (3, 3), (1, 1), (1, 1), (1, 1)),          # 3x3, stride 1: a filter row at a time, one chunk
     (2, 3, 6, 7, 32, (3, 3), (1, 1), (1, 1), (2, 2)),         # the same with four / eight channel chunks, dilated
     (2, 2, 5, 5, 24, (2, 5), (0, 2), (1, 1), (1, 1)),         # 5 wide, three (f32: six) chunks
+    (3, 8, 8, 8, 8, (3, 3), (1, 1), (1, 1), (1, 1)),          # images of >= 256 pixels: gradient rows staged in LDS
+    (2, 16, 5, 6, 12, (3, 3), (0, 0), (1, 1), (1, 1)),        # the same, three chunks of four channels (f32 only)
+    (5, 6, 9, 7, 16, (4, 5), (2, 1), (1, 1), (1, 2)),         # the same, 5 wide, padded and dilated
 ])
 def test_conv2_backward_input_fused(ag, dtype, bs, c, gh, gw, oc, f, p, s, d):
     """agh_conv2_backward_input_<T> = dot with the weight matrix, then col2im (layer.rs:976-988).  On small
