@@ -191,3 +191,60 @@ pub fn max_pool2_backward<T: Scalar>(dx: *mut c_void, dy: *const c_void, bc: usi
         }
     })
 }
+
+/// `Relu` then `MaxPool2` (layer.rs:1253-1267, :1193-1216) in one launch; bit-identical to the two calls.
+pub fn relu_max_pool2<T: Scalar>(x: *const c_void, y: *mut c_void, bc: usize, hw: [usize; 2], size: [usize; 2], strides: [usize; 2]) -> Result<()> {
+    let a = [bc as i64, hw[0] as i64, hw[1] as i64, size[0] as i64, size[1] as i64, strides[0] as i64, strides[1] as i64];
+    check(unsafe {
+        if T::IS_BF16 {
+            sys::agh_relu_max_pool2_bf16(x, y, a[0], a[1], a[2], a[3], a[4], a[5], a[6])
+        } else {
+            sys::agh_relu_max_pool2_f32(x, y, a[0], a[1], a[2], a[3], a[4], a[5], a[6])
+        }
+    })
+}
+
+/// The backward edges of that pair (layer.rs:205-220, :1542-1565) in one launch, from the relu's input `x`;
+/// `nhwc` writes `dx` as the `[bs*ih*iw, c]` matrix of autograd.rs:429-445.  Windows must not overlap.
+#[allow(clippy::too_many_arguments)]
+pub fn max_pool2_relu_backward<T: Scalar>(x: *const c_void, dy: *const c_void, dx: *mut c_void, bs: usize, c: usize, hw: [usize; 2], size: [usize; 2], strides: [usize; 2], nhwc: bool) -> Result<()> {
+    let a = [bs as i64, c as i64, hw[0] as i64, hw[1] as i64, size[0] as i64, size[1] as i64, strides[0] as i64, strides[1] as i64];
+    check(unsafe {
+        if T::IS_BF16 {
+            sys::agh_max_pool2_relu_backward_bf16(x, dy, dx, a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], nhwc as i32)
+        } else {
+            sys::agh_max_pool2_relu_backward_f32(x, dy, dx, a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], nhwc as i32)
+        }
+    })
+}
+
+/// The input-gradient edge of `conv2_im2col` (layer.rs:976-988): `output_grad.dot(&weight_matrix)` and
+/// `col2im_conv2` in one launch.  `g.hw` is the patch grid; an `Err` carrying `AGH_ERANGE` means the filter bank
+/// does not fit in LDS: call `gemm` and `col2im_conv2` instead.
+pub fn conv2_backward_input<T: Scalar>(dy: *const c_void, w: *const c_void, dx: *mut c_void, outputs: usize, g: &ConvGeometry) -> Result<()> {
+    let a = [
+        g.bs as i64, g.c as i64, g.hw[0] as i64, g.hw[1] as i64, outputs as i64, g.filter[0] as i64, g.filter[1] as i64,
+        g.padding[0] as i64, g.padding[1] as i64, g.stride[0] as i64, g.stride[1] as i64, g.dilation[0] as i64, g.dilation[1] as i64,
+    ];
+    check(unsafe {
+        if T::IS_BF16 {
+            sys::agh_conv2_backward_input_bf16(dy, w, dx, a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], a[8], a[9], a[10], a[11], a[12])
+        } else {
+            sys::agh_conv2_backward_input_f32(dy, w, dx, a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], a[8], a[9], a[10], a[11], a[12])
+        }
+    })
+}
+
+/// Runs `f` with the library's second stream current: what `f` launches starts after everything launched
+/// before and runs beside what is launched next, until `join`.  The two sides must write disjoint memory.
+pub fn branch<R>(f: impl FnOnce() -> Result<R>) -> Result<R> {
+    check(unsafe { sys::agh_branch_begin() })?;
+    let out = f();
+    check(unsafe { sys::agh_branch_end() })?;
+    out
+}
+
+/// Later launches wait for every `branch` issued so far.
+pub fn join() -> Result<()> {
+    check(unsafe { sys::agh_branch_join() })
+}
