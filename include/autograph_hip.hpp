@@ -271,6 +271,28 @@ public:
                                                                                  o.strides[1]));
     }
 
+    // Relu then MaxPool2 in one launch (layer.rs:1253-1267, :1193-1216): same bits as relu().max_pool2(o)
+    Tensor relu_max_pool2(const MaxPool2Options &o) const {
+        if (ndim() != 4) bail("relu_max_pool2: expected a 4-D tensor");
+        const Tensor x = as_standard_layout();
+        const auto out = o.output_shape({dim_[2], dim_[3]});
+        Tensor y = uninit({dim_[0], dim_[1], out[0], out[1]});
+        check((kBf16 ? agh_relu_max_pool2_bf16 : agh_relu_max_pool2_f32)(x.data_ptr(), y.buffer_ptr(), dim_[0] * dim_[1], dim_[2], dim_[3],
+                                                                         o.size[0], o.size[1], o.strides[0], o.strides[1]));
+        return y;
+    }
+    // the backward edges of that pair in one launch, *this being the relu's input (layer.rs:205-220, :1542-1565);
+    // `nhwc` returns the gradient as [bs, h, w, c] in standard layout (autograd.rs:429-445).  Windows must not overlap.
+    Tensor max_pool2_relu_backward(const Tensor &output_grad, const MaxPool2Options &o, bool nhwc = false) const {
+        if (ndim() != 4) bail("max_pool2_relu_backward: expected a 4-D tensor");
+        const Tensor x = as_standard_layout(), dy = output_grad.as_standard_layout();
+        Tensor dx = nhwc ? uninit({dim_[0], dim_[2], dim_[3], dim_[1]}) : uninit(dim_);
+        check((kBf16 ? agh_max_pool2_relu_backward_bf16 : agh_max_pool2_relu_backward_f32)(
+            x.data_ptr(), dy.data_ptr(), dx.buffer_ptr(), dim_[0], dim_[1], dim_[2], dim_[3], o.size[0], o.size[1], o.strides[0],
+            o.strides[1], nhwc ? 1 : 0));
+        return dx;
+    }
+
     // -- relu (layer.rs:1269-1510) --
     Tensor relu() const {
         const Tensor x = as_standard_layout();

@@ -173,6 +173,14 @@ static int run_gpu(const char *in_path, const char *out_path) {
     Tensor<float> grad = act.clone();
     grad.max_pool2_backward(Tensor<float>::from_vec(pooled.shape(), std::vector<float>((size_t)pooled.len(), 1.0f)), po);
     append(grad.into_vec());
+    // the fused Relu -> MaxPool2 pair and its backward equal the separate calls bit for bit
+    const Tensor<float> pre = model.conv1.forward(tx);  // [bs,6,24,24], the relu's input
+    REQUIRE(pre.relu_max_pool2(po).into_vec() == pooled.into_vec());
+    const Tensor<float> ones = Tensor<float>::from_vec(pooled.shape(), std::vector<float>((size_t)pooled.len(), 1.0f));
+    const Tensor<float> fused_grad = pre.max_pool2_relu_backward(ones, po);
+    REQUIRE(fused_grad.into_vec() == pre.relu_backward(grad).into_vec());
+    REQUIRE(pre.max_pool2_relu_backward(ones, po, true).into_vec() ==
+            fused_grad.permuted_axes({0, 2, 3, 1}).to_standard_layout().into_vec());
     // a permuted view copies into standard layout
     REQUIRE(act.permuted_axes({0, 2, 3, 1}).to_standard_layout().permuted_axes({0, 3, 1, 2}).into_vec() == act.into_vec());
     device.wait();
