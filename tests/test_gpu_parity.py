@@ -450,6 +450,26 @@ def test_max_pool2_special_values(ag):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_fused_entry_points_empty_and_invalid(ag, dtype):
+    """Empty batches are a no-op (the reference allows zero-length tensors); invalid geometry is an error code,
+    never a launch."""
+    buf = ag.Tensor.zeros((4, 4), dtype)
+    ptr = buf._ptr()
+    lib, check = ag.lib, ag._ffi.check
+    check(getattr(lib, f"agh_relu_max_pool2_{dtype}")(ptr, ptr, 0, 4, 4, 2, 2, 2, 2))
+    check(getattr(lib, f"agh_max_pool2_relu_backward_{dtype}")(ptr, ptr, None, 0, 3, 4, 4, 2, 2, 2, 2, 0))
+    check(getattr(lib, f"agh_conv2_backward_input_{dtype}")(ptr, ptr, None, 0, 3, 4, 4, 8, 3, 3, 0, 0, 1, 1, 1, 1))
+    with pytest.raises(ag.AghError):  # window larger than the image
+        check(getattr(lib, f"agh_relu_max_pool2_{dtype}")(ptr, ptr, 1, 2, 2, 3, 3, 1, 1))
+    with pytest.raises(ag.AghError):  # null output with work to do
+        check(getattr(lib, f"agh_max_pool2_relu_backward_{dtype}")(ptr, ptr, None, 1, 1, 4, 4, 2, 2, 2, 2, 0))
+    with pytest.raises(ag.AghError):  # zero stride
+        check(getattr(lib, f"agh_conv2_backward_input_{dtype}")(ptr, ptr, ptr, 1, 1, 2, 2, 1, 3, 3, 0, 0, 0, 1, 1, 1))
+    with pytest.raises(ag.AghError):  # padding swallows the image
+        check(getattr(lib, f"agh_conv2_backward_input_{dtype}")(ptr, ptr, ptr, 1, 1, 1, 1, 1, 1, 1, 2, 2, 1, 1, 1, 1))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("bs,c,gh,gw,oc,f,p,s,d", [
     (100, 6, 8, 8, 16, (5, 5), (0, 0), (1, 1), (1, 1)),      # conv2 of LeNet5 (its input gradient)
     (3, 5, 7, 9, 7, (3, 2), (1, 0), (1, 1), (1, 1)),          # odd channel counts: element loads
