@@ -95,6 +95,8 @@ int agh_graph_destroy(void *graph_exec);
  * end and the join touch disjoint outputs (e.g. the weight gradient and the input gradient of one
  * layer, autograd.rs:607-627: two `dot` calls on the same `output_grad`).  Works under graph capture:
  * branches become parallel arms of the graph, and a capture must be joined before agh_graph_end.
+ * The branch state belongs to the library, not to the calling thread: while one thread is between begin and
+ * end, entry points called from any thread go to the second stream.
  * The reference has no counterpart (krnl has one queue per device). */
 int agh_branch_begin(void);
 int agh_branch_end(void);
