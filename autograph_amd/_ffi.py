@@ -33,6 +33,8 @@ SIGNATURES = {
     "agh_device_info": ([C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_size_t)], C.c_int),
     "agh_malloc": ([C.POINTER(ptr), C.c_size_t], C.c_int),
     "agh_free": ([ptr], C.c_int),
+    "agh_cache_release": ([], C.c_int),
+    "agh_cache_stats": ([C.POINTER(C.c_size_t)] * 3, C.c_int),
     "agh_memcpy_h2d": ([ptr, ptr, C.c_size_t], C.c_int),
     "agh_memcpy_d2h": ([ptr, ptr, C.c_size_t], C.c_int),
     "agh_memcpy_d2d": ([ptr, ptr, C.c_size_t], C.c_int),

@@ -1,8 +1,13 @@
-// Runtime half of the C ABI: device selection, the single in-order stream, buffers,
-// copies, events.  Replaces what the reference gets from krnl's Device / Buffer.
+// Runtime half of the C ABI: device selection, the in-order streams, the caching buffer
+// allocator, copies, events, graphs.  Replaces what the reference gets from krnl's Device / Buffer.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
+
+#include <map>
+#include <unordered_map>
+#include <vector>
 
 #include "agh_internal.h"
 
@@ -22,9 +27,34 @@ static bool g_side_dirty = false;  // the branch stream has work the main stream
 constexpr int kBranchEvents = 64;
 static hipEvent_t g_events[kBranchEvents];
 static int g_event_next = 0;
-static void *g_ws = nullptr, *g_ws_side = nullptr;
-static size_t g_ws_bytes = 0, g_ws_side_bytes = 0;
+static bool g_capturing = false;   // between agh_graph_begin and agh_graph_end
+static int g_live_graphs = 0;      // graph executables not yet destroyed: their nodes hold workspace pointers
 static thread_local char g_err[512] = "";
+
+// Library-owned workspace of one stream.  A block that a live graph may reference is retired, not
+// freed, when a larger one is needed; retired blocks go at agh_shutdown or when the last graph is
+// destroyed.  Growth at least doubles, so the retired blocks together are smaller than the live one.
+struct Workspace {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+static Workspace g_ws, g_ws_side;
+static std::vector<void *> g_ws_retired;
+
+// ---- caching allocator behind agh_malloc / agh_free ----
+// Freed blocks are kept, by size, and handed out again without touching the driver.  Work is issued in
+// order on one stream, so a block freed by the host while kernels that use it are still queued is safe
+// to reuse: whatever is launched on it later runs after them.  The only other stream is the branch
+// stream: a block freed while that stream had unjoined work remembers the branch it may belong to, and
+// reusing it on the main stream first makes the main stream wait for the branch stream.
+struct CachedBlock {
+    void *ptr;
+    uint64_t side_seq;  // branch number current when it was freed with the branch stream busy, else 0
+};
+static std::multimap<size_t, CachedBlock> g_free_blocks;     // by capacity
+static std::unordered_map<void *, size_t> g_live_blocks;     // capacity of every block handed out
+static size_t g_cached_bytes = 0, g_cache_limit = (size_t)64 << 30;
+static uint64_t g_side_seq = 0, g_side_joined_seq = 0;
 
 std::recursive_mutex &api_mutex() { return g_mutex; }
 hipStream_t stream() { return g_cur; }
@@ -44,21 +74,36 @@ int hip_fail(hipError_t e, const char *what) {
     return (int)e > 0 ? (int)e : 999;
 }
 
+static int release_retired_workspaces() {
+    for (void *p : g_ws_retired) AGH_HIP(hipFree(p));
+    g_ws_retired.clear();
+    return AGH_OK;
+}
+
 int workspace(size_t bytes, void **ptr) {
     const bool side = g_cur == g_side && g_side != nullptr;
-    void *&ws = side ? g_ws_side : g_ws;
-    size_t &have = side ? g_ws_side_bytes : g_ws_bytes;
-    if (bytes > have) {
-        // in-order stream: earlier kernels using the old block must finish first
-        AGH_HIP(hipStreamSynchronize(g_cur));
-        if (ws) AGH_HIP(hipFree(ws));
-        ws = nullptr;
-        have = 0;
+    Workspace &ws = side ? g_ws_side : g_ws;
+    if (bytes > ws.bytes) {
+        if (g_capturing)
+            return fail(AGH_ERANGE, "workspace: %zu bytes needed while capturing a graph, %zu available: run the sequence "
+                        "once eagerly before agh_graph_begin", bytes, ws.bytes);
         size_t want = bytes < (size_t)(8u << 20) ? (size_t)(8u << 20) : bytes;
-        AGH_HIP(hipMalloc(&ws, want));
-        have = want;
+        if (want < 2 * ws.bytes) want = 2 * ws.bytes;
+        void *fresh = nullptr;
+        AGH_HIP(hipMalloc(&fresh, want));
+        if (ws.ptr) {
+            if (g_live_graphs > 0) {
+                g_ws_retired.push_back(ws.ptr);  // a captured node may still name it
+            } else {
+                // in-order stream: earlier kernels using the old block must finish first
+                AGH_HIP(hipStreamSynchronize(g_cur));
+                AGH_HIP(hipFree(ws.ptr));
+            }
+        }
+        ws.ptr = fresh;
+        ws.bytes = want;
     }
-    *ptr = ws;
+    *ptr = ws.ptr;
     return AGH_OK;
 }
 
@@ -66,6 +111,45 @@ static hipEvent_t next_event() {
     hipEvent_t e = g_events[g_event_next];
     g_event_next = (g_event_next + 1) % kBranchEvents;
     return e;
+}
+
+// Later work on the main stream waits for everything issued so far on the branch stream.
+static int join_side() {
+    if (!g_side_dirty) return AGH_OK;
+    hipEvent_t e = next_event();
+    AGH_HIP(hipEventRecord(e, g_side));
+    AGH_HIP(hipStreamWaitEvent(g_stream, e, 0));
+    g_side_joined_seq = g_side_seq;
+    // inside a branch more work for the branch stream may follow: it stays dirty
+    g_side_dirty = g_cur == g_side;
+    return AGH_OK;
+}
+
+// The host waits for both streams.
+static int sync_all() {
+    AGH_HIP(hipStreamSynchronize(g_stream));
+    if (g_side_dirty) {
+        AGH_HIP(hipStreamSynchronize(g_side));
+        g_side_joined_seq = g_side_seq;
+        g_side_dirty = g_cur == g_side;
+    }
+    return AGH_OK;
+}
+
+// capacity classes: 256 B steps up to 4 KiB, then four classes per octave (waste < 25 %)
+static size_t block_capacity(size_t bytes) {
+    if (bytes <= 4096) return bytes ? (bytes + 255) & ~(size_t)255 : 256;
+    size_t top = (size_t)1 << (63 - __builtin_clzll((unsigned long long)bytes));
+    size_t step = top >> 2;
+    return (bytes + step - 1) & ~(step - 1);
+}
+
+static int release_cached_blocks() {
+    if (int rc = sync_all()) return rc;
+    for (auto &kv : g_free_blocks) AGH_HIP(hipFree(kv.second.ptr));
+    g_free_blocks.clear();
+    g_cached_bytes = 0;
+    return AGH_OK;
 }
 
 }  // namespace agh
@@ -97,6 +181,11 @@ int agh_init(int device_index) {
     for (int i = 0; i < kBranchEvents; ++i) AGH_HIP(hipEventCreateWithFlags(&g_events[i], hipEventDisableTiming));
     g_cur = g_stream;
     g_side_dirty = false;
+    g_capturing = false;
+    g_live_graphs = 0;
+    g_side_seq = g_side_joined_seq = 0;
+    if (const char *s = getenv("AGH_CACHE_LIMIT_MB"))
+        if (*s) g_cache_limit = (size_t)strtoull(s, nullptr, 10) << 20;
     g_device = device_index;
     g_init = true;
     return AGH_OK;
@@ -107,10 +196,16 @@ int agh_shutdown(void) {
     if (!g_init) return AGH_OK;
     AGH_HIP(hipStreamSynchronize(g_stream));
     AGH_HIP(hipStreamSynchronize(g_side));
-    if (g_ws) AGH_HIP(hipFree(g_ws));
-    if (g_ws_side) AGH_HIP(hipFree(g_ws_side));
-    g_ws = g_ws_side = nullptr;
-    g_ws_bytes = g_ws_side_bytes = 0;
+    g_side_dirty = false;
+    if (int rc = release_cached_blocks()) return rc;
+    // blocks the caller still holds stay valid (and keep their capacity on record is pointless once the
+    // library is down: a later agh_free after a new agh_init falls back to hipFree)
+    g_live_blocks.clear();
+    if (g_ws.ptr) AGH_HIP(hipFree(g_ws.ptr));
+    if (g_ws_side.ptr) AGH_HIP(hipFree(g_ws_side.ptr));
+    g_ws = Workspace();
+    g_ws_side = Workspace();
+    if (int rc = release_retired_workspaces()) return rc;
     for (int i = 0; i < kBranchEvents; ++i) (void)hipEventDestroy(g_events[i]);
     AGH_HIP(hipStreamDestroy(g_side));
     AGH_HIP(hipStreamDestroy(g_stream));
@@ -138,18 +233,80 @@ int agh_malloc(void **ptr, size_t bytes) {
     AGH_API_ENTER();
     if (!ptr) return fail(AGH_ENULL, "agh_malloc: null out pointer");
     *ptr = nullptr;
-    // zero-length tensors are legal in the reference; hand back a real 256-byte block
-    AGH_HIP(hipMalloc(ptr, bytes ? bytes : 256));
+    if (g_capturing) return fail(AGH_EINVAL, "agh_malloc: not allowed while capturing a graph");
+    // zero-length tensors are legal in the reference; they get a real 256-byte block
+    const size_t cap = block_capacity(bytes);
+    auto it = g_free_blocks.lower_bound(cap);
+    if (it != g_free_blocks.end() && it->first == cap) {
+        CachedBlock blk = it->second;
+        g_free_blocks.erase(it);
+        g_cached_bytes -= cap;
+        // last used by a branch the main stream has not waited for: wait now
+        if (g_cur == g_stream && blk.side_seq > g_side_joined_seq) {
+            if (int rc = join_side()) return rc;
+        }
+        g_live_blocks[blk.ptr] = cap;
+        *ptr = blk.ptr;
+        return AGH_OK;
+    }
+    void *fresh = nullptr;
+    hipError_t e = hipMalloc(&fresh, cap);
+    if (e == hipErrorOutOfMemory) {  // give the cache back to the driver and try once more
+        (void)hipGetLastError();
+        if (int rc = release_cached_blocks()) return rc;
+        e = hipMalloc(&fresh, cap);
+    }
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc");
+    g_live_blocks[fresh] = cap;
+    *ptr = fresh;
     return AGH_OK;
 }
 
 int agh_free(void *ptr) {
     AGH_API_ENTER();
     if (!ptr) return AGH_OK;
-    // the buffer may still be read by queued kernels
-    AGH_HIP(hipStreamSynchronize(g_stream));
-    if (g_side_dirty) AGH_HIP(hipStreamSynchronize(g_side));
-    AGH_HIP(hipFree(ptr));
+    if (g_capturing) return fail(AGH_EINVAL, "agh_free: not allowed while capturing a graph");
+    auto it = g_live_blocks.find(ptr);
+    if (it == g_live_blocks.end()) {
+        // not from this allocator's books (allocated before an agh_shutdown): hand it to the driver
+        if (int rc = sync_all()) return rc;
+        AGH_HIP(hipFree(ptr));
+        return AGH_OK;
+    }
+    const size_t cap = it->second;
+    g_live_blocks.erase(it);
+    if (g_cached_bytes + cap > g_cache_limit) {
+        if (int rc = release_cached_blocks()) return rc;  // waits for both streams
+        if (cap > g_cache_limit) {
+            AGH_HIP(hipFree(ptr));
+            return AGH_OK;
+        }
+    }
+    // No wait: kernels still queued on the main stream run before anything launched on the block later.
+    g_free_blocks.emplace(cap, CachedBlock{ptr, g_side_dirty ? g_side_seq : 0});
+    g_cached_bytes += cap;
+    return AGH_OK;
+}
+
+int agh_cache_release(void) {
+    AGH_API_ENTER();
+    if (g_capturing) return fail(AGH_EINVAL, "agh_cache_release: not allowed while capturing a graph");
+    if (int rc = release_cached_blocks()) return rc;  // waits for both streams
+    if (g_live_graphs == 0) {  // no captured node names the workspaces: they can go too
+        if (g_ws.ptr) AGH_HIP(hipFree(g_ws.ptr));
+        if (g_ws_side.ptr) AGH_HIP(hipFree(g_ws_side.ptr));
+        g_ws = Workspace();
+        g_ws_side = Workspace();
+        return release_retired_workspaces();
+    }
+    return AGH_OK;
+}
+
+int agh_cache_stats(size_t *cached_bytes, size_t *cached_blocks, size_t *live_blocks) {
+    AGH_API_ENTER();
+    if (cached_bytes) *cached_bytes = g_cached_bytes;
+    if (cached_blocks) *cached_blocks = g_free_blocks.size();
+    if (live_blocks) *live_blocks = g_live_blocks.size();
     return AGH_OK;
 }
 
@@ -157,7 +314,7 @@ int agh_memcpy_h2d(void *dst, const void *src, size_t bytes) {
     AGH_API_ENTER();
     if (bytes == 0) return AGH_OK;
     if (!dst || !src) return fail(AGH_ENULL, "agh_memcpy_h2d: null pointer");
-    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_cur));
     return AGH_OK;
 }
 
@@ -165,8 +322,15 @@ int agh_memcpy_d2h(void *dst, const void *src, size_t bytes) {
     AGH_API_ENTER();
     if (bytes == 0) return AGH_OK;
     if (!dst || !src) return fail(AGH_ENULL, "agh_memcpy_d2h: null pointer");
-    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
-    AGH_HIP(hipStreamSynchronize(g_stream));
+    if (g_capturing) return fail(AGH_EINVAL, "agh_memcpy_d2h: waits, not allowed while capturing (use agh_memcpy_d2h_async)");
+    // the bytes may come from a branch that has not been joined: on the main stream, wait for it first
+    if (g_cur == g_stream && g_side_dirty) {
+        AGH_HIP(hipStreamSynchronize(g_side));
+        g_side_joined_seq = g_side_seq;
+        g_side_dirty = false;
+    }
+    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_cur));
+    AGH_HIP(hipStreamSynchronize(g_cur));
     return AGH_OK;
 }
 
@@ -174,7 +338,7 @@ int agh_memcpy_d2d(void *dst, const void *src, size_t bytes) {
     AGH_API_ENTER();
     if (bytes == 0) return AGH_OK;
     if (!dst || !src) return fail(AGH_ENULL, "agh_memcpy_d2d: null pointer");
-    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
+    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_cur));
     return AGH_OK;
 }
 
@@ -182,7 +346,7 @@ int agh_memcpy_d2h_async(void *dst, const void *src, size_t bytes) {
     AGH_API_ENTER();
     if (bytes == 0) return AGH_OK;
     if (!dst || !src) return fail(AGH_ENULL, "agh_memcpy_d2h_async: null pointer");
-    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+    AGH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_cur));
     return AGH_OK;
 }
 
@@ -197,14 +361,19 @@ int agh_host_alloc(void **ptr, size_t bytes) {
 int agh_host_free(void *ptr) {
     AGH_API_ENTER();
     if (!ptr) return AGH_OK;
-    AGH_HIP(hipStreamSynchronize(g_stream));
+    if (int rc = sync_all()) return rc;
     AGH_HIP(hipHostFree(ptr));
     return AGH_OK;
 }
 
 int agh_graph_begin(void) {
     AGH_API_ENTER();
+    if (g_capturing) return fail(AGH_EINVAL, "agh_graph_begin: already capturing");
+    if (g_cur != g_stream) return fail(AGH_EINVAL, "agh_graph_begin: inside a branch");
+    // work left on the branch stream is not part of the graph: the capture starts from a joined state
+    if (int rc = join_side()) return rc;
     AGH_HIP(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal));
+    g_capturing = true;
     return AGH_OK;
 }
 
@@ -212,19 +381,23 @@ int agh_graph_end(void **graph_exec) {
     AGH_API_ENTER();
     if (!graph_exec) return fail(AGH_ENULL, "agh_graph_end: null out pointer");
     *graph_exec = nullptr;
+    if (!g_capturing) return fail(AGH_EINVAL, "agh_graph_end: no capture in progress");
     hipGraph_t graph = nullptr;
     if (g_cur != g_stream) return fail(AGH_EINVAL, "agh_graph_end: still inside a branch");
-    if (g_side_dirty) {  // an arm left open would make the capture invalid
-        hipEvent_t e = next_event();
-        AGH_HIP(hipEventRecord(e, g_side));
-        AGH_HIP(hipStreamWaitEvent(g_stream, e, 0));
-        g_side_dirty = false;
+    // an arm left open would make the capture invalid
+    if (int rc = join_side()) {
+        g_capturing = false;
+        (void)hipStreamEndCapture(g_stream, &graph);
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
     }
+    g_capturing = false;
     AGH_HIP(hipStreamEndCapture(g_stream, &graph));
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
     if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    ++g_live_graphs;
     *graph_exec = (void *)exec;
     return AGH_OK;
 }
@@ -239,19 +412,16 @@ int agh_graph_launch(void *graph_exec) {
 int agh_graph_destroy(void *graph_exec) {
     AGH_API_ENTER();
     if (!graph_exec) return AGH_OK;
-    AGH_HIP(hipStreamSynchronize(g_stream));
+    if (int rc = sync_all()) return rc;
     AGH_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    if (g_live_graphs > 0 && --g_live_graphs == 0) return release_retired_workspaces();
     return AGH_OK;
 }
 
 int agh_sync(void) {
     AGH_API_ENTER();
-    AGH_HIP(hipStreamSynchronize(g_stream));
-    if (g_side_dirty) {
-        AGH_HIP(hipStreamSynchronize(g_side));
-        g_side_dirty = false;
-    }
-    return AGH_OK;
+    if (g_capturing) return fail(AGH_EINVAL, "agh_sync: not allowed while capturing a graph");
+    return sync_all();
 }
 
 int agh_branch_begin(void) {
@@ -262,6 +432,7 @@ int agh_branch_begin(void) {
     AGH_HIP(hipStreamWaitEvent(g_side, e, 0));
     g_cur = g_side;
     g_side_dirty = true;
+    ++g_side_seq;
     return AGH_OK;
 }
 
@@ -275,12 +446,7 @@ int agh_branch_end(void) {
 int agh_branch_join(void) {
     AGH_API_ENTER();
     if (g_cur != g_stream) return fail(AGH_EINVAL, "agh_branch_join: still inside a branch");
-    if (!g_side_dirty) return AGH_OK;
-    hipEvent_t e = next_event();
-    AGH_HIP(hipEventRecord(e, g_side));
-    AGH_HIP(hipStreamWaitEvent(g_stream, e, 0));
-    g_side_dirty = false;
-    return AGH_OK;
+    return join_side();
 }
 
 void *agh_stream(void) { return (void *)g_stream; }

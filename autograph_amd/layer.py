@@ -46,8 +46,11 @@ def conv2_direct_forward(x, weight, padding=(0, 0), stride=(1, 1), dilation=(1, 
     oh, ow = opts.output_shape((ih, iw))
     yshape = (bs, oc, oh // 2, ow // 2) if pool2x2 else (bs, oc, oh, ow)
     y = Tensor.uninit(yshape, x.dtype)
+    # standard-layout copies of strided views are bound to names: they must outlive the launch call
+    w = weight.as_standard_layout()
+    b = bias.as_standard_layout() if bias is not None else None
     check(getattr(lib, f"agh_conv2_direct_{x.dtype}")(
-        x._data_ptr(), weight.as_standard_layout()._data_ptr(), bias._data_ptr() if bias is not None else None,
+        x._data_ptr(), w._data_ptr(), b._data_ptr() if b is not None else None,
         y._ptr(), bs, ic, ih, iw, oc, fh, fw, *padding, *stride, *dilation, 1 if relu else 0, 1 if pool2x2 else 0))
     return y
 
@@ -151,10 +154,10 @@ class LeNet5:
         if out_ptr is None:
             out = Tensor.uninit((bs, 10), x.dtype)
             out_ptr = out._ptr()
-        ws = [self.conv1.weight, self.conv2.weight, self.dense1.weight, self.dense2.weight, self.dense3.weight,
-              self.dense3.bias]
-        check(getattr(lib, f"agh_lenet5_forward_{x.dtype}")(x._data_ptr(), *[w.as_standard_layout()._data_ptr() for w in ws],
-                                                           out_ptr, bs))
+        # standard-layout copies of strided views stay referenced by `ws` until the launch call has returned
+        ws = [w.as_standard_layout() for w in (self.conv1.weight, self.conv2.weight, self.dense1.weight, self.dense2.weight,
+                                               self.dense3.weight, self.dense3.bias)]
+        check(getattr(lib, f"agh_lenet5_forward_{x.dtype}")(x._data_ptr(), *[w._data_ptr() for w in ws], out_ptr, bs))
         return out
 
     # -- graph-captured inference on fixed buffers --
@@ -183,6 +186,9 @@ class LeNet5:
         p1, p2, d1, d2, out = self._bufs
         dt = x.dtype
         bs = x.shape[0]
+        for t in (x, self.conv1.weight, self.conv2.weight):
+            if not t.is_standard_layout():  # raw pointers below: a captured graph cannot own a copy
+                raise AghError(-1, "LeNet5.capture: input and convolution weights must be in standard layout")
         conv = getattr(lib, f"agh_conv2_direct_{dt}")
         gemm = getattr(lib, f"agh_gemm_{dt}_bias_act")
         check(conv(x._data_ptr(), self.conv1.weight._data_ptr(), None, p1._ptr(), bs, 1, 28, 28, 6, 5, 5, 0, 0, 1, 1, 1, 1, 1, 1))
@@ -236,6 +242,8 @@ class LeNet5Trainer:
         self.opt = optimizer if optimizer is not None else SGD()
         bs, dt = batch_size, model.conv1.weight.dtype
         self.dt = dt
+        # `step` passes raw pointers of the input; the parameters are copied into one flat buffer below
+        # (through standard-layout copies), so strided parameter views are fine, a strided x is not
         u = lambda *shape: Tensor.uninit(shape, dt)  # noqa: E731
         self.cols1, self.c1, self.p1 = u(bs * 576, 25), u(bs, 6, 24, 24), u(bs, 6, 12, 12)
         self.cols2, self.c2, self.p2 = u(bs * 64, 150), u(bs, 16, 8, 8), u(bs, 16, 4, 4)
@@ -324,6 +332,8 @@ class LeNet5Trainer:
         """x: [bs,1,28,28] tensor, target: device `Buffer` of bs u8 labels.  The loss lands in pinned
         host memory (`loss()` after a sync)."""
         bs = self.bs
+        if not x.is_standard_layout() or x.shape != (bs, 1, 28, 28):
+            raise AghError(-1, f"LeNet5Trainer.step: x must be a standard-layout [{bs},1,28,28] tensor")
         w1, w2, wd1, wd2, wd3, b3 = self.params
         dw1, dw2, dwd1, dwd2, dwd3, db3 = self.grads
         # forward

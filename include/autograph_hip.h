@@ -55,13 +55,30 @@ const char *agh_last_error_string(void);
 /* Name, compute-unit count and memory size of the active device (krnl DeviceInfo). */
 int agh_device_info(char *name, size_t name_len, int *compute_units, size_t *total_mem_bytes);
 
-/* Buffer allocation: Tensor::uninit (src/tensor.rs:1377-1389) -> hipMalloc. */
+/* Buffer allocation: Tensor::uninit (src/tensor.rs:1377-1389), one per op output in the reference
+ * (src/tensor/linalg.rs:412-419, src/tensor/ops.rs:855-878).  Served by a caching allocator: agh_free
+ * does not wait and does not return the block to the driver, it keeps it (by size class: at most 25 %
+ * larger than asked) for the next agh_malloc.  Reuse is safe because all work is issued in order: a
+ * block freed while kernels that use it are still queued is only touched by work launched after them
+ * (a block last used inside an unjoined branch makes the main stream wait for the branch stream when
+ * it is handed out again).  Cached blocks go back to the driver at agh_shutdown, at
+ * agh_cache_release, when the driver runs out of memory, or when the cache exceeds its limit
+ * (64 GiB, or AGH_CACHE_LIMIT_MB at agh_init). */
 int agh_malloc(void **ptr, size_t bytes);
 int agh_free(void *ptr);
-/* into_device / to_device (src/tensor.rs:1775-1833): host -> device, enqueued on the stream.
+/* Waits for all queued work and returns every cached block to the driver, and the library's own
+ * workspace too unless a graph from agh_graph_end is still alive.  The reference has no counterpart
+ * (krnl frees a buffer when it is dropped). */
+int agh_cache_release(void);
+/* Bytes and blocks held for reuse, blocks currently handed out (any pointer may be null). */
+int agh_cache_stats(size_t *cached_bytes, size_t *cached_blocks, size_t *live_blocks);
+/* into_device / to_device (src/tensor.rs:1775-1833): host -> device, enqueued on the current stream
+ * (the branch stream inside a branch, like every launch).
  * The host range must stay valid until the next agh_sync unless it is pageable memory. */
 int agh_memcpy_h2d(void *dst, const void *src, size_t bytes);
-/* into_array / into_vec (src/tensor.rs:1923-1934): blocks until the bytes are on the host. */
+/* into_array / into_vec (src/tensor.rs:1923-1934): blocks until the bytes are on the host.  Issued
+ * on the current stream; outside a branch it first waits for branches that have not been joined, so
+ * data produced there are complete. */
 int agh_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int agh_memcpy_d2d(void *dst, const void *src, size_t bytes);
 /* Tensor::zeros / fill for byte patterns (src/tensor.rs:1394-1416). */
@@ -80,8 +97,12 @@ void *agh_stream(void);
  * and replayed as one hipGraph: between agh_graph_begin and agh_graph_end every launch entry
  * point and agh_memcpy_d2h_async is captured instead of executed.  No entry point that
  * allocates, frees or waits (agh_malloc, agh_free, agh_sync, agh_memcpy_d2h, a first split-K
- * GEMM that has to grow the workspace) may be called while capturing: run the sequence once
- * eagerly first.  The reference has no counterpart (krnl dispatches kernel by kernel). */
+ * GEMM that has to grow the workspace) may be called while capturing (they return an error): run the
+ * sequence once eagerly first.  The library's workspace (split-K partials, reordered filter banks) is
+ * named by the captured nodes: while any graph from agh_graph_end is alive, a workspace block that
+ * has to grow is retired, not freed, so replays stay valid after larger eager calls; retired blocks
+ * are released when the last graph is destroyed or at agh_shutdown.
+ * The reference has no counterpart (krnl dispatches kernel by kernel). */
 int agh_graph_begin(void);
 int agh_graph_end(void **graph_exec);
 int agh_graph_launch(void *graph_exec);
@@ -90,7 +111,8 @@ int agh_graph_destroy(void *graph_exec);
 /* Independent work.  Everything issued between agh_branch_begin and agh_branch_end goes to a second
  * in-order stream: it starts after all work issued before the begin, and runs concurrently with what
  * the caller issues after the end.  agh_branch_join makes all later work wait for every branch issued
- * so far; agh_sync waits for both streams.  Several begin/end pairs may precede one join (their work
+ * so far; agh_sync waits for both streams (inside a branch too: work issued after it still goes to the
+ * second stream and is still joined).  Several begin/end pairs may precede one join (their work
  * runs in order among itself).  The CALLER guarantees that a branch and the work issued between its
  * end and the join touch disjoint outputs (e.g. the weight gradient and the input gradient of one
  * layer, autograd.rs:607-627: two `dot` calls on the same `output_grad`).  Works under graph capture:

@@ -1,7 +1,8 @@
 //! Raw bindings to `libautograph_hip.so` (the C ABI of `include/autograph_hip.h`), one declaration
 //! per entry point, in header order.  Status codes: 0 ok, negative argument errors (`AGH_E*`),
 //! positive `hipError_t`.  This crate is source only: it has not been compiled (the image it was
-//! written in has no Rust toolchain); `tests/test_abi_cpu.py` checks it against the header.
+//! written in has no Rust toolchain); `gen_bindings.py` writes this file from the header and
+//! `tests/test_abi_cpu.py` checks every argument type against the header.
 #![allow(non_camel_case_types)]
 
 use std::os::raw::{c_char, c_int, c_void};
@@ -22,6 +23,8 @@ extern "C" {
     pub fn agh_device_info(name: *mut c_char, name_len: usize, compute_units: *mut c_int, total_mem_bytes: *mut usize) -> c_int;
     pub fn agh_malloc(ptr: *mut *mut c_void, bytes: usize) -> c_int;
     pub fn agh_free(ptr: *mut c_void) -> c_int;
+    pub fn agh_cache_release() -> c_int;
+    pub fn agh_cache_stats(cached_bytes: *mut usize, cached_blocks: *mut usize, live_blocks: *mut usize) -> c_int;
     pub fn agh_memcpy_h2d(dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     pub fn agh_memcpy_d2h(dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     pub fn agh_memcpy_d2d(dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
@@ -31,13 +34,13 @@ extern "C" {
     pub fn agh_host_free(ptr: *mut c_void) -> c_int;
     pub fn agh_sync() -> c_int;
     pub fn agh_stream() -> *mut c_void;
-    pub fn agh_branch_begin() -> c_int;
-    pub fn agh_branch_end() -> c_int;
-    pub fn agh_branch_join() -> c_int;
     pub fn agh_graph_begin() -> c_int;
     pub fn agh_graph_end(graph_exec: *mut *mut c_void) -> c_int;
     pub fn agh_graph_launch(graph_exec: *mut c_void) -> c_int;
     pub fn agh_graph_destroy(graph_exec: *mut c_void) -> c_int;
+    pub fn agh_branch_begin() -> c_int;
+    pub fn agh_branch_end() -> c_int;
+    pub fn agh_branch_join() -> c_int;
     pub fn agh_event_create(event: *mut *mut c_void) -> c_int;
     pub fn agh_event_destroy(event: *mut c_void) -> c_int;
     pub fn agh_event_record(event: *mut c_void) -> c_int;
@@ -52,6 +55,8 @@ extern "C" {
     pub fn agh_im2col_conv2_bf16(x: *const c_void, y: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
     pub fn agh_col2im_conv2_f32(x: *const c_void, y: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
     pub fn agh_col2im_conv2_bf16(x: *const c_void, y: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
+    pub fn agh_conv2_backward_input_f32(dy: *const c_void, w: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
+    pub fn agh_conv2_backward_input_bf16(dy: *const c_void, w: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
     pub fn agh_conv2_direct_f32(x: *const c_void, w: *const c_void, bias: *const c_void, y: *mut c_void, bs: i64, ic: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64, act: c_int, pool2x2: c_int) -> c_int;
     pub fn agh_conv2_direct_bf16(x: *const c_void, w: *const c_void, bias: *const c_void, y: *mut c_void, bs: i64, ic: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64, act: c_int, pool2x2: c_int) -> c_int;
     pub fn agh_lenet5_forward_f32(x: *const c_void, w1: *const c_void, w2: *const c_void, wd1: *const c_void, wd2: *const c_void, wd3: *const c_void, b3: *const c_void, logits: *mut c_void, bs: i64) -> c_int;
@@ -60,14 +65,12 @@ extern "C" {
     pub fn agh_max_pool2_bf16(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_max_pool2_backward_f32(dx_inout: *mut c_void, dy: *const c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_max_pool2_backward_bf16(dx_inout: *mut c_void, dy: *const c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
-    pub fn agh_relu_f32(x: *const c_void, y: *mut c_void, n: i64) -> c_int;
-    pub fn agh_relu_bf16(x: *const c_void, y: *mut c_void, n: i64) -> c_int;
-    pub fn agh_conv2_backward_input_f32(dy: *const c_void, w: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
-    pub fn agh_conv2_backward_input_bf16(dy: *const c_void, w: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64) -> c_int;
     pub fn agh_relu_max_pool2_f32(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_relu_max_pool2_bf16(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_max_pool2_relu_backward_f32(x: *const c_void, dy: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64, nhwc: c_int) -> c_int;
     pub fn agh_max_pool2_relu_backward_bf16(x: *const c_void, dy: *const c_void, dx: *mut c_void, bs: i64, c: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64, nhwc: c_int) -> c_int;
+    pub fn agh_relu_f32(x: *const c_void, y: *mut c_void, n: i64) -> c_int;
+    pub fn agh_relu_bf16(x: *const c_void, y: *mut c_void, n: i64) -> c_int;
     pub fn agh_relu_backward_f32(x: *const c_void, dy: *const c_void, dx: *mut c_void, n: i64) -> c_int;
     pub fn agh_relu_backward_bf16(x: *const c_void, dy: *const c_void, dx: *mut c_void, n: i64) -> c_int;
     pub fn agh_assign_f32(x: *const c_void, off_x: i64, sx0: i64, sx1: i64, sx2: i64, sx3: i64, y: *mut c_void, off_y: i64, sy0: i64, sy1: i64, sy2: i64, sy3: i64, d0: i64, d1: i64, d2: i64, d3: i64) -> c_int;

@@ -45,14 +45,51 @@ def test_option_shape_formulas():
     assert MaxPool2Options((2, 3), (2, 2)).output_shape((9, 8)) == (orc.pool_out(9, 2, 2), orc.pool_out(8, 3, 2))
 
 
+_C_TO_RUST = {"int": "c_int", "int64_t": "i64", "float": "f32", "size_t": "usize", "char": "c_char", "void": "c_void"}
+
+
+def _rust_type_of(ctype):
+    """The Rust FFI spelling of a C parameter type: pointers keep their depth and the constness of the pointee."""
+    const = re.search(r"\bconst\b", ctype) is not None
+    base = re.sub(r"\bconst\b|\*", " ", ctype).split()
+    assert len(base) == 1, ctype
+    out = _C_TO_RUST[base[0]]
+    for level in range(ctype.count("*")):
+        out = ("*const " if const and level == 0 else "*mut ") + out
+    return out
+
+
 def test_rust_sys_crate_declares_the_header():
     """rust/autograph-hip-sys/src/lib.rs (source only, no Rust toolchain here) must declare every entry
-    point of the header with the same number of arguments."""
+    point of the header with the same argument TYPES in the same order (int64_t <-> i64, int <-> c_int,
+    float <-> f32, size_t <-> usize, pointers with their constness and depth) and the same return type."""
     text = open(os.path.join(ROOT, "include", "autograph_hip.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    c_decls = {n: (0 if a.strip() in ("", "void") else a.count(",") + 1)
-               for n, a in re.findall(r"\b(agh_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text)}
+    c_decls = {}
+    for ret, name, args in re.findall(r"^\s*([a-z_0-9 ]+?\s*\**)\s*\b(agh_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text, flags=re.M):
+        types = []
+        if args.strip() not in ("", "void"):
+            for a in args.split(","):
+                a = " ".join(a.split())
+                types.append(_rust_type_of(re.sub(r"[A-Za-z_][A-Za-z_0-9]*$", "", a)))  # drop the parameter name
+        c_decls[name] = (types, _rust_type_of(ret))
     rs = open(os.path.join(ROOT, "rust", "autograph-hip-sys", "src", "lib.rs")).read()
-    rs_decls = {n: (0 if not a.strip() else a.count(",") + 1) for n, a in re.findall(r"pub fn (agh_[a-z0-9_]+)\(([^)]*)\)", rs)}
-    assert rs_decls == c_decls
+    rs_decls = {}
+    for name, args, ret in re.findall(r"pub fn (agh_[a-z0-9_]+)\(([^)]*)\) -> ([^;]+);", rs):
+        types = [a.split(":", 1)[1].strip() for a in args.split(",")] if args.strip() else []
+        rs_decls[name] = (types, ret.strip())
+    assert sorted(rs_decls) == sorted(c_decls)
+    for name in c_decls:
+        assert rs_decls[name] == c_decls[name], name
     assert sorted(c_decls) == header_symbols()
+    # the ctypes table agrees too (same width and kind per argument)
+    from autograph_amd import _ffi
+    kind = {"c_int": C.c_int, "i64": C.c_int64, "f32": C.c_float, "usize": C.c_size_t}
+    for name, (types, _) in c_decls.items():
+        argtypes = _ffi.SIGNATURES[name][0]
+        assert len(argtypes) == len(types), name
+        for t, ct in zip(types, argtypes):
+            if t.startswith("*"):
+                assert C.sizeof(ct) == C.sizeof(C.c_void_p) and not issubclass(ct, (C.c_int64, C.c_size_t, C.c_float)) or ct is C.c_void_p, (name, t, ct)
+            else:
+                assert ct is kind[t] or (C.sizeof(ct) == C.sizeof(kind[t]) and ct._type_ == kind[t]._type_), (name, t, ct)

@@ -205,6 +205,70 @@ def test_conv2_direct_f32_matrix_core_path(ag, case):
     assert np.array_equal(yi, orc.conv2_naive_f64(xi, wi, p, (1, 1), (1, 1)).astype(np.float32))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_conv2_forward_config3_full_size(ag, dtype):
+    """Conv2 forward of the benchmark list at full size (layer.rs:950-1005): batch 256, 64 -> 128 channels, 56x56,
+    3x3, stride 1, pad 1, both algorithms (im2col + the 802816 x 576 x 128 GEMM, and the implicit GEMM with its
+    3328 tiles walked XCD by XCD).  The oracle's naive f64 convolution is run on the 3x3 windows of sampled
+    output positions (all 128 channels each): the four borders and corners of images, the first and last
+    position of every tile of images that begin or end an XCD's run of tiles, and random ones.  The fused
+    bias + ReLU launch equals the separate ops on the same result bit for bit."""
+    bs, ic, ih, iw, oc = 256, 64, 56, 56, 128
+    rng = np.random.default_rng(29)
+    x = to_dtype(rng.standard_normal((bs, ic, ih, iw), dtype=np.float32), dtype)
+    w = to_dtype((rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9))).astype(np.float32), dtype)
+    b = to_dtype((rng.standard_normal(oc) * 0.1).astype(np.float32), dtype)
+    xf, wf = as_f32(x), as_f32(w)
+    # sampled (image, row, column)
+    pts = []
+    edge_imgs = [0, 1, 31, 32, 63, 64, 127, 128, 191, 192, 223, 224, 254, 255]
+    for img in edge_imgs:
+        for pos in sorted({0, 55, 56, 3080, 3135} | {t * 256 for t in range(13)} | {t * 256 - 1 for t in range(1, 13)}):
+            pts.append((img, pos // iw, pos % iw))
+    for img in (0, 100, 255):
+        for r, c in ((0, 17), (55, 30), (23, 0), (40, 55), (0, 0), (0, 55), (55, 0), (55, 55)):
+            pts.append((img, r, c))
+    for _ in range(600):
+        pts.append((int(rng.integers(bs)), int(rng.integers(ih)), int(rng.integers(iw))))
+    pts = np.array(pts)
+    want = np.empty((len(pts), oc))
+    scale = np.empty((len(pts), oc))
+    pad = {}
+    for n_, (img, r, c) in enumerate(pts):
+        if img not in pad:
+            pad[img] = np.pad(xf[img], ((0, 0), (1, 1), (1, 1)))
+        win = np.ascontiguousarray(pad[img][None, :, r:r + 3, c:c + 3])
+        want[n_] = orc.conv2_naive_f64(win, wf, (0, 0), (1, 1), (1, 1))[0, :, 0, 0]
+        scale[n_] = orc.conv2_naive_f64(np.abs(win), np.abs(wf), (0, 0), (1, 1), (1, 1))[0, :, 0, 0]
+    k = ic * 9
+    tx, tw, tb = ag.Tensor.from_array(x), ag.Tensor.from_array(w), ag.Tensor.from_array(b)
+    results = {}
+    for alg in ("im2col", "direct"):
+        fn = ag.conv2_im2col_forward if alg == "im2col" else ag.conv2_direct_forward
+        y = fn(tx, tw, padding=(1, 1)).into_array()
+        assert y.shape == (bs, oc, ih, iw)
+        got = as_f32(np.ascontiguousarray(y[pts[:, 0], :, pts[:, 1], pts[:, 2]])).astype(np.float64)
+        if dtype == "f32":
+            assert np.all(np.abs(got - want) <= 1e-5 * np.sqrt(k) * scale), alg
+        else:
+            ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0**-126))) - 7)
+            assert np.all(np.abs(got - want) <= ulp + 1e-2 * np.abs(want) + 8 * np.sqrt(k) * 2.0**-24 * scale), alg
+        # nothing left unwritten: every output was produced by this launch
+        assert np.isfinite(as_f32(y[::37].reshape(-1))).all()
+        # bias + relu epilogue against the separate ops on this very result, on whole images
+        yb = fn(tx, tw, padding=(1, 1), bias=tb, relu=True).into_array()
+        for img in (0, 31, 32, 140, 255):
+            flat = np.ascontiguousarray(y[img].reshape(oc, -1).T)
+            ref = orc.relu(orc.bias_add_rows(flat, b)).T.reshape(oc, ih, iw)
+            assert np.array_equal(yb[img], ref), (alg, img)
+        results[alg] = y
+        del yb
+    # the two algorithms add the same products in different orders
+    a_, d_ = as_f32(results["im2col"][::16]).astype(np.float64), as_f32(results["direct"][::16]).astype(np.float64)
+    tol = (2e-5 * np.sqrt(k) if dtype == "f32" else 2.0**-6) * np.maximum(np.abs(a_), 1.0)
+    assert np.all(np.abs(a_ - d_) <= tol)
+
+
 def he(rng, shape, fan_in):  # Uniform(-a, a), a = sqrt(2/fan_in): layer.rs:345-349, :463-467
     a = np.sqrt(2.0 / fan_in)
     return rng.uniform(-a, a, shape).astype(np.float32)

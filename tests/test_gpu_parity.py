@@ -308,6 +308,69 @@ def test_gemm_full_size_sampled_entries_and_identity(ag, dtype, shape):
     assert np.array_equal(out[:, :min(k, n)], a[:, :min(k, n)])
 
 
+def test_gemm_f32_1024_cubed_all_layouts(ag):
+    """The smallest standalone f32 GEMM of the benchmark list, M = N = K = 1024 (the one square shape on which
+    the tile chooser leaves the 256x256 tile): every entry against the f64 product, all four operand layouts."""
+    rng = np.random.default_rng(27)
+    a = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    b = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    ta, tb = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+    assert_f32_gemm_close(ta.dot(tb).into_array(), a, b)
+    assert_f32_gemm_close(ta.t().dot(tb).into_array(), a.T, b)
+    assert_f32_gemm_close(ta.dot(tb.t()).into_array(), a, b.T)
+    assert_f32_gemm_close(ta.t().dot(tb.t()).into_array(), a.T, b.T)
+    eye = ag.Tensor.from_array(np.eye(1024, dtype=np.float32))
+    assert np.array_equal(ta.dot(eye).into_array(), a)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_dense_full_size_bias_relu(ag, dtype):
+    """The Dense-shaped GEMM of the benchmark list at full size: M = 16384 (batch), K = 4096, N = 4096 with the
+    fused bias + ReLU epilogue (layer.rs:1134-1143, :1254-1267).  4096 sampled entries against f64 dot + bias
+    + relu for the fused launch and for its bias-only and relu-only forms; the three are consistent with the
+    plain product bit for bit (epilogue = the separate ops on the rounded dot); A*I through the same epilogue
+    is relu(a + bias) exactly."""
+    m, k, n = 16384, 4096, 4096
+    rng = np.random.default_rng(28)
+    a = to_dtype(rng.normal(0, 0.02, (m, k)).astype(np.float32), dtype)
+    b = to_dtype(rng.normal(0, 0.02, (k, n)).astype(np.float32), dtype)
+    bias = to_dtype(rng.normal(0, 0.02, (n,)).astype(np.float32), dtype)
+    ta, tb, tbias = ag.Tensor.from_array(a), ag.Tensor.from_array(b), ag.Tensor.from_array(bias)
+    ii, jj = rng.integers(0, m, 4096), rng.integers(0, n, 4096)
+    ii[:8], jj[:8] = [0, 0, m - 1, m - 1, 255, 256, 8191, 8192], [0, n - 1, 0, n - 1, 255, 256, 2047, 2048]
+    af, bf, biasf = as_f32(a), as_f32(b), as_f32(bias).astype(np.float64)
+    dot64 = np.einsum("ik,ki->i", af[ii].astype(np.float64), bf[:, jj].astype(np.float64))
+    scale = np.einsum("ik,ki->i", np.abs(af[ii]).astype(np.float64), np.abs(bf[:, jj]).astype(np.float64))
+
+    def close(got, want):
+        got = as_f32(np.ascontiguousarray(got)).astype(np.float64)
+        if dtype == "f32":
+            assert np.all(np.abs(got - want) <= 1e-5 * np.sqrt(k) * (scale + np.abs(biasf[jj])))
+        else:  # two roundings, T(dot) then T(bias + .): a bf16 step of the dot and one of the result
+            assert np.all(np.abs(got - want) <= bf16_ulp(dot64) + bf16_ulp(want) + 1e-2 * np.abs(want) +
+                          8 * np.sqrt(k) * 2.0**-24 * scale)
+
+    plain = ta.dot(tb).into_array()
+    close(plain[ii, jj], dot64)
+    fused = ta.dot(tb, bias=tbias, relu=True).into_array()
+    close(fused[ii, jj], np.maximum(dot64 + biasf[jj], 0))
+    assert (fused.view(np.uint32 if dtype == "f32" else np.uint16) == 0).mean() > 0.3  # the relu did cut
+    # the epilogue is the separate ops applied to the rounded product: bit for bit on whole row blocks
+    rows = np.r_[0:256, 8064:8320, m - 256:m]
+    assert np.array_equal(fused[rows], orc.relu(orc.bias_add_rows(np.ascontiguousarray(plain[rows]), bias)))
+    only_bias = ta.dot(tb, bias=tbias).into_array()
+    assert np.array_equal(only_bias[rows], orc.bias_add_rows(np.ascontiguousarray(plain[rows]), bias))
+    close(only_bias[ii, jj], dot64 + biasf[jj])
+    del only_bias
+    only_relu = ta.dot(tb, relu=True).into_array()
+    assert np.array_equal(only_relu[rows], orc.relu(np.ascontiguousarray(plain[rows])))
+    del only_relu, plain, fused
+    # A * I + bias, relu: exact products, so the result is relu(T(a + bias)) for every entry
+    eye = ag.Tensor.from_array(to_dtype(np.eye(k, n, dtype=np.float32), dtype))
+    out = ta.dot(eye, bias=tbias, relu=True).into_array()
+    assert np.array_equal(out, orc.relu(orc.bias_add_rows(a, bias)))
+
+
 # ------------------------------------------------------------- im2col / col2im ----
 # col2im has a streaming (ring) form for large patch matrices and a gathering form for small ones; the
 # library picks by size, AGH_COL2IM_RING forces either, and the small reference cases must pass on both

@@ -1,0 +1,195 @@
+"""The runtime half of the C ABI on a real MI355X: the caching allocator behind agh_malloc / agh_free
+(the reference allocates one output per op, src/tensor.rs:1377-1389), the library's workspace under live
+graphs, and the branch stream's bookkeeping around waits and copies."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ag():
+    import autograph_amd as ag
+    ag.Device(0)
+    return ag
+
+
+def cache_stats(ag):
+    a, b, c = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    ag._ffi.check(ag.lib.agh_cache_stats(C.byref(a), C.byref(b), C.byref(c)))
+    return a.value, b.value, c.value
+
+
+def test_malloc_free_reuses_blocks_in_stream_order(ag):
+    """alloc -> launch -> free -> alloc -> launch: the second allocation gets the first one's block back while
+    the first launch may still be queued, and every result equals the one computed on fresh memory."""
+    rng = np.random.default_rng(31)
+    a = rng.uniform(-1, 1, (512, 384)).astype(np.float32)
+    b = rng.uniform(-1, 1, (384, 256)).astype(np.float32)
+    ta, tb = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+    first = ta.dot(tb)
+    want = first.into_array()
+    ptr0 = first.buffer.ptr
+    del first
+    _, blocks, live = cache_stats(ag)
+    assert blocks >= 1
+    ptrs = set()
+    for _ in range(20):  # no wait between the iterations: free and reuse race only with queued work
+        out = ta.dot(tb)
+        ptrs.add(out.buffer.ptr)
+        del out
+    # every allocation was served from the cache: the driver was not asked for a single new block
+    assert cache_stats(ag)[1:] == (blocks, live)
+    assert len(ptrs) <= blocks and (blocks > 1 or ptrs == {ptr0})
+    out = ta.dot(tb)
+    assert np.array_equal(out.into_array(), want)
+    # a chain whose intermediates are dropped as soon as the next op is queued (what `Tensor::dot(..)?.relu()` does)
+    x = ta
+    for _ in range(4):
+        x = x.dot(tb).relu().dot(tb.t())
+    got = x.into_array()
+    h = a
+    for _ in range(4):
+        h = np.maximum(h @ b, 0) @ b.T
+    assert np.allclose(got, h, rtol=2e-3, atol=2e-3 * np.abs(h).max())
+
+
+def test_free_of_a_buffer_a_queued_kernel_still_reads(ag):
+    """agh_free returns at once; a kernel queued before it still reads the right bytes even though the block
+    is handed out again and overwritten by a later upload (which is ordered after the kernel)."""
+    rng = np.random.default_rng(32)
+    n = 2048
+    a = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    ta = ag.Tensor.from_array(a)
+    ident = ag.Tensor.from_array(np.eye(n, dtype=np.float32))
+    outs = []
+    for i in range(6):
+        src = ag.Tensor.from_array(a + np.float32(i))      # upload i
+        outs.append(src.dot(ident))                          # queued GEMM reads `src`
+        del src                                              # freed while the GEMM may not have started
+    for i, o in enumerate(outs):
+        assert np.array_equal(o.into_array(), a + np.float32(i)), i
+    del ta
+
+
+def test_cache_release_and_stats(ag):
+    t = ag.Tensor.zeros((1 << 20,), "f32")
+    del t
+    cached, blocks, _ = cache_stats(ag)
+    assert cached >= 4 << 20 and blocks >= 1
+    ag._ffi.check(ag.lib.agh_cache_release())
+    assert cache_stats(ag)[:2] == (0, 0)
+    # zero-length and odd sizes still work
+    p = C.c_void_p()
+    ag._ffi.check(ag.lib.agh_malloc(C.byref(p), 0))
+    assert p.value
+    ag._ffi.check(ag.lib.agh_free(p))
+    ag._ffi.check(ag.lib.agh_free(None))
+
+
+def test_graph_replay_survives_workspace_growth(ag, monkeypatch):
+    """A captured split-K GEMM names the library's workspace in its nodes.  A much larger split-K GEMM run
+    eagerly afterwards needs a bigger workspace: the old block must stay alive for the graph's replays."""
+    rng = np.random.default_rng(33)
+    ag._ffi.check(ag.lib.agh_cache_release())   # earlier tests may have grown the workspace: start from none
+    m, k, n = 6, 57600, 25                      # dW of LeNet5's first convolution: 256 k-groups
+    dy = rng.normal(0, 1, (k, m)).astype(np.float32)
+    cols = rng.normal(0, 1, (k, n)).astype(np.float32)
+    tdy, tcols = ag.Tensor.from_array(dy), ag.Tensor.from_array(cols)
+    out = ag.Tensor.uninit((m, n), "f32")
+    ag.gemm(1.0, tdy.t(), tcols, 0.0, out)      # eager: sizes the workspace
+    want = out.into_array()
+    ag._ffi.check(ag.lib.agh_graph_begin())
+    try:
+        ag.gemm(1.0, tdy.t(), tcols, 0.0, out)
+    finally:
+        g = C.c_void_p()
+        ag._ffi.check(ag.lib.agh_graph_end(C.byref(g)))
+    try:
+        # 16 k-groups x 512 x 512 f32 partials = 16 MiB > the 8 MiB first block
+        big_a = ag.Tensor.from_array(rng.uniform(-1, 1, (512, 2048)).astype(np.float32))
+        big_b = ag.Tensor.from_array(rng.uniform(-1, 1, (2048, 512)).astype(np.float32))
+        big = big_a.dot(big_b)
+        for _ in range(3):
+            ag._ffi.check(ag.lib.agh_memset(out._ptr(), 0xFF, m * n * 4))
+            ag._ffi.check(ag.lib.agh_graph_launch(g))
+            # the large GEMM again, between replays: it now owns the new workspace
+            big2 = big_a.dot(big_b)
+            assert np.array_equal(out.into_array(), want)
+            assert np.array_equal(big2.into_array(), big.into_array())
+        # growth is refused while capturing (nothing may allocate or wait inside a capture)
+        # (allocated before the capture starts; 32 k-groups forced: 128 MiB of partials)
+        huge_a, huge_b = ag.Tensor.uninit((1024, 32768), "f32"), ag.Tensor.uninit((32768, 1024), "f32")
+        huge_c = ag.Tensor.uninit((1024, 1024), "f32")
+        monkeypatch.setenv("AGH_GEMM_SPLITS", "32")
+        ag._ffi.check(ag.lib.agh_graph_begin())
+        try:
+            with pytest.raises(ag.AghError, match="capturing"):
+                ag.gemm(1.0, huge_a, huge_b, 0.0, huge_c)
+        finally:
+            monkeypatch.delenv("AGH_GEMM_SPLITS")
+            g2 = C.c_void_p()
+            rc = ag.lib.agh_graph_end(C.byref(g2))
+            if rc == 0 and g2.value:
+                ag._ffi.check(ag.lib.agh_graph_destroy(g2))
+    finally:
+        ag._ffi.check(ag.lib.agh_graph_destroy(g))
+    ag._ffi.check(ag.lib.agh_sync())
+
+
+def test_sync_and_copies_inside_a_branch(ag):
+    """Tensor.from_array (upload + agh_sync) and into_array inside `with branch():` must neither lose the
+    branch's later launches nor read a result before its producer has run."""
+    rng = np.random.default_rng(34)
+    a = rng.uniform(-1, 1, (300, 200)).astype(np.float32)
+    b = rng.uniform(-1, 1, (200, 100)).astype(np.float32)
+    ta = ag.Tensor.from_array(a)
+    with ag.branch():
+        tb = ag.Tensor.from_array(b)            # upload on the branch stream, then a sync inside the branch
+        side = ta.dot(tb)                        # launched on the branch stream after that sync
+        inside = side.into_array()               # copy inside the branch: waits for the producer
+    main = ta.relu()                             # main stream, beside the branch
+    outside = side.into_array()                  # no join yet: the copy itself must wait for the branch
+    ag.join()
+    want = orc.gemm_f64acc(a, b)
+    assert np.allclose(inside, want, atol=1e-4) and np.array_equal(inside, outside)
+    assert np.array_equal(main.into_array(), np.maximum(a, 0))
+    # a capture with a sync-free branch still closes (the arm is joined by agh_graph_end)
+    out = ag.Tensor.uninit((300, 100), "f32")
+    ag.gemm(1.0, ta, tb, 0.0, out)
+    ag._ffi.check(ag.lib.agh_sync())
+    ag._ffi.check(ag.lib.agh_graph_begin())
+    try:
+        with ag.branch():
+            ag.gemm(1.0, ta, tb, 0.0, out)
+    finally:
+        g = C.c_void_p()
+        ag._ffi.check(ag.lib.agh_graph_end(C.byref(g)))
+    ag._ffi.check(ag.lib.agh_memset(out._ptr(), 0, 300 * 100 * 4))
+    ag._ffi.check(ag.lib.agh_graph_launch(g))
+    assert np.array_equal(out.into_array(), inside)
+    ag._ffi.check(ag.lib.agh_graph_destroy(g))
+
+
+def test_block_freed_under_an_unjoined_branch_is_reused_safely(ag):
+    """A block last used on the branch stream and freed before the join: the main stream's next user of that
+    block waits for the branch."""
+    rng = np.random.default_rng(35)
+    n = 1536
+    a = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    ta = ag.Tensor.from_array(a)
+    ident = ag.Tensor.from_array(np.eye(n, dtype=np.float32))
+    for i in range(4):
+        with ag.branch():
+            tmp = ta.dot(ident)                  # branch stream writes `tmp`
+            res = tmp.dot(ident)                 # and reads it
+        del tmp                                  # freed, branch not joined
+        again = ta.relu()                        # main stream: same size class -> may get tmp's block
+        ag.join()
+        assert np.array_equal(res.into_array(), a), i
+        assert np.array_equal(again.into_array(), np.maximum(a, 0)), i
+        del res, again
