@@ -57,6 +57,7 @@ SIGNATURES = {
     "agh_event_elapsed_ms": ([ptr, ptr, C.POINTER(f32)], C.c_int),
     "agh_gemm_f32": (_GEMM, C.c_int),
     "agh_gemm_bf16": (_GEMM, C.c_int),
+    "agh_gemm_bf16_noalloc": (_GEMM, C.c_int),
     "agh_gemm_f32_bias_act": (_GEMM + [ptr, i64, i64, C.c_int], C.c_int),
     "agh_gemm_bf16_bias_act": (_GEMM + [ptr, i64, i64, C.c_int], C.c_int),
     "agh_gemm_f32_batched": (_GEMM_B, C.c_int),

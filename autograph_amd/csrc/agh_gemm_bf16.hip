@@ -11,6 +11,14 @@ int agh_gemm_bf16(int64_t m, int64_t k, int64_t n, float alpha, const void *a, i
                                            c, off_c, rsc, csc, nullptr, 0, 0, AGH_ACT_NONE);
 }
 
+int agh_gemm_bf16_noalloc(int64_t m, int64_t k, int64_t n, float alpha, const void *a, int64_t off_a, int64_t rsa,
+                          int64_t csa, const void *b, int64_t off_b, int64_t rsb, int64_t csb, float beta, void *c,
+                          int64_t off_c, int64_t rsc, int64_t csc) {
+    // same planning and kernels; split-K partials go to the library's fixed scratch buffer
+    return agh::gemm::gemm_entry<uint16_t>("agh_gemm_bf16_noalloc", m, k, n, alpha, a, off_a, rsa, csa, b, off_b, rsb, csb,
+                                           beta, c, off_c, rsc, csc, nullptr, 0, 0, AGH_ACT_NONE, 1, 0, 0, 0, true);
+}
+
 int agh_gemm_bf16_bias_act(int64_t m, int64_t k, int64_t n, float alpha, const void *a, int64_t off_a, int64_t rsa,
                            int64_t csa, const void *b, int64_t off_b, int64_t rsb, int64_t csb, float beta, void *c,
                            int64_t off_c, int64_t rsc, int64_t csc, const void *bias, int64_t off_bias,

@@ -125,7 +125,8 @@ template <typename T>
 int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, const void *a, int64_t off_a,
                int64_t rsa, int64_t csa, const void *b, int64_t off_b, int64_t rsb, int64_t csb, float beta, void *c,
                int64_t off_c, int64_t rsc, int64_t csc, const void *bias, int64_t off_bias, int64_t bias_stride,
-               int act, int64_t batch = 1, int64_t batch_a = 0, int64_t batch_b = 0, int64_t batch_c = 0) {
+               int act, int64_t batch = 1, int64_t batch_a = 0, int64_t batch_b = 0, int64_t batch_c = 0,
+               bool fixed_scratch = false) {
     AGH_API_ENTER();
     if (m < 0 || k < 0 || n < 0 || batch < 0) return fail(AGH_EINVAL, "%s: negative dimension", name);
     if (batch > 65535) return fail(AGH_ERANGE, "%s: batch count above 65535", name);
@@ -238,7 +239,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     if (splits > 1) {
         void *ws = nullptr;
         const size_t bytes = (size_t)splits * g.NQ * g.NPpad * sizeof(float);
-        if (int rc = workspace(bytes, &ws)) return rc;
+        if (int rc = fixed_scratch ? static_workspace(bytes, &ws) : workspace(bytes, &ws)) return rc;
         g.ws = (float *)ws;
         g.store_mode = ST_SPLITK;
         if (int rc = launch_cfg<T>(best, g, splits, lp, lq, direct)) return rc;

@@ -20,6 +20,8 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t e, const char *what);
 // Scratch owned by the library (split-K partials); grows on demand, never shrinks.
 int workspace(size_t bytes, void **ptr);
+// The fixed scratch buffer of agh_gemm_bf16_noalloc instead: never allocates, fails beyond its size.
+int static_workspace(size_t bytes, void **ptr);
 // Conv2 forward as an implicit GEMM (agh_conv_mfma.hip), T = uint16_t (bf16) or float; 1 = geometry not taken,
 // else a status code
 template <typename T>

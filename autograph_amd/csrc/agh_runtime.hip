@@ -11,6 +11,11 @@
 
 #include "agh_internal.h"
 
+// Fixed scratch of agh_gemm_bf16_noalloc: split-K partials for callers that may not allocate.  In host
+// code this name is only a handle for hipGetSymbolAddress; the device address is looked up once in
+// agh_init (g_scratch_ptr) and that pointer is what kernels receive.
+static __device__ __align__(256) unsigned char scratch[AGH_NOALLOC_SCRATCH_BYTES];
+
 namespace agh {
 
 static std::recursive_mutex g_mutex;
@@ -29,6 +34,7 @@ static hipEvent_t g_events[kBranchEvents];
 static int g_event_next = 0;
 static bool g_capturing = false;   // between agh_graph_begin and agh_graph_end
 static int g_live_graphs = 0;      // graph executables not yet destroyed: their nodes hold workspace pointers
+static void *g_scratch_ptr = nullptr;  // device address of `scratch` on g_device
 static thread_local char g_err[512] = "";
 
 // Library-owned workspace of one stream.  A block that a live graph may reference is retired, not
@@ -107,6 +113,18 @@ int workspace(size_t bytes, void **ptr) {
     return AGH_OK;
 }
 
+int static_workspace(size_t bytes, void **ptr) {
+    if (g_cur != g_stream)
+        return fail(AGH_EINVAL, "agh_gemm_bf16_noalloc: called inside a branch, where it would share the fixed scratch "
+                    "buffer with the main stream's calls");
+    if (bytes > (size_t)AGH_NOALLOC_SCRATCH_BYTES)
+        return fail(AGH_ERANGE, "agh_gemm_bf16_noalloc: this shape needs %zu bytes of split-K scratch, the fixed buffer "
+                    "holds %zu: use agh_gemm_bf16", bytes, (size_t)AGH_NOALLOC_SCRATCH_BYTES);
+    if (!g_scratch_ptr) return fail(AGH_ENOINIT, "agh_gemm_bf16_noalloc: the fixed scratch buffer has no device address");
+    *ptr = g_scratch_ptr;
+    return AGH_OK;
+}
+
 static hipEvent_t next_event() {
     hipEvent_t e = g_events[g_event_next];
     g_event_next = (g_event_next + 1) % kBranchEvents;
@@ -179,6 +197,9 @@ int agh_init(int device_index) {
     AGH_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     AGH_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));  // default priority, like g_stream
     for (int i = 0; i < kBranchEvents; ++i) AGH_HIP(hipEventCreateWithFlags(&g_events[i], hipEventDisableTiming));
+    // this device's copy of the fixed scratch array (the device is current)
+    g_scratch_ptr = nullptr;
+    AGH_HIP(hipGetSymbolAddress(&g_scratch_ptr, HIP_SYMBOL(scratch)));
     g_cur = g_stream;
     g_side_dirty = false;
     g_capturing = false;
@@ -210,6 +231,7 @@ int agh_shutdown(void) {
     AGH_HIP(hipStreamDestroy(g_side));
     AGH_HIP(hipStreamDestroy(g_stream));
     g_stream = g_side = g_cur = nullptr;
+    g_scratch_ptr = nullptr;
     g_init = false;
     g_device = -1;
     return AGH_OK;

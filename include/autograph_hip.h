@@ -150,6 +150,22 @@ int agh_gemm_bf16(int64_t m, int64_t k, int64_t n, float alpha,
                   const void *b, int64_t off_b, int64_t rsb, int64_t csb,
                   float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc);
 
+/* agh_gemm_bf16 for callers that cannot allocate: code under hipGraph capture before any eager run, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments,
+ * same kernels and bit-identical results, but the split-K partial sums (the only memory the GEMM uses
+ * beyond its operands) go to a fixed AGH_NOALLOC_SCRATCH_BYTES buffer that is part of the library image,
+ * so the call never reaches hipMalloc / hipFree or any allocating routine.  A shape whose split-K plan
+ * needs more scratch than that returns AGH_ERANGE and launches nothing.  Every call on the GPU shares the
+ * one buffer: calls are ordered by the library's streams, but a call issued inside a branch
+ * (agh_branch_begin) overlaps the main stream's and would race on it, so inside a branch a call whose
+ * plan needs the scratch returns AGH_EINVAL.  Nothing in the buffer has to start at zero (every partial that is read
+ * was written by the same call). */
+#define AGH_NOALLOC_SCRATCH_BYTES 16777216
+int agh_gemm_bf16_noalloc(int64_t m, int64_t k, int64_t n, float alpha,
+                          const void *a, int64_t off_a, int64_t rsa, int64_t csa,
+                          const void *b, int64_t off_b, int64_t rsb, int64_t csb,
+                          float beta, void *c, int64_t off_c, int64_t rsc, int64_t csc);
+
 /* Dense forward fused into one launch: `input.dot(&weight)` then `add_assign(bias)`
  * (src/learn/neural_network/layer.rs:1134-1143, autograd.rs:571-599) then the Relu
  * layer that follows it (layer.rs:1254-1267, rule x >= 0 ? x : 0 at :1526-1532).

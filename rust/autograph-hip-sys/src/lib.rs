@@ -14,6 +14,7 @@ pub const AGH_ENULL: c_int = -3;
 pub const AGH_ERANGE: c_int = -4;
 pub const AGH_ACT_NONE: c_int = 0;
 pub const AGH_ACT_RELU: c_int = 1;
+pub const AGH_NOALLOC_SCRATCH_BYTES: usize = 16777216;
 
 #[link(name = "autograph_hip")]
 extern "C" {
@@ -47,6 +48,7 @@ extern "C" {
     pub fn agh_event_elapsed_ms(start: *mut c_void, stop: *mut c_void, ms: *mut f32) -> c_int;
     pub fn agh_gemm_f32(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
     pub fn agh_gemm_bf16(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
+    pub fn agh_gemm_bf16_noalloc(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
     pub fn agh_gemm_f32_bias_act(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64, bias: *const c_void, off_bias: i64, bias_stride: i64, act: c_int) -> c_int;
     pub fn agh_gemm_bf16_bias_act(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64, bias: *const c_void, off_bias: i64, bias_stride: i64, act: c_int) -> c_int;
     pub fn agh_gemm_f32_batched(batch: i64, m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, batch_stride_a: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, batch_stride_b: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64, batch_stride_c: i64, bias: *const c_void, off_bias: i64, bias_stride: i64, act: c_int) -> c_int;
