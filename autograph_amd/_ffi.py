@@ -55,6 +55,9 @@ SIGNATURES = {
     "agh_event_destroy": ([ptr], C.c_int),
     "agh_event_record": ([ptr], C.c_int),
     "agh_event_elapsed_ms": ([ptr, ptr, C.POINTER(f32)], C.c_int),
+    "agh_calib_mfma_bf16": ([ptr, C.c_int, C.c_int, C.c_int], C.c_int),
+    "agh_calib_copy": ([ptr, ptr, C.c_size_t, C.c_int], C.c_int),
+    "agh_calib_read": ([ptr, ptr, C.c_size_t, C.c_int], C.c_int),
     "agh_gemm_f32": (_GEMM, C.c_int),
     "agh_gemm_bf16": (_GEMM, C.c_int),
     "agh_gemm_bf16_noalloc": (_GEMM, C.c_int),

@@ -1,0 +1,115 @@
+// Calibration launches: what this GPU can do at best on the two resources the kernels of this library
+// are bound by, measured with the same stream, events and profiler as the kernels themselves.
+//   agh_calib_mfma_bf16  a loop of nothing but independent v_mfma_f32_32x32x16_bf16 (no memory traffic),
+//                        on all-zero operands or on operands shaped like N(0, 0.02^2) bf16 data: the matrix
+//                        pipes' sustained rate under the power limit, the ceiling of any bf16 GEMM on such data
+//   agh_calib_copy       a plain 16-byte copy with a chosen grid: the read+write HBM ceiling, and the pass of
+//                        known size that FETCH_SIZE / WRITE_SIZE counter readings are scaled by
+//   agh_calib_read       a plain 16-byte read with a chosen grid: the read-only HBM ceiling
+#include "agh_internal.h"
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t lcg(uint32_t &s) {
+    s = s * 1664525u + 1013904223u;
+    return s;
+}
+
+// bf16 values with random sign and mantissa and an exponent around 2^-6, like N(0, 0.02^2) samples
+__device__ __forceinline__ bf16x8_t operand_fragment(uint32_t &s, bool zero) {
+    bf16x8_t v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t r = lcg(s);
+        const uint16_t bits = zero ? (uint16_t)0 : (uint16_t)(((r >> 16) & 0x807Fu) | ((118u + ((r >> 8) & 3u)) << 7));
+        v[i] = __builtin_bit_cast(__bf16, bits);
+    }
+    return v;
+}
+
+// 4 waves per workgroup, one per SIMD; each wave keeps 16 accumulator tiles (256 registers) and issues
+// 16 independent MFMAs per iteration on 4 + 4 operand fragments: the register shape of the GEMM's inner loop.
+__global__ __launch_bounds__(256) void mfma_only_kernel(float *out, int iters, int zero) {
+    uint32_t s = threadIdx.x * 2654435761u + blockIdx.x * 97u + 12345u;
+    bf16x8_t a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a[i] = operand_fragment(s, zero != 0);
+        b[i] = operand_fragment(s, zero != 0);
+    }
+    f32x16 acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = (f32x16)(0.0f);
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i * 4 + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i * 4 + j], 0, 0, 0);
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sum += acc[i][r];
+    if (sum == 12345.0f) out[threadIdx.x] = sum;  // keeps the loop alive; practically never true
+}
+
+__global__ __launch_bounds__(256) void copy16_kernel(const u32x4_t *__restrict__ src, u32x4_t *__restrict__ dst, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+__global__ __launch_bounds__(256) void read16_kernel(const u32x4_t *__restrict__ src, uint32_t *out, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint32_t acc = 0;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) {
+        const u32x4_t v = __builtin_nontemporal_load(src + i);
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9E3779B9u) out[0] = acc;  // keeps the loads alive
+}
+
+}  // namespace
+
+using namespace agh;
+
+extern "C" {
+
+int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks) {
+    AGH_API_ENTER();
+    if (!sink) return fail(AGH_ENULL, "agh_calib_mfma_bf16: null sink (1 KiB of device memory)");
+    if (iters < 1 || blocks < 1) return fail(AGH_EINVAL, "agh_calib_mfma_bf16: iters and blocks must be positive");
+    hipLaunchKernelGGL(mfma_only_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), (float *)sink, iters, zero_operands);
+    AGH_LAUNCH_CHECK("agh_calib_mfma_bf16");
+    return AGH_OK;
+}
+
+int agh_calib_copy(const void *src, void *dst, size_t bytes, int blocks) {
+    AGH_API_ENTER();
+    if (bytes == 0) return AGH_OK;
+    if (!src || !dst) return fail(AGH_ENULL, "agh_calib_copy: null pointer");
+    if (bytes % 16 != 0 || (((uintptr_t)src | (uintptr_t)dst) & 15) != 0 || blocks < 1)
+        return fail(AGH_EINVAL, "agh_calib_copy: 16-byte aligned pointers, a multiple of 16 bytes and blocks >= 1");
+    hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), (const u32x4_t *)src, (u32x4_t *)dst, bytes / 16);
+    AGH_LAUNCH_CHECK("agh_calib_copy");
+    return AGH_OK;
+}
+
+int agh_calib_read(const void *src, void *sink, size_t bytes, int blocks) {
+    AGH_API_ENTER();
+    if (bytes == 0) return AGH_OK;
+    if (!src || !sink) return fail(AGH_ENULL, "agh_calib_read: null pointer");
+    if (bytes % 16 != 0 || ((uintptr_t)src & 15) != 0 || blocks < 1)
+        return fail(AGH_EINVAL, "agh_calib_read: a 16-byte aligned pointer, a multiple of 16 bytes and blocks >= 1");
+    hipLaunchKernelGGL(read16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), (const u32x4_t *)src, (uint32_t *)sink, bytes / 16);
+    AGH_LAUNCH_CHECK("agh_calib_read");
+    return AGH_OK;
+}
+
+}  // extern "C"

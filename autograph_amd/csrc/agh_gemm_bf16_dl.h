@@ -300,46 +300,32 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
         // carries no bias or activation state through its unrolled body
         auto staged = [&](auto plainc) {
             constexpr bool PLAIN = decltype(plainc)::value;
-            // A bias along p (C's unit-stride axis) is added after the transposition, where a lane
-            // holds 8 consecutive p of a row and needs the same 8 bias values for every row it stores:
-            // they are loaded once.  (bias and activation act on the already rounded product, so the
-            // result is the same as applying them before staging.)
+            // Bias and activation are applied after the transposition, on the already rounded product (the
+            // reference's three separate ops: T(dot), then T(. + bias), then relu), where a lane holds 8
+            // consecutive p of one q row.  A bias along p (C's unit-stride axis) is then the same 8 values
+            // for every row the lane stores: they are widened to f32 once.  A bias along q is one value
+            // per stored row.
             const int chunk = lane % CPRW;
-            T bp[8];
+            const bool post_bias = has_bias && bias_p, row_bias = has_bias && !bias_p, relu = g.act == AGH_ACT_RELU;
+            float bpf[8];
             if constexpr (!PLAIN) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    bp[e] = 0;
-                    if (has_bias && bias_p) bp[e] = bias[(int64_t)min(pwb + chunk * 8 + e, g.NP - 1) * g.bias_stride];
+                    bpf[e] = 0.0f;
+                    if (post_bias) bpf[e] = bf16_raw_f32(bias[(int64_t)min(pwb + chunk * 8 + e, g.NP - 1) * g.bias_stride]);
                 }
             }
-            const bool post_bias = has_bias && bias_p, relu = g.act == AGH_ACT_RELU;
+            const float alpha = g.alpha;
             static_for<TQ>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
-                T bq = 0;
-                bool pre_bias = false;
-                if constexpr (!PLAIN) {
-                    const int q = qwb + j * 32 + (int)lrow;
-                    pre_bias = has_bias && !bias_p;
-                    if (q < g.NQ && pre_bias) bq = bias[(int64_t)q * g.bias_stride];
-                }
                 static_for<TP>([&](auto ic) {
                     constexpr int i = decltype(ic)::value;
                     static_for<4>([&](auto bc) {
                         constexpr int blk = decltype(bc)::value;
                         const int pl = i * 32 + blk * 8 + (int)lg * 4;  // p inside the wave tile
-                        T o[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) o[e] = finish_plain<T>(acc[i][j][blk * 4 + e], g.alpha);
-                        if constexpr (!PLAIN) {
-                            if (pre_bias) {  // wave-uniform
-#pragma unroll
-                                for (int e = 0; e < 4; ++e)
-                                    o[e] = Elem<T>::from_f32(Elem<T>::to_f32(bq) + Elem<T>::to_f32(o[e]));
-                            }
-                        }
-                        *(uint2 *)(region + lrow * EPITCH + pl * 2) =
-                            make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
+                        const uint32_t w0 = f32x2_to_bf16x2(alpha * acc[i][j][blk * 4 + 0], alpha * acc[i][j][blk * 4 + 1]);
+                        const uint32_t w1 = f32x2_to_bf16x2(alpha * acc[i][j][blk * 4 + 2], alpha * acc[i][j][blk * 4 + 3]);
+                        *(uint2 *)(region + lrow * EPITCH + pl * 2) = make_uint2(w0, w1);
                     });
                 });
                 // same wave, LDS executes in order: the reads below see the writes above
@@ -347,27 +333,30 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
                     constexpr int r = decltype(rc)::value;
                     const int row = r * RPI + lane / CPRW;
                     uint4 v = *(const uint4 *)(region + row * EPITCH + chunk * 16);
+                    const int qq = qwb + j * 32 + row, pp = pwb + chunk * 8;
                     if constexpr (!PLAIN) {
                         uint32_t w[4] = {v.x, v.y, v.z, v.w};
-                        if (post_bias) {  // wave-uniform
+                        float brow = 0.0f;
+                        if (row_bias) brow = bf16_raw_f32(bias[(int64_t)min(qq, g.NQ - 1) * g.bias_stride]);  // wave-uniform branch
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                const T lo = Elem<T>::from_f32(Elem<T>::to_f32(bp[2 * e]) + Elem<T>::to_f32((T)(w[e] & 0xFFFFu)));
-                                const T hi = Elem<T>::from_f32(Elem<T>::to_f32(bp[2 * e + 1]) + Elem<T>::to_f32((T)(w[e] >> 16)));
-                                w[e] = (uint32_t)lo | ((uint32_t)hi << 16);
+                        for (int e = 0; e < 4; ++e) {
+                            // the two bf16 values as f32 (exact); an addition quiets a signalling NaN by itself
+                            float lo = __uint_as_float(w[e] << 16), hi = __uint_as_float(w[e] & 0xFFFF0000u);
+                            if (has_bias) {  // wave-uniform
+                                lo = (post_bias ? bpf[2 * e] : brow) + lo;
+                                hi = (post_bias ? bpf[2 * e + 1] : brow) + hi;
                             }
-                        }
-                        if (relu) {  // wave-uniform; keeps x when x >= 0 (so -0 stays, NaN goes to 0)
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                const bool klo = __uint_as_float(w[e] << 16) >= 0.0f;
-                                const bool khi = __uint_as_float(w[e] & 0xFFFF0000u) >= 0.0f;
-                                w[e] = (klo ? (w[e] & 0xFFFFu) : 0u) | (khi ? (w[e] & 0xFFFF0000u) : 0u);
+                            // relu keeps x when x >= 0 (so -0 stays, NaN goes to 0).  Taken on the f32 sum before it is
+                            // rounded: rounding to bf16 changes neither the sign nor NaN-ness, and a sum of two bf16
+                            // values is zero or at least the smallest bf16 subnormal, so it cannot round to -0.
+                            if (relu) {  // wave-uniform
+                                lo = lo >= 0.0f ? lo : 0.0f;
+                                hi = hi >= 0.0f ? hi : 0.0f;
                             }
+                            w[e] = f32x2_to_bf16x2(lo, hi);
                         }
                         v = make_uint4(w[0], w[1], w[2], w[3]);
                     }
-                    const int qq = qwb + j * 32 + row, pp = pwb + chunk * 8;
                     // streaming store: C is not read again by this launch, and keeping it out of the last-level
                     // cache leaves that cache to the operand panels, which every tile row / column re-reads
                     if (qq < g.NQ && pp < g.NP)
