@@ -5,13 +5,18 @@
 // channels per step; 8 for f32, where a step is four v_mfma_f32_32x32x2_f32 per tile) without a single
 // barrier: the A operand of v_mfma_f32_32x32x16_bf16 (32 positions x 16 channels of one tap) is a
 // 16-byte LDS read per lane, the B operand (32 output channels x the same 16 k) comes straight from
-// a fragment-ordered copy of the filter bank, which is small and stays in L2.  When the rows of all
+// a fragment-ordered copy of the filter bank, which is small and stays in L2.  A wave owns ALL 256
+// positions of the tile and 32 output channels: per k step it reads eight A fragments from LDS (the
+// four waves read the same ones; LDS serves 16-byte reads at 256 bytes per clock, this takes half) and
+// ONE B fragment from memory, so the filter bank crosses the vector memory path once per workgroup.  When the rows of all
 // input channels do not fit in half a CU's LDS, the channels are taken in passes of a power-of-two
 // count each (stage, k loop over all taps, stage the next ...), accumulators staying in registers:
 // two workgroups share a CU, so one's staging and epilogue run under the other's k loop.  HBM traffic is the image in and the activation out, a tenth of
 // what im2col + GEMM move; bias and ReLU are applied in the epilogue in the order the separate
 // layers round.  Sums are f32 in k order (tap, channel), one rounding at the end (none for f32), so
 // results agree with the im2col chain within the GEMM tolerances, not bit for bit.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "agh_internal.h"
@@ -24,15 +29,24 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 constexpr int kThreads = 256;
-constexpr int kTilePos = 256;  // output positions per workgroup (8 MFMA tiles of 32)
-constexpr int kTileOc = 128;   // output channels per workgroup (4 MFMA tiles of 32)
+constexpr int kTileOc = 128;   // output channels per workgroup (4 MFMA tiles of 32, one per wave)
+constexpr int kBRing = 8, kBAhead = kBRing - 1;  // register sets of B fragments, and how many steps ahead they are requested
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
 
 // Element-type geometry: a 16-byte chunk holds CPC channels, a k step covers two chunks (one per half-wave).
 template <typename T> struct Geo {
     static constexpr int ES = (int)sizeof(T);
     static constexpr int CPC = 16 / ES;           // channels per 16-byte chunk = pixels per 16-byte vector of a row
     static constexpr int CPI = 4 / ES;            // channels one staging item packs into a 4-byte LDS write
-    static constexpr int EPITCH = 128 * ES + 16;  // bytes per staged output-channel row in the epilogue (128 positions + pad)
+    static constexpr int EPI_POS = 256 / ES;      // positions the epilogue transposes at a time (256 bytes of an output row)
+    static constexpr int EPITCH = 256 + 16;       // bytes per staged output-channel row in the epilogue (EPI_POS positions + pad)
 };
 
 struct ConvMfmaParams {
@@ -41,8 +55,7 @@ struct ConvMfmaParams {
     int npos, tiles_per_img, oc_tiles;
     int lcols;     // staged columns: iw + 2*pw
     int icc, npass;  // channels staged per pass (a power of two), passes = ic / icc
-    int nch_mask;  // 16-byte chunks per staged pixel - 1 (a power of two)
-    int kshift;    // log2(pixels per 256 bytes): see the swizzle key below
+    int nchunk;    // 16-byte chunks per staged pixel
     int K;         // fh*fw*ic
     int per_xcd;   // workgroups per XCD when the grid divides by 8, else 0
     FastDiv div_ow, div_tiles, div_octiles, div_vec;
@@ -67,15 +80,17 @@ __global__ __launch_bounds__(kThreads) void pack_filter_kernel(const T *__restri
     wp[dst] = w[e];
 }
 
-template <typename T>
-__global__ __launch_bounds__(kThreads, 2) void conv2_mfma_kernel(const T *__restrict__ x, const T *__restrict__ wp,
+// kTilePos output positions per workgroup (kMT MFMA tiles of 32), kWgs workgroups per CU.
+template <typename T, int kTilePos, int kWgs>
+__global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__restrict__ x, const T *__restrict__ wp,
                                                                                   const T *__restrict__ bias, T *__restrict__ y,
                                                                                   ConvMfmaParams p) {
     extern __shared__ __align__(16) unsigned char lds[];
-    constexpr int ES = Geo<T>::ES, CPC = Geo<T>::CPC, CPI = Geo<T>::CPI, PV = Geo<T>::CPC, kEpitch = Geo<T>::EPITCH;
+    constexpr int ES = Geo<T>::ES, CPC = Geo<T>::CPC, PV = Geo<T>::CPC, kEpitch = Geo<T>::EPITCH, kEpiPos = Geo<T>::EPI_POS;
+    constexpr int kMT = kTilePos / 32, kEpiMT = kEpiPos / 32;
+    static_assert(kTilePos % kEpiPos == 0, "the epilogue takes whole groups of position tiles");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave & 1, wn = wave >> 1;
     uint32_t t0, oct, b, tile;
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a run of consecutive
     // tiles, so that the input rows two neighbouring position tiles share are fetched from HBM once
@@ -88,163 +103,152 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_kernel(const T *__rest
     const int lrows = ho_last - ho_first + p.fh;  // staged input rows
     const int pix_bytes = p.icc * ES;
 
-    // ---- staging of one pass: items = (row, channel pair or channel, 16-byte vector of the row) ----
-    // The 16-byte channel chunks of pixel q are stored at chunk ^ key(q), key(q) = ((q >> kshift) + (q >> 4)) &
-    // nch_mask.  The lanes of a ds_read_b128 of the k loop address 16 consecutive pixels and the same chunk:
-    // the first term puts those 16 reads on 16 different 16-byte columns of the 256-byte LDS row.  The lanes
-    // of a staging write address pixels 8 apart: the second term spreads those as well.
+    // ---- staging of one pass ----
+    // A staged pixel is its icc channels (pix_bytes) plus 16 bytes of padding.  The lanes of a ds_read_b128 of the
+    // k loop address consecutive pixels and the same chunk: with a pitch of pix_bytes + 16 (4 banks more than a
+    // multiple of 8 banks) any 16 consecutive pixels fall on 16 different 16-byte bank groups, whatever the tap,
+    // so the k loop needs no swizzle and its addresses are one add away from a per-lane constant.
+    const int pitch = pix_bytes + 16;
     auto stage = [&](int pass) {
-        const int nvec = p.iw / PV, npair = p.icc / CPI;  // an item packs CPI channels of PV pixels into PV 4-byte writes
-        const uint32_t items = (uint32_t)lrows * npair * nvec;
+        // An item is CPC channels x PV (= CPC) pixels: CPC 16-byte loads, one per channel plane, transposed in
+        // registers (bf16: one v_perm_b32 per output dword; f32: the transposition is register renaming) into
+        // PV 16-byte LDS writes, one whole channel chunk of one pixel each.  Consecutive lanes take the
+        // consecutive channel chunks of the same pixels, so a write instruction covers whole staged pixels
+        // (contiguous bytes: no bank conflict).
+        const int nvec = p.iw / PV, ngrp = p.icc / CPC;
+        const uint32_t items = (uint32_t)lrows * ngrp * nvec;
         const T *ximg = x + ((size_t)b * p.ic + (size_t)pass * p.icc) * p.ih * (size_t)p.iw;
-        // batches of SB items per thread: all global loads of a batch are issued before the first LDS write
-        constexpr int SB = 4;
+        const size_t plane = (size_t)p.ih * p.iw;
+        // two items per thread and trip: all 2 * CPC loads are requested before the first LDS write, so a
+        // workgroup's staging waits for memory about once (448 items at the 64-channel 56 x 56 layer)
+        constexpr int SB = 2;
         for (uint32_t it0 = tid; it0 < items; it0 += kThreads * SB) {
-            uint4 r0[SB], r1[SB];
-            int base[SB], pix0[SB], cpart[SB];
+            uint4 r[SB][CPC];
+            int dst[SB];
 #pragma unroll
             for (int u = 0; u < SB; ++u) {
                 const uint32_t it = it0 + u * kThreads;
-                uint32_t rc, v, lr, c2;
-                p.div_vec.divmod(it, rc, v);
-                lr = rc / (uint32_t)npair;
-                c2 = rc - lr * npair;
+                uint32_t rv, v, lr, cg;
+                rv = it / (uint32_t)ngrp;
+                cg = it - rv * ngrp;
+                p.div_vec.divmod(rv, lr, v);
                 const int hi = ho_first - p.ph + (int)lr;
-                r0[u] = make_uint4(0, 0, 0, 0);
-                r1[u] = r0[u];
+#pragma unroll
+                for (int i = 0; i < CPC; ++i) r[u][i] = make_uint4(0, 0, 0, 0);
                 if (it < items && hi >= 0 && hi < p.ih) {
-                    const T *src = ximg + ((size_t)(CPI * c2) * p.ih + hi) * (size_t)p.iw + v * PV;
-                    r0[u] = *(const uint4 *)src;
-                    if constexpr (CPI == 2) r1[u] = *(const uint4 *)(src + (size_t)p.ih * p.iw);
+                    const T *src = ximg + ((size_t)(CPC * cg) * p.ih + hi) * (size_t)p.iw + v * PV;
+#pragma unroll
+                    for (int i = 0; i < CPC; ++i) r[u][i] = *(const uint4 *)(src + i * plane);
                 }
-                const int c = CPI * (int)c2;
-                pix0[u] = (int)lr * p.lcols + p.pw + (int)v * PV;
-                base[u] = it < items ? pix0[u] * pix_bytes + (c % CPC) * ES : -1;
-                cpart[u] = c / CPC;
+                dst[u] = it < items ? ((int)lr * p.lcols + p.pw + (int)v * PV) * pitch + ((int)cg << 4) : -1;
             }
 #pragma unroll
             for (int u = 0; u < SB; ++u) {
-                if (base[u] < 0) continue;
-                const uint32_t lo[4] = {r0[u].x, r0[u].y, r0[u].z, r0[u].w}, hi2[4] = {r1[u].x, r1[u].y, r1[u].z, r1[u].w};
+                if (dst[u] < 0) continue;
 #pragma unroll
                 for (int j = 0; j < PV; ++j) {
-                    uint32_t word;
-                    if constexpr (CPI == 2) word = ((lo[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu) | (((hi2[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu) << 16);
-                    else word = lo[j];
-                    const int q = pix0[u] + j;
-                    const int addr = base[u] + j * pix_bytes + ((cpart[u] ^ (((q >> p.kshift) + (q >> 4)) & p.nch_mask)) << 4);
-                    *(uint32_t *)(lds + addr) = word;
+                    uint4 o;
+                    if constexpr (ES == 2) {
+                        // pixel j's value is half (j & 1) of dword j >> 1 of every channel row; dword d of the chunk
+                        // packs channels 2d (low half) and 2d + 1 (high half)
+                        constexpr uint32_t kLow = 0x05040100u, kHigh = 0x07060302u;
+                        const uint32_t sel = (j & 1) ? kHigh : kLow;
+                        auto word = [&](const uint4 &q) { return (j >> 1) == 0 ? q.x : (j >> 1) == 1 ? q.y : (j >> 1) == 2 ? q.z : q.w; };
+                        o.x = __builtin_amdgcn_perm(word(r[u][1 % CPC]), word(r[u][0]), sel);
+                        o.y = __builtin_amdgcn_perm(word(r[u][3 % CPC]), word(r[u][2 % CPC]), sel);
+                        o.z = __builtin_amdgcn_perm(word(r[u][5 % CPC]), word(r[u][4 % CPC]), sel);
+                        o.w = __builtin_amdgcn_perm(word(r[u][7 % CPC]), word(r[u][6 % CPC]), sel);
+                    } else {
+                        auto word = [&](const uint4 &q) { return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w; };
+                        o = make_uint4(word(r[u][0]), word(r[u][1 % CPC]), word(r[u][2 % CPC]), word(r[u][3 % CPC]));
+                    }
+                    *(uint4 *)(lds + dst[u] + j * pitch) = o;
                 }
             }
         }
         if (pass == 0) {  // padding columns left and right of the image: no pass writes them again
-            const int npadcol = p.lcols - p.iw, nch = p.nch_mask + 1;
+            const int npadcol = p.lcols - p.iw, nch = p.nchunk;
             const uint32_t pads = (uint32_t)lrows * npadcol * nch;
             for (uint32_t it = tid; it < pads; it += kThreads) {
                 const uint32_t ch = it % nch, rc = it / nch;
                 const uint32_t k = rc % npadcol, lr = rc / npadcol;
                 const int col = (int)k < p.pw ? (int)k : p.iw + (int)k;
-                *(uint4 *)(lds + ((int)lr * p.lcols + col) * pix_bytes + (ch << 4)) = make_uint4(0, 0, 0, 0);
+                *(uint4 *)(lds + ((int)lr * p.lcols + col) * pitch + (ch << 4)) = make_uint4(0, 0, 0, 0);
             }
         }
     };
 
     // ---- per-lane operand addressing ----
     const int kg = lane >> 5, l32 = lane & 31;
-    int apix[4], abase[4];  // the lane's staged pixel for tap (0,0) of each position tile, and its byte address
+    int abase[kMT];  // byte address of the lane's chunk (half-wave kg) of its staged pixel for tap (0,0), per position tile
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-        const int pp = min(p0 + (wm * 4 + mt) * 32 + l32, p.npos - 1);  // clamped: a duplicate, never stored
+    for (int mt = 0; mt < kMT; ++mt) {
+        const int pp = min(p0 + mt * 32 + l32, p.npos - 1);  // clamped: a duplicate, never stored
         uint32_t ho, wo;
         p.div_ow.divmod((uint32_t)pp, ho, wo);
-        apix[mt] = ((int)ho - ho_first) * p.lcols + (int)wo;
-        abase[mt] = apix[mt] * pix_bytes;
+        abase[mt] = (((int)ho - ho_first) * p.lcols + (int)wo) * pitch + (kg << 4);
     }
     const int ncc = p.icc / (2 * CPC);          // k steps per tap in one pass
     const int nsteps = p.fh * p.fw * ncc;       // k steps per pass
-    const int oc0 = oct * kTileOc + wn * 64;
+    const int oc0 = oct * kTileOc + wave * 32;
     const bool wave_live = oc0 < p.oc;  // oc is a multiple of 64
-    const T *brow[2];
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt)  // fragment-ordered bank: block (tile of 32 channels, step), CPC elements per lane
-        brow[nt] = wp + ((size_t)(min(oc0 + nt * 32, p.oc - 32) >> 5) * nsteps * p.npass * 64 + lane) * CPC;
+    // fragment-ordered bank: block (tile of 32 channels, step), 16 bytes per lane.  The block address is
+    // wave-uniform (scalar registers), the lane adds 16 * lane.
+    const unsigned char *bbank = (const unsigned char *)wp + (size_t)(min(oc0, p.oc - 32) >> 5) * nsteps * p.npass * 1024;
+    const uint32_t blane = (uint32_t)lane * 16u;
 
-    f32x16 acc[4][2];
+    f32x16 acc[kMT];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt) acc[mt][nt] = (f32x16)(0.0f);
+    for (int mt = 0; mt < kMT; ++mt) acc[mt] = (f32x16)(0.0f);
 
-    // ---- k loop of a pass: taps outer, 2*CPC channels per step, operands of step s+1 requested before the MFMAs of step s ----
+    // ---- k loop of a pass: taps outer, 2*CPC channels per step ----
     int fi = 0, fj = 0, cc = 0;  // position of the NEXT step to load
-    int akey[4];                 // swizzle key of the current tap, << 4
-    const int kg16 = kg << 4;
-    // A fragments: next step's LDS reads are issued before this step's MFMAs.  B fragments come from L2
-    // (several hundred cycles away), so they are requested three steps ahead into a ring of four
-    // register sets.  The main loop takes four steps per trip so every register index is static, and
-    // it contains no branch around a load: a load that would run past the last step re-reads a valid
-    // location instead (with conditional loads the compiler can no longer count outstanding loads and
-    // waits for all of them before every MFMA group, which serialises the L2 latency into each step).
-    int tapbytes_next = 0, chunk16_next = kg16;  // of the step the next load_a_part calls will fetch
-    auto prepare_a = [&](int s) {  // scalar / per-lane state for fetching step s's A fragments
-        tapbytes_next = s < nsteps ? (fi * p.lcols + fj) * pix_bytes : 0;
-        chunk16_next = kg16 + ((s < nsteps ? cc : 0) << 5);
-    };
-    auto load_a_part = [&](uint4(&a)[4], auto mtc) {
+    // A fragments: the fragment of tile mt for step s+1 is read from LDS into the same registers right after
+    // the MFMA of tile mt of step s has been issued (eight MFMAs, 256 clocks, ahead of its use); its address
+    // is the lane's constant plus a wave-uniform step offset.  B fragments come from L2 (several hundred
+    // cycles away), so they are requested kBAhead steps ahead into a ring of register sets.  The main loop
+    // takes a whole ring of steps per trip so every register index is static, and it contains no branch around
+    // a load: a load that would run past the last step re-reads a valid location instead (with conditional
+    // loads the compiler can no longer count outstanding loads and waits for all of them before every MFMA
+    // group, which serialises the L2 latency into each step).
+    int aoff_next = 0;  // wave-uniform byte offset of the step the next load_a calls will fetch
+    auto prepare_a = [&](int s) { aoff_next = s < nsteps ? (fi * p.lcols + fj) * pitch + (cc << 5) : 0; };
+    auto load_a = [&](uint4(&a)[kMT], auto mtc) {
         constexpr int mt = decltype(mtc)::value;
-        a[mt] = *(const uint4 *)(lds + abase[mt] + tapbytes_next + (chunk16_next ^ akey[mt]));
-    };
-    auto set_keys = [&]() {
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-            const int q = apix[mt] + fi * p.lcols + fj;
-            akey[mt] = (((q >> p.kshift) + (q >> 4)) & p.nch_mask) << 4;
-        }
+        a[mt] = *(const uint4 *)(lds + abase[mt] + aoff_next);
     };
     auto advance_a = [&]() {
         if (++cc == ncc) {
             cc = 0;
             if (++fj == p.fw) { fj = 0; ++fi; }
-            set_keys();
         }
     };
-    auto load_b_part = [&](uint4(&bq)[2], int s, auto ntc) {
-        constexpr int nt = decltype(ntc)::value;
-        bq[nt] = *(const uint4 *)(brow[nt] + (size_t)min(s, nsteps - 1) * (64 * CPC));
-    };
-    auto mma = [&](const uint4(&a)[4], const uint4(&bq)[2], auto nc) {
-        constexpr int n = decltype(nc)::value, mt = n >> 1, nt = n & 1;
+    auto load_b = [&](uint4 &bq, int s) { bq = *(const uint4 *)(bbank + (size_t)min(s, nsteps - 1) * 1024 + blane); };
+    auto mma = [&](const uint4(&a)[kMT], const uint4 &bq, auto mtc) {
+        constexpr int mt = decltype(mtc)::value;
         if constexpr (ES == 2) {
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[mt]), __builtin_bit_cast(bf16x8_t, bq[nt]),
-                                                                  acc[mt][nt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[mt]), __builtin_bit_cast(bf16x8_t, bq), acc[mt], 0, 0, 0);
         } else {  // lanes 0-31 hold channels c..c+3, lanes 32-63 channels c+4..c+7: element j of both is one k pair
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].x), __uint_as_float(bq[nt].x), acc[mt][nt], 0, 0, 0);
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].y), __uint_as_float(bq[nt].y), acc[mt][nt], 0, 0, 0);
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].z), __uint_as_float(bq[nt].z), acc[mt][nt], 0, 0, 0);
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].w), __uint_as_float(bq[nt].w), acc[mt][nt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].x), __uint_as_float(bq.x), acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].y), __uint_as_float(bq.y), acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].z), __uint_as_float(bq.z), acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].w), __uint_as_float(bq.w), acc[mt], 0, 0, 0);
         }
     };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    using I2 = std::integral_constant<int, 2>;
-    using I3 = std::integral_constant<int, 3>;
-    using I4 = std::integral_constant<int, 4>;
-    using I5 = std::integral_constant<int, 5>;
-    using I6 = std::integral_constant<int, 6>;
-    using I7 = std::integral_constant<int, 7>;
-    // One step: the eight MFMA groups of step s on (a, b), with the fetches of step s+1's A fragments (into an)
-    // and of step s+3's B fragments (into bn) handed out between them, one per group.  sched_barrier pins
-    // the order, so the matrix pipe gets new work back to back while the other requests trickle out.
-    auto step = [&](const uint4(&a)[4], const uint4(&bq)[2], uint4(&an)[4], uint4(&bn)[2], int s) {
+    // One step: the eight MFMA groups of step s on (a, bq); the A fragment of each tile is refreshed for step s+1
+    // right behind its MFMA, the B fragment of the step kBAhead ahead is requested (into bn) in the middle; the
+    // tap bookkeeping for step s+2 runs at the end of the step, after the last refresh.  sched_barrier pins the order, so the matrix pipe gets
+    // new work back to back while the other requests trickle out.
+    auto step = [&](uint4(&a)[kMT], const uint4 &bq, uint4 &bn, int s) {
         prepare_a(s + 1);
-        mma(a, bq, I0{}); load_a_part(an, I0{}); __builtin_amdgcn_sched_barrier(0);
-        mma(a, bq, I1{}); load_a_part(an, I1{}); __builtin_amdgcn_sched_barrier(0);
-        mma(a, bq, I2{}); load_a_part(an, I2{}); __builtin_amdgcn_sched_barrier(0);
-        mma(a, bq, I3{}); load_a_part(an, I3{}); __builtin_amdgcn_sched_barrier(0);
-        mma(a, bq, I4{}); load_b_part(bn, s + 3, I0{}); __builtin_amdgcn_sched_barrier(0);
-        mma(a, bq, I5{}); load_b_part(bn, s + 3, I1{}); __builtin_amdgcn_sched_barrier(0);
-        mma(a, bq, I6{}); advance_a(); __builtin_amdgcn_sched_barrier(0);
-        mma(a, bq, I7{}); __builtin_amdgcn_sched_barrier(0);
+        static_for<kMT>([&](auto mtc) {
+            constexpr int mt = decltype(mtc)::value;
+            mma(a, bq, mtc);
+            load_a(a, mtc);
+            if constexpr (mt == 3) load_b(bn, s + kBAhead);
+            if constexpr (mt == kMT - 1) advance_a();
+            __builtin_amdgcn_sched_barrier(0);
+        });
     };
 
     for (int pass = 0; pass < p.npass; ++pass) {
@@ -252,68 +256,73 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_kernel(const T *__rest
         stage(pass);
         __syncthreads();
         if (wave_live) {
-            uint4 a0[4], a1[4], b0[2], b1[2], b2[2], b3[2];
-            load_b_part(b0, 0, I0{}); load_b_part(b0, 0, I1{});
-            load_b_part(b1, 1, I0{}); load_b_part(b1, 1, I1{});
-            load_b_part(b2, 2, I0{}); load_b_part(b2, 2, I1{});
+            uint4 a[kMT], bf[kBRing];
+            static_for<kBAhead>([&](auto ic) { load_b(bf[decltype(ic)::value], decltype(ic)::value); });
             fi = 0; fj = 0; cc = 0;
-            set_keys();
             prepare_a(0);
-            load_a_part(a0, I0{}); load_a_part(a0, I1{}); load_a_part(a0, I2{}); load_a_part(a0, I3{});
+            static_for<kMT>([&](auto mtc) { load_a(a, mtc); });
             advance_a();
             int s = 0;
-            for (; s + 4 <= nsteps; s += 4) {
-                step(a0, b0, a1, b3, s);
-                step(a1, b1, a0, b0, s + 1);
-                step(a0, b2, a1, b1, s + 2);
-                step(a1, b3, a0, b2, s + 3);
-            }
-            // up to three steps left: their B fragments are in b0, b1, b2 and the first one's A fragments in a0
+            for (; s + kBRing <= nsteps; s += kBRing)
+                static_for<kBRing>([&](auto ic) {
+                    constexpr int i = decltype(ic)::value;
+                    step(a, bf[i], bf[(i + kBAhead) % kBRing], s + i);
+                });
+            // fewer than a ring of steps left: their B fragments are in bf[0 ..]; the requests these steps
+            // make land in the one set no remaining step reads
             const int left = nsteps - s;
-            if (left >= 1) step(a0, b0, a1, b3, s);
-            if (left >= 2) step(a1, b1, a0, b3, s + 1);
-            if (left >= 3) step(a0, b2, a1, b3, s + 2);
-            brow[0] += (size_t)nsteps * (64 * CPC);
-            brow[1] += (size_t)nsteps * (64 * CPC);
+            static_for<kBRing - 1>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                if (i < left) step(a, bf[i], bf[kBRing - 1], s + i);
+            });
+            bbank += (size_t)nsteps * 1024;
         }
     }
     __syncthreads();  // every wave is done with the staged image: LDS becomes the epilogue's transposition space
 
-    // ---- epilogue: round, bias, ReLU, transpose 32 channels x 128 positions through LDS, 16-byte stores ----
+    // ---- epilogue: round, bias, ReLU, transpose 32 channels x 128 positions at a time through LDS, 16-byte stores ----
     if (wave_live) {
         unsigned char *region = lds + wave * 32 * kEpitch;
         const bool relu = p.act == AGH_ACT_RELU;
+        const int o_lane = oc0 + l32;
+        float bq = 0.0f;
+        if (p.has_bias) bq = Elem<T>::to_f32(bias[min(o_lane, p.oc - 1)]);
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-            const int o_lane = oc0 + nt * 32 + l32;
-            float bq = 0.0f;
-            if (p.has_bias) bq = Elem<T>::to_f32(bias[min(o_lane, p.oc - 1)]);
+        for (int part = 0; part < kTilePos / kEpiPos; ++part) {
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
+            for (int m4 = 0; m4 < kEpiMT; ++m4)
 #pragma unroll
                 for (int blk = 0; blk < 4; ++blk) {
-                    const int pl = mt * 32 + blk * 8 + kg * 4;  // position inside the wave's 128
+                    const int mt = part * kEpiMT + m4;
+                    const int pl = m4 * 32 + blk * 8 + kg * 4;  // position inside this part
                     if constexpr (ES == 2) {
                         // two packed conversions give the four rounded values as two dwords
-                        uint32_t w[2] = {f32x2_to_bf16x2(acc[mt][nt][blk * 4 + 0], acc[mt][nt][blk * 4 + 1]),
-                                         f32x2_to_bf16x2(acc[mt][nt][blk * 4 + 2], acc[mt][nt][blk * 4 + 3])};
-                        if (p.has_bias) {  // wave-uniform: bias + rounded product, rounded again
-#pragma unroll
-                            for (int h = 0; h < 2; ++h)
-                                w[h] = f32x2_to_bf16x2(bq + __uint_as_float(w[h] << 16), bq + __uint_as_float(w[h] & 0xFFFF0000u));
-                        }
-                        if (relu) {  // wave-uniform; keeps x when x >= 0 (so -0 stays, NaN goes to 0)
+                        uint32_t w[2] = {f32x2_to_bf16x2(acc[mt][blk * 4 + 0], acc[mt][blk * 4 + 1]),
+                                         f32x2_to_bf16x2(acc[mt][blk * 4 + 2], acc[mt][blk * 4 + 3])};
+                        if (p.has_bias || relu) {  // wave-uniform
 #pragma unroll
                             for (int h = 0; h < 2; ++h) {
-                                const bool klo = __uint_as_float(w[h] << 16) >= 0.0f, khi = __uint_as_float(w[h] & 0xFFFF0000u) >= 0.0f;
-                                w[h] = (klo ? (w[h] & 0xFFFFu) : 0u) | (khi ? (w[h] & 0xFFFF0000u) : 0u);
+                                // the rounded products as f32 (exact); bias + product is rounded again by the conversion below
+                                float lo = __uint_as_float(w[h] << 16), hi = __uint_as_float(w[h] & 0xFFFF0000u);
+                                if (p.has_bias) {
+                                    lo = bq + lo;
+                                    hi = bq + hi;
+                                }
+                                // relu keeps x when x >= 0 (so -0 stays, NaN goes to 0).  Taken on the f32 value before the
+                                // final rounding: rounding changes neither sign nor NaN-ness, and a sum of two bf16 values is
+                                // zero or at least the smallest bf16 subnormal, so it cannot round to -0.
+                                if (relu) {
+                                    lo = lo >= 0.0f ? lo : 0.0f;
+                                    hi = hi >= 0.0f ? hi : 0.0f;
+                                }
+                                w[h] = f32x2_to_bf16x2(lo, hi);
                             }
                         }
                         *(uint2 *)(region + l32 * kEpitch + pl * 2) = make_uint2(w[0], w[1]);
                     } else {
                         float v[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = acc[mt][nt][blk * 4 + e];
+                        for (int e = 0; e < 4; ++e) v[e] = acc[mt][blk * 4 + e];
                         if (p.has_bias) {
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = bq + v[e];
@@ -325,13 +334,14 @@ __global__ __launch_bounds__(kThreads, 2) void conv2_mfma_kernel(const T *__rest
                         *(float4 *)(region + l32 * kEpitch + pl * 4) = make_float4(v[0], v[1], v[2], v[3]);
                     }
                 }
-            // same wave, LDS executes in order: the reads below see the writes above
-            constexpr int CPRW = 128 * ES / 16, RPI = 64 / CPRW, NST = 32 / RPI;  // chunks per row, rows per instruction
+            // same wave, LDS executes in order: the reads below see the writes above, and the next part's
+            // writes come after these reads.  A staged row is 256 bytes = 16 chunks: a store instruction covers 4 rows.
+            constexpr int CPRW = 16, RPI = 64 / CPRW, NST = 32 / RPI;
 #pragma unroll
             for (int r = 0; r < NST; ++r) {
                 const int row = r * RPI + lane / CPRW, chunk = lane % CPRW;
                 const uint4 v = *(const uint4 *)(region + row * kEpitch + chunk * 16);
-                const int pos = p0 + wm * 128 + chunk * CPC, o = oc0 + nt * 32 + row;
+                const int pos = p0 + part * kEpiPos + chunk * CPC, o = oc0 + row;
                 if (pos < p.npos && o < p.oc) *(uint4 *)(y + ((size_t)b * p.oc + o) * p.npos + pos) = v;
             }
         }
@@ -344,8 +354,8 @@ namespace agh {
 
 // Returns 1 when the geometry is not one this kernel takes (the caller goes on to its other paths),
 // otherwise a status code.  The API lock is held by the caller.
-template <typename T>
-int conv2_mfma_try(const char *name, const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic, int64_t ih,
+template <typename T, int kTilePos, int kWgs>
+static int conv2_mfma_launch(const char *name, const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic, int64_t ih,
                    int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t oh, int64_t ow, int act) {
     constexpr int ES = Geo<T>::ES, CPC = Geo<T>::CPC;
     const int64_t npos = oh * ow;
@@ -355,11 +365,11 @@ int conv2_mfma_try(const char *name, const void *x, const void *w, const void *b
     if (ic * fh * fw < 128 || npos < 256) return 1;
     const int64_t lcols = iw + 2 * pw;
     const int64_t rows_out = std::min<int64_t>(oh, (kTilePos - 1) / ow + 2);
-    // two workgroups per CU (160 KB of LDS): the largest power-of-two channel count whose rows fit in half
-    const int64_t lds_limit = 80 * 1024;
+    // kWgs workgroups per CU (160 KB of LDS): the largest power-of-two channel count whose rows fit in a share
+    const int64_t lds_limit = 160 * 1024 / kWgs;
     int64_t icc = ic & -ic;  // channels per pass: a power of two that divides ic
-    while (icc > 2 * CPC && (rows_out + fh - 1) * lcols * icc * ES > lds_limit) icc >>= 1;
-    const int64_t tile_bytes = (rows_out + fh - 1) * lcols * icc * ES;
+    while (icc > 2 * CPC && (rows_out + fh - 1) * lcols * (icc * ES + 16) > lds_limit) icc >>= 1;
+    const int64_t tile_bytes = (rows_out + fh - 1) * lcols * (icc * ES + 16);  // staged pixels are padded by 16 bytes
     const int64_t smem = std::max<int64_t>(tile_bytes, 4 * 32 * Geo<T>::EPITCH);
     if (smem > lds_limit) return 1;
     const int64_t tiles = (npos + kTilePos - 1) / kTilePos, octiles = (oc + kTileOc - 1) / kTileOc;
@@ -379,9 +389,7 @@ int conv2_mfma_try(const char *name, const void *x, const void *w, const void *b
     p.act = act; p.has_bias = bias != nullptr;
     p.npos = npos; p.tiles_per_img = tiles; p.oc_tiles = octiles; p.lcols = lcols;
     p.icc = icc; p.npass = ic / icc;
-    p.nch_mask = icc / CPC - 1;
-    const int64_t pix_bytes = icc * ES;  // pixels per 256 bytes = 256 / pix_bytes (at least 1)
-    p.kshift = pix_bytes >= 256 ? 0 : (pix_bytes == 128 ? 1 : (pix_bytes == 64 ? 2 : 3));
+    p.nchunk = icc / CPC;
     p.K = fh * fw * ic;
     p.per_xcd = blocks % 8 == 0 ? (int)(blocks / 8) : 0;
     p.div_ow = FastDiv((uint32_t)ow);
@@ -390,13 +398,27 @@ int conv2_mfma_try(const char *name, const void *x, const void *w, const void *b
     p.div_vec = FastDiv((uint32_t)(iw / CPC));
     static bool attr_done = false;
     if (!attr_done) {
-        AGH_HIP(hipFuncSetAttribute((const void *)conv2_mfma_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
+        AGH_HIP(hipFuncSetAttribute((const void *)(conv2_mfma_kernel<T, kTilePos, kWgs>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
         attr_done = true;
     }
-    hipLaunchKernelGGL(conv2_mfma_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), (size_t)smem, stream(), (const T *)x,
+    hipLaunchKernelGGL((conv2_mfma_kernel<T, kTilePos, kWgs>), dim3((unsigned)blocks), dim3(kThreads), (size_t)smem, stream(), (const T *)x,
                        (const T *)wperm, (const T *)bias, (T *)y, p);
     AGH_LAUNCH_CHECK(name);
     return AGH_OK;
+}
+
+template <typename T>
+int conv2_mfma_try(const char *name, const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic, int64_t ih,
+                   int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t oh, int64_t ow, int act) {
+    // f32: 128 positions per workgroup and three workgroups per CU; while one stages its rows or writes its outputs
+    // (memory latency), two others keep the matrix pipes fed (measured 132 against 124 TFLOP/s at the 256 x 64 x 56 x 56
+    // layer).  bf16, whose k loop is eight times shorter per byte staged: 256 positions and two per CU (halo rows are
+    // a smaller share; 878 against 796 TFLOP/s).  AGH_CONV_TILE=128|256 overrides.
+    const char *e = getenv("AGH_CONV_TILE");
+    const int tile = e && *e ? atoi(e) : (sizeof(T) == 4 ? 128 : 256);
+    if (tile == 128)
+        return conv2_mfma_launch<T, 128, 3>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
+    return conv2_mfma_launch<T, 256, 2>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
 }
 
 template int conv2_mfma_try<uint16_t>(const char *, const void *, const void *, const void *, void *, int64_t, int64_t, int64_t, int64_t,
