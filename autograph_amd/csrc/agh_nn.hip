@@ -1047,6 +1047,7 @@ int conv2_backward_input_launch(const char *name, const void *dy, const void *w,
 struct PoolParams {
     int ih, iw, oh, ow, h, w, sh, sw;
     FastDiv div_ow, div_oh;
+    FastDiv div_gpr;  // 2x2 vector kernels: 16-byte groups per input row
 };
 
 template <typename T>
@@ -1100,103 +1101,123 @@ __global__ __launch_bounds__(kThreads) void max_pool2_backward_kernel(T *__restr
         }
 }
 
-// 2x2 windows, stride 2, rows a multiple of 8 elements: one thread takes four neighbouring windows of
-// an output row, i.e. 8 input elements from each of two rows, with 16-byte accesses.  Same visiting
-// order inside a window as the general kernel: (0,0), (0,1), (1,0), (1,1), strictly-greater wins.
+// 2x2 windows, stride 2, rows of whole 16-byte vectors: a work item is one 16-byte vector from each of the two
+// rows of a row pair (4 f32 / 8 bf16 elements: 2 / 4 neighbouring windows), so every load instruction of a wave
+// covers 1 KB of contiguous memory, and the 8 bytes of results leave as one streaming store.  The grid is sized to
+// the chip and strides over the items two at a time: both items' loads are in flight before the first compare.
+// Same visiting order inside a window as the general kernel: (0,0), (0,1), (1,0), (1,1), strictly-greater wins.
 template <typename T>
-struct Row8 {
-    T e[8];
+struct PoolVec {
+    static constexpr int VEC = 16 / (int)sizeof(T), NW = VEC / 2;
+    T e[VEC];
 };
-template <typename T>
-__device__ __forceinline__ Row8<T> load_row8(const T *p) {
-    Row8<T> r;
-    if constexpr (sizeof(T) == 4) {
-        *(u32x4 *)&r.e[0] = __builtin_nontemporal_load((const u32x4 *)p);
-        *(u32x4 *)&r.e[4] = __builtin_nontemporal_load((const u32x4 *)p + 1);
-    } else {
-        *(u32x4 *)&r.e[0] = __builtin_nontemporal_load((const u32x4 *)p);
-    }
-    return r;
-}
-template <typename T>
-__device__ __forceinline__ void store_row8(T *p, const Row8<T> &r) {
-    if constexpr (sizeof(T) == 4) {
-        *((u32x4 *)p) = *(const u32x4 *)&r.e[0];
-        *((u32x4 *)p + 1) = *(const u32x4 *)&r.e[4];
-    } else {
-        *((u32x4 *)p) = *(const u32x4 *)&r.e[0];
-    }
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct Pool2x2Item {
+    size_t in_off, out_off;  // element offsets of the row pair's vector and of its outputs
+};
+__device__ __forceinline__ Pool2x2Item pool2x2_item(const PoolParams &p, uint32_t g, int vec) {
+    uint32_t orow, gi, plane, ho;
+    p.div_gpr.divmod(g, orow, gi);     // orow = plane * oh + ho
+    p.div_oh.divmod(orow, plane, ho);
+    Pool2x2Item it;
+    it.in_off = ((size_t)plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)gi * vec;
+    it.out_off = (size_t)orow * p.ow + (size_t)gi * (vec / 2);
+    return it;
 }
 
 template <typename T>
 __global__ __launch_bounds__(kThreads) void max_pool2_2x2_kernel(const T *__restrict__ x, T *__restrict__ y,
-                                                                  PoolParams p, size_t groups) {
-    const size_t g = (size_t)blockIdx.x * kThreads + threadIdx.x;
-    if (g >= groups) return;
-    const uint32_t gpr = (uint32_t)p.ow >> 2;  // groups per output row
-    const size_t orow = g / gpr;               // plane * oh + ho
-    const uint32_t gi = (uint32_t)(g - orow * gpr);
-    const size_t plane = orow / p.oh;
-    const uint32_t ho = (uint32_t)(orow - plane * p.oh);
-    const T *src = x + (plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)gi * 8;
-    const Row8<T> r0 = load_row8(src), r1 = load_row8(src + p.iw);
-    __align__(16) T out[4];
+                                                                  PoolParams p, uint32_t groups) {
+    constexpr int VEC = PoolVec<T>::VEC, NW = PoolVec<T>::NW;
+    const uint32_t stride = gridDim.x * kThreads;
+    for (uint32_t g0 = blockIdx.x * kThreads + threadIdx.x; g0 < groups; g0 += 2 * stride) {
+        const uint32_t g1 = g0 + stride;
+        const bool two = g1 < groups;
+        const Pool2x2Item it0 = pool2x2_item(p, g0, VEC), it1 = pool2x2_item(p, two ? g1 : g0, VEC);
+        PoolVec<T> r[2][2];
+        *(u32x4 *)r[0][0].e = __builtin_nontemporal_load((const u32x4 *)(x + it0.in_off));
+        *(u32x4 *)r[0][1].e = __builtin_nontemporal_load((const u32x4 *)(x + it0.in_off + p.iw));
+        *(u32x4 *)r[1][0].e = __builtin_nontemporal_load((const u32x4 *)(x + it1.in_off));
+        *(u32x4 *)r[1][1].e = __builtin_nontemporal_load((const u32x4 *)(x + it1.in_off + p.iw));
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        T m = r0.e[2 * k];
-        float mf = Elem<T>::to_f32(m);
-        const T c[3] = {r0.e[2 * k + 1], r1.e[2 * k], r1.e[2 * k + 1]};
+        for (int u = 0; u < 2; ++u) {
+            if (u == 1 && !two) break;
+            __align__(8) T out[NW];
 #pragma unroll
-        for (int q = 0; q < 3; ++q) {
-            const float vf = Elem<T>::to_f32(c[q]);
-            if (vf > mf) { m = c[q]; mf = vf; }
+            for (int k = 0; k < NW; ++k) {
+                T m = r[u][0].e[2 * k];
+                float mf = Elem<T>::to_f32(m);
+                const T c[3] = {r[u][0].e[2 * k + 1], r[u][1].e[2 * k], r[u][1].e[2 * k + 1]};
+#pragma unroll
+                for (int q = 0; q < 3; ++q) {
+                    const float vf = Elem<T>::to_f32(c[q]);
+                    if (vf > mf) { m = c[q]; mf = vf; }
+                }
+                out[k] = m;
+            }
+            __builtin_nontemporal_store(*(const u32x2 *)out, (u32x2 *)(y + (u ? it1.out_off : it0.out_off)));
         }
-        out[k] = m;
     }
-    T *dst = y + orow * p.ow + (size_t)gi * 4;
-    if constexpr (sizeof(T) == 4) *(u32x4 *)dst = *(const u32x4 *)out;
-    else *(uint2 *)dst = *(const uint2 *)out;
 }
 
 template <typename T>
 __global__ __launch_bounds__(kThreads) void max_pool2_backward_2x2_kernel(T *__restrict__ dx, const T *__restrict__ dy,
-                                                                           PoolParams p, size_t groups) {
-    const size_t g = (size_t)blockIdx.x * kThreads + threadIdx.x;
-    if (g >= groups) return;
-    const uint32_t gpr = (uint32_t)p.ow >> 2;
-    const size_t orow = g / gpr;
-    const uint32_t gi = (uint32_t)(g - orow * gpr);
-    const size_t plane = orow / p.oh;
-    const uint32_t ho = (uint32_t)(orow - plane * p.oh);
-    T *win = dx + (plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)gi * 8;
-    Row8<T> r0 = load_row8(win), r1 = load_row8(win + p.iw);
-    __align__(16) T gy[4];
-    const T *gsrc = dy + orow * p.ow + (size_t)gi * 4;
-    if constexpr (sizeof(T) == 4) *(u32x4 *)gy = *(const u32x4 *)gsrc;
-    else *(uint2 *)gy = *(const uint2 *)gsrc;
+                                                                           PoolParams p, uint32_t groups) {
+    constexpr int VEC = PoolVec<T>::VEC, NW = PoolVec<T>::NW;
+    const uint32_t stride = gridDim.x * kThreads;
+    for (uint32_t g0 = blockIdx.x * kThreads + threadIdx.x; g0 < groups; g0 += 2 * stride) {
+        const uint32_t g1 = g0 + stride;
+        const bool two = g1 < groups;
+        const Pool2x2Item it0 = pool2x2_item(p, g0, VEC), it1 = pool2x2_item(p, two ? g1 : g0, VEC);
+        PoolVec<T> r[2][2];
+        __align__(8) T gy[2][NW];
+        *(u32x4 *)r[0][0].e = __builtin_nontemporal_load((const u32x4 *)(dx + it0.in_off));
+        *(u32x4 *)r[0][1].e = __builtin_nontemporal_load((const u32x4 *)(dx + it0.in_off + p.iw));
+        *(u32x2 *)gy[0] = __builtin_nontemporal_load((const u32x2 *)(dy + it0.out_off));
+        *(u32x4 *)r[1][0].e = __builtin_nontemporal_load((const u32x4 *)(dx + it1.in_off));
+        *(u32x4 *)r[1][1].e = __builtin_nontemporal_load((const u32x4 *)(dx + it1.in_off + p.iw));
+        *(u32x2 *)gy[1] = __builtin_nontemporal_load((const u32x2 *)(dy + it1.out_off));
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        float mf = Elem<T>::to_f32(r0.e[2 * k]);
-        int am = 0;
-        const T c[3] = {r0.e[2 * k + 1], r1.e[2 * k], r1.e[2 * k + 1]};
+        for (int u = 0; u < 2; ++u) {
+            if (u == 1 && !two) break;
 #pragma unroll
-        for (int q = 0; q < 3; ++q) {
-            const float vf = Elem<T>::to_f32(c[q]);
-            if (vf > mf) { mf = vf; am = q + 1; }
+            for (int k = 0; k < NW; ++k) {
+                float mf = Elem<T>::to_f32(r[u][0].e[2 * k]);
+                int am = 0;
+                const T c[3] = {r[u][0].e[2 * k + 1], r[u][1].e[2 * k], r[u][1].e[2 * k + 1]};
+#pragma unroll
+                for (int q = 0; q < 3; ++q) {
+                    const float vf = Elem<T>::to_f32(c[q]);
+                    if (vf > mf) { mf = vf; am = q + 1; }
+                }
+                // `0 + dy` in T, as the host's `+=` on the zeroed cell computes it
+                const T gv = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(gy[u][k]));
+                r[u][0].e[2 * k] = am == 0 ? gv : Elem<T>::zero();
+                r[u][0].e[2 * k + 1] = am == 1 ? gv : Elem<T>::zero();
+                r[u][1].e[2 * k] = am == 2 ? gv : Elem<T>::zero();
+                r[u][1].e[2 * k + 1] = am == 3 ? gv : Elem<T>::zero();
+            }
+            T *win = dx + (u ? it1.in_off : it0.in_off);
+            __builtin_nontemporal_store(*(const u32x4 *)r[u][0].e, (u32x4 *)win);
+            __builtin_nontemporal_store(*(const u32x4 *)r[u][1].e, (u32x4 *)(win + p.iw));
         }
-        // `0 + dy` in T, as the host's `+=` on the zeroed cell computes it
-        const T gv = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(gy[k]));
-        r0.e[2 * k] = am == 0 ? gv : Elem<T>::zero();
-        r0.e[2 * k + 1] = am == 1 ? gv : Elem<T>::zero();
-        r1.e[2 * k] = am == 2 ? gv : Elem<T>::zero();
-        r1.e[2 * k + 1] = am == 3 ? gv : Elem<T>::zero();
     }
-    store_row8(win, r0);
-    store_row8(win + p.iw, r1);
 }
 
-inline bool pool_2x2_fast(const PoolParams &p, const void *a, const void *b) {
-    return p.h == 2 && p.w == 2 && p.sh == 2 && p.sw == 2 && p.iw % 8 == 0 && (((uintptr_t)a | (uintptr_t)b) & 15) == 0;
+template <typename T>
+inline bool pool_2x2_fast(const PoolParams &p, const void *a, const void *b, size_t total) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    return p.h == 2 && p.w == 2 && p.sh == 2 && p.sw == 2 && p.iw % VEC == 0 && (((uintptr_t)a | (uintptr_t)b) & 15) == 0 &&
+           total / (VEC / 2) < 0x7FFFFFFFull;
+}
+// blocks for a grid-stride pass over `groups` items, two per thread and trip.  Measured at 256 x 64 x 56 x 56: a grid
+// of 16 workgroups per CU (several trips per thread) is 7 % slower than one that gives most threads a single trip,
+// so the cap only bounds the grid for very large inputs
+inline unsigned pool_2x2_grid(size_t groups) {
+    const size_t want = (groups + 2 * kThreads - 1) / (2 * kThreads);
+    const size_t cap = (size_t)(compute_units() > 0 ? compute_units() : 256) * 64;
+    return (unsigned)std::max<size_t>(1, std::min(want, cap));
 }
 
 // Overlapping windows: the host visits windows of a plane one after another and each sees
@@ -1251,10 +1272,12 @@ int max_pool2_launch(const char *name, const void *x, void *y, int64_t bc, int64
     if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
     size_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
-    if (pool_2x2_fast(p, x, y)) {
-        const size_t groups = total / 4;
-        hipLaunchKernelGGL(max_pool2_2x2_kernel<T>, dim3((unsigned)((groups + kThreads - 1) / kThreads)), dim3(kThreads),
-                           0, stream(), (const T *)x, (T *)y, p, groups);
+    if (pool_2x2_fast<T>(p, x, y, total)) {
+        constexpr int VEC = 16 / (int)sizeof(T);
+        const size_t groups = total / (VEC / 2);
+        p.div_gpr = FastDiv((uint32_t)(p.iw / VEC));
+        hipLaunchKernelGGL(max_pool2_2x2_kernel<T>, dim3(pool_2x2_grid(groups)), dim3(kThreads),
+                           0, stream(), (const T *)x, (T *)y, p, (uint32_t)groups);
         AGH_LAUNCH_CHECK(name);
         return AGH_OK;
     }
@@ -1273,10 +1296,12 @@ int max_pool2_backward_launch(const char *name, void *dx, const void *dy, int64_
     const size_t total = (size_t)bc * p.oh * p.ow;
     if (total == 0) return AGH_OK;
     if (!dx || !dy) return fail(AGH_ENULL, "%s: null buffer", name);
-    if (pool_2x2_fast(p, dx, dy) && total / 4 <= 0x7FFFFFFFull * kThreads) {
-        const size_t groups = total / 4;
-        hipLaunchKernelGGL(max_pool2_backward_2x2_kernel<T>, dim3((unsigned)((groups + kThreads - 1) / kThreads)),
-                           dim3(kThreads), 0, stream(), (T *)dx, (const T *)dy, p, groups);
+    if (pool_2x2_fast<T>(p, dx, dy, total)) {
+        constexpr int VEC = 16 / (int)sizeof(T);
+        const size_t groups = total / (VEC / 2);
+        p.div_gpr = FastDiv((uint32_t)(p.iw / VEC));
+        hipLaunchKernelGGL(max_pool2_backward_2x2_kernel<T>, dim3(pool_2x2_grid(groups)),
+                           dim3(kThreads), 0, stream(), (T *)dx, (const T *)dy, p, (uint32_t)groups);
     } else if (sh >= h && sw >= w) {
         size_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
