@@ -40,6 +40,121 @@ __global__ __launch_bounds__(kThreads) void assign_kernel(const T *__restrict__ 
     }
 }
 
+// Batched 2-D transposition through LDS, for copies whose source and destination are both contiguous, but along
+// different dimensions (NHWC <-> NCHW, `t().to_standard_layout()`): index space [b0, b1, R, C] with the source
+// contiguous along R and the destination along C.  A workgroup moves a 64 x 64 tile: 16-byte loads along R, one
+// 32-bit LDS slot per element in a tile of odd pitch (both the scattering writes and the gathering reads are
+// conflict-free), 16-byte stores along C.  VEC = 1 is the same walk element by element for unaligned views.
+struct TransposeParams {
+    int64_t sx_b0, sx_b1, sx_c;  // source strides of the batch dimensions and of C (its stride along R is 1)
+    int64_t sy_b0, sy_b1, sy_r;  // destination strides of the batch dimensions and of R (its stride along C is 1)
+    int R, C, tiles_r, tiles_c;
+    FastDiv div_tiles, div_tc, div_b1;
+};
+constexpr int kTT = 64, kTPitch = kTT + 1;
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kThreads) void transpose_tile_kernel(const T *__restrict__ x, T *__restrict__ y, TransposeParams p) {
+    __shared__ uint32_t tile[kTT * kTPitch];
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int EPW = 4 / (int)sizeof(T);  // elements per 32-bit word of a vector register
+    uint32_t bidx, t, tr, tc, b0, b1;
+    p.div_tiles.divmod(blockIdx.x, bidx, t);
+    p.div_tc.divmod(t, tr, tc);
+    p.div_b1.divmod(bidx, b0, b1);
+    const int r_base = tr * kTT, c_base = tc * kTT;
+    const T *xs = x + (int64_t)b0 * p.sx_b0 + (int64_t)b1 * p.sx_b1;
+    T *yd = y + (int64_t)b0 * p.sy_b0 + (int64_t)b1 * p.sy_b1;
+    constexpr int VPT = kTT * kTT / VEC / kThreads, VPL = kTT / VEC;  // vectors per thread, vectors per tile line
+    // ---- load along R ----
+    u32x4 reg[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int v = threadIdx.x + k * kThreads, rv = v % VPL, c = v / VPL;
+        const int r = r_base + rv * VEC, cg = c_base + c;
+        reg[k] = u32x4{0, 0, 0, 0};
+        if (r < p.R && cg < p.C) {
+            const T *src = xs + (int64_t)cg * p.sx_c + r;
+            if constexpr (VEC * sizeof(T) == 16) reg[k] = __builtin_nontemporal_load((const u32x4 *)src);
+            else reg[k].x = (uint32_t)*src;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int v = threadIdx.x + k * kThreads, rv = v % VPL, c = v / VPL;
+        const uint32_t w[4] = {reg[k].x, reg[k].y, reg[k].z, reg[k].w};
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            uint32_t e = w[i / EPW];
+            if constexpr (sizeof(T) == 2) e = (e >> (16 * (i % EPW))) & 0xFFFFu;
+            tile[(rv * VEC + i) * kTPitch + c] = e;
+        }
+    }
+    __syncthreads();
+    // ---- store along C ----
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int v = threadIdx.x + k * kThreads, cv = v % VPL, r = v / VPL;
+        const int rg = r_base + r, c = c_base + cv * VEC;
+        if (rg < p.R && c < p.C) {
+            uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const uint32_t e = tile[r * kTPitch + cv * VEC + i];
+                if constexpr (sizeof(T) == 2) w[i / EPW] |= e << (16 * (i % EPW));
+                else w[i] = e;
+            }
+            T *dst = yd + (int64_t)rg * p.sy_r + c;
+            if constexpr (VEC * sizeof(T) == 16) __builtin_nontemporal_store(u32x4{w[0], w[1], w[2], w[3]}, (u32x4 *)dst);
+            else *dst = (T)w[0];
+        }
+    }
+}
+
+// Recognises the transposition pattern after dropping unit dimensions and merging dimensions that are contiguous
+// in both views; returns 1 when the copy is not of that kind (the caller takes the element-wise kernel).
+template <typename T>
+int transpose_try(const char *name, const T *x, const int64_t (&sx)[4], T *y, const int64_t (&sy)[4], const int64_t (&d)[4]) {
+    int64_t dd[4], ax[4], ay[4];
+    int n = 0;
+    for (int i = 0; i < 4; ++i) {
+        if (d[i] == 1) continue;
+        if (n > 0 && ax[n - 1] == sx[i] * d[i] && ay[n - 1] == sy[i] * d[i]) {  // dimension n-1 and i are one dimension
+            dd[n - 1] *= d[i]; ax[n - 1] = sx[i]; ay[n - 1] = sy[i];
+        } else {
+            dd[n] = d[i]; ax[n] = sx[i]; ay[n] = sy[i]; ++n;
+        }
+    }
+    int ir = -1, ic = -1;
+    for (int i = 0; i < n; ++i) {
+        if (ax[i] == 1 && ir < 0) ir = i;
+        if (ay[i] == 1 && ic < 0) ic = i;
+    }
+    if (ir < 0 || ic < 0 || ir == ic || dd[ir] < 16 || dd[ic] < 16) return 1;
+    int64_t bd[2] = {1, 1}, bsx[2] = {0, 0}, bsy[2] = {0, 0};
+    int nb = 0;
+    for (int i = 0; i < n; ++i)
+        if (i != ir && i != ic) { bd[nb] = dd[i]; bsx[nb] = ax[i]; bsy[nb] = ay[i]; ++nb; }
+    TransposeParams p;
+    p.sx_b0 = bsx[0]; p.sx_b1 = bsx[1]; p.sx_c = ax[ic];
+    p.sy_b0 = bsy[0]; p.sy_b1 = bsy[1]; p.sy_r = ay[ir];
+    p.R = (int)dd[ir]; p.C = (int)dd[ic];
+    p.tiles_r = (p.R + kTT - 1) / kTT; p.tiles_c = (p.C + kTT - 1) / kTT;
+    const int64_t tiles = (int64_t)p.tiles_r * p.tiles_c, blocks = tiles * bd[0] * bd[1];
+    if (blocks > 0x7FFFFFFFll) return 1;
+    p.div_tiles = FastDiv((uint32_t)tiles);
+    p.div_tc = FastDiv((uint32_t)p.tiles_c);
+    p.div_b1 = FastDiv((uint32_t)bd[1]);
+    constexpr int V = 16 / (int)sizeof(T);
+    auto mult = [](int64_t v) { return v % V == 0; };
+    const bool vec = p.R % V == 0 && p.C % V == 0 && mult(p.sx_c) && mult(p.sx_b0) && mult(p.sx_b1) && mult(p.sy_r) &&
+                     mult(p.sy_b0) && mult(p.sy_b1) && (((uintptr_t)x | (uintptr_t)y) & 15) == 0;
+    if (vec) hipLaunchKernelGGL((transpose_tile_kernel<T, V>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), x, y, p);
+    else hipLaunchKernelGGL((transpose_tile_kernel<T, 1>), dim3((unsigned)blocks), dim3(kThreads), 0, stream(), x, y, p);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
 template <typename T>
 int assign_launch(const char *name, const void *x, int64_t off_x, const int64_t (&sx)[4], void *y, int64_t off_y,
                   const int64_t (&sy)[4], const int64_t (&d)[4]) {
@@ -53,6 +168,11 @@ int assign_launch(const char *name, const void *x, int64_t off_x, const int64_t 
     }
     if (total == 0) return AGH_OK;
     if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+    // large transposing copies go through LDS tiles; everything else one element per thread
+    if (total >= 4096) {
+        const int rc = transpose_try<T>(name, (const T *)x + off_x, sx, (T *)y + off_y, sy, d);
+        if (rc != 1) return rc;
+    }
     AssignParams p;
     for (int i = 0; i < 4; ++i) { p.sx[i] = sx[i]; p.sy[i] = sy[i]; }
     p.div1 = FastDiv((uint32_t)(d[1] * d[2] * d[3]));

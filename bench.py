@@ -256,6 +256,14 @@ def main():
                 x._ptr(), w4._ptr(), bcv._ptr(), yc._ptr(), bs, ci, hw, hw, co, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0)),
                 2.0 * bs * hw * hw * 576 * co, "TFLOP/s", peak)
             del yc, bcv, w4
+            # NHWC -> NCHW copy of the layer's activation (`permuted_axes([0,3,1,2]).to_standard_layout()`, which the
+            # reference's conv2_im2col ends with): the LDS-tiled transposition in agh_assign
+            nhwc, nchw = ag.Tensor.uninit((bs, hw, hw, co), dt), ag.Tensor.uninit((bs, co, hw, hw), dt)
+            fn_a = getattr(ag.lib, f"agh_assign_{dt}")
+            run(f"assign_nhwc_to_nchw_{dt}_256x128x56x56", lambda: ag._ffi.check(fn_a(
+                nhwc._ptr(), 0, hw * hw * co, 1, hw * co, co, nchw._ptr(), 0, co * hw * hw, hw * hw, hw, 1, bs, co, hw, hw)),
+                2.0 * es * bs * co * hw * hw, "GB/s", PEAK_HBM_GBS)
+            del nhwc, nchw
             dx = ag.Tensor.uninit((bs, ci, hw, hw), dt)
             run(f"col2im_{dt}_conv3x3_b256", lambda: ag._ffi.check(fn_c(cols._ptr(), dx._ptr(), bs, ci, hw, hw, 3, 3, 1, 1, 1, 1, 1, 1)),
                 bytes_, "GB/s", PEAK_HBM_GBS)

@@ -53,6 +53,34 @@ def test_assign_strided_views(ag, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_assign_large_transposing_copies(ag, dtype):
+    """`to_standard_layout` of permuted views whose source and destination are contiguous along different axes
+    (src/tensor/ops.rs:257-318, the NHWC <-> NCHW copies of layer.rs:1000-1004 and autograd.rs:396-445): these
+    take the LDS-tiled path.  Bit-exact against the oracle's strided copy: whole and partial 64 x 64 tiles, the
+    16-byte and the element-wise form (odd sizes, views at odd offsets), one and two batch dimensions,
+    and the Conv2 activation of the benchmark list (256 x 128 x 56 x 56) in both directions."""
+    rng = np.random.default_rng(44)
+    cases = [((4, 64, 64), (0, 2, 1)), ((3, 128, 200), (0, 2, 1)), ((2, 3, 72, 40), (0, 1, 3, 2)), ((5, 17, 33), (0, 2, 1)),
+             ((1, 100, 1000), (0, 2, 1)), ((2, 56, 56, 128), (0, 3, 1, 2)), ((2, 128, 56, 56), (0, 2, 3, 1)),
+             ((7, 19, 23, 16), (0, 3, 1, 2)), ((300, 70), (1, 0)), ((4, 5, 96, 80), (1, 0, 3, 2))]
+    for shape, axes in cases:
+        base = to_dtype(rng.standard_normal(shape), dtype)
+        got = ag.Tensor.from_array(base).permuted_axes(axes).to_standard_layout().into_array()
+        assert np.array_equal(got, orc.to_standard_layout(base.transpose(axes))), (shape, axes)
+    # a view at an odd element offset with an odd row stride: the element-wise tiles
+    big = to_dtype(rng.standard_normal((3, 131, 77)), dtype)
+    t = ag.Tensor.from_array(big)
+    view = ag.Tensor(t.buffer, (3, 64, 129), (131 * 77, 1, 77), 1 * 77 + 5, dtype)  # big[:, 1:130, 5:69] transposed
+    assert np.array_equal(view.to_standard_layout().into_array(), np.ascontiguousarray(big[:, 1:130, 5:69].transpose(0, 2, 1)))
+    # the benchmark's activation, NHWC -> NCHW and back
+    act = to_dtype(rng.standard_normal((256, 56, 56, 128), dtype=np.float32), dtype)
+    nchw = ag.Tensor.from_array(act).permuted_axes((0, 3, 1, 2)).to_standard_layout()
+    assert np.array_equal(nchw.into_array(), orc.to_standard_layout(act.transpose(0, 3, 1, 2)))
+    back = nchw.permuted_axes((0, 2, 3, 1)).to_standard_layout().into_array()
+    assert np.array_equal(back, act)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_scaled_add_sgd_sum_axis0_bit_exact(ag, dtype):
     rng = np.random.default_rng(42)
     for n in (1, 255, 46920, 300001):
