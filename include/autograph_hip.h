@@ -262,7 +262,11 @@ int agh_conv2_backward_input_bf16(const void *dy, const void *w, void *dx, int64
  * whole 16-byte vectors (returns AGH_ERANGE otherwise: use im2col + gemm).  Same result as the
  * conv2_im2col chain (src/learn/neural_network/layer.rs:950-1005) up to f32 summation order;
  * the reference's host has the analogous conv_direct path (layer/conv_direct.rs:23-83).
- * x: [bs,ic,ih,iw], w: [oc,ic,fh,fw], bias: null or [oc] (conv2's add_assign, layer.rs:944-946),
+ * x: [bs,ic,ih,iw], w: [oc,ic,fh,fw], bias: null or [oc], added PER OUTPUT CHANNEL (bias[o] to every
+ * y[b,o,:,:]).  The reference's conv2 calls `output.add_assign(bias)` (layer.rs:944-946), whose broadcast
+ * (autograd.rs:571-599) aligns a [oc] vector with the TRAILING axis of [bs,oc,oh,ow] and so only accepts
+ * ow == oc; no reference test or benchmark gives Conv2 a bias, so the per-channel reading is this
+ * library's and is not pinned by the reference.
  * act: the Relu layer that follows (layer.rs:1254-1267), pool2x2 != 0: also the MaxPool2 with
  * filter [2,2] and stride [2,2] that follows (layer.rs:1193-1216) with its first-strict-max rule.
  * y: [bs,oc,oh,ow], or [bs,oc,oh/2,ow/2] with the pool.  Rounding order as the separate
