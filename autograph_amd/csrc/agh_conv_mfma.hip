@@ -30,7 +30,6 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
 constexpr int kThreads = 256;
 constexpr int kTileOc = 128;   // output channels per workgroup (4 MFMA tiles of 32, one per wave)
-constexpr int kBRing = 8, kBAhead = kBRing - 1;  // register sets of B fragments, and how many steps ahead they are requested
 
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F &&f) {
@@ -80,15 +79,16 @@ __global__ __launch_bounds__(kThreads) void pack_filter_kernel(const T *__restri
     wp[dst] = w[e];
 }
 
-// kTilePos output positions per workgroup (kMT MFMA tiles of 32), kWgs workgroups per CU.
-template <typename T, int kTilePos, int kWgs>
+// kTilePos output positions per workgroup (kMT MFMA tiles of 32), kWgs workgroups per CU, kBRing register sets of B
+// fragments (requested kBRing - 1 steps ahead).
+template <typename T, int kTilePos, int kWgs, int kBRing>
 __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__restrict__ x, const T *__restrict__ wp,
                                                                                   const T *__restrict__ bias, T *__restrict__ y,
                                                                                   ConvMfmaParams p) {
     extern __shared__ __align__(16) unsigned char lds[];
     constexpr int ES = Geo<T>::ES, CPC = Geo<T>::CPC, PV = Geo<T>::CPC, kEpitch = Geo<T>::EPITCH, kEpiPos = Geo<T>::EPI_POS;
-    constexpr int kMT = kTilePos / 32, kEpiMT = kEpiPos / 32;
-    static_assert(kTilePos % kEpiPos == 0, "the epilogue takes whole groups of position tiles");
+    constexpr int kMT = kTilePos / 32, kEpiMT = kEpiPos / 32, kBAhead = kBRing - 1;
+    static_assert(kTilePos % 32 == 0, "whole MFMA tiles");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     uint32_t t0, oct, b, tile;
@@ -119,9 +119,9 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
         const uint32_t items = (uint32_t)lrows * ngrp * nvec;
         const T *ximg = x + ((size_t)b * p.ic + (size_t)pass * p.icc) * p.ih * (size_t)p.iw;
         const size_t plane = (size_t)p.ih * p.iw;
-        // two items per thread and trip: all 2 * CPC loads are requested before the first LDS write, so a
-        // workgroup's staging waits for memory about once (448 items at the 64-channel 56 x 56 layer)
-        constexpr int SB = 2;
+        // SB items per thread and trip: all SB * CPC loads are requested before the first LDS write (with two, a
+        // workgroup's staging waits for memory about once: 448 items at the 64-channel 56 x 56 layer)
+        constexpr int SB = kWgs >= 3 ? 1 : 2;  // three workgroups per CU leave 170 registers: one item at a time
         for (uint32_t it0 = tid; it0 < items; it0 += kThreads * SB) {
             uint4 r[SB][CPC];
             int dst[SB];
@@ -287,10 +287,12 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
         const int o_lane = oc0 + l32;
         float bq = 0.0f;
         if (p.has_bias) bq = Elem<T>::to_f32(bias[min(o_lane, p.oc - 1)]);
+        // the position tiles leave in groups of kEpiMT (256 bytes of every output row), the last group may be smaller
+        static_for<(kMT + kEpiMT - 1) / kEpiMT>([&](auto partc) {
+            constexpr int part = decltype(partc)::value;
+            constexpr int NMT = (kMT - part * kEpiMT) < kEpiMT ? (kMT - part * kEpiMT) : kEpiMT;
 #pragma unroll
-        for (int part = 0; part < kTilePos / kEpiPos; ++part) {
-#pragma unroll
-            for (int m4 = 0; m4 < kEpiMT; ++m4)
+            for (int m4 = 0; m4 < NMT; ++m4)
 #pragma unroll
                 for (int blk = 0; blk < 4; ++blk) {
                     const int mt = part * kEpiMT + m4;
@@ -335,16 +337,18 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
                     }
                 }
             // same wave, LDS executes in order: the reads below see the writes above, and the next part's
-            // writes come after these reads.  A staged row is 256 bytes = 16 chunks: a store instruction covers 4 rows.
-            constexpr int CPRW = 16, RPI = 64 / CPRW, NST = 32 / RPI;
+            // writes come after these reads.  A staged row of NMT tiles is NMT * 64 bytes = 4 * NMT chunks (in either
+            // element type: 32 positions are 64 or 128 bytes, and kEpiMT is 4 or 2).
+            constexpr int CPRW = NMT * 32 * ES / 16, TOTAL = 32 * CPRW, NST = (TOTAL + 63) / 64;
 #pragma unroll
             for (int r = 0; r < NST; ++r) {
-                const int row = r * RPI + lane / CPRW, chunk = lane % CPRW;
+                const int idx = r * 64 + lane, row = idx / CPRW, chunk = idx % CPRW;
+                if (TOTAL % 64 != 0 && idx >= TOTAL) continue;
                 const uint4 v = *(const uint4 *)(region + row * kEpitch + chunk * 16);
                 const int pos = p0 + part * kEpiPos + chunk * CPC, o = oc0 + row;
                 if (pos < p.npos && o < p.oc) *(uint4 *)(y + ((size_t)b * p.oc + o) * p.npos + pos) = v;
             }
-        }
+        });
     }
 }
 
@@ -354,7 +358,7 @@ namespace agh {
 
 // Returns 1 when the geometry is not one this kernel takes (the caller goes on to its other paths),
 // otherwise a status code.  The API lock is held by the caller.
-template <typename T, int kTilePos, int kWgs>
+template <typename T, int kTilePos, int kWgs, int kBRing>
 static int conv2_mfma_launch(const char *name, const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic, int64_t ih,
                    int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t oh, int64_t ow, int act) {
     constexpr int ES = Geo<T>::ES, CPC = Geo<T>::CPC;
@@ -398,10 +402,10 @@ static int conv2_mfma_launch(const char *name, const void *x, const void *w, con
     p.div_vec = FastDiv((uint32_t)(iw / CPC));
     static bool attr_done = false;
     if (!attr_done) {
-        AGH_HIP(hipFuncSetAttribute((const void *)(conv2_mfma_kernel<T, kTilePos, kWgs>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
+        AGH_HIP(hipFuncSetAttribute((const void *)(conv2_mfma_kernel<T, kTilePos, kWgs, kBRing>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
         attr_done = true;
     }
-    hipLaunchKernelGGL((conv2_mfma_kernel<T, kTilePos, kWgs>), dim3((unsigned)blocks), dim3(kThreads), (size_t)smem, stream(), (const T *)x,
+    hipLaunchKernelGGL((conv2_mfma_kernel<T, kTilePos, kWgs, kBRing>), dim3((unsigned)blocks), dim3(kThreads), (size_t)smem, stream(), (const T *)x,
                        (const T *)wperm, (const T *)bias, (T *)y, p);
     AGH_LAUNCH_CHECK(name);
     return AGH_OK;
@@ -417,8 +421,8 @@ int conv2_mfma_try(const char *name, const void *x, const void *w, const void *b
     const char *e = getenv("AGH_CONV_TILE");
     const int tile = e && *e ? atoi(e) : (sizeof(T) == 4 ? 128 : 256);
     if (tile == 128)
-        return conv2_mfma_launch<T, 128, 3>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
-    return conv2_mfma_launch<T, 256, 2>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
+        return conv2_mfma_launch<T, 128, 3, 8>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
+    return conv2_mfma_launch<T, 256, 2, 8>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
 }
 
 template int conv2_mfma_try<uint16_t>(const char *, const void *, const void *, const void *, void *, int64_t, int64_t, int64_t, int64_t,
