@@ -73,6 +73,8 @@ SIGNATURES = {
     "agh_conv2_direct_bf16": ([ptr, ptr, ptr, ptr] + [i64] * 13 + [C.c_int, C.c_int], C.c_int),
     "agh_lenet5_forward_f32": ([ptr] * 8 + [i64], C.c_int),
     "agh_lenet5_forward_bf16": ([ptr] * 8 + [i64], C.c_int),
+    "agh_lenet5_forward_train_f32": ([ptr] * 16 + [i64], C.c_int),
+    "agh_lenet5_forward_train_bf16": ([ptr] * 16 + [i64], C.c_int),
     "agh_max_pool2_f32": (_POOL, C.c_int),
     "agh_max_pool2_bf16": (_POOL, C.c_int),
     "agh_max_pool2_backward_f32": (_POOL, C.c_int),

@@ -329,11 +329,42 @@ __device__ __forceinline__ float relu_pool_window(const float (&acc)[2][WT][OCT]
     return mf;  // activations stay in LDS as f32 copies of the T values
 }
 
+// What a training step needs from the forward pass besides the logits (all [bs, ...] in standard layout): the
+// convolution outputs before the relu (c1 [6,24,24], c2 [16,8,8]), the pooled activations (p1 [6,12,12], p2 [16,4,4]),
+// and the dense layers' outputs before (d1 [128], d2 [84]) and after (a1, a2) the relu.
 template <typename T>
+struct LenetSaves {
+    T *c1, *p1, *c2, *p2, *d1, *a1, *d2, *a2;
+};
+
+// N consecutive activations (N * sizeof(T) a multiple of 4 bytes, destination aligned to that size) rounded to T and
+// stored with the widest vector stores
+template <typename T, int N>
+__device__ __forceinline__ void store_rounded(T *dst, const float (&v)[N]) {
+    if constexpr (sizeof(T) == 4) {
+        if constexpr (N % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < N; i += 4) *(float4 *)((float *)dst + i) = make_float4(v[i], v[i + 1], v[i + 2], v[i + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < N; i += 2) *(float2 *)((float *)dst + i) = make_float2(v[i], v[i + 1]);
+        }
+    } else {
+        uint32_t w[N / 2];
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) w[i] = f32x2_to_bf16x2(v[2 * i], v[2 * i + 1]);
+        if constexpr (N == 8) *(uint4 *)dst = make_uint4(w[0], w[1], w[2], w[3]);
+        else if constexpr (N == 4) *(uint2 *)dst = make_uint2(w[0], w[1]);
+        else *(uint32_t *)dst = w[0];
+    }
+}
+
+template <typename T, bool SAVE>
 __global__ __launch_bounds__(512) void lenet5_forward_kernel(const T *__restrict__ x, const T *__restrict__ w1,
                                                               const T *__restrict__ w2, const T *__restrict__ wd1,
                                                               const T *__restrict__ wd2, const T *__restrict__ wd3,
-                                                              const T *__restrict__ b3, T *__restrict__ out, int bs) {
+                                                              const T *__restrict__ b3, T *__restrict__ out, int bs,
+                                                              LenetSaves<T> sv) {
     constexpr int IMGS = 4;
     __shared__ __align__(16) float xs[IMGS * 28 * 28];     // input images, pitch 28
     __shared__ __align__(16) float w1s[25 * 6];            // [tap][oc]
@@ -381,6 +412,25 @@ __global__ __launch_bounds__(512) void lenet5_forward_kernel(const T *__restrict
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 p1[((img * 6 + grp * 2 + o) * 12 + row) * 12 + wb * 4 + j] = relu_pool_window<T, 2, 8>(acc, j, o);
+        if constexpr (SAVE) {
+            if (img < nimg) {
+#pragma unroll
+                for (int o = 0; o < 2; ++o) {
+                    const size_t plane = (size_t)(b0 + img) * 6 + grp * 2 + o;
+#pragma unroll
+                    for (int a = 0; a < 2; ++a) {
+                        float v[8];
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) v[t] = acc[a][t][o];
+                        store_rounded<T, 8>(sv.c1 + (plane * 24 + 2 * row + a) * 24 + wb * 8, v);
+                    }
+                    float q[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) q[j] = p1[((img * 6 + grp * 2 + o) * 12 + row) * 12 + wb * 4 + j];
+                    store_rounded<T, 4>(sv.p1 + (plane * 12 + row) * 12 + wb * 4, q);
+                }
+            }
+        }
     }
     __syncthreads();
 
@@ -392,6 +442,20 @@ __global__ __launch_bounds__(512) void lenet5_forward_kernel(const T *__restrict
         rowpair_conv<5, 1, 4>(p1 + img * 864 + 2 * row * 12 + wb * 4, 144, 12, 6, 5, w2s + oc, 16, acc);
 #pragma unroll
         for (int j = 0; j < 2; ++j) p2[img * 256 + (oc * 4 + row) * 4 + wb * 2 + j] = relu_pool_window<T, 1, 4>(acc, j, 0);
+        if constexpr (SAVE) {
+            if (img < nimg) {
+                const size_t plane = (size_t)(b0 + img) * 16 + oc;
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    float v[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) v[t] = acc[a][t][0];
+                    store_rounded<T, 4>(sv.c2 + (plane * 8 + 2 * row + a) * 8 + wb * 4, v);
+                }
+                const float q[2] = {p2[img * 256 + (oc * 4 + row) * 4 + wb * 2], p2[img * 256 + (oc * 4 + row) * 4 + wb * 2 + 1]};
+                store_rounded<T, 2>(sv.p2 + (plane * 4 + row) * 4 + wb * 2, q);
+            }
+        }
     }
     __syncthreads();
 
@@ -436,7 +500,14 @@ __global__ __launch_bounds__(512) void lenet5_forward_kernel(const T *__restrict
         float a = 0.0f;
 #pragma unroll
         for (int kg = 0; kg < 16; ++kg) a += parts[kg * IMGS * 128 + o];
-        d1[o] = Elem<T>::to_f32(round_bias_relu<T>(a, false, Elem<T>::zero(), AGH_ACT_RELU));
+        const T act = round_bias_relu<T>(a, false, Elem<T>::zero(), AGH_ACT_RELU);
+        d1[o] = Elem<T>::to_f32(act);
+        if constexpr (SAVE) {
+            if ((o >> 7) < nimg) {
+                sv.d1[(size_t)b0 * 128 + o] = Elem<T>::from_f32(a);
+                sv.a1[(size_t)b0 * 128 + o] = act;
+            }
+        }
     }
     __syncthreads();
     // dense2 128 -> 84 + relu (weights straight from L2, 32 loads in flight per thread)
@@ -446,7 +517,14 @@ __global__ __launch_bounds__(512) void lenet5_forward_kernel(const T *__restrict
         const float *xr = d1 + r * 128;
 #pragma unroll 32
         for (int k = 0; k < 128; ++k) a = __builtin_fmaf(xr[k], Elem<T>::to_f32(wd2[k * 84 + c]), a);
-        d2[tid] = Elem<T>::to_f32(round_bias_relu<T>(a, false, Elem<T>::zero(), AGH_ACT_RELU));
+        const T act = round_bias_relu<T>(a, false, Elem<T>::zero(), AGH_ACT_RELU);
+        d2[tid] = Elem<T>::to_f32(act);
+        if constexpr (SAVE) {
+            if (r < nimg) {
+                sv.d2[(size_t)b0 * 84 + tid] = Elem<T>::from_f32(a);
+                sv.a2[(size_t)b0 * 84 + tid] = act;
+            }
+        }
     }
     __syncthreads();
     // dense3 84 -> 10 + bias
@@ -610,6 +688,30 @@ int conv2_direct_entry(const char *name, const void *x, const void *w, const voi
 
 }  // namespace
 
+template <typename T>
+int lenet5_forward_entry(const char *name, const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                         const void *wd3, const void *b3, void *logits, int64_t bs, void *const *saves) {
+    AGH_API_ENTER();
+    if (bs < 0 || bs > ((int64_t)1 << 30)) return fail(AGH_EINVAL, "%s: bad batch size", name);
+    if (bs == 0) return AGH_OK;
+    if (!x || !w1 || !w2 || !wd1 || !wd2 || !wd3 || !b3 || !logits) return fail(AGH_ENULL, "%s: null buffer", name);
+    LenetSaves<T> sv = {};
+    if (saves) {
+        for (int i = 0; i < 8; ++i)
+            if (!saves[i]) return fail(AGH_ENULL, "%s: null buffer for a saved activation", name);
+        sv = {(T *)saves[0], (T *)saves[1], (T *)saves[2], (T *)saves[3], (T *)saves[4], (T *)saves[5], (T *)saves[6], (T *)saves[7]};
+        hipLaunchKernelGGL((lenet5_forward_kernel<T, true>), dim3((unsigned)((bs + 3) / 4)), dim3(512), 0, stream(), (const T *)x,
+                           (const T *)w1, (const T *)w2, (const T *)wd1, (const T *)wd2, (const T *)wd3, (const T *)b3,
+                           (T *)logits, (int)bs, sv);
+    } else {
+        hipLaunchKernelGGL((lenet5_forward_kernel<T, false>), dim3((unsigned)((bs + 3) / 4)), dim3(512), 0, stream(), (const T *)x,
+                           (const T *)w1, (const T *)w2, (const T *)wd1, (const T *)wd2, (const T *)wd3, (const T *)b3,
+                           (T *)logits, (int)bs, sv);
+    }
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
 extern "C" {
 
 int agh_conv2_direct_f32(const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic, int64_t ih,
@@ -627,27 +729,23 @@ int agh_conv2_direct_bf16(const void *x, const void *w, const void *bias, void *
 
 int agh_lenet5_forward_f32(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
                            const void *wd3, const void *b3, void *logits, int64_t bs) {
-    AGH_API_ENTER();
-    if (bs < 0 || bs > ((int64_t)1 << 30)) return fail(AGH_EINVAL, "agh_lenet5_forward_f32: bad batch size");
-    if (bs == 0) return AGH_OK;
-    if (!x || !w1 || !w2 || !wd1 || !wd2 || !wd3 || !b3 || !logits) return fail(AGH_ENULL, "agh_lenet5_forward_f32: null buffer");
-    hipLaunchKernelGGL(lenet5_forward_kernel<float>, dim3((unsigned)((bs + 3) / 4)), dim3(512), 0, stream(),
-                       (const float *)x, (const float *)w1, (const float *)w2, (const float *)wd1, (const float *)wd2,
-                       (const float *)wd3, (const float *)b3, (float *)logits, (int)bs);
-    AGH_LAUNCH_CHECK("agh_lenet5_forward_f32");
-    return AGH_OK;
+    return lenet5_forward_entry<float>("agh_lenet5_forward_f32", x, w1, w2, wd1, wd2, wd3, b3, logits, bs, nullptr);
 }
 int agh_lenet5_forward_bf16(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
                             const void *wd3, const void *b3, void *logits, int64_t bs) {
-    AGH_API_ENTER();
-    if (bs < 0 || bs > ((int64_t)1 << 30)) return fail(AGH_EINVAL, "agh_lenet5_forward_bf16: bad batch size");
-    if (bs == 0) return AGH_OK;
-    if (!x || !w1 || !w2 || !wd1 || !wd2 || !wd3 || !b3 || !logits) return fail(AGH_ENULL, "agh_lenet5_forward_bf16: null buffer");
-    hipLaunchKernelGGL(lenet5_forward_kernel<uint16_t>, dim3((unsigned)((bs + 3) / 4)), dim3(512), 0, stream(),
-                       (const uint16_t *)x, (const uint16_t *)w1, (const uint16_t *)w2, (const uint16_t *)wd1,
-                       (const uint16_t *)wd2, (const uint16_t *)wd3, (const uint16_t *)b3, (uint16_t *)logits, (int)bs);
-    AGH_LAUNCH_CHECK("agh_lenet5_forward_bf16");
-    return AGH_OK;
+    return lenet5_forward_entry<uint16_t>("agh_lenet5_forward_bf16", x, w1, w2, wd1, wd2, wd3, b3, logits, bs, nullptr);
+}
+int agh_lenet5_forward_train_f32(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                                 const void *wd3, const void *b3, void *c1, void *p1, void *c2, void *p2, void *d1,
+                                 void *a1, void *d2, void *a2, void *logits, int64_t bs) {
+    void *saves[8] = {c1, p1, c2, p2, d1, a1, d2, a2};
+    return lenet5_forward_entry<float>("agh_lenet5_forward_train_f32", x, w1, w2, wd1, wd2, wd3, b3, logits, bs, saves);
+}
+int agh_lenet5_forward_train_bf16(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                                  const void *wd3, const void *b3, void *c1, void *p1, void *c2, void *p2, void *d1,
+                                  void *a1, void *d2, void *a2, void *logits, int64_t bs) {
+    void *saves[8] = {c1, p1, c2, p2, d1, a1, d2, a2};
+    return lenet5_forward_entry<uint16_t>("agh_lenet5_forward_train_bf16", x, w1, w2, wd1, wd2, wd3, b3, logits, bs, saves);
 }
 
 }  // extern "C"

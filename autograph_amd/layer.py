@@ -236,8 +236,17 @@ class LeNet5Trainer:
     a graph (`capture`) and replayed.  Gradients stay available in `grads` after a step.  `overlap`
     issues the weight gradients beside the input-gradient chain (`branch`); same kernels, same bits."""
 
-    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None, overlap=True):
+    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None, overlap=True, fused_forward=None):
         self.model, self.bs, self.lr = model, batch_size, learning_rate
+        # fused_forward: the forward pass is ONE launch (agh_lenet5_forward_train_*) that also writes every activation
+        # the backward edges read; the patch matrices the weight gradients multiply are then built beside the backward
+        # chain.  False: layer by layer (im2col + GEMM convolutions), eleven launches.  Default: fused in f32, where a
+        # replayed step takes 0.147-0.151 ms against 0.172; layered in bf16, where that launch is slower (0.175-0.181
+        # against 0.164 ms: at batch 100 it is 25 workgroups walking twelve layers one after the other, and its bf16
+        # form takes 30-47 us).
+        if fused_forward is None:
+            fused_forward = model.conv1.weight.dtype == "f32"
+        self.fused_forward = fused_forward
         self._branch = branch if overlap else contextlib.nullcontext
         self.opt = optimizer if optimizer is not None else SGD()
         bs, dt = batch_size, model.conv1.weight.dtype
@@ -337,16 +346,26 @@ class LeNet5Trainer:
         w1, w2, wd1, wd2, wd3, b3 = self.params
         dw1, dw2, dwd1, dwd2, dwd3, db3 = self.grads
         # forward
-        self._conv_forward(x, w1, self.cols1, self.c1)
-        self._relu_pool(self.c1, self.p1)
-        self._conv_forward(self.p1, w2, self.cols2, self.c2)
-        self._relu_pool(self.c2, self.p2)
         f = self.p2.into_shape((bs, 256))
-        gemm(1.0, f, wd1, 0.0, self.d1)
-        self._relu(self.d1, self.a1)
-        gemm(1.0, self.a1, wd2, 0.0, self.d2)
-        self._relu(self.d2, self.a2)
-        gemm(1.0, self.a2, wd3, 0.0, self.logits, bias=b3)
+        if self.fused_forward:
+            check(self._fn("agh_lenet5_forward_train")(
+                x._data_ptr(), w1._data_ptr(), w2._data_ptr(), wd1._data_ptr(), wd2._data_ptr(), wd3._data_ptr(),
+                b3._data_ptr(), self.c1._ptr(), self.p1._ptr(), self.c2._ptr(), self.p2._ptr(), self.d1._ptr(),
+                self.a1._ptr(), self.d2._ptr(), self.a2._ptr(), self.logits._ptr(), bs))
+            # the patch matrices feed only the weight gradients of the convolutions: built beside the backward chain
+            with self._branch():
+                check(self._fn("agh_im2col_conv2")(x._data_ptr(), self.cols1._ptr(), bs, 1, 28, 28, 5, 5, 0, 0, 1, 1, 1, 1))
+                check(self._fn("agh_im2col_conv2")(self.p1._ptr(), self.cols2._ptr(), bs, 6, 12, 12, 5, 5, 0, 0, 1, 1, 1, 1))
+        else:
+            self._conv_forward(x, w1, self.cols1, self.c1)
+            self._relu_pool(self.c1, self.p1)
+            self._conv_forward(self.p1, w2, self.cols2, self.c2)
+            self._relu_pool(self.c2, self.p2)
+            gemm(1.0, f, wd1, 0.0, self.d1)
+            self._relu(self.d1, self.a1)
+            gemm(1.0, self.a1, wd2, 0.0, self.d2)
+            self._relu(self.d2, self.a2)
+            gemm(1.0, self.a2, wd3, 0.0, self.logits, bias=b3)
         # backward.  The loss value and the weight gradients of the dense layers and of conv2 feed nothing
         # before the update:
         # with `overlap` they are issued together, once their operands exist, on the second stream, beside
@@ -372,8 +391,12 @@ class LeNet5Trainer:
         check(self._fn("agh_conv2_backward_input")(self.gm2._ptr(), w2._data_ptr(), self.g_p1._ptr(), bs, 6, 8, 8, 16,
                                                    5, 5, 0, 0, 1, 1, 1, 1))
         self._pool_relu_backward(self.c1, self.g_p1, self.gm1)
-        gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
-        join()
+        if self.fused_forward and self._branch is branch:
+            join()  # the patch matrix of conv1 was built on the second stream
+            gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
+        else:
+            gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
+            join()
         # update: all parameters at once (element-wise, so one launch over the shared buffers)
         self.opt.update(self.lr, self._wflat, self._gflat, self._vflat)
 

@@ -290,6 +290,19 @@ int agh_lenet5_forward_f32(const void *x, const void *w1, const void *w2, const 
 int agh_lenet5_forward_bf16(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
                             const void *wd3, const void *b3, void *logits, int64_t bs);
 
+/* The same forward pass for a training step (benches/neural-network-benches/src/autograph_backend.rs:70-86): one
+ * launch that also writes what the backward edges read (layer.rs:950-1005, :1193-1216, :1253-1267, autograd.rs:607-627):
+ * c1 [bs,6,24,24] and c2 [bs,16,8,8], the convolution outputs BEFORE the relu; p1 [bs,6,12,12] and p2 [bs,16,4,4] after
+ * relu and pooling; d1 [bs,128] and d2 [bs,84], the dense outputs before the relu, a1 and a2 after it.  Every value
+ * is rounded to T where the layer-by-layer path rounds it; convolutions and dense layers sum in f32 in another order
+ * than the GEMM kernels, so results agree with that path up to f32 summation order. */
+int agh_lenet5_forward_train_f32(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                                 const void *wd3, const void *b3, void *c1, void *p1, void *c2, void *p2, void *d1,
+                                 void *a1, void *d2, void *a2, void *logits, int64_t bs);
+int agh_lenet5_forward_train_bf16(const void *x, const void *w1, const void *w2, const void *wd1, const void *wd2,
+                                  const void *wd3, const void *b3, void *c1, void *p1, void *c2, void *p2, void *d1,
+                                  void *a1, void *d2, void *a2, void *logits, int64_t bs);
+
 /* ---------------------------------------------------------------- max pool ---- */
 
 /* MaxPool2 device branch (src/tensor/ops.rs:1117-1133; rule from the host impl

@@ -66,6 +66,8 @@ extern "C" {
     pub fn agh_conv2_direct_bf16(x: *const c_void, w: *const c_void, bias: *const c_void, y: *mut c_void, bs: i64, ic: i64, ih: i64, iw: i64, oc: i64, fh: i64, fw: i64, ph: i64, pw: i64, sh: i64, sw: i64, dh: i64, dw: i64, act: c_int, pool2x2: c_int) -> c_int;
     pub fn agh_lenet5_forward_f32(x: *const c_void, w1: *const c_void, w2: *const c_void, wd1: *const c_void, wd2: *const c_void, wd3: *const c_void, b3: *const c_void, logits: *mut c_void, bs: i64) -> c_int;
     pub fn agh_lenet5_forward_bf16(x: *const c_void, w1: *const c_void, w2: *const c_void, wd1: *const c_void, wd2: *const c_void, wd3: *const c_void, b3: *const c_void, logits: *mut c_void, bs: i64) -> c_int;
+    pub fn agh_lenet5_forward_train_f32(x: *const c_void, w1: *const c_void, w2: *const c_void, wd1: *const c_void, wd2: *const c_void, wd3: *const c_void, b3: *const c_void, c1: *mut c_void, p1: *mut c_void, c2: *mut c_void, p2: *mut c_void, d1: *mut c_void, a1: *mut c_void, d2: *mut c_void, a2: *mut c_void, logits: *mut c_void, bs: i64) -> c_int;
+    pub fn agh_lenet5_forward_train_bf16(x: *const c_void, w1: *const c_void, w2: *const c_void, wd1: *const c_void, wd2: *const c_void, wd3: *const c_void, b3: *const c_void, c1: *mut c_void, p1: *mut c_void, c2: *mut c_void, p2: *mut c_void, d1: *mut c_void, a1: *mut c_void, d2: *mut c_void, a2: *mut c_void, logits: *mut c_void, bs: i64) -> c_int;
     pub fn agh_max_pool2_f32(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_max_pool2_bf16(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_max_pool2_backward_f32(dx_inout: *mut c_void, dy: *const c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;

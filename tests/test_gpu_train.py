@@ -133,8 +133,65 @@ def lenet_params(rng):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("bs", [100, 3])
+def test_lenet5_forward_train_saves_every_activation(ag, dtype, bs):
+    """agh_lenet5_forward_train_<T>: the forward pass of a training step in one launch.  Every saved activation must be
+    what the reference's layer produces from the PREVIOUS saved activation (layer.rs:950-1005, :1134-1143, :1193-1216,
+    :1253-1267): convolutions and dense layers within the GEMM tolerances of the oracle's result on that very
+    input (they sum in f32 in another order), relu and pooling bit for bit."""
+    rng = np.random.default_rng(47)
+    params = [to_dtype(p, dtype) for p in lenet_params(rng)]
+    w1, w2, wd1, wd2, wd3, b3 = params
+    x = to_dtype(rng.uniform(0, 1, (bs, 1, 28, 28)), dtype)
+    shapes = [(bs, 6, 24, 24), (bs, 6, 12, 12), (bs, 16, 8, 8), (bs, 16, 4, 4), (bs, 128), (bs, 128), (bs, 84), (bs, 84), (bs, 10)]
+    outs = [ag.Tensor.zeros(sh, dtype) for sh in shapes]
+    tp = [ag.Tensor.from_array(p) for p in params]
+    tx = ag.Tensor.from_array(x)
+    ag._ffi.check(getattr(ag.lib, f"agh_lenet5_forward_train_{dtype}")(tx._ptr(), *[t._ptr() for t in tp], *[o._ptr() for o in outs], bs))
+    c1, p1, c2, p2, d1, a1, d2, a2, logits = [o.into_array() for o in outs]
+
+    def close(got, want64, scale64, k):
+        g = as_f32(got).astype(np.float64)
+        if dtype == "f32":
+            assert np.all(np.abs(g - want64) <= 1e-5 * np.sqrt(k) * scale64 + 1e-30)
+        else:
+            ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want64), 2.0**-126))) - 7)
+            assert np.all(np.abs(g - want64) <= ulp + 1e-2 * np.abs(want64) + 8 * np.sqrt(k) * 2.0**-24 * scale64)
+
+    f = as_f32
+    close(c1, orc.conv2_naive_f64(f(x), f(w1)), orc.conv2_naive_f64(np.abs(f(x)), np.abs(f(w1))), 25)
+    assert np.array_equal(p1, orc.max_pool2(orc.relu(c1), (2, 2)))
+    close(c2, orc.conv2_naive_f64(f(p1), f(w2)), orc.conv2_naive_f64(np.abs(f(p1)), np.abs(f(w2))), 150)
+    assert np.array_equal(p2, orc.max_pool2(orc.relu(c2), (2, 2)))
+    flat = f(p2).reshape(bs, 256).astype(np.float64)
+    close(d1, flat @ f(wd1).astype(np.float64), np.abs(flat) @ np.abs(f(wd1)).astype(np.float64), 256)
+    assert np.array_equal(a1, orc.relu(d1))
+    a1f = f(a1).astype(np.float64)
+    close(d2, a1f @ f(wd2).astype(np.float64), np.abs(a1f) @ np.abs(f(wd2)).astype(np.float64), 128)
+    assert np.array_equal(a2, orc.relu(d2))
+    a2f = f(a2).astype(np.float64)
+    # dense3: T(dot) then T(. + bias): one more rounding step than a plain product
+    want = a2f @ f(wd3).astype(np.float64) + f(b3).astype(np.float64)
+    scale = np.abs(a2f) @ np.abs(f(wd3)).astype(np.float64) + np.abs(f(b3)).astype(np.float64)
+    g = f(logits).astype(np.float64)
+    if dtype == "f32":
+        assert np.all(np.abs(g - want) <= 1e-5 * np.sqrt(84) * scale)
+    else:
+        ulp = 2.0 ** (np.floor(np.log2(np.maximum(scale, 2.0**-126))) - 7)
+        assert np.all(np.abs(g - want) <= 2 * ulp + 1e-2 * np.abs(want))
+    # the logits are those of the inference launch, bit for bit (same kernel body)
+    inf = ag.Tensor.zeros((bs, 10), dtype)
+    ag._ffi.check(getattr(ag.lib, f"agh_lenet5_forward_{dtype}")(tx._ptr(), *[t._ptr() for t in tp], inf._ptr(), bs))
+    assert np.array_equal(inf.into_array(), logits)
+    with pytest.raises(ag.AghError):  # a missing buffer is an error, never a launch
+        ag._ffi.check(getattr(ag.lib, f"agh_lenet5_forward_train_{dtype}")(tx._ptr(), *[t._ptr() for t in tp],
+                                                                         *[o._ptr() for o in outs[:3]], None, *[o._ptr() for o in outs[4:]], bs))
+
+
+@pytest.mark.parametrize("fused_forward", [True, False])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("momentum", [None, 0.01])
-def test_lenet5_train_step(ag, dtype, momentum):
+def test_lenet5_train_step(ag, dtype, momentum, fused_forward):
     rng = np.random.default_rng(44)
     params = [to_dtype(p, dtype) for p in lenet_params(rng)]
     bs = 100
@@ -143,7 +200,7 @@ def test_lenet5_train_step(ag, dtype, momentum):
     want_loss, want_params, want_grads, want_v = orc.lenet5_train_step(x, t, params, lr=0.01, momentum=momentum)
 
     model = ag.LeNet5.from_arrays(*params)
-    trainer = ag.LeNet5Trainer(model, bs, learning_rate=0.01, optimizer=ag.SGD(momentum))
+    trainer = ag.LeNet5Trainer(model, bs, learning_rate=0.01, optimizer=ag.SGD(momentum), fused_forward=fused_forward)
     tx, tt = ag.Tensor.from_array(x), labels(ag, t)
     trainer.step(tx, tt)
     ag._ffi.check(ag.lib.agh_sync())
