@@ -393,7 +393,7 @@ __global__ __launch_bounds__(kThreads) void col2im_gather_kernel(const T *__rest
 #pragma unroll
             for (int u = 0; u < G; ++u) {
                 const T add = ok[u] ? v[u] : Elem<T>::zero();
-                acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(add));
+                acc = Elem<T>::from_f32(Elem<T>::addend(acc) + Elem<T>::addend(add));
             }
         }
     }
@@ -500,7 +500,7 @@ __global__ __launch_bounds__(kThreads) void col2im_ring_kernel(const T *__restri
                     p.div_sw.divmod((uint32_t)tw, wi, rw);
                     if (rw != 0 || wi >= (uint32_t)p.gw) continue;
                     const T v = sc[wi * p.pitch + fi * p.fw + fj];
-                    acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(v));
+                    acc = Elem<T>::from_f32(Elem<T>::addend(acc) + Elem<T>::addend(v));
                 }
                 ring[slot] = to_slot(acc);
             }
@@ -641,7 +641,7 @@ __global__ __launch_bounds__(kThreads) void col2im_ring_unit_kernel(const T *__r
 #pragma unroll
                             for (int fj = F - 1; fj >= 0; --fj) {
                                 const T v = st[tap_base[j] - fj * tap_step + fi * F];
-                                acc[j][fi] = Elem<T>::from_f32(Elem<T>::to_f32(acc[j][fi]) + Elem<T>::to_f32(v));
+                                acc[j][fi] = Elem<T>::from_f32(Elem<T>::addend(acc[j][fi]) + Elem<T>::addend(v));
                             }
                         }
                     }
@@ -914,7 +914,7 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
 #pragma unroll
             for (int fj = FW - 1; fj >= 0; --fj) {
                 const T add = okj[fj] ? Elem<T>::from_f32(d[fj]) : Elem<T>::zero();
-                acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(add));
+                acc = Elem<T>::from_f32(Elem<T>::addend(acc) + Elem<T>::addend(add));
             }
             continue;
         }
@@ -952,7 +952,7 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
                 for (int o = 0; o < oc; ++o) d = fmaf(Elem<T>::to_f32(g[o]), wt[o], d);
             }
             const T add = ok ? Elem<T>::from_f32(d) : Elem<T>::zero();
-            acc = Elem<T>::from_f32(Elem<T>::to_f32(acc) + Elem<T>::to_f32(add));
+            acc = Elem<T>::from_f32(Elem<T>::addend(acc) + Elem<T>::addend(add));
         }
     }
     y[e] = acc;
