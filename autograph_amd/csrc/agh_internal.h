@@ -94,14 +94,15 @@ __device__ __forceinline__ float bf16_raw_f32(uint16_t h) { return __uint_as_flo
 template <typename T> struct Elem;
 template <> struct Elem<float> {
     static __device__ __forceinline__ float to_f32(float v) { return v; }
-    static __device__ __forceinline__ float addend(float v) { return v; }
+    static __device__ __forceinline__ float raw(float v) { return v; }
     static __device__ __forceinline__ float from_f32(float v) { return v; }
     static __device__ __forceinline__ float zero() { return 0.0f; }
 };
 template <> struct Elem<uint16_t> {
     static __device__ __forceinline__ float to_f32(uint16_t v) { return bf16_to_f32(v); }
-    // for an operand of an addition: the plain widening (the addition quiets a signalling NaN itself)
-    static __device__ __forceinline__ float addend(uint16_t v) { return bf16_raw_f32(v); }
+    // the plain widening, for an operand of an addition or a comparison: the addition quiets a signalling NaN
+    // itself, and a comparison with any NaN is false either way
+    static __device__ __forceinline__ float raw(uint16_t v) { return bf16_raw_f32(v); }
     static __device__ __forceinline__ uint16_t from_f32(float v) { return f32_to_bf16(v); }
     static __device__ __forceinline__ uint16_t zero() { return 0; }
 };

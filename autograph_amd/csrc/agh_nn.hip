@@ -393,7 +393,7 @@ __global__ __launch_bounds__(kThreads) void col2im_gather_kernel(const T *__rest
 #pragma unroll
             for (int u = 0; u < G; ++u) {
                 const T add = ok[u] ? v[u] : Elem<T>::zero();
-                acc = Elem<T>::from_f32(Elem<T>::addend(acc) + Elem<T>::addend(add));
+                acc = Elem<T>::from_f32(Elem<T>::raw(acc) + Elem<T>::raw(add));
             }
         }
     }
@@ -500,7 +500,7 @@ __global__ __launch_bounds__(kThreads) void col2im_ring_kernel(const T *__restri
                     p.div_sw.divmod((uint32_t)tw, wi, rw);
                     if (rw != 0 || wi >= (uint32_t)p.gw) continue;
                     const T v = sc[wi * p.pitch + fi * p.fw + fj];
-                    acc = Elem<T>::from_f32(Elem<T>::addend(acc) + Elem<T>::addend(v));
+                    acc = Elem<T>::from_f32(Elem<T>::raw(acc) + Elem<T>::raw(v));
                 }
                 ring[slot] = to_slot(acc);
             }
@@ -641,7 +641,7 @@ __global__ __launch_bounds__(kThreads) void col2im_ring_unit_kernel(const T *__r
 #pragma unroll
                             for (int fj = F - 1; fj >= 0; --fj) {
                                 const T v = st[tap_base[j] - fj * tap_step + fi * F];
-                                acc[j][fi] = Elem<T>::from_f32(Elem<T>::addend(acc[j][fi]) + Elem<T>::addend(v));
+                                acc[j][fi] = Elem<T>::from_f32(Elem<T>::raw(acc[j][fi]) + Elem<T>::raw(v));
                             }
                         }
                     }
@@ -914,7 +914,7 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
 #pragma unroll
             for (int fj = FW - 1; fj >= 0; --fj) {
                 const T add = okj[fj] ? Elem<T>::from_f32(d[fj]) : Elem<T>::zero();
-                acc = Elem<T>::from_f32(Elem<T>::addend(acc) + Elem<T>::addend(add));
+                acc = Elem<T>::from_f32(Elem<T>::raw(acc) + Elem<T>::raw(add));
             }
             continue;
         }
@@ -952,7 +952,7 @@ __global__ __launch_bounds__(kThreads) void conv2_backward_input_kernel(const T 
                 for (int o = 0; o < oc; ++o) d = fmaf(Elem<T>::to_f32(g[o]), wt[o], d);
             }
             const T add = ok ? Elem<T>::from_f32(d) : Elem<T>::zero();
-            acc = Elem<T>::from_f32(Elem<T>::addend(acc) + Elem<T>::addend(add));
+            acc = Elem<T>::from_f32(Elem<T>::raw(acc) + Elem<T>::raw(add));
         }
     }
     y[e] = acc;
@@ -1062,11 +1062,11 @@ __global__ __launch_bounds__(kThreads) void max_pool2_kernel(const T *__restrict
     p.div_ow.divmod(rem, ho, wo);
     const T *src = x + (plane * p.ih + (size_t)ho * p.sh) * p.iw + (size_t)wo * p.sw;
     T m = src[0];
-    float mf = Elem<T>::to_f32(m);
+    float mf = Elem<T>::raw(m);
     for (int fi = 0; fi < p.h; ++fi)
         for (int fj = 0; fj < p.w; ++fj) {
             T v = src[(size_t)fi * p.iw + fj];
-            float vf = Elem<T>::to_f32(v);
+            float vf = Elem<T>::raw(v);
             if (vf > mf) { m = v; mf = vf; }
         }
     y[e] = m;
@@ -1084,16 +1084,16 @@ __global__ __launch_bounds__(kThreads) void max_pool2_backward_kernel(T *__restr
     uint32_t ho, wo;
     p.div_ow.divmod(rem, ho, wo);
     T *win = dx + (plane * p.ih + (size_t)ho * p.sh) * p.iw + (size_t)wo * p.sw;
-    float mf = Elem<T>::to_f32(win[0]);
+    float mf = Elem<T>::raw(win[0]);
     int am = 0;
     for (int fi = 0; fi < p.h; ++fi)
         for (int fj = 0; fj < p.w; ++fj) {
             int off = fi * p.iw + fj;
-            float vf = Elem<T>::to_f32(win[off]);
+            float vf = Elem<T>::raw(win[off]);
             if (vf > mf) { mf = vf; am = off; }
         }
     // `0 + dy` in T, as the host's `+=` on the zeroed cell computes it
-    const T g = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(dy[e]));
+    const T g = Elem<T>::from_f32(0.0f + Elem<T>::raw(dy[e]));
     for (int fi = 0; fi < p.h; ++fi)
         for (int fj = 0; fj < p.w; ++fj) {
             int off = fi * p.iw + fj;
@@ -1147,11 +1147,11 @@ __global__ __launch_bounds__(kThreads) void max_pool2_2x2_kernel(const T *__rest
 #pragma unroll
             for (int k = 0; k < NW; ++k) {
                 T m = r[u][0].e[2 * k];
-                float mf = Elem<T>::to_f32(m);
+                float mf = Elem<T>::raw(m);
                 const T c[3] = {r[u][0].e[2 * k + 1], r[u][1].e[2 * k], r[u][1].e[2 * k + 1]};
 #pragma unroll
                 for (int q = 0; q < 3; ++q) {
-                    const float vf = Elem<T>::to_f32(c[q]);
+                    const float vf = Elem<T>::raw(c[q]);
                     if (vf > mf) { m = c[q]; mf = vf; }
                 }
                 out[k] = m;
@@ -1183,16 +1183,16 @@ __global__ __launch_bounds__(kThreads) void max_pool2_backward_2x2_kernel(T *__r
             if (u == 1 && !two) break;
 #pragma unroll
             for (int k = 0; k < NW; ++k) {
-                float mf = Elem<T>::to_f32(r[u][0].e[2 * k]);
+                float mf = Elem<T>::raw(r[u][0].e[2 * k]);
                 int am = 0;
                 const T c[3] = {r[u][0].e[2 * k + 1], r[u][1].e[2 * k], r[u][1].e[2 * k + 1]};
 #pragma unroll
                 for (int q = 0; q < 3; ++q) {
-                    const float vf = Elem<T>::to_f32(c[q]);
+                    const float vf = Elem<T>::raw(c[q]);
                     if (vf > mf) { mf = vf; am = q + 1; }
                 }
                 // `0 + dy` in T, as the host's `+=` on the zeroed cell computes it
-                const T gv = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(gy[u][k]));
+                const T gv = Elem<T>::from_f32(0.0f + Elem<T>::raw(gy[u][k]));
                 r[u][0].e[2 * k] = am == 0 ? gv : Elem<T>::zero();
                 r[u][0].e[2 * k + 1] = am == 1 ? gv : Elem<T>::zero();
                 r[u][1].e[2 * k] = am == 2 ? gv : Elem<T>::zero();
@@ -1232,16 +1232,16 @@ __global__ __launch_bounds__(64) void max_pool2_backward_seq_kernel(T *__restric
     for (int ho = 0; ho < p.oh; ++ho)
         for (int wo = 0; wo < p.ow; ++wo) {
             T *win = d + (size_t)ho * p.sh * p.iw + (size_t)wo * p.sw;
-            float mf = Elem<T>::to_f32(win[0]);
+            float mf = Elem<T>::raw(win[0]);
             int am = 0;
             for (int fi = 0; fi < p.h; ++fi)
                 for (int fj = 0; fj < p.w; ++fj) {
                     int off = fi * p.iw + fj;
-                    float vf = Elem<T>::to_f32(win[off]);
+                    float vf = Elem<T>::raw(win[off]);
                     if (vf > mf) { mf = vf; am = off; }
                     win[off] = Elem<T>::zero();
                 }
-            win[am] = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(g[(size_t)ho * p.ow + wo]));
+            win[am] = Elem<T>::from_f32(0.0f + Elem<T>::raw(g[(size_t)ho * p.ow + wo]));
         }
 }
 
@@ -1324,14 +1324,14 @@ __global__ __launch_bounds__(kThreads) void relu_kernel(const T *x, T *y, size_t
     size_t stride = (size_t)gridDim.x * kThreads;
     for (; i < n; i += stride) {
         T v = x[i];
-        y[i] = Elem<T>::to_f32(v) >= 0.0f ? v : Elem<T>::zero();
+        y[i] = Elem<T>::raw(v) >= 0.0f ? v : Elem<T>::zero();
     }
 }
 template <typename T>
 __global__ __launch_bounds__(kThreads) void relu_backward_kernel(const T *x, const T *dy, T *dx, size_t n) {
     size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
     size_t stride = (size_t)gridDim.x * kThreads;
-    for (; i < n; i += stride) dx[i] = Elem<T>::to_f32(x[i]) >= 0.0f ? dy[i] : Elem<T>::zero();
+    for (; i < n; i += stride) dx[i] = Elem<T>::raw(x[i]) >= 0.0f ? dy[i] : Elem<T>::zero();
 }
 
 unsigned grid_for(size_t n) {
@@ -1368,7 +1368,7 @@ int relu_backward_launch(const char *name, const void *x, const void *dy, void *
 // y = max_pool2(relu(x)) without the intermediate: the same element rule as relu_kernel and the same visiting
 // order as max_pool2_kernel, applied to values that never reach memory.
 template <typename T>
-__device__ __forceinline__ T relu_of(T v) { return Elem<T>::to_f32(v) >= 0.0f ? v : Elem<T>::zero(); }
+__device__ __forceinline__ T relu_of(T v) { return Elem<T>::raw(v) >= 0.0f ? v : Elem<T>::zero(); }
 
 template <typename T>
 __global__ __launch_bounds__(kThreads) void relu_max_pool2_kernel(const T *__restrict__ x, T *__restrict__ y,
@@ -1382,11 +1382,11 @@ __global__ __launch_bounds__(kThreads) void relu_max_pool2_kernel(const T *__res
     p.div_ow.divmod(rem, ho, wo);
     const T *src = x + (plane * p.ih + (size_t)ho * p.sh) * p.iw + (size_t)wo * p.sw;
     T m = relu_of(src[0]);
-    float mf = Elem<T>::to_f32(m);
+    float mf = Elem<T>::raw(m);
     for (int fi = 0; fi < p.h; ++fi)
         for (int fj = 0; fj < p.w; ++fj) {
             T v = relu_of(src[(size_t)fi * p.iw + fj]);
-            float vf = Elem<T>::to_f32(v);
+            float vf = Elem<T>::raw(v);
             if (vf > mf) { m = v; mf = vf; }
         }
     y[e] = m;
@@ -1421,17 +1421,17 @@ __global__ __launch_bounds__(kThreads) void max_pool2_relu_backward_kernel(const
     T g = relu_of(xv);
     if (rh < (uint32_t)p.h && rw < (uint32_t)p.w && ho < (uint32_t)p.oh && wo < (uint32_t)p.ow) {
         const T *win = x + ((size_t)plane * p.ih + (size_t)ho * p.sh) * p.iw + (size_t)wo * p.sw;
-        float mf = Elem<T>::to_f32(relu_of(win[0]));
+        float mf = Elem<T>::raw(relu_of(win[0]));
         int am = 0;
         for (int fi = 0; fi < p.h; ++fi)
             for (int fj = 0; fj < p.w; ++fj) {
-                const float vf = Elem<T>::to_f32(relu_of(win[(size_t)fi * p.iw + fj]));
+                const float vf = Elem<T>::raw(relu_of(win[(size_t)fi * p.iw + fj]));
                 if (vf > mf) { mf = vf; am = fi * p.w + fj; }
             }
         const T gy = dy[((size_t)plane * p.oh + ho) * p.ow + wo];
-        g = am == (int)(rh * p.w + rw) ? Elem<T>::from_f32(0.0f + Elem<T>::to_f32(gy)) : Elem<T>::zero();
+        g = am == (int)(rh * p.w + rw) ? Elem<T>::from_f32(0.0f + Elem<T>::raw(gy)) : Elem<T>::zero();
     }
-    const T out = Elem<T>::to_f32(xv) >= 0.0f ? g : Elem<T>::zero();
+    const T out = Elem<T>::raw(xv) >= 0.0f ? g : Elem<T>::zero();
     size_t o = e;
     if (q.nhwc) {
         uint32_t b, ci;
@@ -1459,14 +1459,14 @@ __global__ __launch_bounds__(kThreads) void max_pool2_relu_backward_2x2_kernel(c
     const size_t at = ((size_t)plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)wo * 2;
     const T xv[4] = {x[at], x[at + 1], x[at + p.iw], x[at + p.iw + 1]};
     const T gy = dy[e];
-    float mf = Elem<T>::to_f32(relu_of(xv[0]));
+    float mf = Elem<T>::raw(relu_of(xv[0]));
     int am = 0;
 #pragma unroll
     for (int k = 1; k < 4; ++k) {
-        const float vf = Elem<T>::to_f32(relu_of(xv[k]));
+        const float vf = Elem<T>::raw(relu_of(xv[k]));
         if (vf > mf) { mf = vf; am = k; }
     }
-    const T g = Elem<T>::from_f32(0.0f + Elem<T>::to_f32(gy));
+    const T g = Elem<T>::from_f32(0.0f + Elem<T>::raw(gy));
     size_t o = at, ostep = 1, orow = (size_t)p.iw;
     if (q.nhwc) {
         uint32_t b, ci;
@@ -1478,7 +1478,7 @@ __global__ __launch_bounds__(kThreads) void max_pool2_relu_backward_2x2_kernel(c
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const T cell = am == k ? g : Elem<T>::zero();
-        dx[o + (k >> 1) * orow + (k & 1) * ostep] = Elem<T>::to_f32(xv[k]) >= 0.0f ? cell : Elem<T>::zero();
+        dx[o + (k >> 1) * orow + (k & 1) * ostep] = Elem<T>::raw(xv[k]) >= 0.0f ? cell : Elem<T>::zero();
     }
 }
 
