@@ -6,6 +6,8 @@
 //   agh_calib_copy       a plain 16-byte copy with a chosen grid: the read+write HBM ceiling, and the pass of
 //                        known size that FETCH_SIZE / WRITE_SIZE counter readings are scaled by
 //   agh_calib_read       a plain 16-byte read with a chosen grid: the read-only HBM ceiling
+//   agh_calib_mix        R 16-byte reads from R separate streams per 16-byte write: what the memory system sustains on
+//                        the read:write mix of a gather kernel (col2im of a 3x3 filter reads 9 bytes per byte written)
 #include "agh_internal.h"
 
 namespace {
@@ -75,6 +77,22 @@ __global__ __launch_bounds__(256) void read16_kernel(const u32x4_t *__restrict__
     if (acc == 0x9E3779B9u) out[0] = acc;  // keeps the loads alive
 }
 
+// every 16-byte slot i of dst receives the xor of slot i of `reads` source streams, each `n16` slots long
+template <int R>
+__global__ __launch_bounds__(256) void mix16_kernel(const u32x4_t *__restrict__ src, u32x4_t *__restrict__ dst, size_t n16, int reads) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) {
+        u32x4_t a = u32x4_t{(uint32_t)i, 0u, 0u, 0u};
+        if constexpr (R > 0) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) a ^= __builtin_nontemporal_load(src + i + (size_t)r * n16);
+        } else {
+            for (int r = 0; r < reads; ++r) a ^= __builtin_nontemporal_load(src + i + (size_t)r * n16);
+        }
+        dst[i] = a;
+    }
+}
+
 }  // namespace
 
 using namespace agh;
@@ -109,6 +127,27 @@ int agh_calib_read(const void *src, void *sink, size_t bytes, int blocks) {
         return fail(AGH_EINVAL, "agh_calib_read: a 16-byte aligned pointer, a multiple of 16 bytes and blocks >= 1");
     hipLaunchKernelGGL(read16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), (const u32x4_t *)src, (uint32_t *)sink, bytes / 16);
     AGH_LAUNCH_CHECK("agh_calib_read");
+    return AGH_OK;
+}
+
+int agh_calib_mix(const void *src, void *dst, size_t write_bytes, int reads_per_write, int blocks) {
+    AGH_API_ENTER();
+    if (write_bytes == 0) return AGH_OK;
+    if (!src || !dst) return fail(AGH_ENULL, "agh_calib_mix: null pointer");
+    if (write_bytes % 16 != 0 || (((uintptr_t)src | (uintptr_t)dst) & 15) != 0 || blocks < 1 || reads_per_write < 0 || reads_per_write > 64)
+        return fail(AGH_EINVAL, "agh_calib_mix: 16-byte aligned pointers, a multiple of 16 bytes, 0 <= reads_per_write <= 64 and blocks >= 1");
+    const size_t n16 = write_bytes / 16;
+    auto launch = [&](auto kern) {
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, stream(), (const u32x4_t *)src, (u32x4_t *)dst, n16, reads_per_write);
+    };
+    switch (reads_per_write) {
+        case 1: launch(mix16_kernel<1>); break;
+        case 2: launch(mix16_kernel<2>); break;
+        case 4: launch(mix16_kernel<4>); break;
+        case 9: launch(mix16_kernel<9>); break;
+        default: launch(mix16_kernel<0>); break;
+    }
+    AGH_LAUNCH_CHECK("agh_calib_mix");
     return AGH_OK;
 }
 

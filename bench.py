@@ -172,7 +172,18 @@ def main():
             _, ms = timer.time(lambda: ag._ffi.check(ag.lib.agh_calib_read(cx._ptr(), sink._ptr(), nbytes, grid)), 10, 3)
             extras[f"calib_read_1GiB_grid{grid}"] = {"ms": round(ms, 4), "rate": round(nbytes / ms / 1e6, 1), "unit": "GB/s"}
             log(f"read 1 GiB, grid {grid}: {ms:.3f} ms  {nbytes / ms / 1e6:.0f} GB/s")
-        del cx, cy, sink
+        del cx, cy
+        # the 9:1 read:write mix of col2im at the 256x64x56x56 3x3 case, in its simplest form: 9 coalesced streams in, one out
+        for dt, es in (("f32", 4), ("bf16", 2)):
+            wbytes = 256 * 64 * 56 * 56 * es
+            mx, my = ag.Tensor.zeros((9 * wbytes // 4,), "f32"), ag.Tensor.uninit((wbytes // 4,), "f32")
+            for grid in (2048, 8192):
+                _, ms = timer.time(lambda: ag._ffi.check(ag.lib.agh_calib_mix(mx._ptr(), my._ptr(), wbytes, 9, grid)), 10, 3)
+                extras[f"calib_mix_9to1_{dt}_sized_grid{grid}"] = {"ms": round(ms, 4), "rate": round(10.0 * wbytes / ms / 1e6, 1), "unit": "GB/s",
+                                                                  "bytes_read": 9 * wbytes, "bytes_written": wbytes}
+                log(f"9 reads : 1 write, {wbytes >> 20} MiB written ({dt} col2im size), grid {grid}: {ms:.3f} ms  {10.0 * wbytes / ms / 1e6:.0f} GB/s (read + write)")
+            del mx, my
+        del sink
 
     if not args.no_extras and "kernels" in sections:
         ks, kw = max(3, args.steps // 4), 2

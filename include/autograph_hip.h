@@ -137,10 +137,14 @@ int agh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop
  * like N(0, 0.02^2) samples), 2 * 32*32*16 * 16 * iters * 4 * blocks flop, no memory traffic; `sink` is
  * 1 KiB of device memory that is practically never written.  agh_calib_copy / agh_calib_read: a plain
  * 16-byte nontemporal copy / read of `bytes` bytes with a grid of `blocks` workgroups of 256 threads
- * (grid-stride); also the pass of known size that profiler byte counters are scaled by. */
+ * (grid-stride); also the pass of known size that profiler byte counters are scaled by.  agh_calib_mix:
+ * every 16 bytes of `dst` (`write_bytes` in all) receive the xor of the 16 bytes at the same offset of
+ * `reads_per_write` consecutive source streams of `write_bytes` each (so `src` holds reads_per_write *
+ * write_bytes bytes): the read:write mix of a gather kernel such as col2im in its simplest, fully coalesced form. */
 int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks);
 int agh_calib_copy(const void *src, void *dst, size_t bytes, int blocks);
 int agh_calib_read(const void *src, void *sink, size_t bytes, int blocks);
+int agh_calib_mix(const void *src, void *dst, size_t write_bytes, int reads_per_write, int blocks);
 
 /* --------------------------------------------------------------------- gemm ---- */
 
