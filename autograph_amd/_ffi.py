@@ -59,6 +59,7 @@ SIGNATURES = {
     "agh_calib_copy": ([ptr, ptr, C.c_size_t, C.c_int], C.c_int),
     "agh_calib_read": ([ptr, ptr, C.c_size_t, C.c_int], C.c_int),
     "agh_calib_mix": ([ptr, ptr, C.c_size_t, C.c_int, C.c_int], C.c_int),
+    "agh_calib_mfma_dma": ([ptr, C.c_size_t, ptr, C.c_int, C.c_size_t, C.c_int, C.c_int], C.c_int),
     "agh_gemm_f32": (_GEMM, C.c_int),
     "agh_gemm_bf16": (_GEMM, C.c_int),
     "agh_gemm_bf16_noalloc": (_GEMM, C.c_int),

@@ -6,6 +6,10 @@
 //   agh_calib_copy       a plain 16-byte copy with a chosen grid: the read+write HBM ceiling, and the pass of
 //                        known size that FETCH_SIZE / WRITE_SIZE counter readings are scaled by
 //   agh_calib_read       a plain 16-byte read with a chosen grid: the read-only HBM ceiling
+//   agh_calib_mfma_dma   the MFMA-only loop with direct-to-LDS loads between the MFMAs, one workgroup of 4 waves per CU, every
+//                        workgroup cycling through a window of its own: what the matrix pipes sustain while a CU pulls bytes
+//                        through its L1 at a chosen rate, from L2 (small windows) or from beyond it (large ones).  The bf16
+//                        GEMM's 256x256 tile needs 4 such loads per 16 MFMAs per wave (32 bytes per cycle and CU).
 //   agh_calib_mix        R 16-byte reads from R separate streams per 16-byte write: what the memory system sustains on
 //                        the read:write mix of a gather kernel (col2im of a 3x3 filter reads 9 bytes per byte written)
 #include "agh_internal.h"
@@ -77,6 +81,58 @@ __global__ __launch_bounds__(256) void read16_kernel(const u32x4_t *__restrict__
     if (acc == 0x9E3779B9u) out[0] = acc;  // keeps the loads alive
 }
 
+// 16 independent MFMAs per iteration and wave on all-zero operands (the clock stays up), NLD direct loads of 1 KB spread
+// evenly between them; lane L's 16 bytes land at M0-base + 16 L.  128 KB of LDS per workgroup: one workgroup per CU,
+// one wave per SIMD, as in the GEMM.
+template <int NLD>
+__global__ __launch_bounds__(256) void mfma_dma_kernel(const unsigned char *__restrict__ src, float *out, int iters, size_t wg_stride,
+                                                        int wrap_iters) {
+    __shared__ __align__(1024) unsigned char lds[128 * 1024];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    bf16x8_t a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a[i] = (bf16x8_t)(0);
+        b[i] = (bf16x8_t)(0);
+    }
+    f32x16 acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = (f32x16)(0.0f);
+    constexpr size_t kStep = (size_t)4 * NLD * 1024;  // bytes a workgroup requests per iteration
+    const unsigned char *vp = src + (size_t)blockIdx.x * wg_stride + (size_t)wave * NLD * 1024 + lane * 16;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + wave * NLD * 1024;
+    int phase = 0;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int n = 0; n < 16; ++n) {
+            acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[n / 4], b[n % 4], acc[n], 0, 0, 0);
+            if constexpr (NLD > 0) {
+                constexpr int every = 16 / NLD;
+                if (n % every == 0) {
+                    const int l = n / every;
+                    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(vp + l * 1024), "s"(lds_base + l * 1024)
+                                 : "memory", "m0");
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (++phase == wrap_iters) {
+            phase = 0;
+            vp -= (size_t)(wrap_iters - 1) * kStep;
+        } else {
+            vp += kStep;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sum += acc[i][r];
+    if (sum == 12345.0f) out[threadIdx.x] = sum + lds[threadIdx.x * 16];  // keeps the loop and the loads alive; practically never true
+}
+
 // every 16-byte slot i of dst receives the xor of slot i of `reads` source streams, each `n16` slots long
 template <int R>
 __global__ __launch_bounds__(256) void mix16_kernel(const u32x4_t *__restrict__ src, u32x4_t *__restrict__ dst, size_t n16, int reads) {
@@ -127,6 +183,38 @@ int agh_calib_read(const void *src, void *sink, size_t bytes, int blocks) {
         return fail(AGH_EINVAL, "agh_calib_read: a 16-byte aligned pointer, a multiple of 16 bytes and blocks >= 1");
     hipLaunchKernelGGL(read16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), (const u32x4_t *)src, (uint32_t *)sink, bytes / 16);
     AGH_LAUNCH_CHECK("agh_calib_read");
+    return AGH_OK;
+}
+
+int agh_calib_mfma_dma(const void *src, size_t src_bytes, void *sink, int loads_per_16_mfma, size_t window_bytes, int iters, int blocks) {
+    AGH_API_ENTER();
+    if (!sink) return fail(AGH_ENULL, "agh_calib_mfma_dma: null sink (1 KiB of device memory)");
+    const int nld = loads_per_16_mfma;
+    if (iters < 1 || blocks < 1 || (nld != 0 && nld != 2 && nld != 4 && nld != 8 && nld != 16))
+        return fail(AGH_EINVAL, "agh_calib_mfma_dma: iters and blocks positive, loads_per_16_mfma one of 0, 2, 4, 8, 16");
+    const size_t step = (size_t)4 * nld * 1024;  // bytes per workgroup and iteration
+    size_t wg_stride = 0;
+    int wrap = 1;
+    if (nld > 0) {
+        if (!src) return fail(AGH_ENULL, "agh_calib_mfma_dma: null src");
+        if (((uintptr_t)src & 15) != 0 || window_bytes < step || window_bytes % step != 0 || window_bytes / step > (size_t)1 << 20)
+            return fail(AGH_EINVAL, "agh_calib_mfma_dma: src 16-byte aligned, window_bytes a multiple of 4096 * loads_per_16_mfma");
+        wg_stride = window_bytes + 896;  // windows of neighbouring workgroups start in different L2 channels
+        if (src_bytes < (size_t)blocks * wg_stride)
+            return fail(AGH_ERANGE, "agh_calib_mfma_dma: src holds %zu bytes, %zu needed", src_bytes, (size_t)blocks * wg_stride);
+        wrap = (int)(window_bytes / step);
+    }
+    auto launch = [&](auto kern) {
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, stream(), (const unsigned char *)src, (float *)sink, iters, wg_stride, wrap);
+    };
+    switch (nld) {
+        case 0: launch(mfma_dma_kernel<0>); break;
+        case 2: launch(mfma_dma_kernel<2>); break;
+        case 4: launch(mfma_dma_kernel<4>); break;
+        case 8: launch(mfma_dma_kernel<8>); break;
+        default: launch(mfma_dma_kernel<16>); break;
+    }
+    AGH_LAUNCH_CHECK("agh_calib_mfma_dma");
     return AGH_OK;
 }
 

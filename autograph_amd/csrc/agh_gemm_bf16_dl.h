@@ -4,18 +4,23 @@
 // LDS read itself (ds_read_b64_tr_b16).  The k loop therefore contains only MFMAs, LDS
 // reads, the direct loads and one barrier.
 //
-// Same formulation as agh_gemm_kernel.h:  D[p][q] = sum_k P[p][k] * Q[q][k], 32x32x16 MFMAs,
-// accumulator element r of lane l = D[p0 + 8*(r/4) + 4*(l/32) + r%4][q0 + l%32].
+// Same formulation as agh_gemm_kernel.h:  D[p][q] = sum_k P[p][k] * Q[q][k], on
+// v_mfma_f32_16x16x32_bf16: lane l supplies row l % 16, k = 8 (l / 16) .. + 7 of a 32-deep substep, and
+// accumulator element r of lane l = D[p0 + 4 (l / 16) + r][q0 + l % 16].  The 16x16x32 form does the same
+// flop per cycle as 32x32x16 and reads the same LDS bytes per flop, but moves half as many accumulator
+// registers per flop; on data that toggles like real data the part is power-limited, and a loop of nothing
+// but MFMAs sustains about 15 % more flop per second with this form than with 32x32x16.
 //
 // LDS tile of an operand with BR rows, k-tile of 64:
 //   LD_K (k contiguous in memory):   [row][64 k], 128-byte rows, 16-byte chunk c of row r at
-//        slot c ^ swz(r)  (the layout of agh_gemm_kernel.h); fragment = one ds_read_b128.
+//        slot c ^ swz(r)  (the layout of agh_gemm_kernel.h); fragment = one ds_read_b128 of chunk
+//        l / 16 + 4 s of row l % 16: the 16 lanes the LDS serves together hit 16 different 16-byte bank groups.
 //   LD_R (rows contiguous in memory): [k][BR rows], pitch 2*BR bytes.  A 32-byte group of 16
-//        rows (index m) of k-row kr sits at group slot  m ^ (kr&3) ^ ((m&1)<<2).
+//        rows (index m) of k-row kr sits at group slot  m ^ (kr&3) ^ (((kr>>3)&1)<<2).
 //        Fragment = two ds_read_b64_tr_b16: within a 16-lane group, lanes 4j..4j+3 point at
 //        the 16 rows of k-row k0+j, and lane i receives the 4 k values of row i.  The slot
-//        function spreads the four k-rows a group touches (and the two row groups of a
-//        32-row MFMA tile) over distinct banks.
+//        function spreads the four k-rows a group touches, and the k-rows 8 apart that two
+//        neighbouring lane groups read, over distinct banks.
 // A direct load deposits lane L's 16 bytes at (wave-uniform LDS base) + 16*L, so the swizzles
 // are applied on the global side: each lane computes once which chunk of the tile belongs at
 // its LDS position.
@@ -32,13 +37,10 @@ namespace gemm {
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ uint32_t rslot(uint32_t m, uint32_t kr) { return m ^ (kr & 3u) ^ ((m & 1u) << 2); }
-// inverse of rslot in m for a given kr
-__device__ __forceinline__ uint32_t rslot_inv(uint32_t ms, uint32_t kr) {
-    const uint32_t c = kr & 3u;
-    const uint32_t b0 = (ms ^ c) & 1u;
-    return ms ^ c ^ (b0 << 2);
-}
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+// 32-byte group m (16 rows) of k-row kr sits at group slot m ^ (kr & 3) ^ (((kr >> 3) & 1) << 2): an involution in m
+__device__ __forceinline__ uint32_t rslot(uint32_t m, uint32_t kr) { return m ^ (kr & 3u) ^ (((kr >> 3) & 1u) << 2); }
+__device__ __forceinline__ uint32_t rslot_inv(uint32_t ms, uint32_t kr) { return rslot(ms, kr); }
 
 // 16-byte direct load: lane L's data lands at LDS address lds_base + 16*L (lds_base is
 // wave-uniform and travels in M0).  Issued as inline assembly on purpose: the compiler's
@@ -88,31 +90,32 @@ struct DirectLoad {
     }
 };
 
-// Per-lane LDS byte offsets for the MFMA fragments of one operand (32-row tile index i).
+// Per-lane LDS byte offsets for the MFMA fragments of one operand (16-row tile index i), v_mfma_f32_16x16x32_bf16:
+// lane l supplies row l % 16, k = 8 * (l / 16) .. + 7 of a 32-deep substep.
 template <int MODE, int BR, int NTILE>
 struct FragRead {
     static constexpr int PITCH = BR * 2;
-    // LD_K: off[i] as in agh_gemm_kernel.h (substep s toggles bits 5..6)
-    // LD_R: off[i] = ((8*(l/32) + j) * PITCH + 32*slot + 8*(l%4)), substep s / half h add (16s+4h)*PITCH
+    // LD_K: chunk (l / 16) + 4 s of row rb + l % 16; substep s toggles bit 6 of the offset
+    // LD_R: two transposing reads of 4 k-rows each: k-row 8 (l / 16) + (l % 16) / 4 (+ 4), 16-row group rb / 16
     static __device__ __forceinline__ void offsets(uint32_t (&off)[NTILE], int row_base, int lane) {
 #pragma unroll
         for (int i = 0; i < NTILE; ++i) {
-            const int rb = row_base + i * 32;
+            const int rb = row_base + i * 16;
             if constexpr (MODE == LD_K) {
-                const uint32_t lrow = lane & 31, lg = lane >> 5;
-                off[i] = (uint32_t)(rb + (int)lrow) * 128u + ((lg ^ swz(lrow)) << 4);
+                const uint32_t lrow = (uint32_t)rb + (lane & 15), lg = lane >> 4;
+                off[i] = lrow * 128u + ((lg ^ swz(lrow)) << 4);
             } else {
                 const uint32_t j = (lane & 15) >> 2;
-                const uint32_t m = (uint32_t)(rb >> 4) + ((lane >> 4) & 1);
-                off[i] = (8u * (lane >> 5) + j) * PITCH + 32u * rslot(m, j) + 8u * (lane & 3);
+                const uint32_t kr = 8u * (lane >> 4) + j;
+                off[i] = kr * PITCH + 32u * rslot((uint32_t)(rb >> 4), kr) + 8u * (lane & 3);
             }
         }
     }
     static __device__ __forceinline__ uint4 read(const unsigned char *tile, uint32_t off, int s) {
         if constexpr (MODE == LD_K) {
-            return *(const uint4 *)(tile + (off ^ (uint32_t)(s << 5)));
+            return *(const uint4 *)(tile + (off ^ (uint32_t)(s << 6)));
         } else {
-            const unsigned char *p = tile + off + s * 16 * PITCH;
+            const unsigned char *p = tile + off + s * 32 * PITCH;
             s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3))) *)p);
             s16x4_t hi =
                 __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3))) *)(p + 4 * PITCH));
@@ -129,15 +132,14 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     typedef uint16_t T;
     constexpr int NW = WGP * WGQ;
     constexpr int BK = 64;
-    constexpr int TP = BP / WGP / 32, TQ = BQ / WGQ / 32;
+    constexpr int MT = 16;  // MFMA tile: 16 x 16 outputs, 32 deep
+    constexpr int TP = BP / WGP / MT, TQ = BQ / WGQ / MT;
     constexpr int P_BYTES = BP * 128, Q_BYTES = BQ * 128, STAGE_BYTES = P_BYTES + Q_BYTES;
     typedef DirectLoad<LP, BP, NW> DlP;
     typedef DirectLoad<LQ, BQ, NW> DlQ;
     typedef FragRead<LP, BP, TP> FrP;
     typedef FragRead<LQ, BQ, TQ> FrQ;
 
-    // Two separately declared LDS stages: distinct objects, so the compiler knows a direct load
-    // into one stage cannot alias fragment reads of the other and does not wait for it.
     __shared__ __align__(1024) unsigned char stage0[STAGE_BYTES];
     __shared__ __align__(1024) unsigned char stage1[STAGE_BYTES];
 
@@ -153,7 +155,6 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     const int kend = min(g.K, kbeg + g.k_per_split);
     const int KT = kend > kbeg ? (kend - kbeg) / BK : 0;
 
-    // global source pointers of this lane's direct loads, advanced by one k-tile per iteration
     int64_t offp[DlP::NL], offq[DlQ::NL];
     DlP::offsets(offp, g.ps, g.pk, p0, g.NP, wave, lane);
     DlQ::offsets(offq, g.qs, g.qk, q0, g.NQ, wave, lane);
@@ -167,19 +168,15 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
         gq[i] = (const unsigned char *)g.Q + offq[i] + ((int64_t)kbeg * g.qk + (int64_t)blockIdx.z * g.batch_q) * 2;
 
     uint32_t fp[TP], fq[TQ];
-    FrP::offsets(fp, wp * TP * 32, lane);
-    FrQ::offsets(fq, wq * TQ * 32, lane);
+    FrP::offsets(fp, wp * TP * MT, lane);
+    FrQ::offsets(fq, wq * TQ * MT, lane);
 
-    f32x16 acc[TP][TQ];
+    f32x4_t acc[TP][TQ];
     static_for<TP>([&](auto ic) {
-        static_for<TQ>([&](auto jc) { acc[decltype(ic)::value][decltype(jc)::value] = (f32x16)(0.0f); });
+        static_for<TQ>([&](auto jc) { acc[decltype(ic)::value][decltype(jc)::value] = (f32x4_t)(0.0f); });
     });
 
-    // ---- direct loads: NLT per wave per k-tile (P's first, then Q's), issued one at a time ----
     constexpr int NLP = DlP::NL, NLQ = DlQ::NL, NLT = NLP + NLQ;
-    // `adv_p` / `adv_q` is the k-tile step, or 0 once the pointer is at the last k-tile (so a
-    // load issued past the end re-reads the last tile into a free stage instead of leaving the
-    // matrix; keeping the loads unconditional keeps the MFMA stream free of branches)
     auto issue_load = [&](uint32_t stage_addr, auto lc, int64_t adv_p, int64_t adv_q) {
         constexpr int l = decltype(lc)::value;
         if constexpr (l < NLP) {
@@ -191,113 +188,101 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
         }
     };
 
-    // ---- fragment reads: TP + TQ units per substep, in the order the MFMAs first need them ----
-    // two fragment sets, named separately so every register index is a compile-time constant
+    // two fragment sets of TP + TQ fragments each (one 32-deep substep of the wave's 128 x 128 tile)
     uint4 pfa[TP], qfa[TQ], pfb[TP], qfb[TQ];
     constexpr int NU = TP + TQ;
     auto read_unit = [&](uint4 (&pf)[TP], uint4 (&qf)[TQ], const unsigned char *stage, auto sc, auto uc) {
         constexpr int s = decltype(sc)::value, u = decltype(uc)::value;
-        // unit order: P0, Q0, Q1, ..., Q(TQ-1), P1, ..., P(TP-1)
+        // unit order: P0, Q0, Q1, ..., Q(TQ-1), P1, ..., P(TP-1): the order the row-major MFMA walk first needs them
         if constexpr (u == 0) pf[0] = FrP::read(stage, fp[0], s);
         else if constexpr (u <= TQ) qf[u - 1] = FrQ::read(stage + P_BYTES, fq[u - 1], s);
         else pf[u - TQ] = FrP::read(stage, fp[u - TQ], s);
     };
+    // Issued from inline assembly with the accumulator tied to the accumulation registers and updated in place: given
+    // the builtin, the register allocator moves 16x16 tiles between the two register files inside the loop (several
+    // hundred copies per k-tile).  An accumulator is next touched NM MFMAs later, so no result hazard arises here.
+    auto mma = [&](f32x4_t &c, const uint4 &a, const uint4 &b) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(__builtin_bit_cast(u32x4_t, a)), "v"(__builtin_bit_cast(u32x4_t, b)));
+    };
 
-    // ---- one phase: TP*TQ MFMAs on fragment set X; after MFMA number n the phase issues read
-    // unit n of fragment set Y (if READ) and its share of the direct loads
-    // [L0, L1), spread evenly over the MFMAs.  sched_barrier(0) after each MFMA pins this interleaving: the matrix pipe is
-    // handed a new MFMA every 32 cycles while LDS reads and global loads trickle out between.
+    // One k-tile = 2 substeps (32 k each) of NM MFMAs.  On entry: tile kt is visible in `cur`, its substep-0 fragments
+    // are in set A and the loads of tile kt+1 into `nxt` are in flight.  Every RSTEP-th of the first MFMAs of substep 0
+    // is followed by one fragment read of substep 1 (set B; reading them back to back would ask the LDS for 1 KB per
+    // wave every 16 cycles, its whole bandwidth), after which this wave needs nothing more from `cur`: the barrier at
+    // MFMA NB frees `cur` and publishes `nxt`.  From there on the loads of tile kt+2 go out into `cur`, one every LSTEP
+    // MFMAs, and the first MFMAs of substep 1 are followed by the reads of tile kt+1's substep 0 from `nxt` (set A).
+    // sched_barrier(0) after every MFMA pins this interleaving.
     constexpr int NM = TP * TQ;
-    auto phase = [&](const uint4 (&xp)[TP], const uint4 (&xq)[TQ], uint4 (&yp)[TP], uint4 (&yq)[TQ], auto readc,
-                     const unsigned char *rstage, auto sc, uint32_t lstage_addr, auto l0c, auto l1c, int64_t adv_p,
-                     int64_t adv_q) {
-        constexpr bool READ = decltype(readc)::value;
-        constexpr int L0 = decltype(l0c)::value, L1 = decltype(l1c)::value, NLD = L1 - L0;
-        static_for<NM>([&](auto nc) {
-            constexpr int n = decltype(nc)::value, i = n / TQ, j = n % TQ;
-            Mma<T>::run(acc[i][j], xp[i], xq[j]);
-            if constexpr (READ && n < NU) read_unit(yp, yq, rstage, sc, nc);
-            // loads [n*NLD/NM, (n+1)*NLD/NM) of this phase's share go out after MFMA n
-            constexpr int LA = n * NLD / NM, LB = (n + 1) * NLD / NM;
-            static_for<LB - LA>([&](auto tc) {
-                issue_load(lstage_addr, std::integral_constant<int, L0 + LA + decltype(tc)::value>{}, adv_p, adv_q);
-            });
+    constexpr int RSTEP = 2;                                          // one fragment read every RSTEP MFMAs
+    constexpr int NB = NU * RSTEP + NM / 16 < NM ? NU * RSTEP + NM / 16 : NM;  // barrier: a few MFMAs after the last read
+    constexpr int LSTEP = NM / NLT > 0 ? NM / NLT : 1;                // one direct load every LSTEP MFMAs
+    static_assert(NU * RSTEP <= NM, "fragment reads must fit behind the MFMAs of one substep");
+    static_assert(NB + LSTEP * NLT <= 2 * NM, "the loads of a tile must go out within the tile");
+    auto step = [&](unsigned char *cur, unsigned char *nxt, bool adv) {
+        const uint32_t cur_addr = __builtin_amdgcn_readfirstlane(lds_address(cur));
+        const int64_t ap = adv ? stepP : 0, aq = adv ? stepQ : 0;
+        static_for<2 * NM>([&](auto nc) {
+            constexpr int n = decltype(nc)::value, ph = n / NM, m = n % NM, i = m / TQ, j = m % TQ;
+            if constexpr (n == NB) {
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (ph == 0) {
+                mma(acc[i][j], pfa[i], qfa[j]);
+                if constexpr (m % RSTEP == 0 && m / RSTEP < NU) read_unit(pfb, qfb, cur, std::integral_constant<int, 1>{}, std::integral_constant<int, m / RSTEP>{});
+            } else {
+                mma(acc[i][j], pfb[i], qfb[j]);
+                if constexpr (m % RSTEP == 0 && m / RSTEP < NU) read_unit(pfa, qfa, nxt, std::integral_constant<int, 0>{}, std::integral_constant<int, m / RSTEP>{});
+            }
+            if constexpr (n >= NB && (n - NB) % LSTEP == LSTEP - 1 && (n - NB) / LSTEP < NLT)
+                issue_load(cur_addr, std::integral_constant<int, (n - NB) / LSTEP>{}, ap, aq);
             __builtin_amdgcn_sched_barrier(0);
         });
-    };
-    using S0 = std::integral_constant<int, 0>;
-    using S1 = std::integral_constant<int, 1>;
-    using S2 = std::integral_constant<int, 2>;
-    using S3 = std::integral_constant<int, 3>;
-    using Yes = std::true_type;
-    using L_0 = std::integral_constant<int, 0>;
-    using L_T = std::integral_constant<int, NLT>;
-
-    // One k-tile.  On entry: tile kt is visible in `cur`, its substep-0 fragments are in set A,
-    // and the P share of the loads of tile kt+1 into `nxt` is in flight (issued during the previous
-    // tile's last phase); the Q share goes out during phase 0.  Splitting the requests of a tile over
-    // two phases keeps the memory pipeline's queues from filling up: a wave that cannot issue its
-    // load cannot issue its next MFMA either.  The barrier sits between phase 2 and phase 3: by then
-    // every wave has issued (and waited for) its last reads of `cur`, so `cur` can be refilled with
-    // tile kt+2 while phase 3 multiplies out of registers.  `adv0` / `adv` say whether a tile kt+2 /
-    // kt+3 exists.
-    using L_P = std::integral_constant<int, NLP>;
-    auto step = [&](unsigned char *cur, unsigned char *nxt, bool adv0, bool adv) {
-        const uint32_t nxt_addr = __builtin_amdgcn_readfirstlane(lds_address(nxt));
-        phase(pfa, qfa, pfb, qfb, Yes{}, cur, S1{}, nxt_addr, L_P{}, L_T{}, 0, adv0 ? stepQ : 0);
-        phase(pfb, qfb, pfa, qfa, Yes{}, cur, S2{}, 0u, L_0{}, L_0{}, 0, 0);
-        phase(pfa, qfa, pfb, qfb, Yes{}, cur, S3{}, 0u, L_0{}, L_0{}, 0, 0);
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        const uint32_t cur_addr = __builtin_amdgcn_readfirstlane(lds_address(cur));
-        phase(pfb, qfb, pfa, qfa, Yes{}, nxt, S0{}, cur_addr, L_0{}, L_P{}, adv ? stepP : 0, 0);
     };
 
     if (KT > 0) {
         const uint32_t a0 = __builtin_amdgcn_readfirstlane(lds_address(stage0));
         const uint32_t a1 = __builtin_amdgcn_readfirstlane(lds_address(stage1));
-        // tile 0 -> stage0, P share of tile min(1, KT-1) -> stage1
+        // tile 0 -> stage0, tile min(1, KT-1) -> stage1
         static_for<NLT>([&](auto lc) { issue_load(a0, lc, KT > 1 ? stepP : 0, KT > 1 ? stepQ : 0); });
-        static_for<NLP>([&](auto lc) { issue_load(a1, lc, KT > 2 ? stepP : 0, 0); });
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLP) : "memory");  // tile 0 has landed
+        static_for<NLT>([&](auto lc) { issue_load(a1, lc, KT > 2 ? stepP : 0, KT > 2 ? stepQ : 0); });
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLT) : "memory");  // tile 0 has landed
         __syncthreads();
-        static_for<NU>([&](auto uc) { read_unit(pfa, qfa, stage0, S0{}, uc); });
+        static_for<NU>([&](auto uc) { read_unit(pfa, qfa, stage0, std::integral_constant<int, 0>{}, uc); });
     }
     int kt = 0;
-    for (; kt + 2 <= KT; kt += 2) {
-        step(stage0, stage1, kt + 2 < KT, kt + 3 < KT);
-        step(stage1, stage0, kt + 3 < KT, kt + 4 < KT);
+    for (; kt + 2 <= KT; kt += 2) {  // step kt requests tile kt+2 and moves on if a tile kt+3 exists
+        step(stage0, stage1, kt + 3 < KT);
+        step(stage1, stage0, kt + 4 < KT);
     }
-    if (kt < KT) step(stage0, stage1, false, false);
-    // the last phase may have re-issued loads into a free stage: let every wave's land before
-    // the epilogue reuses LDS
+    if (kt < KT) step(stage0, stage1, false);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     // ------------------------------------------------------------ epilogue ----
-    const uint32_t lrow = lane & 31, lg = lane >> 5;
-    const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
+    // accumulator element r of lane l, tile (i, j) = D[pwb + 16 i + 4 (l / 16) + r][qwb + 16 j + l % 16]
+    const uint32_t l16 = lane & 15, lg = lane >> 4;
+    const int pwb = p0 + wp * TP * MT, qwb = q0 + wq * TQ * MT;
+    const int pw0 = pwb + (int)lg * 4, qw0 = qwb + (int)l16;
     T *D = (T *)g.D + (int64_t)blockIdx.z * g.batch_d;
     const T *bias = (const T *)g.bias;
     const int mode = STAGED ? (int)ST_STAGED : g.store_mode;
     const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;
     if (mode == ST_STAGED) {
-        // beta == 0, D rows 16-byte aligned, NP a multiple of 8.  A lane holds 4 consecutive p of
-        // ONE q row, and the 32 lanes of a half-wave hold 32 different q rows, so storing straight
-        // from the accumulators writes 8 bytes into each of 64 different cache lines per
-        // instruction.  Instead each wave transposes 32 q rows at a time through its own LDS
-        // region and stores whole 16-byte chunks of contiguous row segments.
-        constexpr int EPITCH = TP * 64 + 16;           // bytes per staged q row (padded)
-        constexpr int CPRW = TP * 4;                   // 16-byte chunks per staged row
+        // beta == 0, D rows 16-byte aligned, NP a multiple of 8.  A lane holds 4 consecutive p of ONE q row and the
+        // 16 lanes of a group hold 16 different q rows, so storing straight from the accumulators would write 8 bytes
+        // into each of 64 different cache lines per instruction.  Instead each wave transposes 32 q rows (two tile
+        // columns) at a time through its own LDS region and stores whole 16-byte chunks of contiguous row segments.
+        constexpr int WPB = TP * MT * 2;               // bytes of one q row of the wave's tile
+        constexpr int EPITCH = WPB + 16;               // bytes per staged q row (padded)
+        constexpr int CPRW = WPB / 16;                 // 16-byte chunks per staged row
         constexpr int RPI = 64 / CPRW;                 // rows one store instruction covers
         constexpr int NST = 32 / RPI;                  // store instructions per pass
-        static_assert(4 * 32 * EPITCH <= STAGE_BYTES, "epilogue staging must fit in one LDS stage");
-        unsigned char *region = stage0 + wave * 32 * EPITCH;
-        const int pwb = p0 + wp * TP * 32, qwb = q0 + wq * TQ * 32;
-        // two fully separate instantiations (plain `dot` / bias+activation) so that the plain one
-        // carries no bias or activation state through its unrolled body
+        static_assert(TQ % 2 == 0, "the staged epilogue takes two tile columns per pass");
+        static_assert(4 * 32 * EPITCH <= STAGE_BYTES && NW <= 8, "epilogue staging must fit in the LDS stages");
+        unsigned char *region = (wave < 4 ? stage0 : stage1) + (wave & 3) * 32 * EPITCH;
         auto staged = [&](auto plainc) {
             constexpr bool PLAIN = decltype(plainc)::value;
             // Bias and activation are applied after the transposition, on the already rounded product (the
@@ -316,16 +301,16 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
                 }
             }
             const float alpha = g.alpha;
-            static_for<TQ>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                static_for<TP>([&](auto ic) {
-                    constexpr int i = decltype(ic)::value;
-                    static_for<4>([&](auto bc) {
-                        constexpr int blk = decltype(bc)::value;
-                        const int pl = i * 32 + blk * 8 + (int)lg * 4;  // p inside the wave tile
-                        const uint32_t w0 = f32x2_to_bf16x2(alpha * acc[i][j][blk * 4 + 0], alpha * acc[i][j][blk * 4 + 1]);
-                        const uint32_t w1 = f32x2_to_bf16x2(alpha * acc[i][j][blk * 4 + 2], alpha * acc[i][j][blk * 4 + 3]);
-                        *(uint2 *)(region + lrow * EPITCH + pl * 2) = make_uint2(w0, w1);
+            static_for<TQ / 2>([&](auto jc) {
+                constexpr int jj = decltype(jc)::value;
+                static_for<2>([&](auto hc) {
+                    constexpr int half = decltype(hc)::value, j = 2 * jj + half;
+                    static_for<TP>([&](auto ic) {
+                        constexpr int i = decltype(ic)::value;
+                        const int pl = i * MT + (int)lg * 4;  // p inside the wave tile
+                        const uint32_t w0 = f32x2_to_bf16x2(alpha * acc[i][j][0], alpha * acc[i][j][1]);
+                        const uint32_t w1 = f32x2_to_bf16x2(alpha * acc[i][j][2], alpha * acc[i][j][3]);
+                        *(uint2 *)(region + (half * 16 + l16) * EPITCH + pl * 2) = make_uint2(w0, w1);
                     });
                 });
                 // same wave, LDS executes in order: the reads below see the writes above
@@ -333,7 +318,7 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
                     constexpr int r = decltype(rc)::value;
                     const int row = r * RPI + lane / CPRW;
                     uint4 v = *(const uint4 *)(region + row * EPITCH + chunk * 16);
-                    const int qq = qwb + j * 32 + row, pp = pwb + chunk * 8;
+                    const int qq = qwb + jj * 32 + row, pp = pwb + chunk * 8;
                     if constexpr (!PLAIN) {
                         uint32_t w[4] = {v.x, v.y, v.z, v.w};
                         float brow = 0.0f;
@@ -369,66 +354,59 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     } else if (mode == ST_SPLITK) {
         static_for<TQ>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            const int q = qw0 + j * 32;
+            const int q = qw0 + j * MT;
             float *wrow = g.ws + ((size_t)split * g.NQ + q) * g.NPpad;
             static_for<TP>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                static_for<4>([&](auto bc) {
-                    constexpr int blk = decltype(bc)::value;
-                    const int p = pw0 + i * 32 + blk * 8;
-                    if (q < g.NQ && p < g.NPpad)
-                        *(float4 *)(wrow + p) = make_float4(acc[i][j][blk * 4 + 0], acc[i][j][blk * 4 + 1],
-                                                            acc[i][j][blk * 4 + 2], acc[i][j][blk * 4 + 3]);
-                });
+                const int p = pw0 + i * MT;
+                if (q < g.NQ && p < g.NPpad)
+                    *(float4 *)(wrow + p) = make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
             });
         });
     } else if (mode == ST_VEC) {
         static_for<TQ>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            const int q = qw0 + j * 32;
+            const int q = qw0 + j * MT;
             const bool qok = q < g.NQ;
             T bq = 0;
             if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
             T *drow = D + (int64_t)q * g.dq;
             static_for<TP>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                static_for<4>([&](auto bc) {
-                    constexpr int blk = decltype(bc)::value;
-                    const int p = pw0 + i * 32 + blk * 8;
-                    if (qok && p < g.NP) {
-                        T *dst = drow + p;
-                        __align__(8) T old[4] = {0, 0, 0, 0};
-                        if (g.beta != 0.0f) *(uint2 *)old = *(const uint2 *)dst;
-                        T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
-                        if (has_bias && bias_p) {
-                            b0 = bias[(int64_t)(p + 0) * g.bias_stride];
-                            b1 = bias[(int64_t)(p + 1) * g.bias_stride];
-                            b2 = bias[(int64_t)(p + 2) * g.bias_stride];
-                            b3 = bias[(int64_t)(p + 3) * g.bias_stride];
-                        }
-                        __align__(8) T out[4];
-                        out[0] = finish<T>(acc[i][j][blk * 4 + 0], g.alpha, g.beta, old[0], has_bias, b0, g.act);
-                        out[1] = finish<T>(acc[i][j][blk * 4 + 1], g.alpha, g.beta, old[1], has_bias, b1, g.act);
-                        out[2] = finish<T>(acc[i][j][blk * 4 + 2], g.alpha, g.beta, old[2], has_bias, b2, g.act);
-                        out[3] = finish<T>(acc[i][j][blk * 4 + 3], g.alpha, g.beta, old[3], has_bias, b3, g.act);
-                        *(uint2 *)dst = *(const uint2 *)out;
+                const int p = pw0 + i * MT;
+                if (qok && p < g.NP) {
+                    T *dst = drow + p;
+                    __align__(8) T old[4] = {0, 0, 0, 0};
+                    if (g.beta != 0.0f) *(uint2 *)old = *(const uint2 *)dst;
+                    T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
+                    if (has_bias && bias_p) {
+                        b0 = bias[(int64_t)(p + 0) * g.bias_stride];
+                        b1 = bias[(int64_t)(p + 1) * g.bias_stride];
+                        b2 = bias[(int64_t)(p + 2) * g.bias_stride];
+                        b3 = bias[(int64_t)(p + 3) * g.bias_stride];
                     }
-                });
+                    __align__(8) T out[4];
+                    out[0] = finish<T>(acc[i][j][0], g.alpha, g.beta, old[0], has_bias, b0, g.act);
+                    out[1] = finish<T>(acc[i][j][1], g.alpha, g.beta, old[1], has_bias, b1, g.act);
+                    out[2] = finish<T>(acc[i][j][2], g.alpha, g.beta, old[2], has_bias, b2, g.act);
+                    out[3] = finish<T>(acc[i][j][3], g.alpha, g.beta, old[3], has_bias, b3, g.act);
+                    *(uint2 *)dst = *(const uint2 *)out;
+                }
             });
         });
     } else {
         static_for<TQ>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            const int q = qw0 + j * 32;
+            const int q = qw0 + j * MT;
             const bool qok = q < g.NQ;
             T bq = 0;
             if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
             T *drow = D + (int64_t)q * g.dq;
             static_for<TP>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                static_for<16>([&](auto rc) {
+                static_for<4>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
-                    const int p = pw0 + i * 32 + (r >> 2) * 8 + (r & 3);
+                    const int p = pw0 + i * MT + r;
                     if (qok && p < g.NP) {
                         T *dst = drow + (int64_t)p * g.dp;
                         T old = 0;

@@ -162,6 +162,26 @@ def main():
             extras[name] = {"ms": round(ms, 4), "rate": round(mflop / ms / 1e9, 1), "unit": "TFLOP/s",
                             "frac_of_peak": round(mflop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
             log(f"{name}: {ms:.3f} ms  {mflop / ms / 1e9:.0f} TFLOP/s")
+        # the same MFMA stream (zero operands: full clock) with direct-to-LDS loads between the MFMAs, one workgroup per CU
+        # cycling through a window of its own: 64 KiB windows stay in L2, 512 KiB ones come from the last-level cache,
+        # 4 MiB ones from HBM.  The 256x256 GEMM tile needs 4 loads per 16 MFMAs per wave.
+        dsrc_bytes = (1 << 30) + (1 << 20)
+        dsrc = ag.Tensor.zeros((dsrc_bytes // 4,), "f32")
+        d_iters, d_blocks = 4096, 256
+        dflop = 2.0 * 32 * 32 * 16 * 16 * d_iters * 4 * d_blocks
+        for window, wname in ((64 << 10, "L2"), (512 << 10, "LLC"), (4 << 20, "HBM")):
+            for nld in (0, 2, 4, 8):
+                if nld == 0 and wname != "L2":
+                    continue
+                fn = lambda: ag._ffi.check(ag.lib.agh_calib_mfma_dma(dsrc._ptr(), dsrc_bytes, sink._ptr(), nld, window, d_iters, d_blocks))  # noqa: E731
+                _, ms = timer.time(fn, 10, 3)
+                fill = d_blocks * d_iters * 4.0 * nld * 1024
+                extras[f"calib_mfma_dma_{nld}_loads_per_16_mfma_window_{wname}"] = {
+                    "ms": round(ms, 4), "rate": round(dflop / ms / 1e9, 1), "unit": "TFLOP/s", "fill_GBps": round(fill / ms / 1e6, 1),
+                    "fill_GBps_per_cu": round(fill / ms / 1e6 / d_blocks, 2)}
+                log(f"MFMA + {nld} direct loads per 16 MFMAs, windows in {wname}: {ms:.3f} ms  {dflop / ms / 1e9:.0f} TFLOP/s, "
+                    f"{fill / ms / 1e6:.0f} GB/s through the L1s ({fill / ms / 1e6 / d_blocks:.1f} per CU)")
+        del dsrc
         nbytes = 1 << 30
         cx, cy = ag.Tensor.zeros((nbytes // 4,), "f32"), ag.Tensor.uninit((nbytes // 4,), "f32")
         for grid in (1024, 2048, 4096, 8192, 16384, 65536):

@@ -140,11 +140,18 @@ int agh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop
  * (grid-stride); also the pass of known size that profiler byte counters are scaled by.  agh_calib_mix:
  * every 16 bytes of `dst` (`write_bytes` in all) receive the xor of the 16 bytes at the same offset of
  * `reads_per_write` consecutive source streams of `write_bytes` each (so `src` holds reads_per_write *
- * write_bytes bytes): the read:write mix of a gather kernel such as col2im in its simplest, fully coalesced form. */
+ * write_bytes bytes): the read:write mix of a gather kernel such as col2im in its simplest, fully coalesced form.
+ * agh_calib_mfma_dma: the MFMA-only loop on zero operands (`blocks` workgroups of 4 waves that each take a whole CU,
+ * `iters` times 16 MFMAs per wave) with `loads_per_16_mfma` (0, 2, 4, 8 or 16) direct-to-LDS loads of 1 KiB spread
+ * between the MFMAs of every wave; every workgroup cycles through a window of `window_bytes` of its own inside `src`
+ * (`src_bytes` >= blocks * (window_bytes + 896)), so small windows are served by L2 and large ones from beyond it:
+ * what the matrix pipes sustain while a CU pulls bytes through its L1 at the rate a GEMM tile needs. */
 int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks);
 int agh_calib_copy(const void *src, void *dst, size_t bytes, int blocks);
 int agh_calib_read(const void *src, void *sink, size_t bytes, int blocks);
 int agh_calib_mix(const void *src, void *dst, size_t write_bytes, int reads_per_write, int blocks);
+int agh_calib_mfma_dma(const void *src, size_t src_bytes, void *sink, int loads_per_16_mfma, size_t window_bytes, int iters,
+                       int blocks);
 
 /* --------------------------------------------------------------------- gemm ---- */
 

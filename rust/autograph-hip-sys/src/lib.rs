@@ -50,6 +50,7 @@ extern "C" {
     pub fn agh_calib_copy(src: *const c_void, dst: *mut c_void, bytes: usize, blocks: c_int) -> c_int;
     pub fn agh_calib_read(src: *const c_void, sink: *mut c_void, bytes: usize, blocks: c_int) -> c_int;
     pub fn agh_calib_mix(src: *const c_void, dst: *mut c_void, write_bytes: usize, reads_per_write: c_int, blocks: c_int) -> c_int;
+    pub fn agh_calib_mfma_dma(src: *const c_void, src_bytes: usize, sink: *mut c_void, loads_per_16_mfma: c_int, window_bytes: usize, iters: c_int, blocks: c_int) -> c_int;
     pub fn agh_gemm_f32(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
     pub fn agh_gemm_bf16(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
     pub fn agh_gemm_bf16_noalloc(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
