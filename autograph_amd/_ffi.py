@@ -55,7 +55,7 @@ SIGNATURES = {
     "agh_event_destroy": ([ptr], C.c_int),
     "agh_event_record": ([ptr], C.c_int),
     "agh_event_elapsed_ms": ([ptr, ptr, C.POINTER(f32)], C.c_int),
-    "agh_calib_mfma_bf16": ([ptr, C.c_int, C.c_int, C.c_int], C.c_int),
+    "agh_calib_mfma_bf16": ([ptr, C.c_int, C.c_int, C.c_int, C.c_int], C.c_int),
     "agh_calib_copy": ([ptr, ptr, C.c_size_t, C.c_int], C.c_int),
     "agh_calib_read": ([ptr, ptr, C.c_size_t, C.c_int], C.c_int),
     "agh_calib_mix": ([ptr, ptr, C.c_size_t, C.c_int, C.c_int], C.c_int),

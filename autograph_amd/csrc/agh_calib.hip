@@ -1,6 +1,6 @@
 // Calibration launches: what this GPU can do at best on the two resources the kernels of this library
 // are bound by, measured with the same stream, events and profiler as the kernels themselves.
-//   agh_calib_mfma_bf16  a loop of nothing but independent v_mfma_f32_32x32x16_bf16 (no memory traffic),
+//   agh_calib_mfma_bf16  a loop of nothing but independent v_mfma_f32_32x32x16_bf16 or v_mfma_f32_16x16x32_bf16 (no memory traffic),
 //                        on all-zero operands or on operands shaped like N(0, 0.02^2) bf16 data: the matrix
 //                        pipes' sustained rate under the power limit, the ceiling of any bf16 GEMM on such data
 //   agh_calib_copy       a plain 16-byte copy with a chosen grid: the read+write HBM ceiling, and the pass of
@@ -37,31 +37,58 @@ __device__ __forceinline__ bf16x8_t operand_fragment(uint32_t &s, bool zero) {
     return v;
 }
 
-// 4 waves per workgroup, one per SIMD; each wave keeps 16 accumulator tiles (256 registers) and issues
-// 16 independent MFMAs per iteration on 4 + 4 operand fragments: the register shape of the GEMM's inner loop.
+// 4 waves per workgroup, one per SIMD; each wave keeps 256 accumulator registers, the register shape of the GEMM's
+// inner loop.  SHAPE 0: 16 tiles of 32x32, 16 independent v_mfma_f32_32x32x16_bf16 per iteration on 4 + 4 operand
+// fragments.  SHAPE 1: 64 tiles of 16x16, 64 independent v_mfma_f32_16x16x32_bf16 per iteration on 8 + 8 fragments
+// (twice the flop per iteration), walked row by row like the GEMM walks them.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+template <int SHAPE>
 __global__ __launch_bounds__(256) void mfma_only_kernel(float *out, int iters, int zero) {
     uint32_t s = threadIdx.x * 2654435761u + blockIdx.x * 97u + 12345u;
-    bf16x8_t a[4], b[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        a[i] = operand_fragment(s, zero != 0);
-        b[i] = operand_fragment(s, zero != 0);
-    }
-    f32x16 acc[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = (f32x16)(0.0f);
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i * 4 + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i * 4 + j], 0, 0, 0);
-    }
     float sum = 0.0f;
+    if constexpr (SHAPE == 0) {
+        bf16x8_t a[4], b[4];
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
+        for (int i = 0; i < 4; ++i) {
+            a[i] = operand_fragment(s, zero != 0);
+            b[i] = operand_fragment(s, zero != 0);
+        }
+        f32x16 acc[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sum += acc[i][r];
+        for (int i = 0; i < 16; ++i) acc[i] = (f32x16)(0.0f);
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i * 4 + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i * 4 + j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sum += acc[i][r];
+    } else {
+        bf16x8_t a[8], b[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a[i] = operand_fragment(s, zero != 0);
+            b[i] = operand_fragment(s, zero != 0);
+        }
+        f32x4v acc[64];
+#pragma unroll
+        for (int i = 0; i < 64; ++i) acc[i] = (f32x4v)(0.0f);
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    acc[i * 8 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i * 8 + j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 64; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum += acc[i][r];
+    }
     if (sum == 12345.0f) out[threadIdx.x] = sum;  // keeps the loop alive; practically never true
 }
 
@@ -155,11 +182,15 @@ using namespace agh;
 
 extern "C" {
 
-int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks) {
+int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks, int shape) {
     AGH_API_ENTER();
     if (!sink) return fail(AGH_ENULL, "agh_calib_mfma_bf16: null sink (1 KiB of device memory)");
-    if (iters < 1 || blocks < 1) return fail(AGH_EINVAL, "agh_calib_mfma_bf16: iters and blocks must be positive");
-    hipLaunchKernelGGL(mfma_only_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), (float *)sink, iters, zero_operands);
+    if (iters < 1 || blocks < 1 || (shape != 0 && shape != 1))
+        return fail(AGH_EINVAL, "agh_calib_mfma_bf16: iters and blocks must be positive, shape 0 (32x32x16) or 1 (16x16x32)");
+    if (shape == 0)
+        hipLaunchKernelGGL(mfma_only_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, stream(), (float *)sink, iters, zero_operands);
+    else
+        hipLaunchKernelGGL(mfma_only_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream(), (float *)sink, iters, zero_operands);
     AGH_LAUNCH_CHECK("agh_calib_mfma_bf16");
     return AGH_OK;
 }

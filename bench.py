@@ -151,17 +151,18 @@ def main():
     if args.calib:
         # ceilings measured with the same stream and events as everything else (agh_calib_*)
         sink = ag.Tensor.zeros((256,), "f32")
-        iters, blocks = 8192, 1024
-        mflop = 2.0 * 32 * 32 * 16 * 16 * iters * 4 * blocks
-        for zero in (1, 0):
-            name = "calib_mfma_only_bf16_" + ("zero_operands" if zero else "n002_operands")
-            fn = lambda: ag._ffi.check(ag.lib.agh_calib_mfma_bf16(sink._ptr(), zero, iters, blocks))  # noqa: E731
-            for _ in range(40):  # ~100 ms: let the clocks settle on this load
-                fn()
-            _, ms = timer.time(fn, 20, 5)
-            extras[name] = {"ms": round(ms, 4), "rate": round(mflop / ms / 1e9, 1), "unit": "TFLOP/s",
-                            "frac_of_peak": round(mflop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
-            log(f"{name}: {ms:.3f} ms  {mflop / ms / 1e9:.0f} TFLOP/s")
+        blocks = 1024
+        for shape, sname, iters in ((1, "16x16x32", 4096), (0, "32x32x16", 8192)):
+            mflop = 2.0 * 32 * 32 * 16 * 16 * (1 + shape) * iters * 4 * blocks
+            for zero in (1, 0):
+                name = f"calib_mfma_only_bf16_{sname}_" + ("zero_operands" if zero else "n002_operands")
+                fn = lambda: ag._ffi.check(ag.lib.agh_calib_mfma_bf16(sink._ptr(), zero, iters, blocks, shape))  # noqa: E731
+                for _ in range(40):  # ~100 ms: let the clocks settle on this load
+                    fn()
+                _, ms = timer.time(fn, 20, 5)
+                extras[name] = {"ms": round(ms, 4), "rate": round(mflop / ms / 1e9, 1), "unit": "TFLOP/s",
+                                "frac_of_peak": round(mflop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+                log(f"{name}: {ms:.3f} ms  {mflop / ms / 1e9:.0f} TFLOP/s")
         # the same MFMA stream (zero operands: full clock) with direct-to-LDS loads between the MFMAs, one workgroup per CU
         # cycling through a window of its own: 64 KiB windows stay in L2, 512 KiB ones come from the last-level cache,
         # 4 MiB ones from HBM.  The 256x256 GEMM tile needs 4 loads per 16 MFMAs per wave.
@@ -208,7 +209,7 @@ def main():
     if not args.no_extras and "kernels" in sections:
         ks, kw = max(3, args.steps // 4), 2
 
-        def run(name, fn, work, unit, peak, steps=ks):
+        def run(name, fn, work, unit, peak, steps=ks, hbm_bytes=None):
             try:
                 # the same untimed settle as the headline, shorter: clocks follow the load of the last ~50 ms
                 t_s = time.perf_counter()
@@ -218,7 +219,13 @@ def main():
                 _, ms = timer.time(fn, steps, kw)
                 rate = work / (ms * 1e-3) / (1e12 if unit == "TFLOP/s" else 1e9)
                 extras[name] = {"ms": round(ms, 4), "rate": round(rate, 2), "unit": unit, "frac_of_peak": round(rate / peak, 4)}
-                log(f"{name}: {ms:.3f} ms  {rate:.1f} {unit} ({100 * rate / peak:.1f}%)")
+                note = ""
+                if hbm_bytes is not None:  # a launch that may be bound by its operand bytes rather than by its flop
+                    gbs = hbm_bytes / (ms * 1e-3) / 1e9
+                    extras[name].update({"algorithmic_bytes": int(hbm_bytes), "hbm_GBps": round(gbs, 1),
+                                         "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)})
+                    note = f"; {gbs:.0f} GB/s of operand bytes ({100 * gbs / PEAK_HBM_GBS:.1f}% of HBM peak)"
+                log(f"{name}: {ms:.3f} ms  {rate:.1f} {unit} ({100 * rate / peak:.1f}%){note}")
             except Exception as e:  # an extra must not lose the headline line
                 extras[name] = {"error": str(e)}
                 log(f"{name}: FAILED {e}")
@@ -271,8 +278,11 @@ def main():
             run(f"im2col_{dt}_conv3x3_b256", lambda: ag._ffi.check(fn_i(x._ptr(), cols._ptr(), bs, ci, hw, hw, 3, 3, 1, 1, 1, 1, 1, 1)),
                 bytes_, "GB/s", PEAK_HBM_GBS)
             y = ag.Tensor.uninit((bs * hw * hw, co), dt)
+            # 802816 x 576 patch matrix in, 802816 x 128 out: 0.1 flop-seconds of bf16 MFMA work against 1.13 GB (bf16) of
+            # operand bytes, so in bf16 this product is bound by HBM, not by the matrix cores
             run(f"conv_gemm_{dt}_802816x576x128", lambda: ag.gemm(1.0, cols, wt.t(), 0.0, y), 2.0 * bs * hw * hw * 576 * co,
-                "TFLOP/s", PEAK_F32_TFLOPS if dt == "f32" else PEAK_BF16_TFLOPS)
+                "TFLOP/s", PEAK_F32_TFLOPS if dt == "f32" else PEAK_BF16_TFLOPS,
+                hbm_bytes=es * (bs * hw * hw * (576 + co) + 576 * co))
             del y
             # the same Conv2 forward without the patch matrix: implicit GEMM on the matrix cores, NCHW in, NCHW out
             w4 = wt.into_shape((co, ci, 3, 3))

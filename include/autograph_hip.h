@@ -133,8 +133,9 @@ int agh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop
 /* Calibration launches on the library's stream, for measurement only (no counterpart in the
  * reference): what the part sustains at best on the two resources the kernels here are bound by.
  * agh_calib_mfma_bf16: `blocks` workgroups of 4 waves, each wave `iters` times 16 independent
- * v_mfma_f32_32x32x16_bf16 on register operands (zero_operands != 0: all zero; else bf16 patterns shaped
- * like N(0, 0.02^2) samples), 2 * 32*32*16 * 16 * iters * 4 * blocks flop, no memory traffic; `sink` is
+ * v_mfma_f32_32x32x16_bf16 (shape 0) or 64 independent v_mfma_f32_16x16x32_bf16 (shape 1, the form the bf16
+ * GEMM uses) on register operands (zero_operands != 0: all zero; else bf16 patterns shaped like N(0, 0.02^2)
+ * samples), 2 * 32*32*16 * 16 * (1 + shape) * iters * 4 * blocks flop, no memory traffic; `sink` is
  * 1 KiB of device memory that is practically never written.  agh_calib_copy / agh_calib_read: a plain
  * 16-byte nontemporal copy / read of `bytes` bytes with a grid of `blocks` workgroups of 256 threads
  * (grid-stride); also the pass of known size that profiler byte counters are scaled by.  agh_calib_mix:
@@ -146,7 +147,7 @@ int agh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop
  * between the MFMAs of every wave; every workgroup cycles through a window of `window_bytes` of its own inside `src`
  * (`src_bytes` >= blocks * (window_bytes + 896)), so small windows are served by L2 and large ones from beyond it:
  * what the matrix pipes sustain while a CU pulls bytes through its L1 at the rate a GEMM tile needs. */
-int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks);
+int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks, int shape);
 int agh_calib_copy(const void *src, void *dst, size_t bytes, int blocks);
 int agh_calib_read(const void *src, void *sink, size_t bytes, int blocks);
 int agh_calib_mix(const void *src, void *dst, size_t write_bytes, int reads_per_write, int blocks);

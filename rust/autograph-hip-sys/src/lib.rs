@@ -46,7 +46,7 @@ extern "C" {
     pub fn agh_event_destroy(event: *mut c_void) -> c_int;
     pub fn agh_event_record(event: *mut c_void) -> c_int;
     pub fn agh_event_elapsed_ms(start: *mut c_void, stop: *mut c_void, ms: *mut f32) -> c_int;
-    pub fn agh_calib_mfma_bf16(sink: *mut c_void, zero_operands: c_int, iters: c_int, blocks: c_int) -> c_int;
+    pub fn agh_calib_mfma_bf16(sink: *mut c_void, zero_operands: c_int, iters: c_int, blocks: c_int, shape: c_int) -> c_int;
     pub fn agh_calib_copy(src: *const c_void, dst: *mut c_void, bytes: usize, blocks: c_int) -> c_int;
     pub fn agh_calib_read(src: *const c_void, sink: *mut c_void, bytes: usize, blocks: c_int) -> c_int;
     pub fn agh_calib_mix(src: *const c_void, dst: *mut c_void, write_bytes: usize, reads_per_write: c_int, blocks: c_int) -> c_int;
