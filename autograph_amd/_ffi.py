@@ -77,6 +77,10 @@ SIGNATURES = {
     "agh_lenet5_forward_bf16": ([ptr] * 8 + [i64], C.c_int),
     "agh_lenet5_forward_train_f32": ([ptr] * 16 + [i64], C.c_int),
     "agh_lenet5_forward_train_bf16": ([ptr] * 16 + [i64], C.c_int),
+    "agh_lenet5_backward_f32": ([ptr, ptr, C.c_float] + [ptr] * 13 + [i64], C.c_int),
+    "agh_lenet5_backward_bf16": ([ptr, ptr, C.c_float] + [ptr] * 13 + [i64], C.c_int),
+    "agh_lenet5_dense_weight_grads_f32": ([ptr] * 13 + [i64], C.c_int),
+    "agh_lenet5_dense_weight_grads_bf16": ([ptr] * 13 + [i64], C.c_int),
     "agh_max_pool2_f32": (_POOL, C.c_int),
     "agh_max_pool2_bf16": (_POOL, C.c_int),
     "agh_max_pool2_backward_f32": (_POOL, C.c_int),

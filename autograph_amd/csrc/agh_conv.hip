@@ -538,6 +538,311 @@ __global__ __launch_bounds__(512) void lenet5_forward_kernel(const T *__restrict
     }
 }
 
+// The input-gradient chain of a LeNet5 training step in one launch, one workgroup per image: cross-entropy backward,
+// the three dense layers' input gradients with their relu backward, pooling + relu backward of conv2's output written as
+// the [64, 16] matrix its weight gradient multiplies, conv2's input gradient (dot with the filter bank, then col2im),
+// pooling + relu backward of conv1's output as the [576, 6] matrix.  Every value is rounded to T where the separate
+// launches round it, and every T-typed running sum adds in their order (col2im: filter rows and columns descending,
+// the dot over the output channels ascending), so the results differ from theirs only through the order of the f32
+// adds inside the dense dot products.
+template <typename T>
+struct LenetBackward {
+    const T *logits;            // [bs, 10]
+    const uint8_t *target;      // [bs]
+    const T *c1, *c2, *d1, *d2; // conv outputs before relu [bs,6,24,24], [bs,16,8,8]; dense outputs before relu [bs,128], [bs,84]
+    const T *w2, *wd1, *wd2, *wd3;
+    T *g_logits, *g_d2, *g_d1;  // [bs,10], [bs,84], [bs,128]
+    T *gm2, *gm1;               // [bs*64, 16], [bs*576, 6]
+    float dy;                   // upstream gradient of the summed loss divided by the batch size
+};
+
+// pooling (2x2, stride 2) backward through a relu, one window: g lands on the first maximum of relu(x) and passes where
+// x >= 0 (the rule of max_pool2_relu_backward_2x2_kernel); cell k = 2 * row + column
+template <typename T>
+__device__ __forceinline__ void pool_relu_window_backward(const T (&xv)[4], float gy, T (&cell)[4]) {
+    auto relu_of = [](T v) { return Elem<T>::raw(v) >= 0.0f ? v : Elem<T>::zero(); };
+    float mf = Elem<T>::raw(relu_of(xv[0]));
+    int am = 0;
+#pragma unroll
+    for (int k = 1; k < 4; ++k) {
+        const float vf = Elem<T>::raw(relu_of(xv[k]));
+        if (vf > mf) { mf = vf; am = k; }
+    }
+    const T g = Elem<T>::from_f32(0.0f + gy);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) cell[k] = (am == k && Elem<T>::raw(xv[k]) >= 0.0f) ? g : Elem<T>::zero();
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void lenet5_backward_kernel(LenetBackward<T> a) {
+    __shared__ __align__(16) float wl[150 * 16];   // conv2's filter bank, [ci*25 + fi*5 + fj][oc]
+    __shared__ __align__(16) float gm2s[64 * 16];  // gradient of conv2's output, [y*8 + x][oc]
+    __shared__ float gls[16], gd2s[84], gd1s[128], gfs[256], gp1s[864];
+    constexpr int NT = 256;
+    const int tid = threadIdx.x;
+    const size_t b = blockIdx.x;
+    for (int i = tid; i < 2400; i += NT) {
+        const int o = i / 150, k = i - o * 150;  // coalesced read of w2[o][k]
+        wl[k * 16 + o] = Elem<T>::to_f32(a.w2[i]);
+    }
+    // cross-entropy backward (softmax - one-hot, times dy), rounded to T
+    if (tid < 10) {
+        const T *row = a.logits + b * 10;
+        float m = Elem<T>::to_f32(row[0]);
+        for (int j = 0; j < 10; ++j) m = fmaxf(m, Elem<T>::to_f32(row[j]));
+        float s = 0.0f;
+        for (int j = 0; j < 10; ++j) s += expf(Elem<T>::to_f32(row[j]) - m);
+        const float pr = expf(Elem<T>::to_f32(row[tid]) - m) / s;
+        const T g = Elem<T>::from_f32(a.dy * (pr - (tid == (int)a.target[b] ? 1.0f : 0.0f)));
+        a.g_logits[b * 10 + tid] = g;
+        gls[tid] = Elem<T>::to_f32(g);
+    }
+    __syncthreads();
+    // dense3: g_a2 = g_logits . wd3^T (wd3 [84, 10]), then relu backward on dense2's pre-activation
+    if (tid < 84) {
+        float d = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 10; ++c) d = __builtin_fmaf(gls[c], Elem<T>::to_f32(a.wd3[tid * 10 + c]), d);
+        const T ga = Elem<T>::from_f32(d);
+        const T gd = Elem<T>::raw(a.d2[b * 84 + tid]) >= 0.0f ? ga : Elem<T>::zero();
+        a.g_d2[b * 84 + tid] = gd;
+        gd2s[tid] = Elem<T>::to_f32(gd);
+    }
+    __syncthreads();
+    // dense2: g_a1 = g_d2 . wd2^T (wd2 [128, 84]), relu backward on dense1's pre-activation
+    if (tid < 128) {
+        const T *wr = a.wd2 + tid * 84;
+        float d = 0.0f;
+#pragma unroll 28
+        for (int c = 0; c < 84; ++c) d = __builtin_fmaf(gd2s[c], Elem<T>::to_f32(wr[c]), d);
+        const T ga = Elem<T>::from_f32(d);
+        const T gd = Elem<T>::raw(a.d1[b * 128 + tid]) >= 0.0f ? ga : Elem<T>::zero();
+        a.g_d1[b * 128 + tid] = gd;
+        gd1s[tid] = Elem<T>::to_f32(gd);
+    }
+    __syncthreads();
+    // dense1: g_f = g_d1 . wd1^T (wd1 [256, 128]); 16-byte loads of the thread's weight row
+    {
+        const T *wr = a.wd1 + tid * 128;
+        float d = 0.0f;
+        constexpr int EPV = 16 / (int)sizeof(T);
+#pragma unroll 8
+        for (int c = 0; c < 128; c += EPV) {
+            if constexpr (sizeof(T) == 4) {
+                const float4 w = *(const float4 *)(wr + c);
+                d = __builtin_fmaf(gd1s[c], w.x, d);
+                d = __builtin_fmaf(gd1s[c + 1], w.y, d);
+                d = __builtin_fmaf(gd1s[c + 2], w.z, d);
+                d = __builtin_fmaf(gd1s[c + 3], w.w, d);
+            } else {
+                const uint4 w = *(const uint4 *)(wr + c);
+                const uint32_t q[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    d = __builtin_fmaf(gd1s[c + 2 * e], __uint_as_float(q[e] << 16), d);
+                    d = __builtin_fmaf(gd1s[c + 2 * e + 1], __uint_as_float(q[e] & 0xFFFF0000u), d);
+                }
+            }
+        }
+        gfs[tid] = Elem<T>::to_f32(Elem<T>::from_f32(d));
+    }
+    __syncthreads();
+    // pooling + relu backward of conv2's output: one window per thread (16 channels x 4 x 4 windows)
+    {
+        const int oc = tid >> 4, ho = (tid >> 2) & 3, wo = tid & 3;
+        const T *xp = a.c2 + ((b * 16 + oc) * 8 + 2 * ho) * 8 + 2 * wo;
+        const T xv[4] = {xp[0], xp[1], xp[8], xp[9]};
+        T cell[4];
+        pool_relu_window_backward<T>(xv, gfs[tid], cell);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int pos = (2 * ho + (k >> 1)) * 8 + 2 * wo + (k & 1);
+            gm2s[pos * 16 + oc] = Elem<T>::to_f32(cell[k]);
+            a.gm2[(b * 64 + pos) * 16 + oc] = cell[k];
+        }
+    }
+    __syncthreads();
+    // conv2's input gradient: per pixel of the [6, 12, 12] map, the patch entries that land on it in the host's col2im
+    // order, each an f32 dot over the 16 output channels rounded to T, added in T
+    for (int e = tid; e < 864; e += NT) {
+        const int ci = e / 144, r = e - ci * 144, hy = r / 12, wy = r - hy * 12;
+        T acc = Elem<T>::zero();
+#pragma unroll 1
+        for (int fi = 4; fi >= 0; --fi) {
+            const int th = hy - fi;
+            const bool hok = th >= 0 && th < 8;
+            const int thc = min(max(th, 0), 7);
+#pragma unroll
+            for (int fj = 4; fj >= 0; --fj) {
+                const int tw = wy - fj;
+                const bool ok = hok && tw >= 0 && tw < 8;
+                const float4 *g = (const float4 *)(gm2s + (thc * 8 + min(max(tw, 0), 7)) * 16);
+                const float4 *w = (const float4 *)(wl + (ci * 25 + fi * 5 + fj) * 16);
+                float d = 0.0f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 gv = g[q], wv = w[q];
+                    d = __builtin_fmaf(gv.x, wv.x, d);
+                    d = __builtin_fmaf(gv.y, wv.y, d);
+                    d = __builtin_fmaf(gv.z, wv.z, d);
+                    d = __builtin_fmaf(gv.w, wv.w, d);
+                }
+                const T add = ok ? Elem<T>::from_f32(d) : Elem<T>::zero();
+                acc = Elem<T>::from_f32(Elem<T>::raw(acc) + Elem<T>::raw(add));
+            }
+        }
+        gp1s[e] = Elem<T>::to_f32(acc);
+    }
+    __syncthreads();
+    // pooling + relu backward of conv1's output (6 channels x 12 x 12 windows), written as the [576, 6] matrix
+    for (int e = tid; e < 864; e += NT) {
+        const int ci = e / 144, r = e - ci * 144, ho = r / 12, wo = r - ho * 12;
+        const T *xp = a.c1 + ((b * 6 + ci) * 24 + 2 * ho) * 24 + 2 * wo;
+        const T xv[4] = {xp[0], xp[1], xp[24], xp[25]};
+        T cell[4];
+        pool_relu_window_backward<T>(xv, gp1s[e], cell);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int pos = (2 * ho + (k >> 1)) * 24 + 2 * wo + (k & 1);
+            a.gm1[(b * 576 + pos) * 6 + ci] = cell[k];
+        }
+    }
+}
+
+template <typename T>
+int lenet5_backward_entry(const char *name, const void *logits, const void *target, float dy, const void *c1, const void *c2,
+                          const void *d1, const void *d2, const void *w2, const void *wd1, const void *wd2, const void *wd3,
+                          void *g_logits, void *g_d2, void *g_d1, void *gm2, void *gm1, int64_t bs) {
+    AGH_API_ENTER();
+    if (bs < 0) return fail(AGH_EINVAL, "%s: negative batch size", name);
+    if (bs == 0) return AGH_OK;
+    if (bs > ((int64_t)1 << 24)) return fail(AGH_ERANGE, "%s: batch too large", name);
+    if (!logits || !target || !c1 || !c2 || !d1 || !d2 || !w2 || !wd1 || !wd2 || !wd3 || !g_logits || !g_d2 || !g_d1 || !gm2 || !gm1)
+        return fail(AGH_ENULL, "%s: null buffer", name);
+    if (((uintptr_t)wd1 & 15) != 0) return fail(AGH_EINVAL, "%s: wd1 must be 16-byte aligned", name);
+    LenetBackward<T> a;
+    a.logits = (const T *)logits; a.target = (const uint8_t *)target;
+    a.c1 = (const T *)c1; a.c2 = (const T *)c2; a.d1 = (const T *)d1; a.d2 = (const T *)d2;
+    a.w2 = (const T *)w2; a.wd1 = (const T *)wd1; a.wd2 = (const T *)wd2; a.wd3 = (const T *)wd3;
+    a.g_logits = (T *)g_logits; a.g_d2 = (T *)g_d2; a.g_d1 = (T *)g_d1; a.gm2 = (T *)gm2; a.gm1 = (T *)gm1;
+    a.dy = dy / (float)bs;  // `dy /= batch_size` first, in f32, as the host does
+    hipLaunchKernelGGL(lenet5_backward_kernel<T>, dim3((unsigned)bs), dim3(256), 0, stream(), a);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+// The weight gradients of the three dense layers, the bias gradient and the loss of a LeNet5 training step in one
+// launch: dwd3 = a2^T . g_logits [84, 10], dwd2 = a1^T . g_d2 [128, 84], dwd1 = f^T . g_d1 [256, 128] (each an f32 dot over
+// the batch, rounded once to T, as the GEMM rounds it), db3 = the rows of g_logits added one at a time in T (the axis-0
+// sum of the host), loss = the row losses added in row order (one workgroup, as cross_entropy_loss_kernel).  A
+// workgroup owns a 16 x 16 tile of one product and stages the two 16-column strips it multiplies in LDS.
+template <typename T>
+struct LenetDenseGrads {
+    const T *a2, *a1, *f;               // [bs, 84], [bs, 128], [bs, 256]
+    const T *g_logits, *g_d2, *g_d1;    // [bs, 10], [bs, 84], [bs, 128]
+    T *dwd3, *dwd2, *dwd1, *db3;        // [84, 10], [128, 84], [256, 128], [10]
+    const T *logits;                    // [bs, 10]
+    const uint8_t *target;              // [bs]
+    float *loss;                        // one f32 (device or pinned host memory); may be null
+    int bs;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void lenet5_dense_grads_kernel(LenetDenseGrads<T> q) {
+    constexpr int RCH = 128;  // batch rows per pass
+    __shared__ float as[RCH * 16], gs[RCH * 16];
+    __shared__ float part[256];
+    const int tid = threadIdx.x;
+    int wg = blockIdx.x;
+    // tiles: dwd1 16 x 8, dwd2 8 x 6, dwd3 6 x 1, then the bias gradient, then the loss
+    const T *A, *G;
+    T *D;
+    int K, N, tk, tn;
+    if (wg < 128) { A = q.f; G = q.g_d1; D = q.dwd1; K = 256; N = 128; tk = wg / 8; tn = wg % 8; }
+    else if (wg < 176) { wg -= 128; A = q.a1; G = q.g_d2; D = q.dwd2; K = 128; N = 84; tk = wg / 6; tn = wg % 6; }
+    else if (wg < 182) { wg -= 176; A = q.a2; G = q.g_logits; D = q.dwd3; K = 84; N = 10; tk = wg; tn = 0; }
+    else if (wg == 182) {
+        if (tid < 10) {
+            T acc = Elem<T>::zero();
+            for (int r = 0; r < q.bs; ++r) acc = Elem<T>::from_f32(Elem<T>::raw(acc) + Elem<T>::raw(q.g_logits[(size_t)r * 10 + tid]));
+            q.db3[tid] = acc;
+        }
+        return;
+    } else {
+        if (!q.loss) return;
+        float total = 0.0f;
+        for (int base = 0; base < q.bs; base += 256) {
+            const int r = base + tid;
+            float l = 0.0f;
+            if (r < q.bs) {
+                const T *row = q.logits + (size_t)r * 10;
+                float m = Elem<T>::to_f32(row[0]);
+                for (int j = 0; j < 10; ++j) m = fmaxf(m, Elem<T>::to_f32(row[j]));
+                float sum = 0.0f;
+                for (int j = 0; j < 10; ++j) sum += expf(Elem<T>::to_f32(row[j]) - m);
+                l = logf(sum) - (Elem<T>::to_f32(row[q.target[r]]) - m);
+            }
+            part[tid] = l;
+            __syncthreads();
+            if (tid == 0) {
+                const int cnt = min(256, q.bs - base);
+                for (int i = 0; i < cnt; ++i) total += part[i];
+            }
+            __syncthreads();
+        }
+        if (tid == 0) *q.loss = total;
+        return;
+    }
+    const int k0 = tk * 16, n0 = tn * 16;
+    const int i = tid >> 4, j = tid & 15;
+    float acc = 0.0f;
+    for (int r0 = 0; r0 < q.bs; r0 += RCH) {
+        const int rows = min(RCH, q.bs - r0);
+        __syncthreads();
+        // all 16 elements of a thread are requested before the first is stored: one at a time the staging alone would
+        // be a chain of eight memory latencies
+        T av[RCH * 16 / 256], gv[RCH * 16 / 256];
+#pragma unroll
+        for (int u = 0; u < RCH * 16 / 256; ++u) {
+            const int e = tid + u * 256, r = min(e >> 4, rows - 1), c = e & 15;
+            av[u] = A[(size_t)(r0 + r) * K + min(k0 + c, K - 1)];
+            gv[u] = G[(size_t)(r0 + r) * N + min(n0 + c, N - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < RCH * 16 / 256; ++u) {
+            const int e = tid + u * 256, r = e >> 4, c = e & 15;
+            const bool rok = r < rows;
+            as[e] = rok && k0 + c < K ? Elem<T>::to_f32(av[u]) : 0.0f;
+            gs[e] = rok && n0 + c < N ? Elem<T>::to_f32(gv[u]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int r = 0; r < rows; ++r) acc = __builtin_fmaf(as[r * 16 + i], gs[r * 16 + j], acc);
+    }
+    if (k0 + i < K && n0 + j < N) D[(size_t)(k0 + i) * N + n0 + j] = Elem<T>::from_f32(acc);
+}
+
+template <typename T>
+int lenet5_dense_grads_entry(const char *name, const void *a2, const void *a1, const void *f, const void *g_logits,
+                             const void *g_d2, const void *g_d1, void *dwd3, void *dwd2, void *dwd1, void *db3,
+                             const void *logits, const void *target, void *loss, int64_t bs) {
+    AGH_API_ENTER();
+    if (bs < 0) return fail(AGH_EINVAL, "%s: negative batch size", name);
+    if (bs == 0) return AGH_OK;
+    if (bs > ((int64_t)1 << 24)) return fail(AGH_ERANGE, "%s: batch too large", name);
+    if (!a2 || !a1 || !f || !g_logits || !g_d2 || !g_d1 || !dwd3 || !dwd2 || !dwd1 || !db3)
+        return fail(AGH_ENULL, "%s: null buffer", name);
+    if (loss && (!logits || !target)) return fail(AGH_ENULL, "%s: the loss needs the logits and the labels", name);
+    LenetDenseGrads<T> q;
+    q.a2 = (const T *)a2; q.a1 = (const T *)a1; q.f = (const T *)f;
+    q.g_logits = (const T *)g_logits; q.g_d2 = (const T *)g_d2; q.g_d1 = (const T *)g_d1;
+    q.dwd3 = (T *)dwd3; q.dwd2 = (T *)dwd2; q.dwd1 = (T *)dwd1; q.db3 = (T *)db3;
+    q.logits = (const T *)logits; q.target = (const uint8_t *)target; q.loss = (float *)loss; q.bs = (int)bs;
+    hipLaunchKernelGGL(lenet5_dense_grads_kernel<T>, dim3(184), dim3(256), 0, stream(), q);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
 template <typename T, bool POOL>
 int launch_oct(int oct, dim3 grid, dim3 block, size_t smem, const T *x, const T *w, const T *bias, T *y,
                const ConvParams &p) {
@@ -746,6 +1051,31 @@ int agh_lenet5_forward_train_bf16(const void *x, const void *w1, const void *w2,
                                   void *a1, void *d2, void *a2, void *logits, int64_t bs) {
     void *saves[8] = {c1, p1, c2, p2, d1, a1, d2, a2};
     return lenet5_forward_entry<uint16_t>("agh_lenet5_forward_train_bf16", x, w1, w2, wd1, wd2, wd3, b3, logits, bs, saves);
+}
+
+#define AGH_LENET_BWD_ARGS                                                                                             \
+    const void *logits, const void *target, float dy, const void *c1, const void *c2, const void *d1, const void *d2, \
+        const void *w2, const void *wd1, const void *wd2, const void *wd3, void *g_logits, void *g_d2, void *g_d1,    \
+        void *gm2, void *gm1, int64_t bs
+int agh_lenet5_backward_f32(AGH_LENET_BWD_ARGS) {
+    return lenet5_backward_entry<float>("agh_lenet5_backward_f32", logits, target, dy, c1, c2, d1, d2, w2, wd1, wd2, wd3,
+                                        g_logits, g_d2, g_d1, gm2, gm1, bs);
+}
+int agh_lenet5_backward_bf16(AGH_LENET_BWD_ARGS) {
+    return lenet5_backward_entry<uint16_t>("agh_lenet5_backward_bf16", logits, target, dy, c1, c2, d1, d2, w2, wd1, wd2, wd3,
+                                           g_logits, g_d2, g_d1, gm2, gm1, bs);
+}
+
+#define AGH_LENET_DG_ARGS                                                                                            \
+    const void *a2, const void *a1, const void *f, const void *g_logits, const void *g_d2, const void *g_d1, void *dwd3, \
+        void *dwd2, void *dwd1, void *db3, const void *logits, const void *target, void *loss, int64_t bs
+int agh_lenet5_dense_weight_grads_f32(AGH_LENET_DG_ARGS) {
+    return lenet5_dense_grads_entry<float>("agh_lenet5_dense_weight_grads_f32", a2, a1, f, g_logits, g_d2, g_d1, dwd3, dwd2,
+                                           dwd1, db3, logits, target, loss, bs);
+}
+int agh_lenet5_dense_weight_grads_bf16(AGH_LENET_DG_ARGS) {
+    return lenet5_dense_grads_entry<uint16_t>("agh_lenet5_dense_weight_grads_bf16", a2, a1, f, g_logits, g_d2, g_d1, dwd3,
+                                              dwd2, dwd1, db3, logits, target, loss, bs);
 }
 
 }  // extern "C"

@@ -236,7 +236,8 @@ class LeNet5Trainer:
     a graph (`capture`) and replayed.  Gradients stay available in `grads` after a step.  `overlap`
     issues the weight gradients beside the input-gradient chain (`branch`); same kernels, same bits."""
 
-    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None, overlap=True, fused_forward=None):
+    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None, overlap=True, fused_forward=None,
+                 fused_backward=True):
         self.model, self.bs, self.lr = model, batch_size, learning_rate
         # fused_forward: the forward pass is ONE launch (agh_lenet5_forward_train_*) that also writes every activation
         # the backward edges read; the patch matrices the weight gradients multiply are then built beside the backward
@@ -245,8 +246,12 @@ class LeNet5Trainer:
         # against 0.164 ms: at batch 100 it is 25 workgroups walking twelve layers one after the other, and its bf16
         # form takes 30-47 us).
         if fused_forward is None:
-            fused_forward = model.conv1.weight.dtype == "f32"
+            fused_forward = fused_backward or model.conv1.weight.dtype == "f32"
         self.fused_forward = fused_forward
+        # fused_backward: the input-gradient chain (cross-entropy backward, three dense input gradients with their relu
+        # backward, both pooling + relu backward passes, conv2's input gradient) is ONE launch, agh_lenet5_backward_*,
+        # in place of nine; the weight gradients are the same GEMMs either way
+        self.fused_backward = fused_backward
         self._branch = branch if overlap else contextlib.nullcontext
         self.opt = optimizer if optimizer is not None else SGD()
         bs, dt = batch_size, model.conv1.weight.dtype
@@ -378,25 +383,45 @@ class LeNet5Trainer:
             gemm(1.0, f.t(), self.g_d1, 0.0, dwd1)
             gemm(1.0, self.gm2.t(), self.cols2, 0.0, dw2.into_shape((16, 150)))
 
-        check(self._fn("agh_cross_entropy_backward")(self.logits._ptr(), target.ptr, 1.0, self.g_logits._ptr(), bs, 10))
-        gemm(1.0, self.g_logits, wd3.t(), 0.0, self.g_a2)
-        self._relu_backward(self.d2, self.g_a2, self.g_d2)
-        gemm(1.0, self.g_d2, wd2.t(), 0.0, self.g_a1)
-        self._relu_backward(self.d1, self.g_a1, self.g_d1)
-        gemm(1.0, self.g_d1, wd1.t(), 0.0, self.g_f)
-        self._pool_relu_backward(self.c2, self.g_f.into_shape((bs, 16, 4, 4)), self.gm2)
-        with self._branch():
-            weight_grads()
-        # input gradient of conv2: dot with the weight matrix and col2im (layer.rs:976-988) in one launch
-        check(self._fn("agh_conv2_backward_input")(self.gm2._ptr(), w2._data_ptr(), self.g_p1._ptr(), bs, 6, 8, 8, 16,
-                                                   5, 5, 0, 0, 1, 1, 1, 1))
-        self._pool_relu_backward(self.c1, self.g_p1, self.gm1)
-        if self.fused_forward and self._branch is branch:
-            join()  # the patch matrix of conv1 was built on the second stream
-            gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
-        else:
+        if self.fused_backward:
+            check(self._fn("agh_lenet5_backward")(
+                self.logits._ptr(), target.ptr, 1.0, self.c1._ptr(), self.c2._ptr(), self.d1._ptr(), self.d2._ptr(),
+                w2._data_ptr(), wd1._data_ptr(), wd2._data_ptr(), wd3._data_ptr(), self.g_logits._ptr(), self.g_d2._ptr(),
+                self.g_d1._ptr(), self.gm2._ptr(), self.gm1._ptr(), bs))
+            # everything below only waits for that launch: the weight-gradient products and the loss are dealt to the two
+            # streams in two arms of about equal length (the patch matrices of a one-launch forward pass were built on
+            # the second stream meanwhile: joined first)
+            if self.fused_forward:
+                join()
+            with self._branch():
+                # the dense layers' weight gradients, the bias gradient and the loss: one launch
+                check(self._fn("agh_lenet5_dense_weight_grads")(
+                    self.a2._ptr(), self.a1._ptr(), f._data_ptr(), self.g_logits._ptr(), self.g_d2._ptr(), self.g_d1._ptr(),
+                    dwd3._data_ptr(), dwd2._data_ptr(), dwd1._data_ptr(), db3._data_ptr(), self.logits._ptr(), target.ptr,
+                    self._loss_host, bs))
+                gemm(1.0, self.gm2.t(), self.cols2, 0.0, dw2.into_shape((16, 150)))
             gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
             join()
+        else:
+            check(self._fn("agh_cross_entropy_backward")(self.logits._ptr(), target.ptr, 1.0, self.g_logits._ptr(), bs, 10))
+            gemm(1.0, self.g_logits, wd3.t(), 0.0, self.g_a2)
+            self._relu_backward(self.d2, self.g_a2, self.g_d2)
+            gemm(1.0, self.g_d2, wd2.t(), 0.0, self.g_a1)
+            self._relu_backward(self.d1, self.g_a1, self.g_d1)
+            gemm(1.0, self.g_d1, wd1.t(), 0.0, self.g_f)
+            self._pool_relu_backward(self.c2, self.g_f.into_shape((bs, 16, 4, 4)), self.gm2)
+            with self._branch():
+                weight_grads()
+            # input gradient of conv2: dot with the weight matrix and col2im (layer.rs:976-988) in one launch
+            check(self._fn("agh_conv2_backward_input")(self.gm2._ptr(), w2._data_ptr(), self.g_p1._ptr(), bs, 6, 8, 8, 16,
+                                                       5, 5, 0, 0, 1, 1, 1, 1))
+            self._pool_relu_backward(self.c1, self.g_p1, self.gm1)
+            if self.fused_forward and self._branch is branch:
+                join()  # the patch matrix of conv1 was built on the second stream
+                gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
+            else:
+                gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
+                join()
         # update: all parameters at once (element-wise, so one launch over the shared buffers)
         self.opt.update(self.lr, self._wflat, self._gflat, self._vflat)
 

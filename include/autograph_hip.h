@@ -315,6 +315,36 @@ int agh_lenet5_forward_train_bf16(const void *x, const void *w1, const void *w2,
                                   const void *wd3, const void *b3, void *c1, void *p1, void *c2, void *p2, void *d1,
                                   void *a1, void *d2, void *a2, void *logits, int64_t bs);
 
+/* The input-gradient chain of the same training step in one launch (the backward edges of
+ * src/learn/neural_network/autograd.rs:239-261 in their order: criterion.rs:79-103, autograd.rs:607-627, layer.rs:1253-1267,
+ * :1193-1216, :950-1005): from the logits and the u8 labels, the activations agh_lenet5_forward_train_<T> wrote (c1, c2, d1,
+ * d2) and the weights, it writes what the weight gradients multiply: g_logits [bs,10] = dy / bs * (softmax - one-hot),
+ * g_d2 [bs,84] and g_d1 [bs,128] (gradients of the dense pre-activations), gm2 [bs*64, 16] and gm1 [bs*576, 6] (gradients
+ * of the convolution outputs, as the standard-layout [bs*h*w, c] matrices of layer.rs:976-1003).  dW is then
+ * a2^T . g_logits, a1^T . g_d2, flatten(p2)^T . g_d1, gm2^T . im2col(p1) and gm1^T . im2col(x); db3 the axis-0 sum of
+ * g_logits.  Values are rounded to T where the separate calls (agh_cross_entropy_backward, agh_gemm, agh_relu_backward,
+ * agh_max_pool2_relu_backward, agh_conv2_backward_input) round them; the dense dot products sum in f32 in another
+ * order than the GEMM kernels.  wd1 must be 16-byte aligned. */
+int agh_lenet5_backward_f32(const void *logits, const void *target, float dy, const void *c1, const void *c2,
+                            const void *d1, const void *d2, const void *w2, const void *wd1, const void *wd2,
+                            const void *wd3, void *g_logits, void *g_d2, void *g_d1, void *gm2, void *gm1, int64_t bs);
+int agh_lenet5_backward_bf16(const void *logits, const void *target, float dy, const void *c1, const void *c2,
+                             const void *d1, const void *d2, const void *w2, const void *wd1, const void *wd2,
+                             const void *wd3, void *g_logits, void *g_d2, void *g_d1, void *gm2, void *gm1, int64_t bs);
+
+/* The dense layers' weight gradients, the bias gradient and the loss of that step in one launch (autograd.rs:607-627,
+ * :490-542, criterion.rs:205-226): dwd3 [84,10] = a2^T . g_logits, dwd2 [128,84] = a1^T . g_d2, dwd1 [256,128] =
+ * f^T . g_d1 with f = flatten(p2) [bs,256], each dot summed in f32 over the batch and rounded once to T (as agh_gemm
+ * rounds it); db3 [10] = the rows of g_logits added one at a time in T (agh_sum_axis0); *loss = the summed cross-entropy
+ * of `logits` against the u8 labels, rows added in order (agh_cross_entropy_loss), written as one f32 to device or pinned
+ * host memory; loss may be null (then logits and target are not read). */
+int agh_lenet5_dense_weight_grads_f32(const void *a2, const void *a1, const void *f, const void *g_logits,
+                                      const void *g_d2, const void *g_d1, void *dwd3, void *dwd2, void *dwd1, void *db3,
+                                      const void *logits, const void *target, void *loss, int64_t bs);
+int agh_lenet5_dense_weight_grads_bf16(const void *a2, const void *a1, const void *f, const void *g_logits,
+                                       const void *g_d2, const void *g_d1, void *dwd3, void *dwd2, void *dwd1, void *db3,
+                                       const void *logits, const void *target, void *loss, int64_t bs);
+
 /* ---------------------------------------------------------------- max pool ---- */
 
 /* MaxPool2 device branch (src/tensor/ops.rs:1117-1133; rule from the host impl

@@ -188,10 +188,52 @@ def test_lenet5_forward_train_saves_every_activation(ag, dtype, bs):
                                                                          *[o._ptr() for o in outs[:3]], None, *[o._ptr() for o in outs[4:]], bs))
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_lenet5_backward_one_launch_against_the_separate_launches(ag, dtype):
+    """agh_lenet5_backward_<T> against the nine launches it replaces, on the same activations: the cross-entropy
+    gradient bit for bit, the rest up to the summation order of the dense dot products (every rounding point and the
+    order of the T-typed col2im sums are the same)."""
+    rng = np.random.default_rng(46)
+    params = [to_dtype(p, dtype) for p in lenet_params(rng)]
+    bs = 100
+    x = to_dtype(rng.uniform(0, 1, (bs, 1, 28, 28)), dtype)
+    t = rng.integers(0, 10, bs).astype(np.uint8)
+    tx, tt = ag.Tensor.from_array(x), labels(ag, t)
+    got, want = {}, {}
+    for fused, out in ((True, got), (False, want)):
+        tr = ag.LeNet5Trainer(ag.LeNet5.from_arrays(*params), bs, optimizer=ag.SGD(None), overlap=False,
+                              fused_forward=True, fused_backward=fused)
+        tr.step(tx, tt)
+        ag._ffi.check(ag.lib.agh_sync())
+        for name in ("g_logits", "g_d2", "g_d1", "gm2", "gm1"):
+            out[name] = as_f32(getattr(tr, name).into_array()).astype(np.float64)
+        out["loss"] = tr.loss()
+        for name, g in zip(("dw1", "dw2", "dwd1", "dwd2", "dwd3", "db3"), tr.grads):
+            out[name] = as_f32(g.into_array()).astype(np.float64)
+    assert np.array_equal(got["g_logits"], want["g_logits"])
+    # same rows added in the same order: the bias gradient and the loss of agh_lenet5_dense_weight_grads_<T> are those of
+    # agh_sum_axis0_<T> / agh_cross_entropy_loss_<T> bit for bit; dwd3 multiplies identical operands in another order
+    assert np.array_equal(got["db3"], want["db3"]) and got["loss"] == want["loss"]
+    assert np.abs(got["dwd3"] - want["dwd3"]).max() <= (1e-5 if dtype == "f32" else 2.0**-7) * np.abs(want["dwd3"]).max()
+    for name in ("dw1", "dw2", "dwd1", "dwd2"):
+        sc = np.abs(want[name]).max()
+        assert np.abs(got[name] - want[name]).max() <= (1e-4 if dtype == "f32" else 2.0**-5) * sc, name
+    for name in ("g_d2", "g_d1", "gm2", "gm1"):
+        g, w = got[name], want[name]
+        scale = np.abs(w).max()
+        assert scale > 0
+        assert np.array_equal(g == 0, w == 0) or np.mean((g == 0) != (w == 0)) < 1e-3, name  # same relu / pooling decisions
+        if dtype == "f32":
+            assert np.abs(g - w).max() <= 1e-5 * scale, name
+        else:
+            assert np.abs(g - w).max() <= 2.0**-6 * scale and np.abs(g - w).mean() <= 2.0**-11 * scale, name
+
+
+@pytest.mark.parametrize("fused_backward", [True, False])
 @pytest.mark.parametrize("fused_forward", [True, False])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("momentum", [None, 0.01])
-def test_lenet5_train_step(ag, dtype, momentum, fused_forward):
+def test_lenet5_train_step(ag, dtype, momentum, fused_forward, fused_backward):
     rng = np.random.default_rng(44)
     params = [to_dtype(p, dtype) for p in lenet_params(rng)]
     bs = 100
@@ -200,7 +242,8 @@ def test_lenet5_train_step(ag, dtype, momentum, fused_forward):
     want_loss, want_params, want_grads, want_v = orc.lenet5_train_step(x, t, params, lr=0.01, momentum=momentum)
 
     model = ag.LeNet5.from_arrays(*params)
-    trainer = ag.LeNet5Trainer(model, bs, learning_rate=0.01, optimizer=ag.SGD(momentum), fused_forward=fused_forward)
+    trainer = ag.LeNet5Trainer(model, bs, learning_rate=0.01, optimizer=ag.SGD(momentum), fused_forward=fused_forward,
+                               fused_backward=fused_backward)
     tx, tt = ag.Tensor.from_array(x), labels(ag, t)
     trainer.step(tx, tt)
     ag._ffi.check(ag.lib.agh_sync())
