@@ -578,82 +578,118 @@ __global__ __launch_bounds__(256) void lenet5_backward_kernel(LenetBackward<T> a
     __shared__ __align__(16) float wl[150 * 16];   // conv2's filter bank, [ci*25 + fi*5 + fj][oc]
     __shared__ __align__(16) float gm2s[64 * 16];  // gradient of conv2's output, [y*8 + x][oc]
     __shared__ float gls[16], gd2s[84], gd1s[128], gfs[256], gp1s[864];
+    constexpr int kPmPitch = 151;                  // odd: the col2im reads of neighbouring pixels fall into different banks
+    __shared__ float pm[64 * kPmPitch];            // gm2 . W, every entry rounded to T
     constexpr int NT = 256;
+    constexpr int EPV = 16 / (int)sizeof(T);  // elements per 16-byte load
     const int tid = threadIdx.x;
     const size_t b = blockIdx.x;
-    for (int i = tid; i < 2400; i += NT) {
-        const int o = i / 150, k = i - o * 150;  // coalesced read of w2[o][k]
-        wl[k * 16 + o] = Elem<T>::to_f32(a.w2[i]);
+    // Everything this workgroup reads from memory has an address known now, so all of it is requested here, before the
+    // first use: the stages below are a chain of seven short steps, and a load issued inside a step would add its L2
+    // latency to that chain.  (About 100 registers per thread; the launch is 100 workgroups, occupancy is no concern.)
+    T w2v[10];  // the filter bank, coalesced: element tid + u * 256 of w2[oc][ci*25 + tap]
+#pragma unroll
+    for (int u = 0; u < 10; ++u) w2v[u] = a.w2[min(tid + u * NT, 2399)];
+    T lrow[10];  // the image's logits (used by the ten threads of the first stage)
+#pragma unroll
+    for (int j = 0; j < 10; ++j) lrow[j] = a.logits[b * 10 + j];
+    const int label = a.target[b];
+    T w3v[10];   // row min(tid, 83) of wd3
+#pragma unroll
+    for (int c = 0; c < 10; ++c) w3v[c] = a.wd3[min(tid, 83) * 10 + c];
+    const T d2v = a.d2[b * 84 + min(tid, 83)], d1v = a.d1[b * 128 + (tid & 127)];
+    uint2 w2r[84 * (int)sizeof(T) / 8];  // row tid & 127 of wd2 (84 elements: 8-byte aligned)
+    {
+        const uint2 *src = (const uint2 *)(a.wd2 + (tid & 127) * 84);
+#pragma unroll
+        for (int c = 0; c < 84 * (int)sizeof(T) / 8; ++c) w2r[c] = src[c];
     }
+    uint4 w1r[128 / EPV];  // row tid of wd1
+    {
+        const uint4 *src = (const uint4 *)(a.wd1 + tid * 128);
+#pragma unroll
+        for (int c = 0; c < 128 / EPV; ++c) w1r[c] = src[c];
+    }
+    T x2[4];  // the thread's pooling window of conv2's output
+    {
+        const int oc = tid >> 4, ho = (tid >> 2) & 3, wo = tid & 3;
+        const T *xp = a.c2 + ((b * 16 + oc) * 8 + 2 * ho) * 8 + 2 * wo;
+        x2[0] = xp[0]; x2[1] = xp[1]; x2[2] = xp[8]; x2[3] = xp[9];
+    }
+    T x1[4][4];  // its (up to four) pooling windows of conv1's output
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int e = min(tid + u * NT, 863);
+        const int ci = e / 144, r = e - ci * 144, ho = r / 12, wo = r - ho * 12;
+        const T *xp = a.c1 + ((b * 6 + ci) * 24 + 2 * ho) * 24 + 2 * wo;
+        x1[u][0] = xp[0]; x1[u][1] = xp[1]; x1[u][2] = xp[24]; x1[u][3] = xp[25];
+    }
+    auto elem = [](const auto &packed, int c) -> float {  // element c of a row held as 8- or 16-byte words
+        if constexpr (sizeof(T) == 4) return __uint_as_float(((const uint32_t *)&packed)[c]);
+        else {
+            const uint32_t w = ((const uint32_t *)&packed)[c >> 1];
+            return __uint_as_float((c & 1) ? (w & 0xFFFF0000u) : (w << 16));
+        }
+    };
+
     // cross-entropy backward (softmax - one-hot, times dy), rounded to T
     if (tid < 10) {
-        const T *row = a.logits + b * 10;
-        float m = Elem<T>::to_f32(row[0]);
-        for (int j = 0; j < 10; ++j) m = fmaxf(m, Elem<T>::to_f32(row[j]));
+        float m = Elem<T>::to_f32(lrow[0]);
+#pragma unroll
+        for (int j = 0; j < 10; ++j) m = fmaxf(m, Elem<T>::to_f32(lrow[j]));
         float s = 0.0f;
-        for (int j = 0; j < 10; ++j) s += expf(Elem<T>::to_f32(row[j]) - m);
-        const float pr = expf(Elem<T>::to_f32(row[tid]) - m) / s;
-        const T g = Elem<T>::from_f32(a.dy * (pr - (tid == (int)a.target[b] ? 1.0f : 0.0f)));
+#pragma unroll
+        for (int j = 0; j < 10; ++j) s += expf(Elem<T>::to_f32(lrow[j]) - m);
+        float mine = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 10; ++j) mine = j == tid ? Elem<T>::to_f32(lrow[j]) : mine;
+        const float pr = expf(mine - m) / s;
+        const T g = Elem<T>::from_f32(a.dy * (pr - (tid == label ? 1.0f : 0.0f)));
         a.g_logits[b * 10 + tid] = g;
         gls[tid] = Elem<T>::to_f32(g);
+    }
+#pragma unroll
+    for (int u = 0; u < 10; ++u) {
+        const int i = tid + u * NT;
+        const int o = i / 150, k = i - o * 150;
+        if (i < 2400) wl[k * 16 + o] = Elem<T>::to_f32(w2v[u]);
     }
     __syncthreads();
     // dense3: g_a2 = g_logits . wd3^T (wd3 [84, 10]), then relu backward on dense2's pre-activation
     if (tid < 84) {
         float d = 0.0f;
 #pragma unroll
-        for (int c = 0; c < 10; ++c) d = __builtin_fmaf(gls[c], Elem<T>::to_f32(a.wd3[tid * 10 + c]), d);
+        for (int c = 0; c < 10; ++c) d = __builtin_fmaf(gls[c], Elem<T>::to_f32(w3v[c]), d);
         const T ga = Elem<T>::from_f32(d);
-        const T gd = Elem<T>::raw(a.d2[b * 84 + tid]) >= 0.0f ? ga : Elem<T>::zero();
+        const T gd = Elem<T>::raw(d2v) >= 0.0f ? ga : Elem<T>::zero();
         a.g_d2[b * 84 + tid] = gd;
         gd2s[tid] = Elem<T>::to_f32(gd);
     }
     __syncthreads();
     // dense2: g_a1 = g_d2 . wd2^T (wd2 [128, 84]), relu backward on dense1's pre-activation
     if (tid < 128) {
-        const T *wr = a.wd2 + tid * 84;
         float d = 0.0f;
-#pragma unroll 28
-        for (int c = 0; c < 84; ++c) d = __builtin_fmaf(gd2s[c], Elem<T>::to_f32(wr[c]), d);
+#pragma unroll
+        for (int c = 0; c < 84; ++c) d = __builtin_fmaf(gd2s[c], elem(w2r, c), d);
         const T ga = Elem<T>::from_f32(d);
-        const T gd = Elem<T>::raw(a.d1[b * 128 + tid]) >= 0.0f ? ga : Elem<T>::zero();
+        const T gd = Elem<T>::raw(d1v) >= 0.0f ? ga : Elem<T>::zero();
         a.g_d1[b * 128 + tid] = gd;
         gd1s[tid] = Elem<T>::to_f32(gd);
     }
     __syncthreads();
-    // dense1: g_f = g_d1 . wd1^T (wd1 [256, 128]); 16-byte loads of the thread's weight row
+    // dense1: g_f = g_d1 . wd1^T (wd1 [256, 128])
     {
-        const T *wr = a.wd1 + tid * 128;
         float d = 0.0f;
-        constexpr int EPV = 16 / (int)sizeof(T);
-#pragma unroll 8
-        for (int c = 0; c < 128; c += EPV) {
-            if constexpr (sizeof(T) == 4) {
-                const float4 w = *(const float4 *)(wr + c);
-                d = __builtin_fmaf(gd1s[c], w.x, d);
-                d = __builtin_fmaf(gd1s[c + 1], w.y, d);
-                d = __builtin_fmaf(gd1s[c + 2], w.z, d);
-                d = __builtin_fmaf(gd1s[c + 3], w.w, d);
-            } else {
-                const uint4 w = *(const uint4 *)(wr + c);
-                const uint32_t q[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    d = __builtin_fmaf(gd1s[c + 2 * e], __uint_as_float(q[e] << 16), d);
-                    d = __builtin_fmaf(gd1s[c + 2 * e + 1], __uint_as_float(q[e] & 0xFFFF0000u), d);
-                }
-            }
-        }
+        for (int c = 0; c < 128; ++c) d = __builtin_fmaf(gd1s[c], elem(w1r, c), d);
         gfs[tid] = Elem<T>::to_f32(Elem<T>::from_f32(d));
     }
     __syncthreads();
     // pooling + relu backward of conv2's output: one window per thread (16 channels x 4 x 4 windows)
     {
         const int oc = tid >> 4, ho = (tid >> 2) & 3, wo = tid & 3;
-        const T *xp = a.c2 + ((b * 16 + oc) * 8 + 2 * ho) * 8 + 2 * wo;
-        const T xv[4] = {xp[0], xp[1], xp[8], xp[9]};
         T cell[4];
-        pool_relu_window_backward<T>(xv, gfs[tid], cell);
+        pool_relu_window_backward<T>(x2, gfs[tid], cell);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const int pos = (2 * ho + (k >> 1)) * 8 + 2 * wo + (k & 1);
@@ -662,12 +698,43 @@ __global__ __launch_bounds__(256) void lenet5_backward_kernel(LenetBackward<T> a
         }
     }
     __syncthreads();
-    // conv2's input gradient: per pixel of the [6, 12, 12] map, the patch entries that land on it in the host's col2im
-    // order, each an f32 dot over the 16 output channels rounded to T, added in T
+    // conv2's input gradient in two steps, as the host does it.  First the product gm2 . W, a [64, 150] matrix whose
+    // entries are f32 dots over the 16 output channels (ascending) rounded to T: a thread owns 4 positions x 10 taps and
+    // keeps its four gradient rows in registers, so an entry costs a fraction of the LDS reads a per-pixel walk would need.
+    if (tid < 240) {
+        const int pg = tid / 15, kg = tid - pg * 15;
+        float4 g[4][4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) g[r][q] = *(const float4 *)(gm2s + (pg * 4 + r) * 16 + q * 4);
+#pragma unroll 2
+        for (int kk = 0; kk < 10; ++kk) {
+            const int k = kg * 10 + kk;
+            float4 w[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) w[q] = *(const float4 *)(wl + k * 16 + q * 4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float d = 0.0f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    d = __builtin_fmaf(g[r][q].x, w[q].x, d);
+                    d = __builtin_fmaf(g[r][q].y, w[q].y, d);
+                    d = __builtin_fmaf(g[r][q].z, w[q].z, d);
+                    d = __builtin_fmaf(g[r][q].w, w[q].w, d);
+                }
+                pm[(pg * 4 + r) * kPmPitch + k] = Elem<T>::to_f32(Elem<T>::from_f32(d));
+            }
+        }
+    }
+    __syncthreads();
+    // then col2im: per pixel of the [6, 12, 12] map the patch entries that land on it, added in T in the host's order
+    // (filter rows and columns descending)
     for (int e = tid; e < 864; e += NT) {
         const int ci = e / 144, r = e - ci * 144, hy = r / 12, wy = r - hy * 12;
         T acc = Elem<T>::zero();
-#pragma unroll 1
+#pragma unroll
         for (int fi = 4; fi >= 0; --fi) {
             const int th = hy - fi;
             const bool hok = th >= 0 && th < 8;
@@ -676,35 +743,26 @@ __global__ __launch_bounds__(256) void lenet5_backward_kernel(LenetBackward<T> a
             for (int fj = 4; fj >= 0; --fj) {
                 const int tw = wy - fj;
                 const bool ok = hok && tw >= 0 && tw < 8;
-                const float4 *g = (const float4 *)(gm2s + (thc * 8 + min(max(tw, 0), 7)) * 16);
-                const float4 *w = (const float4 *)(wl + (ci * 25 + fi * 5 + fj) * 16);
-                float d = 0.0f;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 gv = g[q], wv = w[q];
-                    d = __builtin_fmaf(gv.x, wv.x, d);
-                    d = __builtin_fmaf(gv.y, wv.y, d);
-                    d = __builtin_fmaf(gv.z, wv.z, d);
-                    d = __builtin_fmaf(gv.w, wv.w, d);
-                }
-                const T add = ok ? Elem<T>::from_f32(d) : Elem<T>::zero();
-                acc = Elem<T>::from_f32(Elem<T>::raw(acc) + Elem<T>::raw(add));
+                const float v = pm[(thc * 8 + min(max(tw, 0), 7)) * kPmPitch + ci * 25 + fi * 5 + fj];
+                acc = Elem<T>::from_f32(Elem<T>::raw(acc) + (ok ? v : 0.0f));
             }
         }
         gp1s[e] = Elem<T>::to_f32(acc);
     }
     __syncthreads();
     // pooling + relu backward of conv1's output (6 channels x 12 x 12 windows), written as the [576, 6] matrix
-    for (int e = tid; e < 864; e += NT) {
-        const int ci = e / 144, r = e - ci * 144, ho = r / 12, wo = r - ho * 12;
-        const T *xp = a.c1 + ((b * 6 + ci) * 24 + 2 * ho) * 24 + 2 * wo;
-        const T xv[4] = {xp[0], xp[1], xp[24], xp[25]};
-        T cell[4];
-        pool_relu_window_backward<T>(xv, gp1s[e], cell);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int pos = (2 * ho + (k >> 1)) * 24 + 2 * wo + (k & 1);
-            a.gm1[(b * 576 + pos) * 6 + ci] = cell[k];
+    for (int u = 0; u < 4; ++u) {
+        const int e = tid + u * NT;
+        if (e < 864) {
+            const int ci = e / 144, r = e - ci * 144, ho = r / 12, wo = r - ho * 12;
+            T cell[4];
+            pool_relu_window_backward<T>(x1[u], gp1s[e], cell);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int pos = (2 * ho + (k >> 1)) * 24 + 2 * wo + (k & 1);
+                a.gm1[(b * 576 + pos) * 6 + ci] = cell[k];
+            }
         }
     }
 }
@@ -719,7 +777,8 @@ int lenet5_backward_entry(const char *name, const void *logits, const void *targ
     if (bs > ((int64_t)1 << 24)) return fail(AGH_ERANGE, "%s: batch too large", name);
     if (!logits || !target || !c1 || !c2 || !d1 || !d2 || !w2 || !wd1 || !wd2 || !wd3 || !g_logits || !g_d2 || !g_d1 || !gm2 || !gm1)
         return fail(AGH_ENULL, "%s: null buffer", name);
-    if (((uintptr_t)wd1 & 15) != 0) return fail(AGH_EINVAL, "%s: wd1 must be 16-byte aligned", name);
+    if (((uintptr_t)wd1 & 15) != 0 || ((uintptr_t)wd2 & 7) != 0)
+        return fail(AGH_EINVAL, "%s: wd1 must be 16-byte and wd2 8-byte aligned", name);
     LenetBackward<T> a;
     a.logits = (const T *)logits; a.target = (const uint8_t *)target;
     a.c1 = (const T *)c1; a.c2 = (const T *)c2; a.d1 = (const T *)d1; a.d2 = (const T *)d2;
@@ -762,11 +821,23 @@ __global__ __launch_bounds__(256) void lenet5_dense_grads_kernel(LenetDenseGrads
     else if (wg < 176) { wg -= 128; A = q.a1; G = q.g_d2; D = q.dwd2; K = 128; N = 84; tk = wg / 6; tn = wg % 6; }
     else if (wg < 182) { wg -= 176; A = q.a2; G = q.g_logits; D = q.dwd3; K = 84; N = 10; tk = wg; tn = 0; }
     else if (wg == 182) {
-        if (tid < 10) {
-            T acc = Elem<T>::zero();
-            for (int r = 0; r < q.bs; ++r) acc = Elem<T>::from_f32(Elem<T>::raw(acc) + Elem<T>::raw(q.g_logits[(size_t)r * 10 + tid]));
-            q.db3[tid] = acc;
+        // the rows go through LDS, 200 at a time: read straight from memory the hundred dependent additions of a column
+        // would each wait for their own load
+        T acc = Elem<T>::zero();
+        for (int r0 = 0; r0 < q.bs; r0 += 200) {
+            const int cnt = min(200, q.bs - r0) * 10;
+            __syncthreads();
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = q.g_logits[(size_t)r0 * 10 + min(tid + u * 256, cnt - 1)];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (tid + u * 256 < cnt) as[tid + u * 256] = Elem<T>::to_f32(v[u]);
+            __syncthreads();
+            if (tid < 10)
+                for (int r = 0; r < cnt / 10; ++r) acc = Elem<T>::from_f32(Elem<T>::raw(acc) + as[r * 10 + tid]);
         }
+        if (tid < 10) q.db3[tid] = acc;
         return;
     } else {
         if (!q.loss) return;

@@ -324,7 +324,7 @@ int agh_lenet5_forward_train_bf16(const void *x, const void *w1, const void *w2,
  * a2^T . g_logits, a1^T . g_d2, flatten(p2)^T . g_d1, gm2^T . im2col(p1) and gm1^T . im2col(x); db3 the axis-0 sum of
  * g_logits.  Values are rounded to T where the separate calls (agh_cross_entropy_backward, agh_gemm, agh_relu_backward,
  * agh_max_pool2_relu_backward, agh_conv2_backward_input) round them; the dense dot products sum in f32 in another
- * order than the GEMM kernels.  wd1 must be 16-byte aligned. */
+ * order than the GEMM kernels.  wd1 must be 16-byte aligned, wd2 8-byte aligned. */
 int agh_lenet5_backward_f32(const void *logits, const void *target, float dy, const void *c1, const void *c2,
                             const void *d1, const void *d2, const void *w2, const void *wd1, const void *wd2,
                             const void *wd3, void *g_logits, void *g_d2, void *g_d1, void *gm2, void *gm1, int64_t bs);
