@@ -359,8 +359,11 @@ __device__ __forceinline__ void store_rounded(T *dst, const float (&v)[N]) {
     }
 }
 
+// waves_per_eu(2, 2): eight waves per workgroup are two per SIMD whatever the register count; without the hint the
+// compiler aimed the bf16 training instantiation at 128 registers and gave up the early weight loads for it (30 us
+// instead of 20)
 template <typename T, bool SAVE>
-__global__ __launch_bounds__(512) void lenet5_forward_kernel(const T *__restrict__ x, const T *__restrict__ w1,
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void lenet5_forward_kernel(const T *__restrict__ x, const T *__restrict__ w1,
                                                               const T *__restrict__ w2, const T *__restrict__ wd1,
                                                               const T *__restrict__ wd2, const T *__restrict__ wd3,
                                                               const T *__restrict__ b3, T *__restrict__ out, int bs,
