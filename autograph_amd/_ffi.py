@@ -81,6 +81,8 @@ SIGNATURES = {
     "agh_lenet5_backward_bf16": ([ptr, ptr, C.c_float] + [ptr] * 13 + [i64], C.c_int),
     "agh_lenet5_dense_weight_grads_f32": ([ptr] * 13 + [i64], C.c_int),
     "agh_lenet5_dense_weight_grads_bf16": ([ptr] * 13 + [i64], C.c_int),
+    "agh_lenet5_conv_weight_grads_f32": ([ptr] * 6 + [i64], C.c_int),
+    "agh_lenet5_conv_weight_grads_bf16": ([ptr] * 6 + [i64], C.c_int),
     "agh_max_pool2_f32": (_POOL, C.c_int),
     "agh_max_pool2_bf16": (_POOL, C.c_int),
     "agh_max_pool2_backward_f32": (_POOL, C.c_int),

@@ -917,6 +917,161 @@ int lenet5_dense_grads_entry(const char *name, const void *a2, const void *a1, c
     return AGH_OK;
 }
 
+// The weight gradients of the two convolutions of a LeNet5 training step without their patch matrices:
+// dw2[oc][ci][fi][fj] = sum over images and output positions of gm2[(y, x)][oc] * p1[ci][y + fi][x + fj] (the product
+// gm2^T . im2col(p1) of layer.rs:990-1003), dw1 likewise from gm1 and x.  One workgroup per image forms the image's f32
+// partial sums from operands staged in LDS; a second launch adds the partials in image order and rounds once to T, as
+// the split-K GEMM does.
+constexpr int kLenetPartPitch = 2560;  // per image: 2400 entries of dw2, 150 of dw1
+template <typename T>
+__global__ __launch_bounds__(512) void lenet5_conv_grads_kernel(const T *__restrict__ x, const T *__restrict__ p1,
+                                                                  const T *__restrict__ gm1, const T *__restrict__ gm2,
+                                                                  float *__restrict__ part) {
+    __shared__ __align__(16) float g2[64 * 16];   // [y*8 + x][oc]
+    __shared__ __align__(8) float g1[576 * 6];    // [y*24 + x][oc]
+    __shared__ float p1s[864], xs[784];
+    __shared__ float q2[16 * 150], q1[8 * 150];   // partial sums: conv2 second half of the positions; conv1 by row group
+    constexpr int NT = 512;
+    const int tid = threadIdx.x;
+    const size_t b = blockIdx.x;
+    {
+        // every element is requested before the first is stored
+        T v2[2], vp[2], vx[2], v1[7];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            v2[u] = gm2[b * 1024 + tid + u * NT];
+            vp[u] = p1[b * 864 + min(tid + u * NT, 863)];
+            vx[u] = x[b * 784 + min(tid + u * NT, 783)];
+        }
+#pragma unroll
+        for (int u = 0; u < 7; ++u) v1[u] = gm1[b * 3456 + min(tid + u * NT, 3455)];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int i = tid + u * NT;
+            g2[i] = Elem<T>::to_f32(v2[u]);
+            if (i < 864) p1s[i] = Elem<T>::to_f32(vp[u]);
+            if (i < 784) xs[i] = Elem<T>::to_f32(vx[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 7; ++u)
+            if (tid + u * NT < 3456) g1[tid + u * NT] = Elem<T>::to_f32(v1[u]);
+    }
+    __syncthreads();
+    float *out = part + b * kLenetPartPitch;
+    float acc2[16];
+    if (tid < 300) {
+        // conv2: one tap (ci, fi, fj) x 16 output channels over half of the 64 positions (ascending); the gradient row is
+        // a broadcast read
+        const int half = tid / 150, k = tid - half * 150;
+        const int ci = k / 25, t = k - ci * 25, fi = t / 5, fj = t - fi * 5;
+#pragma unroll
+        for (int o = 0; o < 16; ++o) acc2[o] = 0.0f;
+#pragma unroll
+        for (int yy = 0; yy < 4; ++yy) {
+            const int y = half * 4 + yy;
+#pragma unroll
+            for (int xx = 0; xx < 8; ++xx) {
+                const float v = p1s[ci * 144 + (y + fi) * 12 + xx + fj];
+                const float4 *g = (const float4 *)(g2 + (y * 8 + xx) * 16);
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd) {
+                    const float4 gv = g[qd];
+                    acc2[4 * qd + 0] = __builtin_fmaf(gv.x, v, acc2[4 * qd + 0]);
+                    acc2[4 * qd + 1] = __builtin_fmaf(gv.y, v, acc2[4 * qd + 1]);
+                    acc2[4 * qd + 2] = __builtin_fmaf(gv.z, v, acc2[4 * qd + 2]);
+                    acc2[4 * qd + 3] = __builtin_fmaf(gv.w, v, acc2[4 * qd + 3]);
+                }
+            }
+        }
+        if (half == 1) {
+#pragma unroll
+            for (int o = 0; o < 16; ++o) q2[o * 150 + k] = acc2[o];
+        }
+    } else if (tid < 500) {
+        // conv1: one tap x 6 output channels over three of the 24 output rows
+        const int t = tid - 300, rg = t / 25, tap = t - rg * 25, fi = tap / 5, fj = tap - fi * 5;
+        float acc[6];
+#pragma unroll
+        for (int o = 0; o < 6; ++o) acc[o] = 0.0f;
+#pragma unroll
+        for (int yy = 0; yy < 3; ++yy) {
+            const int y = 3 * rg + yy;
+#pragma unroll 12
+            for (int xx = 0; xx < 24; ++xx) {
+                const float v = xs[(y + fi) * 28 + xx + fj];
+                const float2 *g = (const float2 *)(g1 + (y * 24 + xx) * 6);
+                const float2 ga = g[0], gb = g[1], gc = g[2];
+                acc[0] = __builtin_fmaf(ga.x, v, acc[0]);
+                acc[1] = __builtin_fmaf(ga.y, v, acc[1]);
+                acc[2] = __builtin_fmaf(gb.x, v, acc[2]);
+                acc[3] = __builtin_fmaf(gb.y, v, acc[3]);
+                acc[4] = __builtin_fmaf(gc.x, v, acc[4]);
+                acc[5] = __builtin_fmaf(gc.y, v, acc[5]);
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < 6; ++o) q1[rg * 150 + o * 25 + tap] = acc[o];
+    }
+    __syncthreads();
+    if (tid < 150) {
+#pragma unroll
+        for (int o = 0; o < 16; ++o) out[o * 150 + tid] = acc2[o] + q2[o * 150 + tid];
+    } else if (tid >= 300 && tid < 450) {
+        const int k = tid - 300;
+        float s = q1[k];
+#pragma unroll
+        for (int rg = 1; rg < 8; ++rg) s += q1[rg * 150 + k];
+        out[2400 + k] = s;
+    }
+}
+
+// 64 outputs per workgroup; wave j adds the images of the j-th quarter of the batch (its loads all in flight together),
+// the four sums are then added in a fixed order
+template <typename T>
+__global__ __launch_bounds__(256) void lenet5_conv_grads_reduce_kernel(const float *__restrict__ part, T *__restrict__ dw1,
+                                                                         T *__restrict__ dw2, int bs) {
+    __shared__ float sums[4][64];
+    const int lane = threadIdx.x & 63, j = threadIdx.x >> 6;
+    const int k = min((int)blockIdx.x * 64 + lane, 2549);
+    const int per = (bs + 3) / 4, b0 = j * per, b1 = min(bs, b0 + per);
+    float s = 0.0f;
+    int b = b0;
+    for (; b + 8 <= b1; b += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = part[(size_t)(b + u) * kLenetPartPitch + k];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; b < b1; ++b) s += part[(size_t)b * kLenetPartPitch + k];
+    sums[j][lane] = s;
+    __syncthreads();
+    if (j == 0 && (int)blockIdx.x * 64 + lane < 2550) {
+        const float tot = (sums[0][lane] + sums[1][lane]) + (sums[2][lane] + sums[3][lane]);
+        if (k < 2400) dw2[k] = Elem<T>::from_f32(tot);
+        else dw1[k - 2400] = Elem<T>::from_f32(tot);
+    }
+}
+
+template <typename T>
+int lenet5_conv_grads_entry(const char *name, const void *x, const void *p1, const void *gm1, const void *gm2, void *dw1,
+                            void *dw2, int64_t bs) {
+    AGH_API_ENTER();
+    if (bs < 0) return fail(AGH_EINVAL, "%s: negative batch size", name);
+    if (bs == 0) return AGH_OK;
+    if (bs > ((int64_t)1 << 20)) return fail(AGH_ERANGE, "%s: batch too large", name);
+    if (!x || !p1 || !gm1 || !gm2 || !dw1 || !dw2) return fail(AGH_ENULL, "%s: null buffer", name);
+    void *ws = nullptr;
+    if (int rc = workspace((size_t)bs * kLenetPartPitch * sizeof(float), &ws)) return rc;
+    hipLaunchKernelGGL(lenet5_conv_grads_kernel<T>, dim3((unsigned)bs), dim3(512), 0, stream(), (const T *)x, (const T *)p1,
+                       (const T *)gm1, (const T *)gm2, (float *)ws);
+    AGH_LAUNCH_CHECK(name);
+    hipLaunchKernelGGL(lenet5_conv_grads_reduce_kernel<T>, dim3(40), dim3(256), 0, stream(), (const float *)ws, (T *)dw1,
+                       (T *)dw2, (int)bs);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
 template <typename T, bool POOL>
 int launch_oct(int oct, dim3 grid, dim3 block, size_t smem, const T *x, const T *w, const T *bias, T *y,
                const ConvParams &p) {
@@ -1150,6 +1305,15 @@ int agh_lenet5_dense_weight_grads_f32(AGH_LENET_DG_ARGS) {
 int agh_lenet5_dense_weight_grads_bf16(AGH_LENET_DG_ARGS) {
     return lenet5_dense_grads_entry<uint16_t>("agh_lenet5_dense_weight_grads_bf16", a2, a1, f, g_logits, g_d2, g_d1, dwd3,
                                               dwd2, dwd1, db3, logits, target, loss, bs);
+}
+
+int agh_lenet5_conv_weight_grads_f32(const void *x, const void *p1, const void *gm1, const void *gm2, void *dw1, void *dw2,
+                                     int64_t bs) {
+    return lenet5_conv_grads_entry<float>("agh_lenet5_conv_weight_grads_f32", x, p1, gm1, gm2, dw1, dw2, bs);
+}
+int agh_lenet5_conv_weight_grads_bf16(const void *x, const void *p1, const void *gm1, const void *gm2, void *dw1, void *dw2,
+                                      int64_t bs) {
+    return lenet5_conv_grads_entry<uint16_t>("agh_lenet5_conv_weight_grads_bf16", x, p1, gm1, gm2, dw1, dw2, bs);
 }
 
 }  // extern "C"

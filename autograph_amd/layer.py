@@ -236,7 +236,7 @@ class LeNet5Trainer:
     a graph (`capture`) and replayed.  Gradients stay available in `grads` after a step.  `overlap`
     issues the weight gradients beside the input-gradient chain (`branch`); same kernels, same bits."""
 
-    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None, overlap=True, fused_forward=None,
+    def __init__(self, model, batch_size, learning_rate=0.01, optimizer=None, overlap=None, fused_forward=None,
                  fused_backward=True):
         self.model, self.bs, self.lr = model, batch_size, learning_rate
         # fused_forward: the forward pass is ONE launch (agh_lenet5_forward_train_*) that also writes every activation
@@ -252,6 +252,11 @@ class LeNet5Trainer:
         # backward, both pooling + relu backward passes, conv2's input gradient) is ONE launch, agh_lenet5_backward_*,
         # in place of nine; the weight gradients are the same GEMMs either way
         self.fused_backward = fused_backward
+        # overlap: issue the weight gradients on the second stream beside the input-gradient chain.  Default: only for the
+        # layer-by-layer backward pass; with the one-launch forms a step is six kernels, and the fork and join of a second
+        # stream cost more (about 10 us) than the one launch they would hide
+        if overlap is None:
+            overlap = not fused_backward
         self._branch = branch if overlap else contextlib.nullcontext
         self.opt = optimizer if optimizer is not None else SGD()
         bs, dt = batch_size, model.conv1.weight.dtype
@@ -357,10 +362,12 @@ class LeNet5Trainer:
                 x._data_ptr(), w1._data_ptr(), w2._data_ptr(), wd1._data_ptr(), wd2._data_ptr(), wd3._data_ptr(),
                 b3._data_ptr(), self.c1._ptr(), self.p1._ptr(), self.c2._ptr(), self.p2._ptr(), self.d1._ptr(),
                 self.a1._ptr(), self.d2._ptr(), self.a2._ptr(), self.logits._ptr(), bs))
-            # the patch matrices feed only the weight gradients of the convolutions: built beside the backward chain
-            with self._branch():
-                check(self._fn("agh_im2col_conv2")(x._data_ptr(), self.cols1._ptr(), bs, 1, 28, 28, 5, 5, 0, 0, 1, 1, 1, 1))
-                check(self._fn("agh_im2col_conv2")(self.p1._ptr(), self.cols2._ptr(), bs, 6, 12, 12, 5, 5, 0, 0, 1, 1, 1, 1))
+            if not self.fused_backward:
+                # the patch matrices feed only the weight gradients of the convolutions: built beside the backward chain
+                # (the one-launch backward path forms those gradients without them)
+                with self._branch():
+                    check(self._fn("agh_im2col_conv2")(x._data_ptr(), self.cols1._ptr(), bs, 1, 28, 28, 5, 5, 0, 0, 1, 1, 1, 1))
+                    check(self._fn("agh_im2col_conv2")(self.p1._ptr(), self.cols2._ptr(), bs, 6, 12, 12, 5, 5, 0, 0, 1, 1, 1, 1))
         else:
             self._conv_forward(x, w1, self.cols1, self.c1)
             self._relu_pool(self.c1, self.p1)
@@ -388,19 +395,16 @@ class LeNet5Trainer:
                 self.logits._ptr(), target.ptr, 1.0, self.c1._ptr(), self.c2._ptr(), self.d1._ptr(), self.d2._ptr(),
                 w2._data_ptr(), wd1._data_ptr(), wd2._data_ptr(), wd3._data_ptr(), self.g_logits._ptr(), self.g_d2._ptr(),
                 self.g_d1._ptr(), self.gm2._ptr(), self.gm1._ptr(), bs))
-            # everything below only waits for that launch: the weight-gradient products and the loss are dealt to the two
-            # streams in two arms of about equal length (the patch matrices of a one-launch forward pass were built on
-            # the second stream meanwhile: joined first)
-            if self.fused_forward:
-                join()
+            # everything below only waits for that launch: the dense layers' weight gradients, the bias gradient and the
+            # loss are one launch on the second stream, the convolutions' weight gradients (formed without patch
+            # matrices) two on the first
             with self._branch():
-                # the dense layers' weight gradients, the bias gradient and the loss: one launch
                 check(self._fn("agh_lenet5_dense_weight_grads")(
                     self.a2._ptr(), self.a1._ptr(), f._data_ptr(), self.g_logits._ptr(), self.g_d2._ptr(), self.g_d1._ptr(),
                     dwd3._data_ptr(), dwd2._data_ptr(), dwd1._data_ptr(), db3._data_ptr(), self.logits._ptr(), target.ptr,
                     self._loss_host, bs))
-                gemm(1.0, self.gm2.t(), self.cols2, 0.0, dw2.into_shape((16, 150)))
-            gemm(1.0, self.gm1.t(), self.cols1, 0.0, dw1.into_shape((6, 25)))
+            check(self._fn("agh_lenet5_conv_weight_grads")(x._data_ptr(), self.p1._ptr(), self.gm1._ptr(), self.gm2._ptr(),
+                                                           dw1._data_ptr(), dw2._data_ptr(), bs))
             join()
         else:
             check(self._fn("agh_cross_entropy_backward")(self.logits._ptr(), target.ptr, 1.0, self.g_logits._ptr(), bs, 10))

@@ -446,7 +446,7 @@ def main():
                 if g_ms is None:
                     g_ms = e_ms
                 rec = {"gpu_ms": round(g_ms, 4), "gpu_eager_ms": round(e_ms, 4), "last_loss": round(trainer.loss(), 4),
-                       "what": "forward + summed cross-entropy + backward + SGD(momentum 0.01) update: the forward pass and the input-gradient chain one launch each, the dense weight gradients + bias gradient + loss one launch, two im2col launches, the convolutions' weight gradients two split-K GEMMs, one update launch; second stream beside the first; gpu_ms: "
+                       "what": "forward + summed cross-entropy + backward + SGD(momentum 0.01) update in six kernels on one stream: the forward pass, the input-gradient chain, the dense weight gradients + bias gradient + loss, the convolutions' weight gradients (per-image partial sums, then their reduction), the update; gpu_ms: "
                                "graph replay, wall clock per step including the host-side wait for the loss; "
                                "gpu_eager_ms: the same launches issued one by one from the host"}
                 if not args.no_cpu:

@@ -345,6 +345,15 @@ int agh_lenet5_dense_weight_grads_bf16(const void *a2, const void *a1, const voi
                                        const void *g_d2, const void *g_d1, void *dwd3, void *dwd2, void *dwd1, void *db3,
                                        const void *logits, const void *target, void *loss, int64_t bs);
 
+/* The two convolutions' weight gradients of that step without their patch matrices (layer.rs:990-1003:
+ * output_grad^T . im2col(input)): dw2 [16,6,5,5] from gm2 [bs*64,16] and p1 [bs,6,12,12], dw1 [6,1,5,5] from gm1
+ * [bs*576,6] and x [bs,1,28,28].  Per image the sums run in f32 over the output positions; the images' partial sums
+ * (in the library's workspace) are added in image order and rounded once to T, as a split-K agh_gemm rounds. */
+int agh_lenet5_conv_weight_grads_f32(const void *x, const void *p1, const void *gm1, const void *gm2, void *dw1, void *dw2,
+                                     int64_t bs);
+int agh_lenet5_conv_weight_grads_bf16(const void *x, const void *p1, const void *gm1, const void *gm2, void *dw1, void *dw2,
+                                      int64_t bs);
+
 /* ---------------------------------------------------------------- max pool ---- */
 
 /* MaxPool2 device branch (src/tensor/ops.rs:1117-1133; rule from the host impl

@@ -74,6 +74,8 @@ extern "C" {
     pub fn agh_lenet5_backward_bf16(logits: *const c_void, target: *const c_void, dy: f32, c1: *const c_void, c2: *const c_void, d1: *const c_void, d2: *const c_void, w2: *const c_void, wd1: *const c_void, wd2: *const c_void, wd3: *const c_void, g_logits: *mut c_void, g_d2: *mut c_void, g_d1: *mut c_void, gm2: *mut c_void, gm1: *mut c_void, bs: i64) -> c_int;
     pub fn agh_lenet5_dense_weight_grads_f32(a2: *const c_void, a1: *const c_void, f: *const c_void, g_logits: *const c_void, g_d2: *const c_void, g_d1: *const c_void, dwd3: *mut c_void, dwd2: *mut c_void, dwd1: *mut c_void, db3: *mut c_void, logits: *const c_void, target: *const c_void, loss: *mut c_void, bs: i64) -> c_int;
     pub fn agh_lenet5_dense_weight_grads_bf16(a2: *const c_void, a1: *const c_void, f: *const c_void, g_logits: *const c_void, g_d2: *const c_void, g_d1: *const c_void, dwd3: *mut c_void, dwd2: *mut c_void, dwd1: *mut c_void, db3: *mut c_void, logits: *const c_void, target: *const c_void, loss: *mut c_void, bs: i64) -> c_int;
+    pub fn agh_lenet5_conv_weight_grads_f32(x: *const c_void, p1: *const c_void, gm1: *const c_void, gm2: *const c_void, dw1: *mut c_void, dw2: *mut c_void, bs: i64) -> c_int;
+    pub fn agh_lenet5_conv_weight_grads_bf16(x: *const c_void, p1: *const c_void, gm1: *const c_void, gm2: *const c_void, dw1: *mut c_void, dw2: *mut c_void, bs: i64) -> c_int;
     pub fn agh_max_pool2_f32(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_max_pool2_bf16(x: *const c_void, y: *mut c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
     pub fn agh_max_pool2_backward_f32(dx_inout: *mut c_void, dy: *const c_void, bc: i64, ih: i64, iw: i64, h: i64, w: i64, sh: i64, sw: i64) -> c_int;
