@@ -306,12 +306,23 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    uint4 rp[NRP], rq[NRQ];
+    // Small tiles (a k-tile is a few hundred matrix-pipe cycles, less than a trip to L2) keep TWO k-tiles in
+    // flight: the loads requested during k-tile kt are written to LDS during k-tile kt + 1, out of a second set
+    // of staging registers, so a load has a whole k-tile and a half to arrive instead of half of one.
+    constexpr bool SPREAD = LP != LD_S && LQ != LD_S;
+    constexpr bool DEEP = SPREAD && BP + BQ <= 160;
+    constexpr int NSET = DEEP ? 2 : 1;
+    uint4 rp[NSET][NRP], rq[NSET][NRQ];
     if (KT > 0) {
-        LdP::load(rp, P, g.ps, g.pk, p0, g.NP, kbeg, kend, tid);
-        LdQ::load(rq, Q, g.qs, g.qk, q0, g.NQ, kbeg, kend, tid);
-        LdP::store(rp, smem, kbeg, kend, tid);
-        LdQ::store(rq, smem + BP * 128, kbeg, kend, tid);
+        LdP::load(rp[0], P, g.ps, g.pk, p0, g.NP, kbeg, kend, tid);
+        LdQ::load(rq[0], Q, g.qs, g.qk, q0, g.NQ, kbeg, kend, tid);
+        LdP::store(rp[0], smem, kbeg, kend, tid);
+        LdQ::store(rq[0], smem + BP * 128, kbeg, kend, tid);
+        if constexpr (DEEP) {  // the second k-tile (or the first again, never used), published during the first
+            const int k1 = kbeg + min(1, KT - 1) * BK;
+            LdP::load(rp[1], P, g.ps, g.pk, p0, g.NP, k1, kend, tid);
+            LdQ::load(rq[1], Q, g.qs, g.qk, q0, g.NQ, k1, kend, tid);
+        }
     }
     __syncthreads();
 
@@ -356,17 +367,20 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     // its next MFMA either); past the last tile the same tile is fetched again and never used.  The element
     // loader keeps its guarded loads together in front of the MFMAs.  Then the barrier publishes that
     // stage, and the last substep multiplies out of registers while the first fragments of the next tile are read.
-    constexpr bool SPREAD = LP != LD_S && LQ != LD_S;
     constexpr int NPP = LdP::NPIECE, NPT = LdP::NPIECE + LdQ::NPIECE;
-    for (int kt = 0; kt < KT; ++kt) {
+    // `parc` is kt & 1 when two k-tiles are in flight (it selects the staging register sets), else 0
+    auto ktile = [&](int kt, auto parc) {
+        constexpr int LS = DEEP ? decltype(parc)::value : 0;      // set the loads fill: k-tile kt's, already in LDS
+        constexpr int SS = DEEP ? 1 - decltype(parc)::value : 0;  // set the stores drain: k-tile kt + 1's
         const bool more = kt + 1 < KT;
-        const int k0 = kbeg + (more ? kt + 1 : kt) * BK;
+        const int k0 = kbeg + (more ? kt + 1 : kt) * BK;                   // the k-tile the stores publish
+        const int kl = DEEP ? kbeg + min(kt + 2, KT - 1) * BK : k0;         // the k-tile the loads request
         const unsigned char *cur = smem + (kt & 1) * STAGE_BYTES;
         unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
         if constexpr (!SPREAD) {
             if (more) {
-                LdP::load(rp, P, g.ps, g.pk, p0, g.NP, k0, kend, tid);
-                LdQ::load(rq, Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
+                LdP::load(rp[0], P, g.ps, g.pk, p0, g.NP, k0, kend, tid);
+                LdQ::load(rq[0], Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
             }
         }
         phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 1, [&](auto mc) {
@@ -374,8 +388,8 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
                 constexpr int m = decltype(mc)::value, LA = m * NPT / SLOTS, LB = (m + 1) * NPT / SLOTS;
                 static_for<LB - LA>([&](auto tc) {
                     constexpr int l = LA + decltype(tc)::value;
-                    if constexpr (l < NPP) LdP::template load_piece<l>(rp, P, g.ps, g.pk, p0, g.NP, k0, kend, tid);
-                    else LdQ::template load_piece<l - NPP>(rq, Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
+                    if constexpr (l < NPP) LdP::template load_piece<l>(rp[LS], P, g.ps, g.pk, p0, g.NP, kl, kend, tid);
+                    else LdQ::template load_piece<l - NPP>(rq[LS], Q, g.qs, g.qk, q0, g.NQ, kl, kend, tid);
                 });
             }
         });
@@ -385,20 +399,28 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
                 constexpr int m = decltype(mc)::value, LA = m * NPT / SLOTS, LB = (m + 1) * NPT / SLOTS;
                 static_for<LB - LA>([&](auto tc) {
                     constexpr int l = LA + decltype(tc)::value;
-                    if constexpr (l < NPP) LdP::template store_piece<l>(rp, nxt, k0, kend, tid);
-                    else LdQ::template store_piece<l - NPP>(rq, nxt + BP * 128, k0, kend, tid);
+                    if constexpr (l < NPP) LdP::template store_piece<l>(rp[SS], nxt, k0, kend, tid);
+                    else LdQ::template store_piece<l - NPP>(rq[SS], nxt + BP * 128, k0, kend, tid);
                 });
             }
         });
         if constexpr (!SPREAD) {
             if (more) {
-                LdP::store(rp, nxt, k0, kend, tid);
-                LdQ::store(rq, nxt + BP * 128, k0, kend, tid);
+                LdP::store(rp[0], nxt, k0, kend, tid);
+                LdQ::store(rq[0], nxt + BP * 128, k0, kend, tid);
             }
         }
         __syncthreads();
         // after the last tile `nxt` holds stale data: the fragments read from it are never used
         phase(pfb, qfb, pfa, qfa, nxt + wave_p, nxt + wave_q, 0, [](auto) {});
+    };
+    if constexpr (DEEP) {
+        for (int kt = 0; kt < KT; kt += 2) {
+            ktile(kt, std::integral_constant<int, 0>{});
+            if (kt + 1 < KT) ktile(kt + 1, std::integral_constant<int, 1>{});
+        }
+    } else {
+        for (int kt = 0; kt < KT; ++kt) ktile(kt, std::integral_constant<int, 0>{});
     }
 
     // ------------------------------------------------------------ epilogue ----
