@@ -306,22 +306,27 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    // Small tiles (a k-tile is a few hundred matrix-pipe cycles, less than a trip to L2) keep TWO k-tiles in
-    // flight: the loads requested during k-tile kt are written to LDS during k-tile kt + 1, out of a second set
-    // of staging registers, so a load has a whole k-tile and a half to arrive instead of half of one.
+    // Small tiles (a k-tile is a few hundred matrix-pipe cycles, far less than a trip to memory, and every CU asks
+    // for a k-tile's new lines at about the same time, so somebody's request is always the first) keep NSET
+    // k-tiles in flight: the loads requested during k-tile kt are those of k-tile kt + NSET and are written to LDS
+    // during k-tile kt + NSET - 1, out of one of NSET sets of staging registers (two to four registers each), so a
+    // load has NSET - 1/2 k-tiles to arrive instead of half of one.
     constexpr bool SPREAD = LP != LD_S && LQ != LD_S;
     constexpr bool DEEP = SPREAD && BP + BQ <= 160;
-    constexpr int NSET = DEEP ? 2 : 1;
+    constexpr int NSET = DEEP ? 2 : 1;  // four measured no faster than two (f32 1024^3: 29-33 us either way)
     uint4 rp[NSET][NRP], rq[NSET][NRQ];
     if (KT > 0) {
         LdP::load(rp[0], P, g.ps, g.pk, p0, g.NP, kbeg, kend, tid);
         LdQ::load(rq[0], Q, g.qs, g.qk, q0, g.NQ, kbeg, kend, tid);
         LdP::store(rp[0], smem, kbeg, kend, tid);
         LdQ::store(rq[0], smem + BP * 128, kbeg, kend, tid);
-        if constexpr (DEEP) {  // the second k-tile (or the first again, never used), published during the first
-            const int k1 = kbeg + min(1, KT - 1) * BK;
-            LdP::load(rp[1], P, g.ps, g.pk, p0, g.NP, k1, kend, tid);
-            LdQ::load(rq[1], Q, g.qs, g.qk, q0, g.NQ, k1, kend, tid);
+        if constexpr (DEEP) {  // k-tiles 1 .. NSET - 1 (past the last one: the last again, never used)
+            static_for<NSET - 1>([&](auto sc) {
+                constexpr int s = decltype(sc)::value + 1;
+                const int ks = kbeg + min(s, KT - 1) * BK;
+                LdP::load(rp[s], P, g.ps, g.pk, p0, g.NP, ks, kend, tid);
+                LdQ::load(rq[s], Q, g.qs, g.qk, q0, g.NQ, ks, kend, tid);
+            });
         }
     }
     __syncthreads();
@@ -368,13 +373,13 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     // loader keeps its guarded loads together in front of the MFMAs.  Then the barrier publishes that
     // stage, and the last substep multiplies out of registers while the first fragments of the next tile are read.
     constexpr int NPP = LdP::NPIECE, NPT = LdP::NPIECE + LdQ::NPIECE;
-    // `parc` is kt & 1 when two k-tiles are in flight (it selects the staging register sets), else 0
+    // `parc` is kt % NSET (it selects the staging register sets)
     auto ktile = [&](int kt, auto parc) {
-        constexpr int LS = DEEP ? decltype(parc)::value : 0;      // set the loads fill: k-tile kt's, already in LDS
-        constexpr int SS = DEEP ? 1 - decltype(parc)::value : 0;  // set the stores drain: k-tile kt + 1's
+        constexpr int LS = decltype(parc)::value;               // set the loads fill: k-tile kt's, already in LDS
+        constexpr int SS = (decltype(parc)::value + 1) % NSET;  // set the stores drain: k-tile kt + 1's
         const bool more = kt + 1 < KT;
         const int k0 = kbeg + (more ? kt + 1 : kt) * BK;                   // the k-tile the stores publish
-        const int kl = DEEP ? kbeg + min(kt + 2, KT - 1) * BK : k0;         // the k-tile the loads request
+        const int kl = DEEP ? kbeg + min(kt + NSET, KT - 1) * BK : k0;      // the k-tile the loads request
         const unsigned char *cur = smem + (kt & 1) * STAGE_BYTES;
         unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
         if constexpr (!SPREAD) {
@@ -410,15 +415,17 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
                 LdQ::store(rq[0], nxt + BP * 128, k0, kend, tid);
             }
         }
-        __syncthreads();
+        // the barrier publishes LDS writes only; __syncthreads() would also wait for every global load in flight
+        // (the requests of the k-tiles ahead), once per k-tile
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         // after the last tile `nxt` holds stale data: the fragments read from it are never used
         phase(pfb, qfb, pfa, qfa, nxt + wave_p, nxt + wave_q, 0, [](auto) {});
     };
     if constexpr (DEEP) {
-        for (int kt = 0; kt < KT; kt += 2) {
-            ktile(kt, std::integral_constant<int, 0>{});
-            if (kt + 1 < KT) ktile(kt + 1, std::integral_constant<int, 1>{});
-        }
+        for (int kt = 0; kt < KT; kt += NSET)
+            static_for<NSET>([&](auto ic) {
+                if (kt + decltype(ic)::value < KT) ktile(kt + decltype(ic)::value, ic);
+            });
     } else {
         for (int kt = 0; kt < KT; ++kt) ktile(kt, std::integral_constant<int, 0>{});
     }
