@@ -354,8 +354,11 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
                      const unsigned char *sq, int s, auto &&after) {
         static_for<SLOTS>([&](auto mc) {  // part-major: consecutive MFMAs write different accumulators
             constexpr int m = decltype(mc)::value, e = m / NM, n = m % NM, i = n / TQ, j = n % TQ;
+            // with a single MFMA tile per wave a substep is only PARTS MFMAs long: all of the next substep's
+            // fragments are requested in front of its first MFMA, or the last read has half a substep to arrive
+            if constexpr (NM == 1 && m == 0) static_for<NU>([&](auto uc) { read_unit(yp, yq, sp, sq, s, uc); });
             Mma<T>::template part<e>(acc[i][j], xp[i], xq[j]);
-            if constexpr (m < NU) read_unit(yp, yq, sp, sq, s, mc);
+            if constexpr (NM > 1 && m < NU) read_unit(yp, yq, sp, sq, s, mc);
             after(mc);
             __builtin_amdgcn_sched_barrier(0);
         });
