@@ -166,11 +166,37 @@ struct Loader {
         }
     }
 
+    // The same for a k-tile that lies wholly inside [kbeg, kend): no clamp on k, and the address is written as a
+    // per-lane part that does not change from k-tile to k-tile plus a wave-uniform part in k0, so that a piece costs
+    // one or two vector instructions instead of a 64-bit multiply per load (vector loaders only).
+    template <int i>
+    static __device__ __forceinline__ void load_piece_full(Regs &reg, const T *base, int64_t rs, int64_t ks, int r0, int NR,
+                                                           int k0, int tid) {
+        static_assert(MODE == LD_K || MODE == LD_R, "vector loaders only");
+        if constexpr (MODE == LD_K) {
+            const int id = min(tid + i * NT, TOTAL - 1);
+            const int r = id >> 3, c = id & 7;
+            const int row = min(r0 + r, NR - 1);
+            const T *lane_base = base + (int64_t)row * rs + c * EPC;
+            reg[i] = *(const uint4 *)(lane_base + k0);
+        } else {
+            const int id = min(tid + i * NT, NBLK_TOTAL - 1);
+            const int kb = id & 7, rb = id >> 3;
+            int row = r0 + rb * EPC;
+            if (row >= NR) row = NR - EPC;  // NR is a multiple of EPC on this path
+            const T *lane_base = base + row + (int64_t)(kb * EPC) * ks;
+            const T *p = lane_base + (int64_t)k0 * ks;
+#pragma unroll
+            for (int e = 0; e < EPC; ++e) reg[i * EPC + e] = *(const uint4 *)(p + (int64_t)e * ks);
+        }
+    }
+
     // registers -> LDS stage (tile base address `lds`, bytes); k0 / kend as given to load
     static __device__ __forceinline__ void store(const Regs &reg, unsigned char *lds, int k0, int kend, int tid) {
         static_for<NPIECE>([&](auto ic) { store_piece<decltype(ic)::value>(reg, lds, k0, kend, tid); });
     }
-    template <int i>
+    // FULL: the k-tile lies wholly below kend, nothing to zero
+    template <int i, bool FULL = false>
     static __device__ __forceinline__ void store_piece(const Regs &reg, unsigned char *lds, int k0, int kend, int tid) {
         if constexpr (MODE == LD_R) {
             int id = tid + i * NT;
@@ -179,7 +205,7 @@ struct Loader {
             uint4 in[EPC];  // in[e] = EPC rows at k = kb*EPC + e
 #pragma unroll
             for (int e = 0; e < EPC; ++e) {
-                const bool ok = k0 + kb * EPC + e < kend;
+                const bool ok = FULL || k0 + kb * EPC + e < kend;
                 const uint4 &src = reg[i * EPC + e];
                 in[e] = make_uint4(ok ? src.x : 0u, ok ? src.y : 0u, ok ? src.z : 0u, ok ? src.w : 0u);
             }
@@ -218,7 +244,7 @@ struct Loader {
         } else {
             int id = tid + i * NT;
             int r = id >> 3, c = id & 7;
-            const bool ok = MODE != LD_K || k0 + c * EPC < kend;
+            const bool ok = FULL || MODE != LD_K || k0 + c * EPC < kend;
             const uint4 v = make_uint4(ok ? reg[i].x : 0u, ok ? reg[i].y : 0u, ok ? reg[i].z : 0u, ok ? reg[i].w : 0u);
             if (TOTAL % NT == 0 || id < TOTAL) *(uint4 *)(lds + lds_off(r, c)) = v;
         }
@@ -391,27 +417,55 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
                 LdQ::load(rq[0], Q, g.qs, g.qk, q0, g.NQ, k0, kend, tid);
             }
         }
-        phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 1, [&](auto mc) {
+        // small tiles: whole k-tiles (all but possibly the last) take the loaders' short forms; next to sixteen
+        // MFMAs the clamps, the zeroing selects and a 64-bit multiply per load of the general forms are most of the
+        // instructions of a k-tile
+        const bool req_full = DEEP && kl + BK <= kend, pub_full = DEEP && k0 + BK <= kend;
+        auto request = [&](auto mc) {
             if constexpr (SPREAD) {
                 constexpr int m = decltype(mc)::value, LA = m * NPT / SLOTS, LB = (m + 1) * NPT / SLOTS;
                 static_for<LB - LA>([&](auto tc) {
                     constexpr int l = LA + decltype(tc)::value;
+                    if constexpr (DEEP) {
+                        if (req_full) {
+                            if constexpr (l < NPP) LdP::template load_piece_full<l>(rp[LS], P, g.ps, g.pk, p0, g.NP, kl, tid);
+                            else LdQ::template load_piece_full<l - NPP>(rq[LS], Q, g.qs, g.qk, q0, g.NQ, kl, tid);
+                            return;
+                        }
+                    }
                     if constexpr (l < NPP) LdP::template load_piece<l>(rp[LS], P, g.ps, g.pk, p0, g.NP, kl, kend, tid);
                     else LdQ::template load_piece<l - NPP>(rq[LS], Q, g.qs, g.qk, q0, g.NQ, kl, kend, tid);
                 });
             }
-        });
-        phase(pfb, qfb, pfa, qfa, cur + wave_p, cur + wave_q, 2, [](auto) {});
-        phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 3, [&](auto mc) {
+        };
+        auto publish = [&](auto mc) {
             if constexpr (SPREAD) {
                 constexpr int m = decltype(mc)::value, LA = m * NPT / SLOTS, LB = (m + 1) * NPT / SLOTS;
                 static_for<LB - LA>([&](auto tc) {
                     constexpr int l = LA + decltype(tc)::value;
+                    if constexpr (DEEP) {
+                        if (pub_full) {
+                            if constexpr (l < NPP) LdP::template store_piece<l, true>(rp[SS], nxt, k0, kend, tid);
+                            else LdQ::template store_piece<l - NPP, true>(rq[SS], nxt + BP * 128, k0, kend, tid);
+                            return;
+                        }
+                    }
                     if constexpr (l < NPP) LdP::template store_piece<l>(rp[SS], nxt, k0, kend, tid);
                     else LdQ::template store_piece<l - NPP>(rq[SS], nxt + BP * 128, k0, kend, tid);
                 });
             }
-        });
+        };
+        if constexpr (DEEP) {
+            // the pieces to publish arrived a k-tile ago and the other stage is free since the last barrier: they
+            // go to LDS first, so that the barrier below never waits for an LDS write; the new requests follow
+            phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 1, publish);
+            phase(pfb, qfb, pfa, qfa, cur + wave_p, cur + wave_q, 2, request);
+            phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 3, [](auto) {});
+        } else {
+            phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 1, request);
+            phase(pfb, qfb, pfa, qfa, cur + wave_p, cur + wave_q, 2, [](auto) {});
+            phase(pfa, qfa, pfb, qfb, cur + wave_p, cur + wave_q, 3, publish);
+        }
         if constexpr (!SPREAD) {
             if (more) {
                 LdP::store(rp[0], nxt, k0, kend, tid);
