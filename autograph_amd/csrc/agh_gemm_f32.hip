@@ -1,4 +1,6 @@
 // f32 GEMM entry points (v_mfma_f32_32x32x2_f32: full f32 multiplies and accumulation).
+#define AGH_GEMM_WITH_F32_DIRECT
+#include "agh_gemm_f32_dl.h"
 #include "agh_gemm_host.h"
 
 extern "C" {

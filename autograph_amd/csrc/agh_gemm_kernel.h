@@ -295,6 +295,101 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_p, int tiles_q, i
     tq = in_group / gsz;
 }
 
+// ------------------------------------------------------------ epilogue ----
+// Stores a wave's TP x TQ tiles of 32 x 32 accumulators (element r of lane l of tile (i, j) is
+// D[p0 + 32 (wp TP + i) + 8 (r / 4) + 4 (l / 32) + r % 4][q0 + 32 (wq TQ + j) + l % 32]).  One loop nest per store
+// mode, each small enough to unroll fully: the accumulators must only ever be indexed by compile-time constants
+// or they would be demoted to scratch.
+template <typename T, int TP, int TQ>
+__device__ __forceinline__ void store_tile(const Args &g, const f32x16 (&acc)[TP][TQ], int p0, int q0, int wp, int wq,
+                                           int lane, int split) {
+    const uint32_t lrow = lane & 31, lg = lane >> 5;
+    const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
+    T *D = (T *)g.D + (int64_t)blockIdx.z * g.batch_d;
+    const T *bias = (const T *)g.bias;
+    const int mode = g.store_mode;
+    const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;
+    if (mode == ST_SPLITK) {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            float *wrow = g.ws + ((size_t)split * g.NQ + q) * g.NPpad;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<4>([&](auto bc) {
+                    constexpr int blk = decltype(bc)::value;
+                    const int p = pw0 + i * 32 + blk * 8;
+                    if (q < g.NQ && p < g.NPpad)
+                        *(float4 *)(wrow + p) = make_float4(acc[i][j][blk * 4 + 0], acc[i][j][blk * 4 + 1],
+                                                            acc[i][j][blk * 4 + 2], acc[i][j][blk * 4 + 3]);
+                });
+            });
+        });
+    } else if (mode == ST_VEC) {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            const bool qok = q < g.NQ;
+            T bq = 0;
+            if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
+            T *drow = D + (int64_t)q * g.dq;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<4>([&](auto bc) {
+                    constexpr int blk = decltype(bc)::value;
+                    const int p = pw0 + i * 32 + blk * 8;
+                    if (qok && p < g.NP) {  // NP is a multiple of 4 on this path
+                        T *dst = drow + p;
+                        __align__(16) T old[4] = {0, 0, 0, 0};
+                        if (g.beta != 0.0f) {
+                            if constexpr (sizeof(T) == 4) *(uint4 *)old = *(const uint4 *)dst;
+                            else *(uint2 *)old = *(const uint2 *)dst;
+                        }
+                        T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
+                        if (has_bias && bias_p) {
+                            b0 = bias[(int64_t)(p + 0) * g.bias_stride];
+                            b1 = bias[(int64_t)(p + 1) * g.bias_stride];
+                            b2 = bias[(int64_t)(p + 2) * g.bias_stride];
+                            b3 = bias[(int64_t)(p + 3) * g.bias_stride];
+                        }
+                        __align__(16) T out[4];
+                        out[0] = finish<T>(acc[i][j][blk * 4 + 0], g.alpha, g.beta, old[0], has_bias, b0, g.act);
+                        out[1] = finish<T>(acc[i][j][blk * 4 + 1], g.alpha, g.beta, old[1], has_bias, b1, g.act);
+                        out[2] = finish<T>(acc[i][j][blk * 4 + 2], g.alpha, g.beta, old[2], has_bias, b2, g.act);
+                        out[3] = finish<T>(acc[i][j][blk * 4 + 3], g.alpha, g.beta, old[3], has_bias, b3, g.act);
+                        if constexpr (sizeof(T) == 4) *(uint4 *)dst = *(const uint4 *)out;
+                        else *(uint2 *)dst = *(const uint2 *)out;
+                    }
+                });
+            });
+        });
+    } else {
+        static_for<TQ>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int q = qw0 + j * 32;
+            const bool qok = q < g.NQ;
+            T bq = 0;
+            if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
+            T *drow = D + (int64_t)q * g.dq;
+            static_for<TP>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    const int p = pw0 + i * 32 + (r >> 2) * 8 + (r & 3);
+                    if (qok && p < g.NP) {
+                        T *dst = drow + (int64_t)p * g.dp;
+                        T old = 0;
+                        if (g.beta != 0.0f) old = *dst;
+                        T bv = bq;
+                        if (has_bias && bias_p) bv = bias[(int64_t)p * g.bias_stride];
+                        *dst = finish<T>(acc[i][j][r], g.alpha, g.beta, old, has_bias, bv, g.act);
+                    }
+                });
+            });
+        });
+    }
+}
+
 template <typename T, int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
 __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
     constexpr int NT = WGP * WGQ * 64;
@@ -487,93 +582,7 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_kernel(Args g) {
         for (int kt = 0; kt < KT; ++kt) ktile(kt, std::integral_constant<int, 0>{});
     }
 
-    // ------------------------------------------------------------ epilogue ----
-    // One loop nest per store mode, each small enough to unroll fully: the accumulators must
-    // only ever be indexed by compile-time constants or they would be demoted to scratch.
-    const int pw0 = p0 + wp * TP * 32 + (int)lg * 4, qw0 = q0 + wq * TQ * 32 + (int)lrow;
-    T *D = (T *)g.D + (int64_t)blockIdx.z * g.batch_d;
-    const T *bias = (const T *)g.bias;
-    const int mode = g.store_mode;
-    const bool has_bias = g.has_bias != 0, bias_p = g.bias_on_p != 0;
-    if (mode == ST_SPLITK) {
-        static_for<TQ>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const int q = qw0 + j * 32;
-            float *wrow = g.ws + ((size_t)split * g.NQ + q) * g.NPpad;
-            static_for<TP>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<4>([&](auto bc) {
-                    constexpr int blk = decltype(bc)::value;
-                    const int p = pw0 + i * 32 + blk * 8;
-                    if (q < g.NQ && p < g.NPpad)
-                        *(float4 *)(wrow + p) = make_float4(acc[i][j][blk * 4 + 0], acc[i][j][blk * 4 + 1],
-                                                            acc[i][j][blk * 4 + 2], acc[i][j][blk * 4 + 3]);
-                });
-            });
-        });
-    } else if (mode == ST_VEC) {
-        static_for<TQ>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const int q = qw0 + j * 32;
-            const bool qok = q < g.NQ;
-            T bq = 0;
-            if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
-            T *drow = D + (int64_t)q * g.dq;
-            static_for<TP>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<4>([&](auto bc) {
-                    constexpr int blk = decltype(bc)::value;
-                    const int p = pw0 + i * 32 + blk * 8;
-                    if (qok && p < g.NP) {  // NP is a multiple of 4 on this path
-                        T *dst = drow + p;
-                        __align__(16) T old[4] = {0, 0, 0, 0};
-                        if (g.beta != 0.0f) {
-                            if constexpr (sizeof(T) == 4) *(uint4 *)old = *(const uint4 *)dst;
-                            else *(uint2 *)old = *(const uint2 *)dst;
-                        }
-                        T b0 = bq, b1 = bq, b2 = bq, b3 = bq;
-                        if (has_bias && bias_p) {
-                            b0 = bias[(int64_t)(p + 0) * g.bias_stride];
-                            b1 = bias[(int64_t)(p + 1) * g.bias_stride];
-                            b2 = bias[(int64_t)(p + 2) * g.bias_stride];
-                            b3 = bias[(int64_t)(p + 3) * g.bias_stride];
-                        }
-                        __align__(16) T out[4];
-                        out[0] = finish<T>(acc[i][j][blk * 4 + 0], g.alpha, g.beta, old[0], has_bias, b0, g.act);
-                        out[1] = finish<T>(acc[i][j][blk * 4 + 1], g.alpha, g.beta, old[1], has_bias, b1, g.act);
-                        out[2] = finish<T>(acc[i][j][blk * 4 + 2], g.alpha, g.beta, old[2], has_bias, b2, g.act);
-                        out[3] = finish<T>(acc[i][j][blk * 4 + 3], g.alpha, g.beta, old[3], has_bias, b3, g.act);
-                        if constexpr (sizeof(T) == 4) *(uint4 *)dst = *(const uint4 *)out;
-                        else *(uint2 *)dst = *(const uint2 *)out;
-                    }
-                });
-            });
-        });
-    } else {
-        static_for<TQ>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const int q = qw0 + j * 32;
-            const bool qok = q < g.NQ;
-            T bq = 0;
-            if (qok && has_bias && !bias_p) bq = bias[(int64_t)q * g.bias_stride];
-            T *drow = D + (int64_t)q * g.dq;
-            static_for<TP>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<16>([&](auto rc) {
-                    constexpr int r = decltype(rc)::value;
-                    const int p = pw0 + i * 32 + (r >> 2) * 8 + (r & 3);
-                    if (qok && p < g.NP) {
-                        T *dst = drow + (int64_t)p * g.dp;
-                        T old = 0;
-                        if (g.beta != 0.0f) old = *dst;
-                        T bv = bq;
-                        if (has_bias && bias_p) bv = bias[(int64_t)p * g.bias_stride];
-                        *dst = finish<T>(acc[i][j][r], g.alpha, g.beta, old, has_bias, bv, g.act);
-                    }
-                });
-            });
-        });
-    }
+    store_tile<T, TP, TQ>(g, acc, p0, q0, wp, wq, lane, split);
 }
 
 // Second pass of split-K: sum the partials in split order (deterministic), then the same
