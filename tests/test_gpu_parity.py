@@ -323,6 +323,55 @@ def test_gemm_f32_1024_cubed_all_layouts(ag):
     assert np.array_equal(ta.dot(eye).into_array(), a)
 
 
+def test_gemm_f32_direct_small_tiles(ag, monkeypatch):
+    """The f32 kernel that loads 64 x 64 tiles straight into LDS (both operands vector-loadable, k a multiple of
+    32): one to five k-tiles (its ring holds four), tile rows and columns cut off by the matrix edge, all four operand
+    layouts, a batch, split-K partials, alpha / beta / bias / ReLU, integer data exactly, and the register-staged
+    kernel on the same inputs."""
+    rng = np.random.default_rng(31)
+    for (m, k, n) in [(64, 32, 64), (64, 64, 64), (100, 96, 76), (132, 128, 200), (60, 160, 68), (256, 1024, 192)]:
+        a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        at, bt = np.ascontiguousarray(a.T), np.ascontiguousarray(b.T)
+        ta, tb, tat, tbt = (ag.Tensor.from_array(x) for x in (a, b, at, bt))
+        outs = [ta.dot(tb).into_array(), tat.t().dot(tb).into_array(), ta.dot(tbt.t()).into_array(),
+                tat.t().dot(tbt.t()).into_array()]
+        for out in outs:
+            assert_f32_gemm_close(out, a, b)
+        monkeypatch.setenv("AGH_GEMM_DIRECT", "0")
+        staged = ta.dot(tb).into_array()
+        monkeypatch.delenv("AGH_GEMM_DIRECT")
+        assert np.abs(outs[0] - staged).max() <= 1e-5 * np.sqrt(k) * np.abs(staged).max()
+        # small integers: every product and partial sum is exact in f32, whatever the order
+        ai = rng.integers(-8, 9, (m, k)).astype(np.float32)
+        bi = rng.integers(-8, 9, (k, n)).astype(np.float32)
+        assert np.array_equal(ag.Tensor.from_array(ai).dot(ag.Tensor.from_array(bi)).into_array(), ai @ bi)
+    # alpha, beta, bias and ReLU through the shared epilogue
+    m, k, n = 96, 64, 80
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    c = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    tc = ag.Tensor.from_array(c)
+    ag.gemm(0.5, ag.Tensor.from_array(a), ag.Tensor.from_array(b), -2.0, tc)
+    want = 0.5 * (a.astype(np.float64) @ b.astype(np.float64)) - 2.0 * c
+    assert np.abs(tc.into_array() - want).max() <= 1e-5 * np.sqrt(k) * np.abs(want).max()
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    got = ag.Dense(ag.Tensor.from_array(b), ag.Tensor.from_array(bias)).forward(ag.Tensor.from_array(a), relu=True).into_array()
+    want = np.maximum(a.astype(np.float64) @ b.astype(np.float64) + bias, 0.0)
+    assert np.abs(got - want).max() <= 1e-5 * np.sqrt(k) * max(np.abs(want).max(), 1.0)
+    # split-K partials (forced) and the result's independence of the run
+    monkeypatch.setenv("AGH_GEMM_CFG", "4")
+    monkeypatch.setenv("AGH_GEMM_SPLITS", "3")
+    a = rng.uniform(-1, 1, (70, 320)).astype(np.float32)
+    b = rng.uniform(-1, 1, (320, 90)).astype(np.float32)
+    out = ag.Tensor.from_array(a).dot(ag.Tensor.from_array(b)).into_array()
+    again = ag.Tensor.from_array(a).dot(ag.Tensor.from_array(b)).into_array()
+    monkeypatch.delenv("AGH_GEMM_CFG")
+    monkeypatch.delenv("AGH_GEMM_SPLITS")
+    assert np.array_equal(out, again)
+    assert_f32_gemm_close(out, a, b)
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 def test_dense_full_size_bias_relu(ag, dtype):
     """The Dense-shaped GEMM of the benchmark list at full size: M = 16384 (batch), K = 4096, N = 4096 with the
