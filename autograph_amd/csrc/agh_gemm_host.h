@@ -58,13 +58,14 @@ inline int env_int(const char *name, int dflt);
 
 #ifdef AGH_GEMM_WITH_F32_DIRECT
 // direct-to-LDS f32 kernel for 64 x 64 tiles (agh_gemm_f32_dl.h)
-template <int LP, int LQ>
+template <int TP, int TQ, int NS, int LP, int LQ>
 int launch_f32_dl(const Args &g, int splits) {
-    auto kern = gemm_f32_dl_kernel<LP, LQ>;
-    constexpr size_t smem = 4 * 2 * 8 * 1152;  // four stages of two operands of eight 1152-byte load images
+    auto kern = gemm_f32_dl_kernel<TP, TQ, NS, LP, LQ>;
+    constexpr size_t smem = F32DlGeo<TP, TQ, NS, LP, LQ>::SMEM_BYTES;
     static bool attr_done = false;
     if (!attr_done) {
-        AGH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        if (smem > 48 * 1024)
+            AGH_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_done = true;
     }
     dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits, (unsigned)g.batch);
@@ -77,15 +78,17 @@ int launch_f32_dl(const Args &g, int splits) {
 template <typename T, int BP, int BQ, int WGP, int WGQ, bool SCALAR_OK>
 int launch_loaders(const Args &g, int splits, int lp, int lq, bool direct) {
 #ifdef AGH_GEMM_WITH_F32_DIRECT
-    if constexpr (std::is_same<T, float>::value && BP == 64 && BQ == 64) {
+    if constexpr (std::is_same<T, float>::value && ((BP == 64 && BQ == 64) || (BP == 128 && BQ == 128))) {
         // both operands vector-loadable and k (hence every split's range) a multiple of the 32-wide k-tile
-        // (AGH_GEMM_DIRECT=0 forces the register-staged kernel)
+        // (AGH_GEMM_DIRECT=0 forces the register-staged kernel).  64 x 64: a ring of four stages, one or two
+        // workgroups per CU; 128 x 128: two stages (a k-tile is four times as long), two workgroups per CU.
+        constexpr int TPW = BP / 64, TQW = BQ / 64, NS = BP == 64 ? 4 : 2;
         if (lp != LD_S && lq != LD_S && g.K > 0 && g.K % 32 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0) {
             switch (lp * 3 + lq) {
-                case LD_K * 3 + LD_K: return launch_f32_dl<LD_K, LD_K>(g, splits);
-                case LD_K * 3 + LD_R: return launch_f32_dl<LD_K, LD_R>(g, splits);
-                case LD_R * 3 + LD_K: return launch_f32_dl<LD_R, LD_K>(g, splits);
-                case LD_R * 3 + LD_R: return launch_f32_dl<LD_R, LD_R>(g, splits);
+                case LD_K * 3 + LD_K: return launch_f32_dl<TPW, TQW, NS, LD_K, LD_K>(g, splits);
+                case LD_K * 3 + LD_R: return launch_f32_dl<TPW, TQW, NS, LD_K, LD_R>(g, splits);
+                case LD_R * 3 + LD_K: return launch_f32_dl<TPW, TQW, NS, LD_R, LD_K>(g, splits);
+                case LD_R * 3 + LD_R: return launch_f32_dl<TPW, TQW, NS, LD_R, LD_R>(g, splits);
                 default: break;
             }
         }
@@ -234,11 +237,13 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         // where the direct-to-LDS bf16 kernel applies (the four large tiles), the register-staged small tiles
         // are a poor second: measured 2x slower at 1024^3 although they put four times as many CUs to work
         double eff = (direct_ok && !kCfgs[i].scalar_ok) || !direct_ok ? t.eff : t.eff * 0.4;
-        // f32: the 64 x 64 tile has a direct-to-LDS kernel of its own (agh_gemm_f32_dl.h), measured at 0.8 of the
-        // 256 x 256 tile's rate per CU (3072^3: 118 TFLOP/s, where 144 tiles of 256 x 256 leave 112 CUs idle)
-        const bool f32_direct = sizeof(T) == 4 && t.bp == 64 && t.bq == 64 && !any_scalar && g.K > 0 && g.K % 32 == 0 &&
-                                env_int("AGH_GEMM_DIRECT", 1) != 0;
+        // the 64 x 64 direct tile is measured at 0.8 of the 256 x 256 tile's rate per CU (3072^3: 118 TFLOP/s, where
+        // 144 tiles of 256 x 256 leave 112 CUs idle)
+        // f32: the 64 x 64 and 128 x 128 tiles have direct-to-LDS kernels (agh_gemm_f32_dl.h)
+        const bool f32_dl_ok = sizeof(T) == 4 && !any_scalar && g.K > 0 && g.K % 32 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0;
+        const bool f32_direct = f32_dl_ok && t.bp == 64 && t.bq == 64;
         if (f32_direct) eff = 0.80;
+        if (f32_dl_ok && t.bp == 128 && t.bq == 128) eff = 0.95;  // 4096^3: 135 TFLOP/s, the 256 x 256 tile's rate
         // a tile's prologue and epilogue cost about four k-tiles of time when the CU holds one workgroup, next
         // to nothing when a second workgroup multiplies meanwhile: decides short-k shapes (conv GEMM, k = 576).
         // The f32 direct kernel's k-tile is short (sixteen MFMAs a wave): filling its four-stage ring and storing
