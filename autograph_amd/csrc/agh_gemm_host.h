@@ -78,10 +78,11 @@ int launch_f32_dl(const Args &g, int splits) {
 template <typename T, int BP, int BQ, int WGP, int WGQ, bool SCALAR_OK>
 int launch_loaders(const Args &g, int splits, int lp, int lq, bool direct) {
 #ifdef AGH_GEMM_WITH_F32_DIRECT
-    if constexpr (std::is_same<T, float>::value && ((BP == 64 && BQ == 64) || (BP == 128 && BQ == 128))) {
+    if constexpr (std::is_same<T, float>::value && BP % 64 == 0 && BQ % 64 == 0) {
         // both operands vector-loadable and k (hence every split's range) a multiple of the 32-wide k-tile
         // (AGH_GEMM_DIRECT=0 forces the register-staged kernel).  64 x 64: a ring of four stages, one or two
-        // workgroups per CU; 128 x 128: two stages (a k-tile is four times as long), two workgroups per CU.
+        // workgroups per CU; 128 x 128: two stages (a k-tile is four times as long), two workgroups per CU; the
+        // larger tiles: two stages, one workgroup per CU.
         constexpr int TPW = BP / 64, TQW = BQ / 64, NS = BP == 64 ? 4 : 2;
         if (lp != LD_S && lq != LD_S && g.K > 0 && g.K % 32 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0) {
             switch (lp * 3 + lq) {
