@@ -55,12 +55,40 @@ def conv2_direct_forward(x, weight, padding=(0, 0), stride=(1, 1), dilation=(1, 
     return y
 
 
+def _device_param(pair, dtype):
+    """(array, is_bf16) of autograph_amd.serde -> device tensor, checked against an expected element type"""
+    if pair is None:
+        return None
+    array, is_bf16 = pair
+    got = "bf16" if is_bf16 else "f32"
+    if not is_bf16 and array.dtype != np.float32:
+        raise AghError(-1, "serde: parameters are f32 or bf16 here")
+    if dtype is not None and dtype != got:
+        raise AghError(-1, f"Expected {dtype} found {got}")
+    return Tensor.from_array(array)
+
+
 class Conv2:
     """`Conv2` (layer.rs:844-1047): weight [outputs, inputs, fh, fw], optional bias [outputs]."""
 
     def __init__(self, weight, bias=None, padding=(0, 0), stride=(1, 1), dilation=(1, 1)):
         self.weight, self.bias = weight, bias
         self.padding, self.stride, self.dilation = tuple(padding), tuple(stride), tuple(dilation)
+
+    # the data model of the reference's derive (layer.rs:833-848), as serde_json writes it; see autograph_amd/serde.py
+    def to_json(self):
+        import json
+        from . import serde
+        bf16 = self.weight.dtype == "bf16"
+        return json.dumps(serde.conv2_to_value(self.weight.into_array(), None if self.bias is None else self.bias.into_array(),
+                                               self.padding, self.stride, self.dilation, bf16=bf16), separators=(",", ":"))
+
+    @classmethod
+    def from_json(cls, text, dtype=None):
+        import json
+        from . import serde
+        f = serde.conv2_from_value(json.loads(text))
+        return cls(_device_param(f["weight"], dtype), _device_param(f["bias"], dtype), f["padding"], f["stride"], f["dilation"])
 
     def forward(self, x, relu=False, pool2x2=False, algorithm="auto"):
         """`conv2` (layer.rs:930-948).  Like the reference's host, which takes a direct kernel when
@@ -87,6 +115,19 @@ class Dense:
     def forward(self, x, relu=False):
         return x.dot(self.weight, bias=self.bias, relu=relu)
 
+    def to_json(self):
+        import json
+        from . import serde
+        return json.dumps(serde.dense_to_value(self.weight.into_array(), None if self.bias is None else self.bias.into_array(),
+                                               bf16=self.weight.dtype == "bf16"), separators=(",", ":"))
+
+    @classmethod
+    def from_json(cls, text, dtype=None):
+        import json
+        from . import serde
+        f = serde.dense_from_value(json.loads(text))
+        return cls(_device_param(f["weight"], dtype), _device_param(f["bias"], dtype))
+
 
 class MaxPool2:
     """`MaxPool2` (layer.rs:1149-1216); stride defaults to the filter (layer.rs:535-539)."""
@@ -97,6 +138,17 @@ class MaxPool2:
 
     def forward(self, x):
         return x.max_pool2(MaxPool2Options(self.filter, self.stride))
+
+    def to_json(self):
+        import json
+        from . import serde
+        return json.dumps(serde.max_pool2_to_value(self.filter, self.stride), separators=(",", ":"))
+
+    @classmethod
+    def from_json(cls, text):
+        import json
+        from . import serde
+        return cls(**serde.max_pool2_from_value(json.loads(text)))
 
 
 class Relu:

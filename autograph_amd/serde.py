@@ -74,10 +74,14 @@ def to_tokens(array, bf16=False):
     return toks
 
 
+def to_value(array, bf16=False):
+    """The tensor as the JSON value serde_json writes: a struct is an object, tuples and tuple structs are arrays."""
+    return {"dim": [int(d) for d in array.shape], "buffer": [scalar_name(array, bf16), int(array.size), _items(array)]}
+
+
 def to_json(array, bf16=False):
-    """What serde_json writes for the same value: a struct is an object, tuples and tuple structs are arrays."""
-    return json.dumps({"dim": [int(d) for d in array.shape],
-                       "buffer": [scalar_name(array, bf16), int(array.size), _items(array)]}, separators=(",", ":"))
+    """What serde_json writes for the same value."""
+    return json.dumps(to_value(array, bf16), separators=(",", ":"))
 
 
 def from_json(text):
@@ -88,6 +92,11 @@ def from_json(text):
         obj = json.loads(text)
     except json.JSONDecodeError as e:
         raise SerdeError(f"not JSON: {e}") from None
+    return from_value(obj)
+
+
+def from_value(obj):
+    """`from_json` for an already parsed JSON value."""
     if not isinstance(obj, dict) or set(obj) != {"dim", "buffer"}:
         raise SerdeError("expected an object with exactly the fields `dim` and `buffer`")
     dim, buf = obj["dim"], obj["buffer"]
@@ -101,3 +110,76 @@ def from_json(text):
     if int(np.prod(dim, dtype=np.int64)) != count:
         raise SerdeError(f"IncompatibleShape: dim {dim} does not hold {count} elements")
     return flat.reshape(dim), name == "BF16"
+
+
+# ---- layers (src/learn/neural_network/layer.rs) ----
+# The reference derives Serialize / Deserialize for its layer structs, so their data model is the field list:
+#   Conv<D>    { weight: Parameter, padding: D, stride: D, dilation: D, bias: Option<Parameter1> }   (layer.rs:833-848)
+#   Dense      { weight: Parameter2, bias: Option<Parameter1> }                                      (layer.rs:1069-1073)
+#   MaxPool<D> { filter: D, stride: D }                                                              (layer.rs:1150-1155)
+#   Relu, Flatten, Identity: unit structs (serde_json: null)                                        (layer.rs:1222-1252)
+#   Parameter  { value: Tensor, optim_state }, `grad` skipped and `optim_state` skipped when it is none, absent ->
+#              none (autograd.rs:639-656); ndarray's fixed-rank dimensions are tuples of integers.
+# No vector of these is held by the reference's tests (its serde tests cover tensors only), so beyond the field
+# names and order of the derive this encoding is unpinned; it is what serde_json makes of that data model.
+# Values here are host arrays: (array, is_bf16) pairs as `from_value` returns them.
+
+
+def _dims(obj, what, rank):
+    if not isinstance(obj, list) or len(obj) != rank or any(not isinstance(d, int) or isinstance(d, bool) or d < 0 for d in obj):
+        raise SerdeError(f"`{what}` must be an array of {rank} unsigned integers")
+    return tuple(obj)
+
+
+def parameter_to_value(array, bf16=False):
+    """A parameter without optimizer state (the state of a freshly built or inference-only layer)."""
+    return {"value": to_value(array, bf16)}
+
+
+def parameter_from_value(obj, rank):
+    if not isinstance(obj, dict) or "value" not in obj or set(obj) - {"value", "optim_state"}:
+        raise SerdeError("expected a parameter object with the field `value`")
+    if obj.get("optim_state") is not None:
+        raise SerdeError("optimizer state in a parameter is not supported here")
+    array, is_bf16 = from_value(obj["value"])
+    if array.ndim != rank:
+        raise SerdeError(f"IncompatibleShape: a parameter of rank {rank} holds a tensor of rank {array.ndim}")
+    return array, is_bf16
+
+
+def conv2_to_value(weight, bias=None, padding=(0, 0), stride=(1, 1), dilation=(1, 1), bf16=False):
+    return {"weight": parameter_to_value(weight, bf16), "padding": [int(v) for v in padding],
+            "stride": [int(v) for v in stride], "dilation": [int(v) for v in dilation],
+            "bias": None if bias is None else parameter_to_value(bias, bf16)}
+
+
+def conv2_from_value(obj):
+    """-> dict(weight=(array, is_bf16), bias=None | (array, is_bf16), padding, stride, dilation)"""
+    fields = {"weight", "padding", "stride", "dilation", "bias"}
+    if not isinstance(obj, dict) or set(obj) != fields:
+        raise SerdeError("expected an object with exactly the fields " + ", ".join(sorted(fields)))
+    return dict(weight=parameter_from_value(obj["weight"], 4),
+                bias=None if obj["bias"] is None else parameter_from_value(obj["bias"], 1),
+                padding=_dims(obj["padding"], "padding", 2), stride=_dims(obj["stride"], "stride", 2),
+                dilation=_dims(obj["dilation"], "dilation", 2))
+
+
+def dense_to_value(weight, bias=None, bf16=False):
+    return {"weight": parameter_to_value(weight, bf16), "bias": None if bias is None else parameter_to_value(bias, bf16)}
+
+
+def dense_from_value(obj):
+    if not isinstance(obj, dict) or set(obj) != {"weight", "bias"}:
+        raise SerdeError("expected an object with exactly the fields `weight` and `bias`")
+    return dict(weight=parameter_from_value(obj["weight"], 2),
+                bias=None if obj["bias"] is None else parameter_from_value(obj["bias"], 1))
+
+
+def max_pool2_to_value(filter, stride):
+    return {"filter": [int(v) for v in filter], "stride": [int(v) for v in stride]}
+
+
+def max_pool2_from_value(obj):
+    if not isinstance(obj, dict) or set(obj) != {"filter", "stride"}:
+        raise SerdeError("expected an object with exactly the fields `filter` and `stride`")
+    return dict(filter=_dims(obj["filter"], "filter", 2), stride=_dims(obj["stride"], "stride", 2))

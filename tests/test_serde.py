@@ -1,5 +1,7 @@
 """The tensor wire format of the reference (src/tensor.rs:1199-1249), pinned by its own token test
-(src/tensor.rs:2236-2277).  CPU only: the encoding is host logic."""
+(src/tensor.rs:2236-2277), and the layer structs' data model around it (layer.rs:833-848, 1069-1073, 1150-1155:
+field lists of the derive; no vector of them exists in the reference).  CPU only but for the device round trips: the
+encoding is host logic."""
 import json
 
 import numpy as np
@@ -78,3 +80,56 @@ def test_device_tensor_round_trip():
         ag.Tensor.from_json(ag.Tensor.from_array(w).to_json(), dtype="bf16")
     with pytest.raises(ag.AghError):
         ag.Tensor.from_json(serde.to_json(np.arange(4, dtype=np.uint32)))
+
+
+def test_layer_values_follow_the_derived_field_lists():
+    rng = np.random.default_rng(5)
+    w = rng.standard_normal((4, 3, 5, 5)).astype(np.float32)
+    b = rng.standard_normal(4).astype(np.float32)
+    v = serde.conv2_to_value(w, b, padding=(2, 1), stride=(1, 2), dilation=(1, 1))
+    assert list(v) == ["weight", "padding", "stride", "dilation", "bias"]          # layer.rs:842-848
+    assert list(v["weight"]) == ["value"] and v["weight"]["value"] == json.loads(serde.to_json(w))
+    assert v["padding"] == [2, 1] and v["stride"] == [1, 2] and v["dilation"] == [1, 1]
+    back = serde.conv2_from_value(json.loads(json.dumps(v)))
+    assert np.array_equal(back["weight"][0], w) and np.array_equal(back["bias"][0], b) and not back["weight"][1]
+    assert (back["padding"], back["stride"], back["dilation"]) == ((2, 1), (1, 2), (1, 1))
+    assert serde.conv2_from_value(serde.conv2_to_value(w))["bias"] is None            # Option::None is null
+    d = serde.dense_to_value(w.reshape(4, 75), None)
+    assert list(d) == ["weight", "bias"] and d["bias"] is None                        # layer.rs:1070-1073
+    assert np.array_equal(serde.dense_from_value(d)["weight"][0], w.reshape(4, 75))
+    assert serde.max_pool2_to_value((2, 2), (2, 2)) == {"filter": [2, 2], "stride": [2, 2]}  # layer.rs:1152-1155
+    assert serde.max_pool2_from_value({"filter": [3, 2], "stride": [1, 1]}) == dict(filter=(3, 2), stride=(1, 1))
+    # an absent optimizer state is the default (none); anything else, unknown or missing fields, wrong ranks are errors
+    assert np.array_equal(serde.parameter_from_value({"value": json.loads(serde.to_json(b)), "optim_state": None}, 1)[0], b)
+    for bad in ({"weight": v["weight"], "bias": None, "extra": 1}, {"weight": v["weight"]},
+                {"weight": {"value": json.loads(serde.to_json(b))}, "bias": None}):
+        with pytest.raises(serde.SerdeError):
+            serde.dense_from_value(bad)
+    with pytest.raises(serde.SerdeError):
+        serde.conv2_from_value({**v, "padding": [1]})
+    with pytest.raises(serde.SerdeError):
+        serde.max_pool2_from_value({"filter": [2, 2]})
+
+
+@pytest.mark.gpu
+def test_device_layer_round_trip():
+    import autograph_amd as ag
+    import oracle as orc
+    ag.Device(0)
+    rng = np.random.default_rng(6)
+    w = rng.standard_normal((6, 1, 5, 5)).astype(np.float32)
+    b = rng.standard_normal(6).astype(np.float32)
+    x = rng.standard_normal((2, 1, 12, 12)).astype(np.float32)
+    for dt, conv in (("f32", lambda a: a), ("bf16", orc.f32_to_bf16)):
+        layer = ag.Conv2(ag.Tensor.from_array(conv(w)), ag.Tensor.from_array(conv(b)), padding=(1, 1))
+        back = ag.Conv2.from_json(layer.to_json(), dtype=dt)
+        assert back.padding == (1, 1) and back.stride == (1, 1) and back.weight.dtype == dt
+        tx = ag.Tensor.from_array(conv(x))
+        assert np.array_equal(back.forward(tx).into_array(), layer.forward(tx).into_array())
+        dense = ag.Dense(ag.Tensor.from_array(conv(w.reshape(6, 25).T.copy())))
+        back = ag.Dense.from_json(dense.to_json())
+        assert back.bias is None and np.array_equal(back.weight.into_array(), dense.weight.into_array())
+        with pytest.raises(ag.AghError):
+            ag.Conv2.from_json(layer.to_json(), dtype="f32" if dt == "bf16" else "bf16")
+    pool = ag.MaxPool2.from_json(ag.MaxPool2((2, 2)).to_json())
+    assert pool.filter == (2, 2) and pool.stride == (2, 2)
