@@ -372,6 +372,45 @@ def test_gemm_f32_direct_small_tiles(ag, monkeypatch):
     assert_f32_gemm_close(out, a, b)
 
 
+def test_gemm_f32_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
+    """150 seeded f32 products with k a multiple of 32 (so that the direct-to-LDS kernels apply wherever the operands
+    are vector-loadable), odd and even m and n, all four layouts, alpha and beta, each in the chooser's tile
+    configuration and forced into the 256 x 256, 128 x 128 and 64 x 64 ones (a forced configuration that has no
+    kernel for the operands' loaders is refused, not miscomputed)."""
+    rng = np.random.default_rng(123)
+    ran = {None: 0, "0": 0, "3": 0, "4": 0}
+    for _ in range(150):
+        m, n, k = int(rng.integers(1, 400)), int(rng.integers(1, 400)), 32 * int(rng.integers(1, 12))
+        if rng.random() < 0.5:
+            m = 4 * max(1, m // 4)
+        if rng.random() < 0.5:
+            n = 4 * max(1, n // 4)
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        a = rng.uniform(-1, 1, (k, m) if ta else (m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (n, k) if tb else (k, n)).astype(np.float32)
+        c0 = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+        alpha, beta = float(rng.choice([1.0, 0.5])), float(rng.choice([0.0, 0.0, 1.0, -0.5]))
+        A, B = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+        av, bv = (a.T if ta else a), (b.T if tb else b)
+        want = alpha * (av.astype(np.float64) @ bv.astype(np.float64)) + beta * c0
+        tol = 1e-5 * np.sqrt(k) * max(np.abs(want).max(), 1e-3) + 1e-6
+        for cfg in ran:
+            if cfg is None:
+                monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
+            else:
+                monkeypatch.setenv("AGH_GEMM_CFG", cfg)
+            C = ag.Tensor.from_array(c0)
+            try:
+                ag.gemm(alpha, A.t() if ta else A, B.t() if tb else B, beta, C)
+            except ag.AghError as e:
+                assert cfg is not None and e.code == -4
+                continue
+            ran[cfg] += 1
+            assert np.abs(C.into_array() - want).max() <= tol, (m, k, n, ta, tb, alpha, beta, cfg)
+    monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
+    assert ran[None] == 150 and min(ran.values()) >= 30, ran
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 def test_dense_full_size_bias_relu(ag, dtype):
     """The Dense-shaped GEMM of the benchmark list at full size: M = 16384 (batch), K = 4096, N = 4096 with the
