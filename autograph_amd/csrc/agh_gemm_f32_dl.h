@@ -21,6 +21,11 @@
 // behind the barrier after which nobody reads that stage any more.  Either way a load has more than NS - 2 k-tiles
 // to land (with two stages: most of one, which for 128-row tiles is 4000 matrix-pipe cycles).
 //
+// KS = 2 splits every k-tile between two waves per 32 x 32-tile position (eight waves, two per SIMD: while one waits
+// for its fragments or at the barrier the other multiplies): a wave takes two of a k-tile's four substeps, and the
+// two partial accumulators are added through LDS in front of the epilogue, always in the same order.  For grids that
+// give a CU a single workgroup.
+//
 // Requirements checked by the host: K and every split's k range multiples of 32, operand base pointers 16-byte
 // aligned, unit stride along k (LD_K) or along rows (LD_R) with the other stride a multiple of 4 elements, rows a
 // multiple of 4 for LD_R.
@@ -51,16 +56,19 @@ struct F32DlGeo {
     static constexpr int SMEM_BYTES = NS * STAGE_BYTES;
 };
 
-template <int TP, int TQ, int NS, int LP, int LQ>
-__global__ __launch_bounds__(256) void gemm_f32_dl_kernel(Args g) {
+template <int TP, int TQ, int NS, int LP, int LQ, int KS = 1>
+__global__ __launch_bounds__(256 * KS) void gemm_f32_dl_kernel(Args g) {
     typedef float T;
     static_assert((LP == LD_K || LP == LD_R) && (LQ == LD_K || LQ == LD_R), "vector layouts only");
+    static_assert(KS == 1 || KS == 2, "a k-tile goes to one wave or is split between two");
+    constexpr int SPW = 4 / KS;  // substeps of a k-tile per wave
     typedef F32DlGeo<TP, TQ, NS, LP, LQ> Geo_;
     typedef typename Geo_::OpP OpP;
     typedef typename Geo_::OpQ OpQ;
     constexpr int BP = Geo_::BP, BQ = Geo_::BQ, BK = 32;
     constexpr int STAGE_BYTES = Geo_::STAGE_BYTES;
-    constexpr int LPWP = OpP::LOADS / 4, LPWQ = OpQ::LOADS / 4, LPW = LPWP + LPWQ;  // direct loads per wave and k-tile
+    constexpr int LPWP = OpP::LOADS / (4 * KS), LPWQ = OpQ::LOADS / (4 * KS), LPW = LPWP + LPWQ;  // direct loads per wave and k-tile
+    static_assert(LPWP >= 1 && LPWQ >= 1, "every wave issues loads of both operands");
     static_assert(NS >= 2 && (NS - 1) * LPW <= 63, "the loads in flight must fit the counter");
     constexpr bool EARLY = NS >= 3;                  // requests in the first substep (see above)
     constexpr int AHEAD = EARLY ? NS - 1 : NS;       // k-tile kt requests k-tile kt + AHEAD; the prologue the AHEAD first
@@ -70,7 +78,8 @@ __global__ __launch_bounds__(256) void gemm_f32_dl_kernel(Args g) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wp = wave & 1, wq = wave >> 1;
+    const int wp = wave & 1, wq = (wave >> 1) & 1;
+    const int kh = wave >> 2;  // which half of every k-tile's substeps (KS == 2)
     int tp, tq;
     tile_coords(blockIdx.x, g.tiles_p, g.tiles_q, tp, tq);
     const int p0 = tp * BP, q0 = tq * BQ;
@@ -132,8 +141,9 @@ __global__ __launch_bounds__(256) void gemm_f32_dl_kernel(Args g) {
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             const uint32_t r = (uint32_t)wave_row + 32u * i + lrow;
-            if constexpr (MODE == LD_K) off[i] = r * 128u + ((lg ^ swz(r)) << 4);  // substep s toggles bit 5
-            else off[i] = lg * (uint32_t)Op::koff(4) + r * 4u;                      // substep s adds koff(8 s)
+            // the wave's first substep is SPW * kh; its later ones toggle bits 5.. (LD_K) or add koff(8 s) (LD_R)
+            if constexpr (MODE == LD_K) off[i] = (r * 128u + ((lg ^ swz(r)) << 4)) ^ (uint32_t)((SPW * kh) << 5);
+            else off[i] = lg * (uint32_t)Op::koff(4) + r * 4u + (uint32_t)(kh * Op::koff(8 * (SPW % 4)));
         }
     };
     frag_offsets(std::common_type<OpP>{}, std::integral_constant<int, LP>{}, std::integral_constant<int, TP>{}, wp * 32 * TP, fp);
@@ -200,8 +210,10 @@ __global__ __launch_bounds__(256) void gemm_f32_dl_kernel(Args g) {
         };
         if constexpr (EARLY) substep(pfa, qfa, pfb, qfb, cur, std::integral_constant<int, 1>{}, requests);
         else substep(pfa, qfa, pfb, qfb, cur, std::integral_constant<int, 1>{}, nothing);
-        substep(pfb, qfb, pfa, qfa, cur, std::integral_constant<int, 2>{}, nothing);
-        substep(pfa, qfa, pfb, qfb, cur, std::integral_constant<int, 3>{}, nothing);
+        if constexpr (SPW == 4) {
+            substep(pfb, qfb, pfa, qfa, cur, std::integral_constant<int, 2>{}, nothing);
+            substep(pfa, qfa, pfb, qfb, cur, std::integral_constant<int, 3>{}, nothing);
+        }
         // k-tile kt + 1 becomes visible: this wave's loads of it have landed (those of the NS - 2 k-tiles after it may
         // still be in flight), every fragment of `cur` has been read, and the barrier says the same of the other waves.
         // Then the first fragments of k-tile kt + 1 between the last MFMAs of this one (and, with two stages, the loads
@@ -213,6 +225,30 @@ __global__ __launch_bounds__(256) void gemm_f32_dl_kernel(Args g) {
         else substep(pfb, qfb, pfa, qfa, nxt, std::integral_constant<int, 0>{}, requests);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the requests past the last k-tile
+    if constexpr (KS == 2) {
+        // the second half's partial sums go to the first half through LDS: [tile][i][j][r][lane], 4 bytes each
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();  // nobody reads a stage any more
+        asm volatile("" ::: "memory");
+        float *xch = (float *)smem + ((wave & 3) * TP * TQ * 16) * 64 + lane;
+        static_assert(4 * TP * TQ * 16 * 64 * 4 <= Geo_::SMEM_BYTES, "the partial sums must fit in the stages");
+        if (kh == 1) {
+#pragma unroll
+            for (int i = 0; i < TP; ++i)
+#pragma unroll
+                for (int j = 0; j < TQ; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) xch[((i * TQ + j) * 16 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (kh == 1) return;
+#pragma unroll
+        for (int i = 0; i < TP; ++i)
+#pragma unroll
+            for (int j = 0; j < TQ; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] += xch[((i * TQ + j) * 16 + r) * 64];
+    }
 
     store_tile<T, TP, TQ>(g, acc, p0, q0, wp, wq, lane, split);
 }

@@ -58,9 +58,16 @@ inline int env_int(const char *name, int dflt);
 
 #ifdef AGH_GEMM_WITH_F32_DIRECT
 // direct-to-LDS f32 kernel for 64 x 64 tiles (agh_gemm_f32_dl.h)
-template <int TP, int TQ, int NS, int LP, int LQ>
+template <int TP, int TQ, int NS, int LP, int LQ, int KS = 1>
 int launch_f32_dl(const Args &g, int splits) {
-    auto kern = gemm_f32_dl_kernel<TP, TQ, NS, LP, LQ>;
+    if constexpr (KS == 1 && TP * TQ <= 4) {
+        // a grid that gives a CU one workgroup at most: eight waves, every k-tile split between two (AGH_GEMM_KSPLIT=0|1
+        // forbids / forces it)
+        const int64_t wgs = (int64_t)g.tiles_p * g.tiles_q * splits * g.batch;
+        const int ks = env_int("AGH_GEMM_KSPLIT", wgs <= (compute_units() > 0 ? compute_units() : 256) ? 1 : 0);
+        if (ks) return launch_f32_dl<TP, TQ, NS, LP, LQ, 2>(g, splits);
+    }
+    auto kern = gemm_f32_dl_kernel<TP, TQ, NS, LP, LQ, KS>;
     constexpr size_t smem = F32DlGeo<TP, TQ, NS, LP, LQ>::SMEM_BYTES;
     static bool attr_done = false;
     if (!attr_done) {
@@ -69,7 +76,7 @@ int launch_f32_dl(const Args &g, int splits) {
         attr_done = true;
     }
     dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits, (unsigned)g.batch);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream(), g);
+    hipLaunchKernelGGL(kern, grid, dim3(256 * KS), smem, stream(), g);
     AGH_LAUNCH_CHECK("gemm kernel launch");
     return AGH_OK;
 }
