@@ -243,8 +243,9 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         // a CU works through ceil(tiles / CUs) tiles; co-resident workgroups share its MFMA rate
         const int64_t rounds = (tiles + cus - 1) / cus;
         // where the direct-to-LDS bf16 kernel applies (the four large tiles), the register-staged small tiles
-        // are a poor second: measured 2x slower at 1024^3 although they put four times as many CUs to work
-        double eff = (direct_ok && !kCfgs[i].scalar_ok) || !direct_ok ? t.eff : t.eff * 0.4;
+        // are a poor second: measured 2x slower at 1024^3 (16.4 us against 8.9 us) although they put four times as
+        // many CUs to work
+        double eff = (direct_ok && !kCfgs[i].scalar_ok) || !direct_ok ? t.eff : t.eff * 0.25;
         // the 64 x 64 direct tile is measured at 0.8 of the 256 x 256 tile's rate per CU (3072^3: 118 TFLOP/s, where
         // 144 tiles of 256 x 256 leave 112 CUs idle)
         // f32: the 64 x 64 and 128 x 128 tiles have direct-to-LDS kernels (agh_gemm_f32_dl.h)
@@ -258,7 +259,23 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         // the tile cost about six of them (at k = 576 the 128 x 128 tile is 9 % faster, from k = 1536 on slower).
         const double kt = (double)((g.K + BK - 1) / BK);
         eff *= kt / (kt + (f32_direct ? 6.0 : t.wgs_per_cu == 1 ? 4.0 : 0.5));
-        const double cost = (double)rounds * t.bp * t.bq / eff;
+        double cost = (double)rounds * t.bp * t.bq / eff;
+        // bf16 direct-to-LDS tiles: a full chip of them runs at the power limit, where the rate depends on the tile
+        // shape (bigger tiles move fewer operand bytes per flop) and not on how many CUs take part, while a
+        // launch that leaves CUs idle runs the busy ones at a higher clock.  Measured per k-tile of a 256 x 256
+        // tile: 1.32 us with 256 workgroups (8192^3, 4096^3), 0.97 us with 144 (3072^3).  The cost is the larger
+        // of the two limits: rounds of co-resident workgroups at the unthrottled rate, all tiles at the power limit.
+        if (direct_ok && !t.scalar_ok) {
+            // kAlone: a 128 x 128 workgroup with a CU to itself (2048^3: 22.8 us) against two sharing it
+            static const double kUnthrottled[4] = {1.36, 0.89, 0.89, 0.946}, kAtPowerLimit[4] = {1.0, 0.83, 0.83, 0.85},
+                                kAlone[4] = {1.36, 0.89, 0.89, 0.59};
+            const int64_t slots = (int64_t)cus * t.wgs_per_cu, rest = tiles % slots;
+            const double area = (double)t.bp * t.bq;
+            const double by_rounds = (double)(tiles / slots) * t.wgs_per_cu * area / kUnthrottled[i] +
+                                     (rest == 0 ? 0.0 : rest <= cus ? area / kAlone[i] : t.wgs_per_cu * area / kUnthrottled[i]);
+            const double by_power = (double)tiles * t.bp * t.bq / (cus * kAtPowerLimit[i]);
+            cost = std::max(by_rounds, by_power) * (kt + (t.wgs_per_cu == 1 ? 4.0 : 2.0)) / kt;
+        }
         if (best < 0 || cost < best_cost) { best = i; best_cost = cost; }
     }
     best = env_int("AGH_GEMM_CFG", best);
