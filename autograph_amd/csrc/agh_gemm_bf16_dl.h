@@ -127,7 +127,10 @@ struct FragRead {
 
 // STAGED: the kernel is only launched with store_mode == ST_STAGED (the common case); the other
 // epilogues are compiled out, which keeps their register demand from spilling accumulators.
-template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ, bool STAGED>
+// NS: LDS stages.  Two serve wherever the CU's matrix pipes are kept busy by a second workgroup or by a k-tile long
+// enough to cover a load's latency; a 128 x 128 workgroup alone on its CU (a grid of at most one per CU) multiplies a
+// k-tile in 512 cycles, a quarter of that latency, and runs a ring of four.
+template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ, bool STAGED, int NS = 2>
 __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     typedef uint16_t T;
     constexpr int NW = WGP * WGQ;
@@ -140,8 +143,9 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     typedef FragRead<LP, BP, TP> FrP;
     typedef FragRead<LQ, BQ, TQ> FrQ;
 
-    __shared__ __align__(1024) unsigned char stage0[STAGE_BYTES];
-    __shared__ __align__(1024) unsigned char stage1[STAGE_BYTES];
+    static_assert(NS >= 2, "tile kt is multiplied while tile kt + 1 lands");
+    __shared__ __align__(1024) unsigned char stages[NS][STAGE_BYTES];
+    unsigned char *const stage0 = stages[0], *const stage1 = stages[1];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -206,10 +210,10 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     };
 
     // One k-tile = 2 substeps (32 k each) of NM MFMAs.  On entry: tile kt is visible in `cur`, its substep-0 fragments
-    // are in set A and the loads of tile kt+1 into `nxt` are in flight.  Every RSTEP-th of the first MFMAs of substep 0
+    // are in set A and the loads of tiles kt+1 .. kt+NS-1 are in flight, those of tile kt+1 into `nxt`.  Every RSTEP-th of the first MFMAs of substep 0
     // is followed by one fragment read of substep 1 (set B; reading them back to back would ask the LDS for 1 KB per
     // wave every 16 cycles, its whole bandwidth), after which this wave needs nothing more from `cur`: the barrier at
-    // MFMA NB frees `cur` and publishes `nxt`.  From there on the loads of tile kt+2 go out into `cur`, one every LSTEP
+    // MFMA NB frees `cur` and publishes `nxt`.  From there on the loads of tile kt+NS go out into `cur`, one every LSTEP
     // MFMAs, and the first MFMAs of substep 1 are followed by the reads of tile kt+1's substep 0 from `nxt` (set A).
     // sched_barrier(0) after every MFMA pins this interleaving.
     constexpr int NM = TP * TQ;
@@ -218,13 +222,13 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     constexpr int LSTEP = NM / NLT > 0 ? NM / NLT : 1;                // one direct load every LSTEP MFMAs
     static_assert(NU * RSTEP <= NM, "fragment reads must fit behind the MFMAs of one substep");
     static_assert(NB + LSTEP * NLT <= 2 * NM, "the loads of a tile must go out within the tile");
-    auto step = [&](unsigned char *cur, unsigned char *nxt, bool adv) {
+    auto step = [&](unsigned char *cur, unsigned char *nxt, bool adv) __attribute__((always_inline)) {
         const uint32_t cur_addr = __builtin_amdgcn_readfirstlane(lds_address(cur));
         const int64_t ap = adv ? stepP : 0, aq = adv ? stepQ : 0;
         static_for<2 * NM>([&](auto nc) {
             constexpr int n = decltype(nc)::value, ph = n / NM, m = n % NM, i = m / TQ, j = m % TQ;
             if constexpr (n == NB) {
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NS - 2) * NLT) : "memory");  // tile kt+1 has landed
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_sched_barrier(0);
@@ -243,21 +247,27 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     };
 
     if (KT > 0) {
+        // tile min(t, KT-1) -> stage t
         const uint32_t a0 = __builtin_amdgcn_readfirstlane(lds_address(stage0));
-        const uint32_t a1 = __builtin_amdgcn_readfirstlane(lds_address(stage1));
-        // tile 0 -> stage0, tile min(1, KT-1) -> stage1
-        static_for<NLT>([&](auto lc) { issue_load(a0, lc, KT > 1 ? stepP : 0, KT > 1 ? stepQ : 0); });
-        static_for<NLT>([&](auto lc) { issue_load(a1, lc, KT > 2 ? stepP : 0, KT > 2 ? stepQ : 0); });
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLT) : "memory");  // tile 0 has landed
+        static_for<NS * NLT>([&](auto nc) {
+            constexpr int t = decltype(nc)::value / NLT, l = decltype(nc)::value % NLT;
+            issue_load(a0 + t * STAGE_BYTES, std::integral_constant<int, l>{}, KT > t + 1 ? stepP : 0, KT > t + 1 ? stepQ : 0);
+        });
+        static_assert((NS - 1) * NLT < 64, "the wait counter holds six bits");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 1) * NLT) : "memory");  // tile 0 has landed
         __syncthreads();
         static_for<NU>([&](auto uc) { read_unit(pfa, qfa, stage0, std::integral_constant<int, 0>{}, uc); });
     }
     int kt = 0;
-    for (; kt + 2 <= KT; kt += 2) {  // step kt requests tile kt+2 and moves on if a tile kt+3 exists
-        step(stage0, stage1, kt + 3 < KT);
-        step(stage1, stage0, kt + 4 < KT);
-    }
-    if (kt < KT) step(stage0, stage1, false);
+    for (; kt + NS <= KT; kt += NS)  // step kt requests tile kt+NS and moves on if a tile kt+NS+1 exists
+        static_for<NS>([&](auto sc) {
+            constexpr int s = decltype(sc)::value;
+            step(stages[s], stages[(s + 1) % NS], kt + s + NS + 1 < KT);
+        });
+    static_for<NS - 1>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
+        if (kt + s < KT) step(stages[s], stages[(s + 1) % NS], false);
+    });
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 

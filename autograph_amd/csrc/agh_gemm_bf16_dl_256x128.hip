@@ -3,6 +3,6 @@
 
 namespace agh {
 namespace gemm {
-AGH_DL_INSTANTIATE(256, 128, 2, 2)
+AGH_DL_INSTANTIATE(256, 128, 2, 2, 2)
 }  // namespace gemm
 }  // namespace agh

@@ -6,23 +6,23 @@
 namespace agh {
 namespace gemm {
 
-template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
+template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ, int NS>
 int launch_one_dl(const Args &g, int splits) {
     dim3 grid((unsigned)(g.tiles_p * g.tiles_q), (unsigned)splits, (unsigned)g.batch);
-    // both LDS stages are static
+    // the LDS stages are static
     if (g.store_mode == ST_STAGED)
-        hipLaunchKernelGGL((gemm_bf16_dl_kernel<BP, BQ, WGP, WGQ, LP, LQ, true>), grid, dim3(WGP * WGQ * 64), 0, stream(), g);
+        hipLaunchKernelGGL((gemm_bf16_dl_kernel<BP, BQ, WGP, WGQ, LP, LQ, true, NS>), grid, dim3(WGP * WGQ * 64), 0, stream(), g);
     else
-        hipLaunchKernelGGL((gemm_bf16_dl_kernel<BP, BQ, WGP, WGQ, LP, LQ, false>), grid, dim3(WGP * WGQ * 64), 0, stream(), g);
+        hipLaunchKernelGGL((gemm_bf16_dl_kernel<BP, BQ, WGP, WGQ, LP, LQ, false, NS>), grid, dim3(WGP * WGQ * 64), 0, stream(), g);
     AGH_LAUNCH_CHECK("gemm (direct-to-LDS) kernel launch");
     return AGH_OK;
 }
 
-#define AGH_DL_INSTANTIATE(BP, BQ, WGP, WGQ)                                          \
-    template int launch_one_dl<BP, BQ, WGP, WGQ, LD_K, LD_K>(const Args &, int);      \
-    template int launch_one_dl<BP, BQ, WGP, WGQ, LD_K, LD_R>(const Args &, int);      \
-    template int launch_one_dl<BP, BQ, WGP, WGQ, LD_R, LD_K>(const Args &, int);      \
-    template int launch_one_dl<BP, BQ, WGP, WGQ, LD_R, LD_R>(const Args &, int);
+#define AGH_DL_INSTANTIATE(BP, BQ, WGP, WGQ, NS)                                          \
+    template int launch_one_dl<BP, BQ, WGP, WGQ, LD_K, LD_K, NS>(const Args &, int);      \
+    template int launch_one_dl<BP, BQ, WGP, WGQ, LD_K, LD_R, NS>(const Args &, int);      \
+    template int launch_one_dl<BP, BQ, WGP, WGQ, LD_R, LD_K, NS>(const Args &, int);      \
+    template int launch_one_dl<BP, BQ, WGP, WGQ, LD_R, LD_R, NS>(const Args &, int);
 
 }  // namespace gemm
 }  // namespace agh

@@ -50,11 +50,28 @@ int launch_one(const Args &g, int splits) {
 #ifdef AGH_GEMM_WITH_BF16_DIRECT
 // direct-to-LDS bf16 kernels: defined and explicitly instantiated in agh_gemm_bf16_dl_<tile>.hip
 // (one translation unit per tile shape, so they compile in parallel)
-template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
+template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ, int NS>
 int launch_one_dl(const Args &g, int splits);
 #endif
 
 inline int env_int(const char *name, int dflt);
+
+#ifdef AGH_GEMM_WITH_BF16_DIRECT
+// Two LDS stages, but a ring of four for a grid of 128 x 128 tiles that gives a CU one workgroup at most and has 20
+// k-tiles or more: alone on its CU such a workgroup waits for loads most of the time (2048^3: 22.8 us with two stages,
+// 17.9 us with four; at 16 k-tiles the four tiles requested up front cost 0.3 us more than they save).
+// AGH_GEMM_RING=2|4 forces either.
+template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
+int launch_dl_ring(const Args &g, int splits) {
+    if constexpr (BP == 128 && BQ == 128) {
+        const int64_t wgs = (int64_t)g.tiles_p * g.tiles_q * splits * g.batch;
+        const bool alone = wgs <= (compute_units() > 0 ? compute_units() : 256) && g.k_per_split >= 20 * 64;
+        if (env_int("AGH_GEMM_RING", alone ? 4 : 2) == 4)
+            return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, 4>(g, splits);
+    }
+    return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, 2>(g, splits);
+}
+#endif
 
 #ifdef AGH_GEMM_WITH_F32_DIRECT
 // direct-to-LDS f32 kernel for 64 x 64 tiles (agh_gemm_f32_dl.h)
@@ -106,10 +123,10 @@ int launch_loaders(const Args &g, int splits, int lp, int lq, bool direct) {
     if constexpr (std::is_same<T, uint16_t>::value && !SCALAR_OK) {
         if (direct) {
             switch (lp * 3 + lq) {
-                case LD_K * 3 + LD_K: return launch_one_dl<BP, BQ, WGP, WGQ, LD_K, LD_K>(g, splits);
-                case LD_K * 3 + LD_R: return launch_one_dl<BP, BQ, WGP, WGQ, LD_K, LD_R>(g, splits);
-                case LD_R * 3 + LD_K: return launch_one_dl<BP, BQ, WGP, WGQ, LD_R, LD_K>(g, splits);
-                case LD_R * 3 + LD_R: return launch_one_dl<BP, BQ, WGP, WGQ, LD_R, LD_R>(g, splits);
+                case LD_K * 3 + LD_K: return launch_dl_ring<BP, BQ, WGP, WGQ, LD_K, LD_K>(g, splits);
+                case LD_K * 3 + LD_R: return launch_dl_ring<BP, BQ, WGP, WGQ, LD_K, LD_R>(g, splits);
+                case LD_R * 3 + LD_K: return launch_dl_ring<BP, BQ, WGP, WGQ, LD_R, LD_K>(g, splits);
+                case LD_R * 3 + LD_R: return launch_dl_ring<BP, BQ, WGP, WGQ, LD_R, LD_R>(g, splits);
                 default: break;
             }
         }
@@ -266,9 +283,10 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         // tile: 1.32 us with 256 workgroups (8192^3, 4096^3), 0.97 us with 144 (3072^3).  The cost is the larger
         // of the two limits: rounds of co-resident workgroups at the unthrottled rate, all tiles at the power limit.
         if (direct_ok && !t.scalar_ok) {
-            // kAlone: a 128 x 128 workgroup with a CU to itself (2048^3: 22.8 us) against two sharing it
-            static const double kUnthrottled[4] = {1.36, 0.89, 0.89, 0.946}, kAtPowerLimit[4] = {1.0, 0.83, 0.83, 0.85},
-                                kAlone[4] = {1.36, 0.89, 0.89, 0.59};
+            // kAlone: a 128 x 128 workgroup with a CU to itself (2048^3: 22.8 us on two LDS stages, 17.9 us on the ring of
+            // four a launch of at most one workgroup per CU and 20 k-tiles or more takes) against two sharing it
+            static const double kUnthrottled[4] = {1.36, 0.89, 0.89, 0.946}, kAtPowerLimit[4] = {1.0, 0.83, 0.83, 0.85};
+            const double kAlone[4] = {1.36, 0.89, 0.89, tiles <= cus && kt >= 20 ? 0.75 : 0.59};
             const int64_t slots = (int64_t)cus * t.wgs_per_cu, rest = tiles % slots;
             const double area = (double)t.bp * t.bq;
             const double by_rounds = (double)(tiles / slots) * t.wgs_per_cu * area / kUnthrottled[i] +

@@ -372,6 +372,48 @@ def test_gemm_f32_direct_small_tiles(ag, monkeypatch):
     assert_f32_gemm_close(out, a, b)
 
 
+def test_gemm_bf16_ring_of_four_stages(ag, monkeypatch):
+    """The 128 x 128 bf16 direct-to-LDS kernel on four LDS stages, the form a launch of at most one workgroup per CU
+    and 20 k-tiles or more takes: k-tile counts 20 to 23 (every length of the ring's tail) by the launch rule, counts
+    1 to 5 forced (fewer tiles than stages: the requests beyond the last tile repeat it), tile rows and columns cut
+    off by the matrix edge, all four operand layouts, bias and ReLU.  Against the oracle, and bit for bit against the
+    same kernel on two stages (the order of every sum is the same)."""
+    rng = np.random.default_rng(77)
+    monkeypatch.setenv("AGH_GEMM_CFG", "3")
+    cases = [(200, 1280, 264, None), (128, 1344, 128, None), (256, 1408, 136, None), (136, 1472, 384, None),
+             (128, 64, 128, "4"), (136, 128, 200, "4"), (128, 192, 128, "4"), (264, 256, 128, "4"), (128, 320, 136, "4")]
+    for (m, k, n, force) in cases:
+        for ta in (False, True):
+            for tb in (False, True):
+                a = to_dtype(rng.uniform(-1, 1, (k, m) if ta else (m, k)), "bf16")
+                b = to_dtype(rng.uniform(-1, 1, (n, k) if tb else (k, n)), "bf16")
+                ta_, tb_ = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+                av, bv = (a.T if ta else a), (b.T if tb else b)
+                tav, tbv = (ta_.t() if ta else ta_), (tb_.t() if tb else tb_)
+                if force:
+                    monkeypatch.setenv("AGH_GEMM_RING", force)
+                out = tav.dot(tbv).into_array()
+                monkeypatch.setenv("AGH_GEMM_RING", "2")
+                two = tav.dot(tbv).into_array()
+                monkeypatch.delenv("AGH_GEMM_RING")
+                assert_bf16_gemm_close(out, orc.gemm_bf16_f32acc(av, bv), av, bv)
+                assert np.array_equal(out, two), (m, k, n, ta, tb)
+    m, k, n = 192, 1536, 256
+    a = to_dtype(rng.uniform(-1, 1, (m, k)), "bf16")
+    w = to_dtype(rng.uniform(-1, 1, (k, n)), "bf16")
+    bias = to_dtype(rng.uniform(-1, 1, n), "bf16")
+    layer = ag.Dense(ag.Tensor.from_array(w), ag.Tensor.from_array(bias))
+    got = layer.forward(ag.Tensor.from_array(a), relu=True).into_array()
+    monkeypatch.setenv("AGH_GEMM_RING", "2")
+    two = layer.forward(ag.Tensor.from_array(a), relu=True).into_array()
+    monkeypatch.delenv("AGH_GEMM_RING")
+    assert np.array_equal(got, two)
+    dot = orc.bf16_to_f32(orc.gemm_bf16_f32acc(a, w))
+    want = np.maximum(orc.bf16_to_f32(orc.f32_to_bf16(dot + orc.bf16_to_f32(bias))), 0.0)
+    gotf = orc.bf16_to_f32(got).astype(np.float64)
+    assert np.all(np.abs(gotf - want) <= 2 * bf16_ulp(want) + 1e-2 * np.abs(want) + 0.05)
+
+
 def test_gemm_f32_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
     """150 seeded f32 products with k a multiple of 32 (so that the direct-to-LDS kernels apply wherever the operands
     are vector-loadable), odd and even m and n, all four layouts, alpha and beta, each in the chooser's tile
