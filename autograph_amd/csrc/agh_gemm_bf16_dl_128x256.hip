@@ -1,8 +1,8 @@
-// Direct-to-LDS bf16 GEMM kernels, 128x256 tile, 2x2 waves: all four loader pairs.
+// Direct-to-LDS bf16 GEMM kernels, 128x256 tile, 2x2 waves, three LDS stages: all four loader pairs.
 #include "agh_gemm_bf16_dl_launch.h"
 
 namespace agh {
 namespace gemm {
-AGH_DL_INSTANTIATE(128, 256, 2, 2, 2)
+AGH_DL_INSTANTIATE(128, 256, 2, 2, 3)
 }  // namespace gemm
 }  // namespace agh

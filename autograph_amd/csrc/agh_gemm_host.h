@@ -69,7 +69,9 @@ int launch_dl_ring(const Args &g, int splits) {
         if (env_int("AGH_GEMM_RING", alone ? 4 : 2) == 4)
             return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, 4>(g, splits);
     }
-    return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, 2>(g, splits);
+    // 128 x 256 and 256 x 128: three stages of 48 KB (a CU holds one such workgroup either way; 3 to 10 % faster than
+    // two at every size measured, 2048^3 to 8192^3)
+    return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, BP * BQ == 128 * 256 ? 3 : 2>(g, splits);
 }
 #endif
 
@@ -280,19 +282,26 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         // bf16 direct-to-LDS tiles: a full chip of them runs at the power limit, where the rate depends on the tile
         // shape (bigger tiles move fewer operand bytes per flop) and not on how many CUs take part, while a
         // launch that leaves CUs idle runs the busy ones at a higher clock.  Measured per k-tile of a 256 x 256
-        // tile: 1.32 us with 256 workgroups (8192^3, 4096^3), 0.97 us with 144 (3072^3).  The cost is the larger
-        // of the two limits: rounds of co-resident workgroups at the unthrottled rate, all tiles at the power limit.
+        // tile: 1.32 us with 256 workgroups (8192^3, 4096^3), 0.97 us with 144 (3072^3).  The cost is summed over
+        // rounds of co-resident workgroups, each round at the lower of the two rates.
         if (direct_ok && !t.scalar_ok) {
-            // kAlone: a 128 x 128 workgroup with a CU to itself (2048^3: 22.8 us on two LDS stages, 17.9 us on the ring of
-            // four a launch of at most one workgroup per CU and 20 k-tiles or more takes) against two sharing it
-            static const double kUnthrottled[4] = {1.36, 0.89, 0.89, 0.946}, kAtPowerLimit[4] = {1.0, 0.83, 0.83, 0.85};
-            const double kAlone[4] = {1.36, 0.89, 0.89, tiles <= cus && kt >= 20 ? 0.75 : 0.59};
+            // rates relative to a 256 x 256 workgroup on a full chip.  kAlone: a 128 x 128 workgroup with a CU to itself
+            // (2048^3: 22.8 us on two LDS stages, 17.9 us on the ring of four a launch of at most one workgroup per CU
+            // and 20 k-tiles or more takes) against two sharing it
+            static const double kUnthrottled[4] = {1.36, 1.0, 1.0, 0.946}, kAtPowerLimit[4] = {1.0, 0.855, 0.855, 0.85};
+            const double kAlone[4] = {1.36, 1.0, 1.0, tiles <= cus && kt >= 20 ? 0.75 : 0.59};
             const int64_t slots = (int64_t)cus * t.wgs_per_cu, rest = tiles % slots;
             const double area = (double)t.bp * t.bq;
-            const double by_rounds = (double)(tiles / slots) * t.wgs_per_cu * area / kUnthrottled[i] +
-                                     (rest == 0 ? 0.0 : rest <= cus ? area / kAlone[i] : t.wgs_per_cu * area / kUnthrottled[i]);
-            const double by_power = (double)tiles * t.bp * t.bq / (cus * kAtPowerLimit[i]);
-            cost = std::max(by_rounds, by_power) * (kt + (t.wgs_per_cu == 1 ? 4.0 : 2.0)) / kt;
+            // a round of n co-resident workgroups: each CU at its unthrottled rate or at its share of the chip's
+            // power-limited rate, whichever is lower
+            auto round_cost = [&](int64_t n) {
+                const bool shared = n > cus;
+                const double rate = std::min(shared ? kUnthrottled[i] : kAlone[i],
+                                             kAtPowerLimit[i] * cus / (double)std::min<int64_t>(n, cus));
+                return (shared ? t.wgs_per_cu : 1) * area / rate;
+            };
+            cost = ((double)(tiles / slots) * round_cost(slots) + (rest ? round_cost(rest) : 0.0)) *
+                   (kt + (t.wgs_per_cu == 1 ? 4.0 : 2.0)) / kt;
         }
         if (best < 0 || cost < best_cost) { best = i; best_cost = cost; }
     }

@@ -453,6 +453,56 @@ def test_gemm_f32_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
     assert ran[None] == 150 and min(ran.values()) >= 30, ran
 
 
+def test_gemm_bf16_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
+    """120 seeded bf16 products with k a multiple of 64 (so that the direct-to-LDS kernels apply wherever the operands
+    are vector-loadable), m and n mostly multiples of 8, all four layouts, beta 0 or 1, each in the chooser's tile
+    configuration and forced into the 256 x 256, 128 x 256, 256 x 128 and 128 x 128 ones (two, three, three and two or
+    four LDS stages; a forced configuration that has no kernel for the operands' loaders is refused, not
+    miscomputed).  The forced configurations must agree bit for bit wherever they take the direct-to-LDS kernel: one
+    f32 sum per output in k order, rounded once."""
+    rng = np.random.default_rng(321)
+    ran = {None: 0, "0": 0, "1": 0, "2": 0, "3": 0}
+    for _ in range(120):
+        m, n, k = int(rng.integers(1, 700)), int(rng.integers(1, 700)), 64 * int(rng.integers(1, 14))
+        if rng.random() < 0.8:
+            m = 8 * max(1, m // 8)
+        if rng.random() < 0.8:
+            n = 8 * max(1, n // 8)
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        a = to_dtype(rng.uniform(-1, 1, (k, m) if ta else (m, k)), "bf16")
+        b = to_dtype(rng.uniform(-1, 1, (n, k) if tb else (k, n)), "bf16")
+        c0 = to_dtype(rng.uniform(-1, 1, (m, n)), "bf16")
+        beta = float(rng.choice([0.0, 0.0, 1.0]))
+        A, B = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+        av, bv = (a.T if ta else a), (b.T if tb else b)
+        want = orc.gemm_bf16_f32acc(av, bv, 1.0, beta, c0)
+        forced = []
+        for cfg in ran:
+            if cfg is None:
+                monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
+            else:
+                monkeypatch.setenv("AGH_GEMM_CFG", cfg)
+            C = ag.Tensor.from_array(c0)
+            try:
+                ag.gemm(1.0, A.t() if ta else A, B.t() if tb else B, beta, C)
+            except ag.AghError as e:
+                assert cfg is not None and e.code == -4
+                continue
+            ran[cfg] += 1
+            got = C.into_array()
+            if beta == 0.0:
+                assert_bf16_gemm_close(got, want, av, bv)
+            else:
+                gf, wf = orc.bf16_to_f32(got).astype(np.float64), orc.bf16_to_f32(want).astype(np.float64)
+                assert np.all(np.abs(gf - wf) <= bf16_ulp(wf) + 1e-2 * np.abs(wf) + 1e-3), (m, k, n, ta, tb, cfg)
+            if cfg is not None:
+                forced.append(got)
+        for other in forced[1:]:
+            assert np.array_equal(forced[0], other), (m, k, n, ta, tb, beta)
+    monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
+    assert ran[None] == 120 and min(ran.values()) >= 40, ran
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 def test_dense_full_size_bias_relu(ag, dtype):
     """The Dense-shaped GEMM of the benchmark list at full size: M = 16384 (batch), K = 4096, N = 4096 with the
