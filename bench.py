@@ -137,7 +137,7 @@ def main():
     flop = 2.0 * n * n * n
     value = flop / (wall_ms * 1e-3) / 1e12
     achieved = flop / (dev_ms * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "kernel": "gemm_bf16_dl_kernel<256,256,2,2,1,0,true> (v_mfma_f32_16x16x32_bf16, direct-to-LDS loads)",
+    roofline = {"bound": "mfma", "kernel": "gemm_bf16_dl_kernel<256,256,2,2,1,0,true,2> (v_mfma_f32_16x16x32_bf16, direct-to-LDS loads)",
                 "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/
