@@ -345,6 +345,12 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         const size_t total = (size_t)g.NQ * g.NP;
         int lanes = 1;  // threads per output element: about eight partials each
         while (lanes < 16 && lanes * 16 <= splits) lanes *= 2;
+        if (lanes == 1 && vec_store && g.NPpad == g.NP) {
+            hipLaunchKernelGGL(splitk_reduce_vec4_kernel<T>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0,
+                               stream(), g, splits);
+            AGH_LAUNCH_CHECK("split-K reduce launch");
+            return AGH_OK;
+        }
         const size_t blocks = (total * lanes + 255) / 256;
         if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: output too large for split-K", name);
         hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream(), g, splits, lanes);

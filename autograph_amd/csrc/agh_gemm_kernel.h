@@ -621,5 +621,46 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(Args g, int splits, 
     *dst = finish<T>(s, g.alpha, g.beta, old, g.has_bias != 0, bv, g.act);
 }
 
+// The same pass for fewer than 16 splits, C rows contiguous along p and whole groups of four: one thread per four
+// neighbouring outputs, the partials read 16 bytes at a time and four splits requested before the first add.  Every
+// output is the sum of its partials in split order from +0, exactly as splitk_reduce_kernel with one lane forms it.
+template <typename T>
+__global__ __launch_bounds__(256) void splitk_reduce_vec4_kernel(Args g, int splits) {
+    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int groups_per_row = g.NP / 4;
+    if (t >= (size_t)g.NQ * groups_per_row) return;
+    const int q = (int)(t / groups_per_row), p = (int)(t - (size_t)q * groups_per_row) * 4;
+    const float4 *wp = (const float4 *)(g.ws + (size_t)q * g.NPpad + p);
+    const size_t zstride = (size_t)g.NQ * g.NPpad / 4;  // in float4
+    float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int z = 0; z < splits; z += 4) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = wp[(size_t)min(z + u, splits - 1) * zstride];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const bool on = z + u < splits;  // s is never -0: adding +0 is exact
+            s[0] += on ? v[u].x : 0.0f;
+            s[1] += on ? v[u].y : 0.0f;
+            s[2] += on ? v[u].z : 0.0f;
+            s[3] += on ? v[u].w : 0.0f;
+        }
+    }
+    T *dst = (T *)g.D + p + (int64_t)q * g.dq;
+    __align__(16) T old[4] = {0, 0, 0, 0}, out[4];
+    if (g.beta != 0.0f) {
+        if constexpr (sizeof(T) == 4) *(uint4 *)old = *(const uint4 *)dst;
+        else *(uint2 *)old = *(const uint2 *)dst;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        T bv = 0;
+        if (g.has_bias) bv = ((const T *)g.bias)[(int64_t)(g.bias_on_p ? p + e : q) * g.bias_stride];
+        out[e] = finish<T>(s[e], g.alpha, g.beta, old[e], g.has_bias != 0, bv, g.act);
+    }
+    if constexpr (sizeof(T) == 4) *(uint4 *)dst = *(const uint4 *)out;
+    else *(uint2 *)dst = *(const uint2 *)out;
+}
+
 }  // namespace gemm
 }  // namespace agh

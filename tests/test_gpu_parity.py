@@ -414,6 +414,49 @@ def test_gemm_bf16_ring_of_four_stages(ag, monkeypatch):
     assert np.all(np.abs(gotf - want) <= 2 * bf16_ulp(want) + 1e-2 * np.abs(want) + 0.05)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_gemm_split_k_second_pass_four_outputs_a_thread(ag, monkeypatch, dtype):
+    """Split-K with fewer than 16 splits into a C whose rows are contiguous and whole groups of four: the second pass
+    that reads the partials 16 bytes at a time.  2 to 15 forced splits (the last one shorter than the others), alpha
+    and beta, a column bias and a row bias with ReLU, against the oracle; and against the one-output-a-thread pass,
+    which a C of 6 more columns takes, on the shared columns of integer data (exact in any order)."""
+    rng = np.random.default_rng(91)
+    m, k, n = 96, 1920, 136
+    a = to_dtype(rng.uniform(-1, 1, (m, k)), dtype)
+    b = to_dtype(rng.uniform(-1, 1, (k, n)), dtype)
+    c0 = to_dtype(rng.uniform(-1, 1, (m, n)), dtype)
+    A, B = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+    for splits in (2, 3, 4, 5, 7, 15):
+        monkeypatch.setenv("AGH_GEMM_SPLITS", str(splits))
+        for alpha, beta in ((1.0, 0.0), (0.5, -1.0)):
+            C = ag.Tensor.from_array(c0)
+            ag.gemm(alpha, A, B, beta, C)
+            got = C.into_array()
+            if dtype == "f32":
+                want = alpha * (a.astype(np.float64) @ b.astype(np.float64)) + beta * c0
+                assert np.abs(got - want).max() <= 1e-5 * np.sqrt(k) * np.abs(want).max()
+            else:
+                want = orc.bf16_to_f32(orc.gemm_bf16_f32acc(a, b, alpha, beta, c0)).astype(np.float64)
+                gf = orc.bf16_to_f32(got).astype(np.float64)
+                assert np.all(np.abs(gf - want) <= bf16_ulp(want) + 1e-2 * np.abs(want) + 1e-3)
+        bias = to_dtype(rng.uniform(-1, 1, n), dtype)
+        got = ag.Dense(B, ag.Tensor.from_array(bias)).forward(A, relu=True).into_array()
+        monkeypatch.delenv("AGH_GEMM_SPLITS")
+        one = ag.Dense(B, ag.Tensor.from_array(bias)).forward(A, relu=True).into_array()
+        gf, of = as_f32(got).astype(np.float64), as_f32(one).astype(np.float64)
+        tol = 1e-5 * np.sqrt(k) * max(np.abs(of).max(), 1.0) if dtype == "f32" else bf16_ulp(of) + 1e-2 * np.abs(of) + 1e-3
+        assert np.all(np.abs(gf - of) <= tol)
+    ai = to_dtype(rng.integers(-4, 5, (m, k)).astype(np.float32), dtype)
+    bi = to_dtype(rng.integers(-4, 5, (k, n + 6)).astype(np.float32), dtype)
+    monkeypatch.setenv("AGH_GEMM_SPLITS", "6")
+    wide = ag.Tensor.from_array(ai).dot(ag.Tensor.from_array(bi)).into_array()
+    narrow = ag.Tensor.from_array(ai).dot(ag.Tensor.from_array(np.ascontiguousarray(bi[:, :n]))).into_array()
+    monkeypatch.delenv("AGH_GEMM_SPLITS")
+    assert np.array_equal(wide[:, :n], narrow)
+    if dtype == "f32":
+        assert np.array_equal(narrow, ai @ bi[:, :n])
+
+
 def test_gemm_f32_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
     """150 seeded f32 products with k a multiple of 32 (so that the direct-to-LDS kernels apply wherever the operands
     are vector-loadable), odd and even m and n, all four layouts, alpha and beta, each in the chooser's tile
