@@ -68,12 +68,47 @@ def _device_param(pair, dtype):
     return Tensor.from_array(array)
 
 
+class OptimizerState:
+    """`State` of a parameter (optimizer.rs:163-173) with its tensors on the device: `name` of the optimizer and
+    `key_values` [(key, Tensor, parameter_device, parameter_type)].  A state read back from JSON is kept and written
+    again, but an optimizer starts a fresh one: the reference skips the optimizer's type id when it writes a state and
+    restores `()`'s (optimizer.rs:169-170, :175-178), which `SGD::init_state` then takes for another optimizer's state
+    and replaces with a zero velocity (optimizer.rs:358-381)."""
+
+    def __init__(self, name, key_values=()):
+        self.name, self.key_values = name, list(key_values)
+
+    def get(self, key):
+        for k, t, _, _ in self.key_values:
+            if k == key:
+                return t
+        return None
+
+
+def _host_state(state):
+    from . import serde
+    if state is None:
+        return None
+    return serde.OptimStateValue(state.name, [(k, t.into_array(), t.dtype == "bf16", pd, pt) for k, t, pd, pt in state.key_values])
+
+
+def _device_state(pair):
+    st = getattr(pair, "optim_state", None)
+    if st is None:
+        return None
+    for _, array, is_bf16, _, _ in st.key_values:
+        if not is_bf16 and array.dtype != np.float32:
+            raise AghError(-1, "serde: optimizer state tensors are f32 or bf16 here")
+    return OptimizerState(st.name, [(k, Tensor.from_array(a), pd, pt) for k, a, _, pd, pt in st.key_values])
+
+
 class Conv2:
     """`Conv2` (layer.rs:844-1047): weight [outputs, inputs, fh, fw], optional bias [outputs]."""
 
     def __init__(self, weight, bias=None, padding=(0, 0), stride=(1, 1), dilation=(1, 1)):
         self.weight, self.bias = weight, bias
         self.padding, self.stride, self.dilation = tuple(padding), tuple(stride), tuple(dilation)
+        self.weight_state = self.bias_state = None  # OptimizerState of each parameter (autograd.rs:655)
 
     # the data model of the reference's derive (layer.rs:833-848), as serde_json writes it; see autograph_amd/serde.py
     def to_json(self):
@@ -81,14 +116,18 @@ class Conv2:
         from . import serde
         bf16 = self.weight.dtype == "bf16"
         return json.dumps(serde.conv2_to_value(self.weight.into_array(), None if self.bias is None else self.bias.into_array(),
-                                               self.padding, self.stride, self.dilation, bf16=bf16), separators=(",", ":"))
+                                               self.padding, self.stride, self.dilation, bf16=bf16,
+                                               weight_state=_host_state(self.weight_state),
+                                               bias_state=_host_state(self.bias_state)), separators=(",", ":"))
 
     @classmethod
     def from_json(cls, text, dtype=None):
         import json
         from . import serde
         f = serde.conv2_from_value(json.loads(text))
-        return cls(_device_param(f["weight"], dtype), _device_param(f["bias"], dtype), f["padding"], f["stride"], f["dilation"])
+        layer = cls(_device_param(f["weight"], dtype), _device_param(f["bias"], dtype), f["padding"], f["stride"], f["dilation"])
+        layer.weight_state, layer.bias_state = _device_state(f["weight"]), _device_state(f["bias"])
+        return layer
 
     def forward(self, x, relu=False, pool2x2=False, algorithm="auto"):
         """`conv2` (layer.rs:930-948).  Like the reference's host, which takes a direct kernel when
@@ -111,6 +150,7 @@ class Dense:
 
     def __init__(self, weight, bias=None):
         self.weight, self.bias = weight, bias
+        self.weight_state = self.bias_state = None  # OptimizerState of each parameter (autograd.rs:655)
 
     def forward(self, x, relu=False):
         return x.dot(self.weight, bias=self.bias, relu=relu)
@@ -119,14 +159,17 @@ class Dense:
         import json
         from . import serde
         return json.dumps(serde.dense_to_value(self.weight.into_array(), None if self.bias is None else self.bias.into_array(),
-                                               bf16=self.weight.dtype == "bf16"), separators=(",", ":"))
+                                               bf16=self.weight.dtype == "bf16", weight_state=_host_state(self.weight_state),
+                                               bias_state=_host_state(self.bias_state)), separators=(",", ":"))
 
     @classmethod
     def from_json(cls, text, dtype=None):
         import json
         from . import serde
         f = serde.dense_from_value(json.loads(text))
-        return cls(_device_param(f["weight"], dtype), _device_param(f["bias"], dtype))
+        layer = cls(_device_param(f["weight"], dtype), _device_param(f["bias"], dtype))
+        layer.weight_state, layer.bias_state = _device_state(f["weight"]), _device_state(f["bias"])
+        return layer
 
 
 class MaxPool2:
@@ -351,6 +394,12 @@ class LeNet5Trainer:
             self.velocities = views(self._vflat)
         else:
             self._vflat, self.velocities = None, [None] * 6
+        # every parameter's optimizer state, as `SGD::init_state` builds it (optimizer.rs:358-381): named "SGD", empty
+        # without momentum, else the velocity (a view of the shared buffer, so it is always current) marked as
+        # following the parameter's device and type
+        states = [OptimizerState("SGD", [] if v is None else [("velocity", v, True, True)]) for v in self.velocities]
+        (m.conv1.weight_state, m.conv2.weight_state, m.dense1.weight_state, m.dense2.weight_state, m.dense3.weight_state,
+         m.dense3.bias_state) = states
         host = C.c_void_p()
         check(lib.agh_host_alloc(C.byref(host), 4))
         self._loss_host = host

@@ -131,30 +131,82 @@ def _dims(obj, what, rank):
     return tuple(obj)
 
 
-def parameter_to_value(array, bf16=False):
-    """A parameter without optimizer state (the state of a freshly built or inference-only layer)."""
-    return {"value": to_value(array, bf16)}
+class OptimStateValue:
+    """`State { name, id (skipped), key_values: Vec<(String, Value)> }` (optimizer.rs:163-173) on the host.
+    `key_values`: [(key, array, is_bf16, parameter_device, parameter_type)]: every value a
+    `Value::Tensor(TensorValue { tensor, parameter_device, parameter_type })` (optimizer.rs:108-131), the only kind
+    the reference's optimizers create (SGD's "velocity", optimizer.rs:367-381)."""
+
+    def __init__(self, name, key_values=()):
+        self.name, self.key_values = str(name), [tuple(kv) for kv in key_values]
+
+
+class ParamValue(tuple):
+    """(array, is_bf16) of a parameter, with its optimizer state (None or an OptimStateValue) as `.optim_state`."""
+
+    def __new__(cls, array, is_bf16, optim_state=None):
+        self = super().__new__(cls, (array, is_bf16))
+        self.optim_state = optim_state
+        return self
+
+
+def optim_state_to_value(state):
+    return {"name": state.name,
+            "key_values": [[str(key), {"Tensor": {"tensor": to_value(array, bf16), "parameter_device": bool(pdev),
+                                                  "parameter_type": bool(ptype)}}]
+                           for (key, array, bf16, pdev, ptype) in state.key_values]}
+
+
+def optim_state_from_value(obj):
+    if not isinstance(obj, dict) or set(obj) != {"name", "key_values"} or not isinstance(obj["name"], str) \
+            or not isinstance(obj["key_values"], list):
+        raise SerdeError("expected an optimizer state with the fields `name` and `key_values`")
+    out = []
+    for kv in obj["key_values"]:
+        if not isinstance(kv, list) or len(kv) != 2 or not isinstance(kv[0], str) or not isinstance(kv[1], dict) \
+                or len(kv[1]) != 1:
+            raise SerdeError("`key_values` must hold [key, {variant: value}] pairs")
+        (variant, value), = kv[1].items()
+        if variant == "Elem":
+            # the element type of Value::Elem is the scalar crate's, whose encoding no file of the reference holds
+            raise SerdeError("optimizer state with a scalar element value is not supported here")
+        if variant != "Tensor" or not isinstance(value, dict) or set(value) != {"tensor", "parameter_device", "parameter_type"} \
+                or not isinstance(value["parameter_device"], bool) or not isinstance(value["parameter_type"], bool):
+            raise SerdeError("expected {\"Tensor\": {tensor, parameter_device, parameter_type}}")
+        array, is_bf16 = from_value(value["tensor"])
+        out.append((kv[0], array, is_bf16, value["parameter_device"], value["parameter_type"]))
+    return OptimStateValue(obj["name"], out)
+
+
+def parameter_to_value(array, bf16=False, optim_state=None):
+    """`value`, then `optim_state` unless it is none (skip_serializing_if, autograd.rs:651-655)."""
+    out = {"value": to_value(array, bf16)}
+    if optim_state is not None:
+        out["optim_state"] = optim_state_to_value(optim_state)
+    return out
 
 
 def parameter_from_value(obj, rank):
+    """-> ParamValue.  An absent `optim_state` is none (`default`); a present one must be a state: the reference's
+    deserializer has no none case (autograd.rs:1141-1151)."""
     if not isinstance(obj, dict) or "value" not in obj or set(obj) - {"value", "optim_state"}:
         raise SerdeError("expected a parameter object with the field `value`")
-    if obj.get("optim_state") is not None:
-        raise SerdeError("optimizer state in a parameter is not supported here")
+    state = optim_state_from_value(obj["optim_state"]) if "optim_state" in obj else None
     array, is_bf16 = from_value(obj["value"])
     if array.ndim != rank:
         raise SerdeError(f"IncompatibleShape: a parameter of rank {rank} holds a tensor of rank {array.ndim}")
-    return array, is_bf16
+    return ParamValue(array, is_bf16, state)
 
 
-def conv2_to_value(weight, bias=None, padding=(0, 0), stride=(1, 1), dilation=(1, 1), bf16=False):
-    return {"weight": parameter_to_value(weight, bf16), "padding": [int(v) for v in padding],
+def conv2_to_value(weight, bias=None, padding=(0, 0), stride=(1, 1), dilation=(1, 1), bf16=False, weight_state=None,
+                   bias_state=None):
+    return {"weight": parameter_to_value(weight, bf16, weight_state), "padding": [int(v) for v in padding],
             "stride": [int(v) for v in stride], "dilation": [int(v) for v in dilation],
-            "bias": None if bias is None else parameter_to_value(bias, bf16)}
+            "bias": None if bias is None else parameter_to_value(bias, bf16, bias_state)}
 
 
 def conv2_from_value(obj):
-    """-> dict(weight=(array, is_bf16), bias=None | (array, is_bf16), padding, stride, dilation)"""
+    """-> dict(weight=ParamValue, bias=None | ParamValue, padding, stride, dilation)"""
     fields = {"weight", "padding", "stride", "dilation", "bias"}
     if not isinstance(obj, dict) or set(obj) != fields:
         raise SerdeError("expected an object with exactly the fields " + ", ".join(sorted(fields)))
@@ -164,8 +216,9 @@ def conv2_from_value(obj):
                 dilation=_dims(obj["dilation"], "dilation", 2))
 
 
-def dense_to_value(weight, bias=None, bf16=False):
-    return {"weight": parameter_to_value(weight, bf16), "bias": None if bias is None else parameter_to_value(bias, bf16)}
+def dense_to_value(weight, bias=None, bf16=False, weight_state=None, bias_state=None):
+    return {"weight": parameter_to_value(weight, bf16, weight_state),
+            "bias": None if bias is None else parameter_to_value(bias, bf16, bias_state)}
 
 
 def dense_from_value(obj):

@@ -99,8 +99,11 @@ def test_layer_values_follow_the_derived_field_lists():
     assert np.array_equal(serde.dense_from_value(d)["weight"][0], w.reshape(4, 75))
     assert serde.max_pool2_to_value((2, 2), (2, 2)) == {"filter": [2, 2], "stride": [2, 2]}  # layer.rs:1152-1155
     assert serde.max_pool2_from_value({"filter": [3, 2], "stride": [1, 1]}) == dict(filter=(3, 2), stride=(1, 1))
-    # an absent optimizer state is the default (none); anything else, unknown or missing fields, wrong ranks are errors
-    assert np.array_equal(serde.parameter_from_value({"value": json.loads(serde.to_json(b)), "optim_state": None}, 1)[0], b)
+    # an absent optimizer state is the default (none); a null one is no state (the deserializer reads a struct,
+    # autograd.rs:1141-1151); unknown or missing fields and wrong ranks are errors
+    assert serde.parameter_from_value({"value": json.loads(serde.to_json(b))}, 1).optim_state is None
+    with pytest.raises(serde.SerdeError):
+        serde.parameter_from_value({"value": json.loads(serde.to_json(b)), "optim_state": None}, 1)
     for bad in ({"weight": v["weight"], "bias": None, "extra": 1}, {"weight": v["weight"]},
                 {"weight": {"value": json.loads(serde.to_json(b))}, "bias": None}):
         with pytest.raises(serde.SerdeError):
@@ -109,6 +112,83 @@ def test_layer_values_follow_the_derived_field_lists():
         serde.conv2_from_value({**v, "padding": [1]})
     with pytest.raises(serde.SerdeError):
         serde.max_pool2_from_value({"filter": [2, 2]})
+
+
+def test_parameter_optimizer_state_follows_the_derived_field_lists():
+    """`optim_state` after `value`, only when there is a state (autograd.rs:647-656); a state is its name and its
+    (key, value) pairs, the optimizer's type id skipped (optimizer.rs:166-173); a value is the externally tagged
+    `Tensor` variant with the tensor and the two flags SGD sets (optimizer.rs:108-131, :373-380)."""
+    rng = np.random.default_rng(8)
+    w = rng.standard_normal((3, 4)).astype(np.float32)
+    vel = rng.standard_normal((3, 4)).astype(np.float32)
+    state = serde.OptimStateValue("SGD", [("velocity", vel, False, True, True)])
+    v = serde.parameter_to_value(w, optim_state=state)
+    assert list(v) == ["value", "optim_state"] and list(v["optim_state"]) == ["name", "key_values"]
+    assert v["optim_state"]["name"] == "SGD"
+    (key, value), = v["optim_state"]["key_values"]
+    assert key == "velocity" and list(value) == ["Tensor"]
+    assert list(value["Tensor"]) == ["tensor", "parameter_device", "parameter_type"]
+    assert value["Tensor"]["tensor"] == json.loads(serde.to_json(vel))
+    assert value["Tensor"]["parameter_device"] is True and value["Tensor"]["parameter_type"] is True
+    back = serde.parameter_from_value(json.loads(json.dumps(v)), 2)
+    assert np.array_equal(back[0], w) and back.optim_state.name == "SGD"
+    (k, a, is_bf16, pdev, ptype), = back.optim_state.key_values
+    assert k == "velocity" and np.array_equal(a, vel) and not is_bf16 and pdev and ptype
+    # SGD without momentum: a state with no values (optimizer.rs:366-381)
+    empty = serde.parameter_to_value(w, optim_state=serde.OptimStateValue("SGD"))
+    assert empty["optim_state"] == {"name": "SGD", "key_values": []}
+    assert serde.parameter_from_value(empty, 2).optim_state.key_values == []
+    # bf16 velocity, inside a layer
+    bits = (vel.view(np.uint32) >> 16).astype(np.uint16)
+    d = serde.dense_to_value(bits, None, bf16=True, weight_state=serde.OptimStateValue("SGD", [("velocity", bits, True, True, True)]))
+    got = serde.dense_from_value(json.loads(json.dumps(d)))["weight"]
+    assert got[1] and got.optim_state.key_values[0][2] and np.array_equal(got.optim_state.key_values[0][1], bits)
+    for bad in ({"name": "SGD"}, {"name": "SGD", "key_values": [["velocity", {"Elem": {"F32": 0.5}}]]},
+                {"name": "SGD", "key_values": [["velocity", {"Tensor": {"tensor": value["Tensor"]["tensor"]}}]]},
+                {"name": "SGD", "key_values": [["velocity"]]}, {"name": 3, "key_values": []}):
+        with pytest.raises(serde.SerdeError):
+            serde.parameter_from_value({"value": v["value"], "optim_state": bad}, 2)
+
+
+@pytest.mark.gpu
+def test_trainer_velocity_is_written_with_the_parameters():
+    """A LeNet5 training step with momentum, then every layer written and read back: the velocity travels as the
+    parameter's optimizer state and is the trainer's, bit for bit; a layer without a trainer writes none."""
+    import autograph_amd as ag
+    ag.Device(0)
+    rng = np.random.default_rng(12)
+
+    def he(shape, fan_in):
+        a = np.sqrt(2.0 / fan_in)
+        return rng.uniform(-a, a, shape).astype(np.float32)
+
+    def lenet():
+        return ag.LeNet5.from_arrays(he((6, 1, 5, 5), 25), he((16, 6, 5, 5), 150), he((256, 128), 256), he((128, 84), 128),
+                                     he((84, 10), 84), he((10,), 84))
+
+    model = lenet()
+    assert "optim_state" not in json.loads(model.dense1.to_json())["weight"]
+    trainer = ag.LeNet5Trainer(model, 16, learning_rate=0.05, optimizer=ag.SGD(momentum=0.9))
+    x = ag.Tensor.from_array(rng.uniform(0, 1, (16, 1, 28, 28)).astype(np.float32))
+    labels = rng.integers(0, 10, 16).astype(np.uint8)
+    t = ag.Buffer(labels.size)
+    ag._ffi.check(ag.lib.agh_memcpy_h2d(t.ptr, labels.ctypes.data, labels.size))
+    ag._ffi.check(ag.lib.agh_sync())
+    trainer.step(x, t)
+    trainer.step(x, t)
+    ag._ffi.check(ag.lib.agh_sync())
+    for layer, vel in ((model.conv1, trainer.velocities[0]), (model.dense1, trainer.velocities[2]), (model.dense3, trainer.velocities[4])):
+        back = type(layer).from_json(layer.to_json())
+        assert back.weight_state.name == "SGD"
+        v = back.weight_state.get("velocity").into_array()
+        assert np.array_equal(v, vel.into_array()) and np.abs(v).max() > 0
+        assert np.array_equal(back.weight.into_array(), layer.weight.into_array())
+        # written again, the state is still there
+        assert json.loads(back.to_json())["weight"]["optim_state"]["name"] == "SGD"
+    back = ag.Dense.from_json(model.dense3.to_json())
+    assert np.array_equal(back.bias_state.get("velocity").into_array(), trainer.velocities[5].into_array())
+    plain = ag.LeNet5Trainer(lenet(), 16)
+    assert json.loads(plain.model.dense2.to_json())["weight"]["optim_state"] == {"name": "SGD", "key_values": []}
 
 
 @pytest.mark.gpu
