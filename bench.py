@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Headline benchmark: bf16 GEMM at 8192^3 on one MI355X, plus the other BASELINE configs
+"""Headline benchmark: bf16 GEMM at 8192^3 on one MI355X, plus the other benchmark configurations
 as `extras`, the MFMA roofline of the dominant kernel and the CPU host-path baseline.
 
     python bench.py --gpus 1 --steps K --warmup W
@@ -319,7 +319,7 @@ def main():
                 es * (2 * nx + ny), "GB/s", PEAK_HBM_GBS)
             del x, wt, cols, dx, py
 
-    # ---------------- LeNet5 f32 inference, batch 1000 (BASELINE configs[0]) ----------------
+    # ---------------- LeNet5 f32 inference, batch 1000 (benchmark configuration 0) ----------------
     lenet = None
     if not args.no_extras and "lenet" in sections:
         try:
@@ -398,7 +398,7 @@ def main():
             extras["lenet5_f32_infer_b1000"] = {"error": str(e)}
             log("lenet5: FAILED", e)
 
-    # ---------------- LeNet5 training step, batch 100 (BASELINE configs[4]) ----------------
+    # ---------------- LeNet5 training step, batch 100 (benchmark configuration 4) ----------------
     if not args.no_extras and "train" in sections:
         for dt in ("bf16", "f32"):
             key = f"lenet5_{dt}_train_b100"

@@ -274,7 +274,7 @@ def test_bf16_output_rounding_matches_reference_rule(ag):
 @pytest.mark.parametrize("dtype,shape", [("f32", (4096, 4096, 4096)), ("bf16", (8192, 8192, 8192)),
                                          ("f32", (8192, 8192, 8192))])
 def test_gemm_full_size_sampled_entries_and_identity(ag, dtype, shape):
-    """BASELINE-size GEMMs: the oracle cannot run 10^12 flops, so check (1) 4096 sampled output
+    """Benchmark-size GEMMs: the oracle cannot run 10^12 flops, so check (1) 4096 sampled output
     entries against f64 dot products of the corresponding row and column, for A*B, A^T*B and
     A*B^T, and (2) A*I == A bit for bit."""
     m, k, n = shape
