@@ -279,6 +279,10 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         const double kt = (double)((g.K + BK - 1) / BK);
         eff *= kt / (kt + (f32_direct ? 6.0 : t.wgs_per_cu == 1 ? 4.0 : 0.5));
         double cost = (double)rounds * t.bp * t.bq / eff;
+        // many small tiles do not run in lockstep rounds: a CU takes the next tile when one of its two is done, and the
+        // launch ends a fraction of a tile after tiles / CUs tile times (3584^3 on 64 x 64 tiles: 12.25 tiles a CU,
+        // 12.5 tile times measured, 790 us against 871 us on the 256 x 256 tile)
+        if (f32_direct && tiles >= 4 * (int64_t)cus) cost = ((double)tiles / cus + 0.25) * t.bp * t.bq / eff;
         // bf16 direct-to-LDS tiles: a full chip of them runs at the power limit, where the rate depends on the tile
         // shape (bigger tiles move fewer operand bytes per flop) and not on how many CUs take part, while a
         // launch that leaves CUs idle runs the busy ones at a higher clock.  Measured per k-tile of a 256 x 256
