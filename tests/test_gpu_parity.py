@@ -398,6 +398,17 @@ def test_gemm_bf16_ring_of_four_stages(ag, monkeypatch):
                 monkeypatch.delenv("AGH_GEMM_RING")
                 assert_bf16_gemm_close(out, orc.gemm_bf16_f32acc(av, bv), av, bv)
                 assert np.array_equal(out, two), (m, k, n, ta, tb)
+    # a batch of three products with a shared B in one launch (agh_gemm_bf16_batched), 22 k-tiles
+    nb, m, k, n = 3, 136, 1408, 128
+    a = to_dtype(rng.uniform(-1, 1, (nb, m, k)), "bf16")
+    b = to_dtype(rng.uniform(-1, 1, (k, n)), "bf16")
+    A, B, Cb = ag.Tensor.from_array(a), ag.Tensor.from_array(b), ag.Tensor.zeros((nb, m, n), "bf16")
+    ag._ffi.check(ag.lib.agh_gemm_bf16_batched(nb, m, k, n, 1.0, A._ptr(), 0, k, 1, m * k, B._ptr(), 0, n, 1, 0, 0.0,
+                                               Cb._ptr(), 0, n, 1, m * n, None, 0, 0, 0))
+    got = Cb.into_array()
+    for i in range(nb):
+        assert_bf16_gemm_close(got[i], orc.gemm_bf16_f32acc(a[i], b), a[i], b)
+        assert np.array_equal(got[i], ag.Tensor.from_array(a[i]).dot(B).into_array())
     m, k, n = 192, 1536, 256
     a = to_dtype(rng.uniform(-1, 1, (m, k)), "bf16")
     w = to_dtype(rng.uniform(-1, 1, (k, n)), "bf16")
