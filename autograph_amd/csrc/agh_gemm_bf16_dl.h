@@ -25,9 +25,10 @@
 // are applied on the global side: each lane computes once which chunk of the tile belongs at
 // its LDS position.
 //
-// Requirements checked by the host: K (and every split's k range) a multiple of 64, operand
-// base pointers 16-byte aligned, unit stride along k (LD_K) or along rows (LD_R) with the
-// other stride a multiple of 8 elements, rows a multiple of 8 for LD_R.
+// Requirements checked by the host: every split's k range but the last a multiple of 64, operand
+// base pointers 16-byte aligned, unit stride along k (LD_K: k a multiple of 8) or along rows (LD_R)
+// with the other stride a multiple of 8 elements, rows a multiple of 8 for LD_R.  A last k-tile
+// shorter than 64 is multiplied after the pipelined loop, its lanes reading zeros behind k = K.
 #pragma once
 #include "agh_gemm_kernel.h"
 
@@ -88,7 +89,21 @@ struct DirectLoad {
             }
         }
     }
+    // whether this lane's 16 bytes of load i lie below k = rem within a k-tile (rem < 64: the last, shorter tile)
+    static __device__ __forceinline__ bool below(int i, int wave, int lane, int rem) {
+        const int inst = wave * NL + i;
+        if constexpr (MODE == LD_K) {
+            const int row = inst * 8 + (lane >> 3);
+            return (((lane & 7) ^ (int)swz((uint32_t)row)) * 8) < rem;
+        } else {
+            return inst * KRPI + lane / CPR < rem;
+        }
+    }
 };
+
+// what the lanes of a shorter last k-tile read in place of elements at k >= K: both operands are zero there, so the
+// products vanish whatever lies behind the end of a row
+__device__ __align__(16) static const uint32_t kZeroChunk[4] = {0u, 0u, 0u, 0u};
 
 // Per-lane LDS byte offsets for the MFMA fragments of one operand (16-row tile index i), v_mfma_f32_16x16x32_bf16:
 // lane l supplies row l % 16, k = 8 * (l / 16) .. + 7 of a 32-deep substep.
@@ -157,7 +172,8 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     const int split = blockIdx.y;
     const int kbeg = split * g.k_per_split;
     const int kend = min(g.K, kbeg + g.k_per_split);
-    const int KT = kend > kbeg ? (kend - kbeg) / BK : 0;
+    const int KT = kend > kbeg ? (kend - kbeg) / BK : 0;     // whole k-tiles
+    const int rem = kend > kbeg ? (kend - kbeg) % BK : 0;    // depth of a shorter last one (the last split's only)
 
     int64_t offp[DlP::NL], offq[DlQ::NL];
     DlP::offsets(offp, g.ps, g.pk, p0, g.NP, wave, lane);
@@ -270,6 +286,32 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     });
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    if (rem > 0) {
+        // The shorter last k-tile, outside the pipeline (one load latency per workgroup, once): the same direct loads
+        // into stage 0, lanes whose bytes lie at k >= K reading zeros instead.  After the loop the pointers stand at
+        // the last whole tile (at this tile when there is none).
+        const uint32_t a0 = __builtin_amdgcn_readfirstlane(lds_address(stage0));
+        const int64_t tp_adv = KT > 0 ? stepP : 0, tq_adv = KT > 0 ? stepQ : 0;
+        static_for<NLT>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            if constexpr (l < NLP) {
+                const void *src = DlP::below(l, wave, lane, rem) ? (const void *)(gp[l] + tp_adv) : (const void *)kZeroChunk;
+                direct_load16(src, a0 + (wave * NLP + l) * 1024);
+            } else {
+                const void *src = DlQ::below(l - NLP, wave, lane, rem) ? (const void *)(gq[l - NLP] + tq_adv) : (const void *)kZeroChunk;
+                direct_load16(src, a0 + P_BYTES + (wave * NLQ + (l - NLP)) * 1024);
+            }
+        });
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        static_for<NU>([&](auto uc) { read_unit(pfa, qfa, stage0, std::integral_constant<int, 0>{}, uc); });
+        static_for<NM>([&](auto mc) { mma(acc[decltype(mc)::value / TQ][decltype(mc)::value % TQ], pfa[decltype(mc)::value / TQ], qfa[decltype(mc)::value % TQ]); });
+        if (rem > 32) {
+            static_for<NU>([&](auto uc) { read_unit(pfb, qfb, stage0, std::integral_constant<int, 1>{}, uc); });
+            static_for<NM>([&](auto mc) { mma(acc[decltype(mc)::value / TQ][decltype(mc)::value % TQ], pfb[decltype(mc)::value / TQ], qfb[decltype(mc)::value % TQ]); });
+        }
+        __syncthreads();  // the epilogue reuses the stages
+    }
 
     // ------------------------------------------------------------ epilogue ----
     // accumulator element r of lane l, tile (i, j) = D[pwb + 16 i + 4 (l / 16) + r][qwb + 16 j + l % 16]

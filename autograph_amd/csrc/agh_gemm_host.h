@@ -251,7 +251,8 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
 
     // ---- tile shape: minimise (rounds of workgroups) x (tile area) / efficiency ----
     const int cus = compute_units() > 0 ? compute_units() : 256;
-    const bool direct_ok = sizeof(T) == 2 && !any_scalar && g.K > 0 && g.K % 64 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0;
+    // (any k: a last k-tile shorter than 64 is loaded with zeros behind k = K)
+    const bool direct_ok = sizeof(T) == 2 && !any_scalar && g.K > 0 && env_int("AGH_GEMM_DIRECT", 1) != 0;
     int best = -1;
     double best_cost = 0;
     for (int i = 0; i < kNumCfgs; ++i) {
@@ -335,7 +336,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     splits = ktiles > 0 ? (ktiles + tiles_per_split - 1) / tiles_per_split : 1;
     g.k_per_split = tiles_per_split * BK;
 
-    // bf16 with both operands vector-loadable and k a multiple of the 64-wide k-tile takes the
+    // bf16 with both operands vector-loadable takes the
     // direct-to-LDS kernel (AGH_GEMM_DIRECT=0 forces the register-staged one)
     const bool direct = direct_ok;
 

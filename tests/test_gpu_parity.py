@@ -468,6 +468,59 @@ def test_gemm_split_k_second_pass_four_outputs_a_thread(ag, monkeypatch, dtype):
         assert np.array_equal(narrow, ai @ bi[:, :n])
 
 
+def test_gemm_bf16_last_k_tile_shorter_than_64(ag, monkeypatch):
+    """The bf16 direct-to-LDS kernels with k not a multiple of their 64-deep k-tile: the last tile is loaded with zeros
+    behind k = K (both operands), outside the pipeline.  k below one tile, one tile and a rest, a rest of at most and of
+    more than 32 (one or both halves of the tile multiplied), 20 tiles and a rest (the four-stage ring), all four
+    layouts, every tile forced; odd k (operands stored k-major, the only vector-loadable form then); forced split-K,
+    whose last split alone has the shorter tile; the register-staged kernel on the same inputs."""
+    rng = np.random.default_rng(99)
+    cases = [(128, k, 128) for k in (8, 24, 40, 56, 72, 104, 200, 1000, 1288)] + [(264, 120, 136), (136, 1096, 264)]
+    for (m, k, n) in cases:
+        for ta in (False, True):
+            for tb in (False, True):
+                a = to_dtype(rng.uniform(-1, 1, (k, m) if ta else (m, k)), "bf16")
+                b = to_dtype(rng.uniform(-1, 1, (n, k) if tb else (k, n)), "bf16")
+                A, B = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+                av, bv = (a.T if ta else a), (b.T if tb else b)
+                want = orc.gemm_bf16_f32acc(av, bv)
+                outs = []
+                for cfg in (None, "0", "1", "2", "3"):
+                    if cfg is None:
+                        monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
+                    else:
+                        monkeypatch.setenv("AGH_GEMM_CFG", cfg)
+                    out = (A.t() if ta else A).dot(B.t() if tb else B).into_array()
+                    assert_bf16_gemm_close(out, want, av, bv)
+                    outs.append(out)
+                monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
+                for other in outs[2:]:
+                    assert np.array_equal(outs[1], other), (m, k, n, ta, tb)  # one f32 sum in k order, rounded once
+    for (m, k, n) in ((96, 77, 200), (96, 3, 200), (104, 1001, 96)):
+        a = to_dtype(rng.uniform(-1, 1, (k, m)), "bf16")
+        b = to_dtype(rng.uniform(-1, 1, (k, n)), "bf16")
+        out = ag.Tensor.from_array(a).t().dot(ag.Tensor.from_array(b)).into_array()
+        assert_bf16_gemm_close(out, orc.gemm_bf16_f32acc(a.T, b), a.T, b)
+        monkeypatch.setenv("AGH_GEMM_DIRECT", "0")
+        staged = ag.Tensor.from_array(a).t().dot(ag.Tensor.from_array(b)).into_array()
+        monkeypatch.delenv("AGH_GEMM_DIRECT")
+        assert_bf16_gemm_close(staged, orc.gemm_bf16_f32acc(a.T, b), a.T, b)
+    m, k, n = 136, 1000, 128
+    a = to_dtype(rng.uniform(-1, 1, (m, k)), "bf16")
+    b = to_dtype(rng.uniform(-1, 1, (k, n)), "bf16")
+    for splits in ("3", "16"):
+        monkeypatch.setenv("AGH_GEMM_SPLITS", splits)
+        out = ag.Tensor.from_array(a).dot(ag.Tensor.from_array(b)).into_array()
+        assert_bf16_gemm_close(out, orc.gemm_bf16_f32acc(a, b), a, b)
+    monkeypatch.delenv("AGH_GEMM_SPLITS")
+    # integer data: exact whatever the order, so any element dropped or counted twice at the tile's edge shows
+    ai = to_dtype(rng.integers(-3, 4, (136, 1016)).astype(np.float32), "bf16")
+    bi = to_dtype(rng.integers(-3, 4, (1016, 264)).astype(np.float32), "bf16")
+    got = orc.bf16_to_f32(ag.Tensor.from_array(ai).dot(ag.Tensor.from_array(bi)).into_array())
+    exact = orc.bf16_to_f32(ai).astype(np.float64) @ orc.bf16_to_f32(bi).astype(np.float64)
+    assert np.array_equal(got, orc.bf16_to_f32(orc.f32_to_bf16(exact.astype(np.float32))))
+
+
 def test_gemm_f32_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
     """150 seeded f32 products with k a multiple of 32 (so that the direct-to-LDS kernels apply wherever the operands
     are vector-loadable), odd and even m and n, all four layouts, alpha and beta, each in the chooser's tile
