@@ -26,9 +26,10 @@
 // two partial accumulators are added through LDS in front of the epilogue, always in the same order.  For grids that
 // give a CU a single workgroup.
 //
-// Requirements checked by the host: K and every split's k range multiples of 32, operand base pointers 16-byte
-// aligned, unit stride along k (LD_K) or along rows (LD_R) with the other stride a multiple of 4 elements, rows a
-// multiple of 4 for LD_R.
+// Requirements checked by the host: every split's k range but the last a multiple of 32, operand base pointers
+// 16-byte aligned, unit stride along k (LD_K: k a multiple of 4) or along rows (LD_R) with the other stride a
+// multiple of 4 elements, rows a multiple of 4 for LD_R.  A last k-tile shorter than 32 is multiplied after the
+// pipelined loop, its lanes reading zeros behind k = K.
 #pragma once
 #include "agh_gemm_bf16_dl.h"
 
@@ -55,6 +56,9 @@ struct F32DlGeo {
     static constexpr int STAGE_BYTES = OpP::BYTES + OpQ::BYTES;
     static constexpr int SMEM_BYTES = NS * STAGE_BYTES;
 };
+
+// what the lanes of a shorter last k-tile read in place of elements at k >= K
+__device__ __align__(16) static const uint32_t kZeroChunkF32[4] = {0u, 0u, 0u, 0u};
 
 template <int TP, int TQ, int NS, int LP, int LQ, int KS = 1>
 __global__ __launch_bounds__(256 * KS) void gemm_f32_dl_kernel(Args g) {
@@ -86,7 +90,8 @@ __global__ __launch_bounds__(256 * KS) void gemm_f32_dl_kernel(Args g) {
     const int split = blockIdx.y;
     const int kbeg = split * g.k_per_split;
     const int kend = min(g.K, kbeg + g.k_per_split);
-    const int KT = kend > kbeg ? (kend - kbeg) / BK : 0;
+    const int KT = kend > kbeg ? (kend - kbeg) / BK : 0;   // whole k-tiles
+    const int rem = kend > kbeg ? (kend - kbeg) % BK : 0;  // depth of a shorter last one (the last split's only)
 
     // ---- the wave's direct loads (instructions wave * n .. wave * n + n - 1 of an operand's loads) ----
     // per-lane global address for k-tile 0, LDS offset of the load's image inside the operand, bytes per k-tile
@@ -225,6 +230,43 @@ __global__ __launch_bounds__(256 * KS) void gemm_f32_dl_kernel(Args g) {
         else substep(pfb, qfb, pfa, qfa, nxt, std::integral_constant<int, 0>{}, requests);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the requests past the last k-tile
+    if (rem > 0) {
+        // The shorter last k-tile, outside the pipeline (one load latency per workgroup, once): the same direct loads
+        // into stage 0, lanes whose 16 bytes lie at k >= K reading zeros instead (in both operands, so the products
+        // vanish whatever follows the end of a row), then every substep of the wave's share out of one fragment set.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();  // nobody reads a stage any more
+        asm volatile("" ::: "memory");
+        auto below = [&](auto opc, auto modec, int inst) {
+            typedef typename decltype(opc)::type Op;
+            if constexpr (decltype(modec)::value == LD_K) {
+                const int row = inst * 8 + (lane >> 3);
+                return (((lane & 7) ^ (int)swz((uint32_t)row)) * 4) < rem;
+            } else {
+                return inst * Op::KRPI + lane / (64 / Op::KRPI) < rem;
+            }
+        };
+        static_for<LPW>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            if constexpr (l < LPWP) {
+                const bool in = below(std::common_type<OpP>{}, std::integral_constant<int, LP>{}, wave * LPWP + l);
+                direct_load16(in ? (const void *)(gp[l] + (int64_t)KT * stepP) : (const void *)kZeroChunkF32, smem_addr + lp[l]);
+            } else {
+                const bool in = below(std::common_type<OpQ>{}, std::integral_constant<int, LQ>{}, wave * LPWQ + (l - LPWP));
+                direct_load16(in ? (const void *)(gq[l - LPWP] + (int64_t)KT * stepQ) : (const void *)kZeroChunkF32,
+                              smem_addr + OpP::BYTES + lq[l - LPWP]);
+            }
+        });
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        static_for<SPW>([&](auto sc) {
+            static_for<NU>([&](auto uc) { read_unit(pfa, qfa, smem, sc, uc); });
+            static_for<SLOTS>([&](auto mc) {
+                constexpr int m = decltype(mc)::value, e = m / NM, n = m % NM, i = n / TQ, j = n % TQ;
+                Mma<T>::template part<e>(acc[i][j], pfa[i], qfa[j]);
+            });
+        });
+    }
     if constexpr (KS == 2) {
         // the second half's partial sums go to the first half through LDS: [tile][i][j][r][lane], 4 bytes each
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");

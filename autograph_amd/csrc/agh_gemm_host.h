@@ -105,12 +105,12 @@ template <typename T, int BP, int BQ, int WGP, int WGQ, bool SCALAR_OK>
 int launch_loaders(const Args &g, int splits, int lp, int lq, bool direct) {
 #ifdef AGH_GEMM_WITH_F32_DIRECT
     if constexpr (std::is_same<T, float>::value && BP % 64 == 0 && BQ % 64 == 0) {
-        // both operands vector-loadable and k (hence every split's range) a multiple of the 32-wide k-tile
+        // both operands vector-loadable (any k: a last k-tile shorter than 32 is loaded with zeros behind k = K)
         // (AGH_GEMM_DIRECT=0 forces the register-staged kernel).  64 x 64: a ring of four stages, one or two
         // workgroups per CU; 128 x 128: two stages (a k-tile is four times as long), two workgroups per CU; the
         // larger tiles: two stages, one workgroup per CU.
         constexpr int TPW = BP / 64, TQW = BQ / 64, NS = BP == 64 ? 4 : 2;
-        if (lp != LD_S && lq != LD_S && g.K > 0 && g.K % 32 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0) {
+        if (lp != LD_S && lq != LD_S && g.K > 0 && env_int("AGH_GEMM_DIRECT", 1) != 0) {
             switch (lp * 3 + lq) {
                 case LD_K * 3 + LD_K: return launch_f32_dl<TPW, TQW, NS, LD_K, LD_K>(g, splits);
                 case LD_K * 3 + LD_R: return launch_f32_dl<TPW, TQW, NS, LD_K, LD_R>(g, splits);
@@ -269,7 +269,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         // the 64 x 64 direct tile is measured at 0.8 of the 256 x 256 tile's rate per CU (3072^3: 118 TFLOP/s, where
         // 144 tiles of 256 x 256 leave 112 CUs idle)
         // f32: the 64 x 64 and 128 x 128 tiles have direct-to-LDS kernels (agh_gemm_f32_dl.h)
-        const bool f32_dl_ok = sizeof(T) == 4 && !any_scalar && g.K > 0 && g.K % 32 == 0 && env_int("AGH_GEMM_DIRECT", 1) != 0;
+        const bool f32_dl_ok = sizeof(T) == 4 && !any_scalar && g.K > 0 && env_int("AGH_GEMM_DIRECT", 1) != 0;
         const bool f32_direct = f32_dl_ok && t.bp == 64 && t.bq == 64;
         if (f32_direct) eff = 0.80;
         if (f32_dl_ok && t.bp == 128 && t.bq == 128) eff = 0.95;  // 4096^3: 135 TFLOP/s, the 256 x 256 tile's rate

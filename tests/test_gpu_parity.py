@@ -521,6 +521,51 @@ def test_gemm_bf16_last_k_tile_shorter_than_64(ag, monkeypatch):
     assert np.array_equal(got, orc.bf16_to_f32(orc.f32_to_bf16(exact.astype(np.float32))))
 
 
+def test_gemm_f32_last_k_tile_shorter_than_32(ag, monkeypatch):
+    """The f32 direct-to-LDS kernels with k not a multiple of their 32-deep k-tile: the last tile is loaded with zeros
+    behind k = K and multiplied after the pipelined loop.  k below one tile, whole tiles and a rest, all four layouts,
+    the 256 x 256, 128 x 128 and 64 x 64 tiles forced, eight waves sharing every k-tile forced on and off, odd k
+    (operands stored k-major), forced split-K (the last split alone has the shorter tile), integer data exactly."""
+    rng = np.random.default_rng(98)
+    cases = [(128, k, 128) for k in (4, 12, 28, 36, 60, 100, 1000)] + [(200, 44, 72), (72, 1028, 264)]
+    for (m, k, n) in cases:
+        for ta in (False, True):
+            for tb in (False, True):
+                a = rng.uniform(-1, 1, (k, m) if ta else (m, k)).astype(np.float32)
+                b = rng.uniform(-1, 1, (n, k) if tb else (k, n)).astype(np.float32)
+                A, B = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+                av, bv = (a.T if ta else a), (b.T if tb else b)
+                for cfg in (None, "0", "3", "4"):
+                    for ks in (None, "0", "1"):
+                        if cfg is None and ks is not None:
+                            continue
+                        if cfg is None:
+                            monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
+                        else:
+                            monkeypatch.setenv("AGH_GEMM_CFG", cfg)
+                        if ks is None:
+                            monkeypatch.delenv("AGH_GEMM_KSPLIT", raising=False)
+                        else:
+                            monkeypatch.setenv("AGH_GEMM_KSPLIT", ks)
+                        out = (A.t() if ta else A).dot(B.t() if tb else B).into_array()
+                        assert_f32_gemm_close(out, av, bv)
+    monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
+    monkeypatch.delenv("AGH_GEMM_KSPLIT", raising=False)
+    for (m, k, n) in ((96, 77, 200), (96, 3, 200), (104, 1001, 96)):
+        a = rng.uniform(-1, 1, (k, m)).astype(np.float32)
+        b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        assert_f32_gemm_close(ag.Tensor.from_array(a).t().dot(ag.Tensor.from_array(b)).into_array(), a.T, b)
+    a = rng.uniform(-1, 1, (136, 1000)).astype(np.float32)
+    b = rng.uniform(-1, 1, (1000, 128)).astype(np.float32)
+    for splits in ("3", "16"):
+        monkeypatch.setenv("AGH_GEMM_SPLITS", splits)
+        assert_f32_gemm_close(ag.Tensor.from_array(a).dot(ag.Tensor.from_array(b)).into_array(), a, b)
+    monkeypatch.delenv("AGH_GEMM_SPLITS")
+    ai = rng.integers(-8, 9, (136, 1012)).astype(np.float32)
+    bi = rng.integers(-8, 9, (1012, 264)).astype(np.float32)
+    assert np.array_equal(ag.Tensor.from_array(ai).dot(ag.Tensor.from_array(bi)).into_array(), ai @ bi)
+
+
 def test_gemm_f32_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
     """150 seeded f32 products with k a multiple of 32 (so that the direct-to-LDS kernels apply wherever the operands
     are vector-loadable), odd and even m and n, all four layouts, alpha and beta, each in the chooser's tile
