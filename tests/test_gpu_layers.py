@@ -350,3 +350,104 @@ def test_lenet5_forward_bf16(ag, bs):
         # every layer may differ from the oracle by one bf16 rounding; six layers compound
         assert np.abs(got - want).max() <= 0.05 * max(1.0, np.abs(want).max()), (name, np.abs(got - want).max())
         assert np.mean(np.abs(got - want)) <= 0.01 * max(1.0, np.abs(want).max()), name
+
+
+def test_random_geometry_im2col_col2im_pool(ag):
+    """200 seeded random geometries (filter 1..5 per axis, padding 0..2, stride 1..3, dilation 1..2, windows 1..3 with
+    equal or other strides, inputs up to 39 x 39, both element types, a third of the pooling inputs quantised so that
+    windows hold ties): im2col, col2im on a random patch matrix of the same geometry, MaxPool2 forward and backward,
+    each bit for bit against the oracle's host loops (src/tensor/ops.rs:842-1037, :1117-1264)."""
+    from autograph_amd.tensor import Col2ImConv2Options, Im2ColConv2Options, MaxPool2Options
+    rng = np.random.default_rng(2718)
+
+    def rnd(shape, dt):
+        x = rng.standard_normal(shape).astype(np.float32)
+        if rng.random() < 0.3:
+            x = np.round(x * 2) / 2
+        return to_dtype(x, dt)
+
+    done = 0
+    for _ in range(200):
+        dt = "bf16" if rng.random() < 0.5 else "f32"
+        bs, c = int(rng.integers(1, 5)), int(rng.integers(1, 20))
+        ih, iw = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        if rng.random() < 0.4:
+            iw = 8 * max(1, iw // 8)
+        fh, fw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        if rng.random() < 0.5:
+            fw = fh
+        pad = (int(rng.integers(0, 3)), int(rng.integers(0, 3)))
+        st = (1, 1) if rng.random() < 0.6 else (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        dl = (1, 1) if rng.random() < 0.7 else (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        tag = (dt, bs, c, ih, iw, fh, fw, pad, st, dl)
+        if ih + 2 * pad[0] >= dl[0] * (fh - 1) + 1 and iw + 2 * pad[1] >= dl[1] * (fw - 1) + 1:
+            oh, ow = orc.conv_out(ih, fh, pad[0], st[0], dl[0]), orc.conv_out(iw, fw, pad[1], st[1], dl[1])
+            x = rnd((bs, c, ih, iw), dt)
+            got = ag.Tensor.from_array(x).im2col_conv2(Im2ColConv2Options((fh, fw), pad, st, dl)).into_array()
+            assert np.array_equal(got, orc.im2col_conv2(x, (fh, fw), pad, st, dl)), tag
+            o2h, o2w = orc.col2im_out(oh, fh, pad[0], st[0], dl[0]), orc.col2im_out(ow, fw, pad[1], st[1], dl[1])
+            if o2h >= 1 and o2w >= 1:
+                cols = rnd((bs * oh * ow, c * fh * fw), dt)
+                got = ag.Tensor.from_array(cols).col2im_conv2(Col2ImConv2Options((oh, ow), (fh, fw), pad, st, dl)).into_array()
+                assert np.array_equal(got, orc.col2im_conv2(cols, (oh, ow), (fh, fw), pad, st, dl)), tag
+            done += 1
+        kh, kw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        ps = (kh, kw) if rng.random() < 0.6 else (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        if ih >= kh and iw >= kw:
+            x = rnd((bs, c, ih, iw), dt)
+            want = orc.max_pool2(x, (kh, kw), ps)
+            assert np.array_equal(ag.Tensor.from_array(x).max_pool2(MaxPool2Options((kh, kw), ps)).into_array(), want), (tag, kh, kw, ps)
+            dy = rnd(want.shape, dt)
+            tb = ag.Tensor.from_array(x)
+            tb.max_pool2_backward(ag.Tensor.from_array(dy), MaxPool2Options((kh, kw), ps))
+            assert np.array_equal(tb.into_array(), orc.max_pool2_backward(x, dy, (kh, kw), ps)), (tag, kh, kw, ps)
+    assert done >= 150
+
+
+def test_random_geometry_conv2_forward(ag):
+    """80 seeded random convolutions, more than half of them shaped for the matrix-core kernel (16..64 input channels, 64
+    or 128 output channels, rows of whole vectors, unit stride), the rest small with strides and dilations: both
+    algorithms against the naive f64 convolution (f32: 1e-5 sqrt(K); bf16: 1 ulp + 1e-2 relative + a floor where the
+    sum cancels), and bias + ReLU bit-identical to the separate ops on that very result (layer.rs:950-1005)."""
+    rng = np.random.default_rng(31415)
+    direct = 0
+    for _ in range(80):
+        dt = "bf16" if rng.random() < 0.5 else "f32"
+        if rng.random() < 0.6:
+            bs, ic, oc = int(rng.integers(1, 4)), 16 * int(rng.integers(1, 5)), 64 * int(rng.integers(1, 3))
+            ih, iw = int(rng.integers(6, 40)), 8 * int(rng.integers(2, 6))
+            st = dl = (1, 1)
+        else:
+            bs, ic, oc = int(rng.integers(1, 4)), int(rng.integers(1, 9)), int(rng.integers(1, 20))
+            ih, iw = int(rng.integers(4, 30)), int(rng.integers(4, 30))
+            st = (1, 1) if rng.random() < 0.6 else (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+            dl = (1, 1) if rng.random() < 0.8 else (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        fh, fw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        pad = (int(rng.integers(0, 3)), int(rng.integers(0, 3)))
+        if ih + 2 * pad[0] < dl[0] * (fh - 1) + 1 or iw + 2 * pad[1] < dl[1] * (fw - 1) + 1:
+            continue
+        x = to_dtype(rng.standard_normal((bs, ic, ih, iw)), dt)
+        w = to_dtype(rng.standard_normal((oc, ic, fh, fw)) * np.sqrt(2.0 / (ic * fh * fw)), dt)
+        b = to_dtype(rng.standard_normal(oc), dt)
+        want = orc.conv2_naive_f64(as_f32(x), as_f32(w), pad, st, dl)
+        tag = (dt, bs, ic, ih, iw, oc, fh, fw, pad, st, dl)
+        tx, tw, tb = ag.Tensor.from_array(x), ag.Tensor.from_array(w), ag.Tensor.from_array(b)
+        scale = max(np.abs(want).max(), 1e-6)
+        for alg in ("im2col", "direct"):
+            fn = ag.conv2_im2col_forward if alg == "im2col" else ag.conv2_direct_forward
+            try:
+                y = fn(tx, tw, padding=pad, stride=st, dilation=dl).into_array()
+                yb = fn(tx, tw, padding=pad, stride=st, dilation=dl, bias=tb, relu=True).into_array()
+            except ag.AghError as e:
+                assert alg == "direct" and e.code == -4, (alg, tag)   # the layer does not fit the direct kernels
+                continue
+            direct += alg == "direct"
+            yf = as_f32(y).astype(np.float64)
+            if dt == "f32":
+                assert np.abs(yf - want).max() <= 1e-5 * np.sqrt(ic * fh * fw) * scale, (alg, tag)
+                assert np.array_equal(yb, np.maximum(y + b[None, :, None, None], 0.0)), (alg, tag)
+            else:
+                assert np.all(np.abs(yf - want) <= 2.0**-7 * np.abs(want) + 1e-2 * np.abs(want) + 2e-3 * scale), (alg, tag)
+                s1 = orc.f32_to_bf16(as_f32(y) + as_f32(b)[None, :, None, None])
+                assert np.array_equal(as_f32(yb), np.maximum(as_f32(s1), 0.0)), (alg, tag)
+    assert direct >= 30
