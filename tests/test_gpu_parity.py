@@ -158,6 +158,69 @@ def test_gemm_strides_offsets_alpha_beta(ag, dtype):
                 assert np.all(np.abs(gotf - want) <= bf16_ulp(want) + 1e-2 * np.abs(want) + 1e-5 * absprod)
 
 
+def test_gemm_random_views(ag):
+    """150 seeded products over random views of larger buffers, as `fn gemm` receives them (linalg.rs:281-299): row and
+    column steps of 1 to 3 elements, either sign, transposed or not, any offset, for A, B and C independently, both
+    element types, alpha in {1, 0.5, -1.25} and beta in {0, 1, 2}.  The result against the f64 product under the
+    element type's bound, and every element of C's buffer outside the view unchanged."""
+    rng = np.random.default_rng(1618)
+
+    def rand_view(big, r, c):
+        rows, cols = big.shape
+        for _ in range(100):
+            tr = rng.random() < 0.5
+            rr, cc = (c, r) if tr else (r, c)
+            sr, sc = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+            if (rr - 1) * sr + 1 > rows or (cc - 1) * sc + 1 > cols:
+                continue
+            r0, c0 = int(rng.integers(0, rows - (rr - 1) * sr)), int(rng.integers(0, cols - (cc - 1) * sc))
+            v = big[r0:r0 + (rr - 1) * sr + 1:sr, c0:c0 + (cc - 1) * sc + 1:sc]
+            if rng.random() < 0.3:
+                v = v[::-1]
+            if rng.random() < 0.3:
+                v = v[:, ::-1]
+            return v.T if tr else v
+        return None
+
+    done = 0
+    for _ in range(150):
+        dtype = "bf16" if rng.random() < 0.5 else "f32"
+        m, k, n = int(rng.integers(1, 150)), int(rng.integers(1, 200)), int(rng.integers(1, 150))
+        if rng.random() < 0.4:
+            m, k, n = 8 * max(1, m // 8), 8 * max(1, k // 8), 8 * max(1, n // 8)
+        big_a = to_dtype(rng.uniform(-1, 1, (460, 620)), dtype)
+        big_b = to_dtype(rng.uniform(-1, 1, (620, 460)), dtype)
+        big_c = to_dtype(rng.uniform(-1, 1, (460, 460)), dtype)
+        av, bv, cv = rand_view(big_a, m, k), rand_view(big_b, k, n), rand_view(big_c, m, n)
+        if av is None or bv is None or cv is None:
+            continue
+        alpha, beta = float(rng.choice([1.0, 0.5, -1.25])), float(rng.choice([0.0, 0.0, 1.0, 2.0]))
+        ta, tb, tc = ag.Tensor.from_array(big_a), ag.Tensor.from_array(big_b), ag.Tensor.from_array(big_c)
+
+        def view(t, v):
+            _, off, rs, cs = orc._view(v)
+            return ag.Tensor(t.buffer, v.shape, (rs, cs), off, t.dtype)
+
+        ag.gemm(alpha, view(ta, av), view(tb, bv), beta, view(tc, cv))
+        full = tc.into_array().reshape(-1)
+        _, off, rs, cs = orc._view(cv)
+        idx = off + np.arange(m)[:, None] * rs + np.arange(n)[None, :] * cs
+        mask = np.ones(big_c.size, bool)
+        mask[idx.reshape(-1)] = False
+        tag = (dtype, m, k, n, orc._view(av)[1:], orc._view(bv)[1:], orc._view(cv)[1:], alpha, beta)
+        assert np.array_equal(full[mask], big_c.reshape(-1)[mask]), tag
+        want = orc.gemm_f64acc(av, bv, alpha, beta, cv)
+        f64 = lambda v: as_f32(np.ascontiguousarray(v)).astype(np.float64)  # noqa: E731
+        absprod = abs(alpha) * (np.abs(f64(av)) @ np.abs(f64(bv))) + abs(beta) * np.abs(f64(cv))
+        got = f64(full[idx])
+        if dtype == "f32":
+            assert np.all(np.abs(got - want) <= 1e-5 * np.sqrt(k) * absprod + 1e-30), tag
+        else:
+            assert np.all(np.abs(got - want) <= bf16_ulp(want) + 1e-2 * np.abs(want) + 1e-5 * absprod), tag
+        done += 1
+    assert done >= 120
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_gemm_beta_zero_never_reads_c_and_k_zero(ag, dtype):
     rng = np.random.default_rng(12)
