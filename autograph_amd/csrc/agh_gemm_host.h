@@ -65,7 +65,10 @@ template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
 int launch_dl_ring(const Args &g, int splits) {
     if constexpr (BP == 128 && BQ == 128) {
         const int64_t wgs = (int64_t)g.tiles_p * g.tiles_q * splits * g.batch;
-        const bool alone = wgs <= (compute_units() > 0 ? compute_units() : 256) && g.k_per_split >= 20 * 64;
+        // split-K streams its operands from HBM once (no second workgroup re-reads them out of L2), where the deeper
+        // ring pays from 8 k-tiles on (128x4096x4096 in 8 splits: 19.5 against 20.5 us; in 4: 17.2 against 20.1)
+        const bool alone = wgs <= (compute_units() > 0 ? compute_units() : 256) &&
+                           (g.k_per_split >= 20 * 64 || (splits > 1 && g.k_per_split >= 8 * 64));
         if (env_int("AGH_GEMM_RING", alone ? 4 : 2) == 4)
             return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, 4>(g, splits);
     }
@@ -324,7 +327,10 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     const int ktiles = (g.K + BK - 1) / BK;
     if (tiles * 2 <= slots && ktiles >= 32 && batch == 1) {
         int64_t s = slots / tiles;
-        if (s > ktiles / 4) s = ktiles / 4;
+        // at least four k-tiles a split; twelve for the bf16 128 x 128 direct tile, whose four-stage ring makes fewer,
+        // longer splits the better trade (128x4096x4096: 17.0-17.2 us in 4 to 6 splits, 19.5 in 8)
+        const int kmin = direct_ok && best == 3 ? 12 : 4;
+        if (s > ktiles / kmin) s = ktiles / kmin;
         if (s > 256) s = 256;
         if (s > 1) splits = (int)s;
     }
