@@ -35,6 +35,7 @@ SIGNATURES = {
     "agh_free": ([ptr], C.c_int),
     "agh_cache_release": ([], C.c_int),
     "agh_cache_stats": ([C.POINTER(C.c_size_t)] * 3, C.c_int),
+    "agh_workspace_stats": ([C.POINTER(C.c_size_t)] * 2, C.c_int),
     "agh_memcpy_h2d": ([ptr, ptr, C.c_size_t], C.c_int),
     "agh_memcpy_d2h": ([ptr, ptr, C.c_size_t], C.c_int),
     "agh_memcpy_d2d": ([ptr, ptr, C.c_size_t], C.c_int),
@@ -55,11 +56,6 @@ SIGNATURES = {
     "agh_event_destroy": ([ptr], C.c_int),
     "agh_event_record": ([ptr], C.c_int),
     "agh_event_elapsed_ms": ([ptr, ptr, C.POINTER(f32)], C.c_int),
-    "agh_calib_mfma_bf16": ([ptr, C.c_int, C.c_int, C.c_int, C.c_int], C.c_int),
-    "agh_calib_copy": ([ptr, ptr, C.c_size_t, C.c_int], C.c_int),
-    "agh_calib_read": ([ptr, ptr, C.c_size_t, C.c_int], C.c_int),
-    "agh_calib_mix": ([ptr, ptr, C.c_size_t, C.c_int, C.c_int], C.c_int),
-    "agh_calib_mfma_dma": ([ptr, C.c_size_t, ptr, C.c_int, C.c_size_t, C.c_int, C.c_int], C.c_int),
     "agh_gemm_f32": (_GEMM, C.c_int),
     "agh_gemm_bf16": (_GEMM, C.c_int),
     "agh_gemm_bf16_noalloc": (_GEMM, C.c_int),
@@ -101,6 +97,8 @@ SIGNATURES = {
     "agh_assign_bf16": ([ptr] + [i64] * 5 + [ptr] + [i64] * 9, C.c_int),
     "agh_scaled_add_f32": ([ptr, f32, ptr, i64], C.c_int),
     "agh_scaled_add_bf16": ([ptr, f32, ptr, i64], C.c_int),
+    "agh_scaled_add_strided_f32": ([ptr] + [i64] * 5 + [f32, ptr] + [i64] * 9, C.c_int),
+    "agh_scaled_add_strided_bf16": ([ptr] + [i64] * 5 + [f32, ptr] + [i64] * 9, C.c_int),
     "agh_sgd_momentum_f32": ([ptr, ptr, f32, f32, ptr, i64], C.c_int),
     "agh_sgd_momentum_bf16": ([ptr, ptr, f32, f32, ptr, i64], C.c_int),
     "agh_sum_axis0_f32": ([ptr, ptr, i64, i64], C.c_int),
@@ -109,6 +107,8 @@ SIGNATURES = {
     "agh_cross_entropy_loss_bf16": ([ptr, ptr, i64, i64, ptr], C.c_int),
     "agh_cross_entropy_backward_f32": ([ptr, ptr, f32, ptr, i64, i64], C.c_int),
     "agh_cross_entropy_backward_bf16": ([ptr, ptr, f32, ptr, i64, i64], C.c_int),
+    "agh_accuracy_f32": ([ptr, ptr, i64, i64, ptr], C.c_int),
+    "agh_accuracy_bf16": ([ptr, ptr, i64, i64, ptr], C.c_int),
 }
 
 for _name, (_args, _res) in SIGNATURES.items():

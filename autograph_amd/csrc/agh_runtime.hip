@@ -29,9 +29,11 @@ static hipStream_t g_stream = nullptr;
 static hipStream_t g_side = nullptr;
 static hipStream_t g_cur = nullptr;
 static bool g_side_dirty = false;  // the branch stream has work the main stream has not waited for
+// Fork / join events.  Eager work and a capture in progress draw from separate rings, so an event that a captured
+// graph's edges were built from is never re-recorded by eager work (and the other way round).
 constexpr int kBranchEvents = 64;
-static hipEvent_t g_events[kBranchEvents];
-static int g_event_next = 0;
+static hipEvent_t g_events[kBranchEvents], g_capture_events[kBranchEvents];
+static int g_event_next = 0, g_capture_event_next = 0;
 static bool g_capturing = false;   // between agh_graph_begin and agh_graph_end
 static int g_live_graphs = 0;      // graph executables not yet destroyed: their nodes hold workspace pointers
 static void *g_scratch_ptr = nullptr;  // device address of `scratch` on g_device
@@ -60,6 +62,13 @@ struct CachedBlock {
 static std::multimap<size_t, CachedBlock> g_free_blocks;     // by capacity
 static std::unordered_map<void *, size_t> g_live_blocks;     // capacity of every block handed out
 static size_t g_cached_bytes = 0, g_cache_limit = (size_t)64 << 30;
+// Blocks freed while a graph is being captured: they can neither be handed to the driver nor (their capacity class
+// being taken by agh_malloc, which a capture refuses anyway) reused before the capture ends; agh_graph_end files them.
+struct DeferredFree {
+    void *ptr;
+    size_t cap;  // 0: not from this allocator's books, goes back to the driver
+};
+static std::vector<DeferredFree> g_deferred_frees;
 static uint64_t g_side_seq = 0, g_side_joined_seq = 0;
 
 std::recursive_mutex &api_mutex() { return g_mutex; }
@@ -126,6 +135,11 @@ int static_workspace(size_t bytes, void **ptr) {
 }
 
 static hipEvent_t next_event() {
+    if (g_capturing) {
+        hipEvent_t e = g_capture_events[g_capture_event_next];
+        g_capture_event_next = (g_capture_event_next + 1) % kBranchEvents;
+        return e;
+    }
     hipEvent_t e = g_events[g_event_next];
     g_event_next = (g_event_next + 1) % kBranchEvents;
     return e;
@@ -170,6 +184,24 @@ static int release_cached_blocks() {
     return AGH_OK;
 }
 
+// Files the blocks that were freed during a capture (called once the capture has ended, successfully or not).
+static int flush_deferred_frees() {
+    std::vector<DeferredFree> todo;
+    todo.swap(g_deferred_frees);
+    for (const DeferredFree &d : todo) {
+        if (d.cap == 0 || d.cap > g_cache_limit) {
+            if (int rc = sync_all()) return rc;
+            AGH_HIP(hipFree(d.ptr));
+            continue;
+        }
+        if (g_cached_bytes + d.cap > g_cache_limit)
+            if (int rc = release_cached_blocks()) return rc;
+        g_free_blocks.emplace(d.cap, CachedBlock{d.ptr, g_side_dirty ? g_side_seq : 0});
+        g_cached_bytes += d.cap;
+    }
+    return AGH_OK;
+}
+
 }  // namespace agh
 
 using namespace agh;
@@ -196,7 +228,10 @@ int agh_init(int device_index) {
     g_cus = prop.multiProcessorCount;
     AGH_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     AGH_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));  // default priority, like g_stream
-    for (int i = 0; i < kBranchEvents; ++i) AGH_HIP(hipEventCreateWithFlags(&g_events[i], hipEventDisableTiming));
+    for (int i = 0; i < kBranchEvents; ++i) {
+        AGH_HIP(hipEventCreateWithFlags(&g_events[i], hipEventDisableTiming));
+        AGH_HIP(hipEventCreateWithFlags(&g_capture_events[i], hipEventDisableTiming));
+    }
     // this device's copy of the fixed scratch array (the device is current)
     g_scratch_ptr = nullptr;
     AGH_HIP(hipGetSymbolAddress(&g_scratch_ptr, HIP_SYMBOL(scratch)));
@@ -227,7 +262,10 @@ int agh_shutdown(void) {
     g_ws = Workspace();
     g_ws_side = Workspace();
     if (int rc = release_retired_workspaces()) return rc;
-    for (int i = 0; i < kBranchEvents; ++i) (void)hipEventDestroy(g_events[i]);
+    for (int i = 0; i < kBranchEvents; ++i) {
+        (void)hipEventDestroy(g_events[i]);
+        (void)hipEventDestroy(g_capture_events[i]);
+    }
     AGH_HIP(hipStreamDestroy(g_side));
     AGH_HIP(hipStreamDestroy(g_stream));
     g_stream = g_side = g_cur = nullptr;
@@ -287,8 +325,18 @@ int agh_malloc(void **ptr, size_t bytes) {
 int agh_free(void *ptr) {
     AGH_API_ENTER();
     if (!ptr) return AGH_OK;
-    if (g_capturing) return fail(AGH_EINVAL, "agh_free: not allowed while capturing a graph");
     auto it = g_live_blocks.find(ptr);
+    if (g_capturing) {
+        // No wait, no driver call and no reuse inside a capture: the block is set aside and filed by agh_graph_end.
+        // (Typical case: a host-side temporary dropped by the garbage collector while a step is being recorded.)
+        if (it == g_live_blocks.end()) {
+            g_deferred_frees.push_back(DeferredFree{ptr, 0});
+        } else {
+            g_deferred_frees.push_back(DeferredFree{ptr, it->second});
+            g_live_blocks.erase(it);
+        }
+        return AGH_OK;
+    }
     if (it == g_live_blocks.end()) {
         // not from this allocator's books (allocated before an agh_shutdown): hand it to the driver
         if (int rc = sync_all()) return rc;
@@ -329,6 +377,13 @@ int agh_cache_stats(size_t *cached_bytes, size_t *cached_blocks, size_t *live_bl
     if (cached_bytes) *cached_bytes = g_cached_bytes;
     if (cached_blocks) *cached_blocks = g_free_blocks.size();
     if (live_blocks) *live_blocks = g_live_blocks.size();
+    return AGH_OK;
+}
+
+int agh_workspace_stats(size_t *workspace_bytes, size_t *retired_blocks) {
+    AGH_API_ENTER();
+    if (workspace_bytes) *workspace_bytes = g_ws.bytes + g_ws_side.bytes;
+    if (retired_blocks) *retired_blocks = g_ws_retired.size();
     return AGH_OK;
 }
 
@@ -411,22 +466,35 @@ int agh_graph_end(void **graph_exec) {
         g_capturing = false;
         (void)hipStreamEndCapture(g_stream, &graph);
         if (graph) (void)hipGraphDestroy(graph);
+        (void)flush_deferred_frees();
         return rc;
     }
     g_capturing = false;
-    AGH_HIP(hipStreamEndCapture(g_stream, &graph));
+    const hipError_t ec = hipStreamEndCapture(g_stream, &graph);
+    if (ec != hipSuccess) {
+        (void)flush_deferred_frees();
+        return hip_fail(ec, "hipStreamEndCapture");
+    }
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
-    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    if (e != hipSuccess) {
+        (void)flush_deferred_frees();
+        return hip_fail(e, "hipGraphInstantiate");
+    }
     ++g_live_graphs;
     *graph_exec = (void *)exec;
-    return AGH_OK;
+    return flush_deferred_frees();
 }
 
 int agh_graph_launch(void *graph_exec) {
     AGH_API_ENTER();
     if (!graph_exec) return fail(AGH_ENULL, "agh_graph_launch: null graph");
+    if (g_capturing) return fail(AGH_EINVAL, "agh_graph_launch: not allowed while capturing a graph");
+    if (g_cur != g_stream) return fail(AGH_EINVAL, "agh_graph_launch: inside a branch");
+    // A graph captured with a branch names the branch stream's workspace in its fork arm; eager branch work that has
+    // not been joined may still be using that block, so the replay is ordered behind it.
+    if (int rc = join_side()) return rc;
     AGH_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, g_stream));
     return AGH_OK;
 }

@@ -194,6 +194,48 @@ __global__ __launch_bounds__(kThreads) void scaled_add_kernel(T *__restrict__ y,
     }
 }
 
+// The same operation on views: index space [d0, d1, d2, d3] walked with d3 fastest, signed element strides, a
+// stride 0 on x broadcasts.  VEC > 1: d3 is walked in groups of VEC elements that are contiguous in y (sy3 == 1)
+// and either contiguous (sx3 == 1) or one broadcast element (sx3 == 0) in x; groups are 16-byte loads and stores.
+struct ScaledAddParams {
+    int64_t sx[4], sy[4];
+    FastDiv div1, div2, div3;  // by d1*d2*g3, d2*g3, g3 with g3 = d3 / VEC
+};
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kThreads) void scaled_add_strided_kernel(T *__restrict__ y, float alpha, const T *__restrict__ x,
+                                                                       ScaledAddParams p, uint32_t total) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const float a = Elem<T>::to_f32(Elem<T>::from_f32(alpha));
+    for (uint32_t e = blockIdx.x * kThreads + threadIdx.x; e < total; e += gridDim.x * kThreads) {
+        uint32_t i0, r0, i1, r1, i2, i3;
+        p.div1.divmod(e, i0, r0);
+        p.div2.divmod(r0, i1, r1);
+        p.div3.divmod(r1, i2, i3);
+        const int64_t ix = i0 * p.sx[0] + i1 * p.sx[1] + i2 * p.sx[2] + (int64_t)(i3 * VEC) * p.sx[3];
+        const int64_t iy = i0 * p.sy[0] + i1 * p.sy[1] + i2 * p.sy[2] + (int64_t)(i3 * VEC) * p.sy[3];
+        if constexpr (VEC == 1) {
+            const T prod = Elem<T>::from_f32(a * Elem<T>::to_f32(x[ix]));
+            y[iy] = Elem<T>::from_f32(Elem<T>::to_f32(prod) + Elem<T>::to_f32(y[iy]));
+        } else {
+            T xv[VEC], yv[VEC];
+            *(u32x4 *)yv = *(const u32x4 *)(y + iy);
+            if (p.sx[3] != 0) *(u32x4 *)xv = *(const u32x4 *)(x + ix);
+            else {
+                const T b = x[ix];
+#pragma unroll
+                for (int u = 0; u < VEC; ++u) xv[u] = b;
+            }
+#pragma unroll
+            for (int u = 0; u < VEC; ++u) {
+                const T prod = Elem<T>::from_f32(a * Elem<T>::to_f32(xv[u]));
+                yv[u] = Elem<T>::from_f32(Elem<T>::to_f32(prod) + Elem<T>::to_f32(yv[u]));
+            }
+            *(u32x4 *)(y + iy) = *(const u32x4 *)yv;
+        }
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kThreads) void sgd_momentum_kernel(T *__restrict__ w, const T *__restrict__ dw, float lr, float m,
                                                                  T *__restrict__ v, size_t n) {
@@ -278,6 +320,50 @@ __global__ __launch_bounds__(kThreads) void cross_entropy_backward_kernel(const 
     }
 }
 
+// ---------------------------------------------------------------- accuracy ----
+// One thread per row: the prediction counts when the target's score is strictly greater than every other score of the
+// row (a tie, a NaN or a target >= classes does not count).  Every workgroup adds up its rows' flags in LDS and
+// writes one count: straight to `out` when the grid is a single workgroup, else to its slot of `partial`, which
+// accuracy_sum_kernel adds up.  No atomics, so `out` may be pinned host memory.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void accuracy_kernel(const T *__restrict__ x, const uint8_t *__restrict__ t, int64_t bs,
+                                                             int classes, uint32_t *__restrict__ partial, uint32_t *__restrict__ out) {
+    __shared__ uint32_t cnt[kThreads / 64];
+    uint32_t mine = 0;
+    for (int64_t r = (int64_t)blockIdx.x * kThreads + threadIdx.x; r < bs; r += (int64_t)gridDim.x * kThreads) {
+        const int tr = t[r];
+        if (tr >= classes) continue;
+        const T *row = x + r * classes;
+        const float xt = Elem<T>::raw(row[tr]);
+        bool ok = true;
+        for (int j = 0; j < classes; ++j) ok = ok && (j == tr || xt > Elem<T>::raw(row[j]));
+        mine += ok ? 1u : 0u;
+    }
+    for (int off = 32; off > 0; off >>= 1) mine += __shfl_down(mine, off, 64);
+    if ((threadIdx.x & 63) == 0) cnt[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t s = 0;
+        for (int w = 0; w < kThreads / 64; ++w) s += cnt[w];
+        if (gridDim.x == 1) *out = s;
+        else partial[blockIdx.x] = s;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void accuracy_sum_kernel(const uint32_t *__restrict__ partial, int n, uint32_t *__restrict__ out) {
+    __shared__ uint32_t cnt[kThreads / 64];
+    uint32_t mine = 0;
+    for (int i = threadIdx.x; i < n; i += kThreads) mine += partial[i];
+    for (int off = 32; off > 0; off >>= 1) mine += __shfl_down(mine, off, 64);
+    if ((threadIdx.x & 63) == 0) cnt[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t s = 0;
+        for (int w = 0; w < kThreads / 64; ++w) s += cnt[w];
+        *out = s;
+    }
+}
+
 template <typename T>
 int scaled_add_launch(const char *name, void *y, float alpha, const void *x, int64_t n) {
     AGH_API_ENTER();
@@ -287,6 +373,71 @@ int scaled_add_launch(const char *name, void *y, float alpha, const void *x, int
     hipLaunchKernelGGL(scaled_add_kernel<T>, dim3(grid_for((size_t)n)), dim3(kThreads), 0, stream(), (T *)y,
                        alpha, (const T *)x, (size_t)n);
     AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+template <typename T>
+int scaled_add_strided_launch(const char *name, void *y, int64_t off_y, const int64_t (&sy)[4], float alpha, const void *x,
+                              int64_t off_x, const int64_t (&sx)[4], const int64_t (&d)[4]) {
+    AGH_API_ENTER();
+    int64_t total = 1;
+    for (int i = 0; i < 4; ++i) {
+        if (d[i] < 0) return fail(AGH_EINVAL, "%s: negative dimension", name);
+        if (d[i] > ((int64_t)1 << 30)) return fail(AGH_ERANGE, "%s: dimension too large", name);
+        total *= d[i];
+        if (total > ((int64_t)1 << 31) - 1) return fail(AGH_ERANGE, "%s: more than 2^31-1 elements", name);
+    }
+    if (total == 0) return AGH_OK;
+    if (!x || !y) return fail(AGH_ENULL, "%s: null buffer", name);
+    for (int i = 0; i < 4; ++i)
+        if (d[i] > 1 && sy[i] == 0) return fail(AGH_EINVAL, "%s: the destination cannot be a broadcast view (stride 0 along dimension %d)", name, i);
+    const T *xp = (const T *)x + off_x;
+    T *yp = (T *)y + off_y;
+    constexpr int V = 16 / (int)sizeof(T);
+    auto mult = [](int64_t v) { return v % V == 0; };
+    // 16-byte groups along d3: y contiguous there, x contiguous or broadcast, every other step a whole number of groups
+    bool vec = d[3] % V == 0 && sy[3] == 1 && (sx[3] == 1 || sx[3] == 0) && ((uintptr_t)yp & 15) == 0;
+    for (int i = 0; i < 3 && vec; ++i) vec = d[i] == 1 || (mult(sy[i]) && (sx[3] == 0 || mult(sx[i])));
+    if (vec && sx[3] == 1) vec = ((uintptr_t)xp & 15) == 0;
+    const int64_t g3 = vec ? d[3] / V : d[3];
+    ScaledAddParams p;
+    for (int i = 0; i < 4; ++i) { p.sx[i] = sx[i]; p.sy[i] = sy[i]; }
+    p.div1 = FastDiv((uint32_t)(d[1] * d[2] * g3));
+    p.div2 = FastDiv((uint32_t)(d[2] * g3));
+    p.div3 = FastDiv((uint32_t)g3);
+    const uint32_t items = (uint32_t)(total / d[3] * g3);
+    if (vec)
+        hipLaunchKernelGGL((scaled_add_strided_kernel<T, V>), dim3(grid_for(items)), dim3(kThreads), 0, stream(), yp, alpha, xp, p, items);
+    else
+        hipLaunchKernelGGL((scaled_add_strided_kernel<T, 1>), dim3(grid_for(items)), dim3(kThreads), 0, stream(), yp, alpha, xp, p, items);
+    AGH_LAUNCH_CHECK(name);
+    return AGH_OK;
+}
+
+template <typename T>
+int accuracy_launch(const char *name, const void *x, const void *t, int64_t bs, int64_t classes, void *correct_out) {
+    uint32_t *correct = (uint32_t *)correct_out;
+    AGH_API_ENTER();
+    if (bs < 0 || classes < 1) return fail(AGH_EINVAL, "%s: invalid shape", name);
+    if (classes > 256) return fail(AGH_ERANGE, "%s: targets are u8, at most 256 classes", name);
+    if (!correct) return fail(AGH_ENULL, "%s: null output", name);
+    if (bs > 0 && (!x || !t)) return fail(AGH_ENULL, "%s: null buffer", name);
+    int64_t blocks = (bs + kThreads - 1) / kThreads;
+    if (blocks < 1) blocks = 1;
+    if (blocks > 1024) blocks = 1024;
+    uint32_t *partial = nullptr;
+    if (blocks > 1) {
+        void *ws = nullptr;
+        if (int rc = workspace((size_t)blocks * sizeof(uint32_t), &ws)) return rc;
+        partial = (uint32_t *)ws;
+    }
+    hipLaunchKernelGGL(accuracy_kernel<T>, dim3((unsigned)blocks), dim3(kThreads), 0, stream(), (const T *)x, (const uint8_t *)t, bs,
+                       (int)classes, partial, correct);
+    AGH_LAUNCH_CHECK(name);
+    if (blocks > 1) {
+        hipLaunchKernelGGL(accuracy_sum_kernel, dim3(1), dim3(kThreads), 0, stream(), partial, (int)blocks, correct);
+        AGH_LAUNCH_CHECK(name);
+    }
     return AGH_OK;
 }
 
@@ -371,6 +522,25 @@ int agh_scaled_add_f32(void *y, float alpha, const void *x, int64_t n) {
 }
 int agh_scaled_add_bf16(void *y, float alpha, const void *x, int64_t n) {
     return scaled_add_launch<uint16_t>("agh_scaled_add_bf16", y, alpha, x, n);
+}
+
+#define AGH_SCALED_ADD_STRIDED_ARGS                                                                              \
+    void *y, int64_t off_y, int64_t sy0, int64_t sy1, int64_t sy2, int64_t sy3, float alpha, const void *x,     \
+        int64_t off_x, int64_t sx0, int64_t sx1, int64_t sx2, int64_t sx3, int64_t d0, int64_t d1, int64_t d2, int64_t d3
+int agh_scaled_add_strided_f32(AGH_SCALED_ADD_STRIDED_ARGS) {
+    const int64_t sx[4] = {sx0, sx1, sx2, sx3}, sy[4] = {sy0, sy1, sy2, sy3}, d[4] = {d0, d1, d2, d3};
+    return scaled_add_strided_launch<float>("agh_scaled_add_strided_f32", y, off_y, sy, alpha, x, off_x, sx, d);
+}
+int agh_scaled_add_strided_bf16(AGH_SCALED_ADD_STRIDED_ARGS) {
+    const int64_t sx[4] = {sx0, sx1, sx2, sx3}, sy[4] = {sy0, sy1, sy2, sy3}, d[4] = {d0, d1, d2, d3};
+    return scaled_add_strided_launch<uint16_t>("agh_scaled_add_strided_bf16", y, off_y, sy, alpha, x, off_x, sx, d);
+}
+
+int agh_accuracy_f32(const void *x, const void *target_u8, int64_t bs, int64_t classes, void *correct) {
+    return accuracy_launch<float>("agh_accuracy_f32", x, target_u8, bs, classes, correct);
+}
+int agh_accuracy_bf16(const void *x, const void *target_u8, int64_t bs, int64_t classes, void *correct) {
+    return accuracy_launch<uint16_t>("agh_accuracy_bf16", x, target_u8, bs, classes, correct);
 }
 
 int agh_sgd_momentum_f32(void *w, const void *dw, float learning_rate, float momentum, void *velocity, int64_t n) {

@@ -152,8 +152,16 @@ class Dense:
         self.weight, self.bias = weight, bias
         self.weight_state = self.bias_state = None  # OptimizerState of each parameter (autograd.rs:655)
 
-    def forward(self, x, relu=False):
-        return x.dot(self.weight, bias=self.bias, relu=relu)
+    def forward(self, x, relu=False, fused=True):
+        """`Dense::forward` (layer.rs:1134-1143): `input.dot(&weight)` then `output.add_assign(&bias)`, and the Relu
+        layer behind it when `relu`.  fused (default): one launch, bias and relu in the GEMM epilogue; fused=False runs
+        the reference's separate calls (dot, broadcast add_assign, relu), bit-identical to the fused launch."""
+        if fused:
+            return x.dot(self.weight, bias=self.bias, relu=relu)
+        out = x.dot(self.weight)
+        if self.bias is not None:
+            out.add_assign(self.bias)
+        return out.relu() if relu else out
 
     def to_json(self):
         import json

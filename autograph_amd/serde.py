@@ -158,7 +158,8 @@ def optim_state_to_value(state):
 
 
 def optim_state_from_value(obj):
-    if not isinstance(obj, dict) or set(obj) != {"name", "key_values"} or not isinstance(obj["name"], str) \
+    # the derives set no `deny_unknown_fields`: keys they do not know are skipped, like serde's derive skips them
+    if not isinstance(obj, dict) or not {"name", "key_values"} <= set(obj) or not isinstance(obj["name"], str) \
             or not isinstance(obj["key_values"], list):
         raise SerdeError("expected an optimizer state with the fields `name` and `key_values`")
     out = []
@@ -170,7 +171,7 @@ def optim_state_from_value(obj):
         if variant == "Elem":
             # the element type of Value::Elem is the scalar crate's, whose encoding no file of the reference holds
             raise SerdeError("optimizer state with a scalar element value is not supported here")
-        if variant != "Tensor" or not isinstance(value, dict) or set(value) != {"tensor", "parameter_device", "parameter_type"} \
+        if variant != "Tensor" or not isinstance(value, dict) or not {"tensor", "parameter_device", "parameter_type"} <= set(value) \
                 or not isinstance(value["parameter_device"], bool) or not isinstance(value["parameter_type"], bool):
             raise SerdeError("expected {\"Tensor\": {tensor, parameter_device, parameter_type}}")
         array, is_bf16 = from_value(value["tensor"])
@@ -189,7 +190,7 @@ def parameter_to_value(array, bf16=False, optim_state=None):
 def parameter_from_value(obj, rank):
     """-> ParamValue.  An absent `optim_state` is none (`default`); a present one must be a state: the reference's
     deserializer has no none case (autograd.rs:1141-1151)."""
-    if not isinstance(obj, dict) or "value" not in obj or set(obj) - {"value", "optim_state"}:
+    if not isinstance(obj, dict) or "value" not in obj:
         raise SerdeError("expected a parameter object with the field `value`")
     state = optim_state_from_value(obj["optim_state"]) if "optim_state" in obj else None
     array, is_bf16 = from_value(obj["value"])
@@ -207,11 +208,13 @@ def conv2_to_value(weight, bias=None, padding=(0, 0), stride=(1, 1), dilation=(1
 
 def conv2_from_value(obj):
     """-> dict(weight=ParamValue, bias=None | ParamValue, padding, stride, dilation)"""
-    fields = {"weight", "padding", "stride", "dilation", "bias"}
-    if not isinstance(obj, dict) or set(obj) != fields:
-        raise SerdeError("expected an object with exactly the fields " + ", ".join(sorted(fields)))
+    # As the derive reads it (layer.rs:833-848, no `deny_unknown_fields`): unknown keys are skipped, a missing
+    # `Option` field (`bias`) is None, any other missing field is an error.
+    fields = {"weight", "padding", "stride", "dilation"}
+    if not isinstance(obj, dict) or not fields <= set(obj):
+        raise SerdeError("missing field: expected an object with the fields " + ", ".join(sorted(fields)) + " (and `bias`)")
     return dict(weight=parameter_from_value(obj["weight"], 4),
-                bias=None if obj["bias"] is None else parameter_from_value(obj["bias"], 1),
+                bias=None if obj.get("bias") is None else parameter_from_value(obj["bias"], 1),
                 padding=_dims(obj["padding"], "padding", 2), stride=_dims(obj["stride"], "stride", 2),
                 dilation=_dims(obj["dilation"], "dilation", 2))
 
@@ -222,10 +225,11 @@ def dense_to_value(weight, bias=None, bf16=False, weight_state=None, bias_state=
 
 
 def dense_from_value(obj):
-    if not isinstance(obj, dict) or set(obj) != {"weight", "bias"}:
-        raise SerdeError("expected an object with exactly the fields `weight` and `bias`")
+    # layer.rs:1069-1073: a missing `bias` is None, unknown keys are skipped
+    if not isinstance(obj, dict) or "weight" not in obj:
+        raise SerdeError("missing field `weight`")
     return dict(weight=parameter_from_value(obj["weight"], 2),
-                bias=None if obj["bias"] is None else parameter_from_value(obj["bias"], 1))
+                bias=None if obj.get("bias") is None else parameter_from_value(obj["bias"], 1))
 
 
 def max_pool2_to_value(filter, stride):
@@ -233,6 +237,6 @@ def max_pool2_to_value(filter, stride):
 
 
 def max_pool2_from_value(obj):
-    if not isinstance(obj, dict) or set(obj) != {"filter", "stride"}:
-        raise SerdeError("expected an object with exactly the fields `filter` and `stride`")
+    if not isinstance(obj, dict) or not {"filter", "stride"} <= set(obj):
+        raise SerdeError("missing field: expected an object with the fields `filter` and `stride`")
     return dict(filter=_dims(obj["filter"], "filter", 2), stride=_dims(obj["stride"], "stride", 2))

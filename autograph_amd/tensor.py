@@ -317,13 +317,39 @@ class Tensor:
 
     # -- scaled_add / sum_axis / cross entropy (src/tensor/ops.rs:257-318, reduce.rs:59-113, learn/criterion.rs) --
     def scaled_add(self, alpha, rhs):
-        """In place: self = alpha * rhs + self, each operation rounded to the element type."""
-        if self.dtype != rhs.dtype or self.shape != rhs.shape:
-            raise AghError(-1, f"scaled_add: {self.dtype}{self.shape} vs {rhs.dtype}{rhs.shape}")
-        if not self.is_standard_layout():
-            raise AghError(-1, "scaled_add: destination must be in standard layout")
-        x = rhs.as_standard_layout()
-        check(self._fn("agh_scaled_add")(self._data_ptr(), alpha, x._data_ptr(), len(self)))
+        """In place: self += alpha * rhs with `rhs` broadcast to self's shape, the product and the sum each rounded to
+        the element type (src/tensor/ops.rs:192-204 -> `assign(BinaryOp::Add, ..)`, :257-318).  Both sides may be any
+        views of up to four dimensions."""
+        if self.dtype != rhs.dtype:
+            raise AghError(-1, f"scaled_add: {self.dtype} vs {rhs.dtype}")
+        x = rhs.broadcast(self.shape)
+        if x is None:
+            raise AghError(-1, f"Broadcast not possible! {rhs.shape} -> {self.shape}")  # ops.rs:287-291
+        if self.is_standard_layout() and x.is_standard_layout() and x.shape == rhs.shape:
+            check(self._fn("agh_scaled_add")(self._data_ptr(), alpha, x._data_ptr(), len(self)))
+            return
+        if self.ndim > 4:
+            raise AghError(-1, "scaled_add: more than 4 dimensions")
+        pad = 4 - self.ndim
+        dims = [1] * pad + list(self.shape)
+        sy = [0] * pad + list(self.strides)
+        sx = [0] * pad + list(x.strides)
+        check(self._fn("agh_scaled_add_strided")(self._ptr(), self.offset, *sy, alpha, x._ptr(), x.offset, *sx, *dims))
+
+    def add_assign(self, rhs):
+        """`AddAssign` (src/tensor/ops.rs:245-255): `self.scaled_add(T::one(), &rhs)`."""
+        self.scaled_add(1.0, rhs)
+
+    def accuracy(self, target):
+        """`Accuracy::accuracy` (src/learn/criterion.rs:22-118): the number of rows whose target class has the strictly
+        largest score.  `target`: u8 class indices on the device (a `Buffer`).  Blocking."""
+        x = self.as_standard_layout()
+        bs, classes = x.shape
+        tmp = Buffer(4)
+        check(self._fn("agh_accuracy")(x._data_ptr(), target.ptr, bs, classes, tmp.ptr))
+        out = np.empty(1, dtype=np.uint32)
+        check(lib.agh_memcpy_d2h(out.ctypes.data, tmp.ptr, 4))
+        return int(out[0])
 
     def sum_axis0(self):
         x = self.as_standard_layout()

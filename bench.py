@@ -149,14 +149,16 @@ def main():
     del c
 
     if args.calib:
-        # ceilings measured with the same stream and events as everything else (agh_calib_*)
+        # ceilings measured with the same stream and events as everything else (benchlib/, a library of its own)
+        import benchlib as cal
+        cstream = ag.lib.agh_stream()
         sink = ag.Tensor.zeros((256,), "f32")
         blocks = 1024
         for shape, sname, iters in ((1, "16x16x32", 4096), (0, "32x32x16", 8192)):
             mflop = 2.0 * 32 * 32 * 16 * 16 * (1 + shape) * iters * 4 * blocks
             for zero in (1, 0):
                 name = f"calib_mfma_only_bf16_{sname}_" + ("zero_operands" if zero else "n002_operands")
-                fn = lambda: ag._ffi.check(ag.lib.agh_calib_mfma_bf16(sink._ptr(), zero, iters, blocks, shape))  # noqa: E731
+                fn = lambda: cal.check(cal.lib.calib_mfma_bf16(cstream, sink._ptr(), zero, iters, blocks, shape))  # noqa: E731
                 for _ in range(40):  # ~100 ms: let the clocks settle on this load
                     fn()
                 _, ms = timer.time(fn, 20, 5)
@@ -174,7 +176,7 @@ def main():
             for nld in (0, 2, 4, 8):
                 if nld == 0 and wname != "L2":
                     continue
-                fn = lambda: ag._ffi.check(ag.lib.agh_calib_mfma_dma(dsrc._ptr(), dsrc_bytes, sink._ptr(), nld, window, d_iters, d_blocks))  # noqa: E731
+                fn = lambda: cal.check(cal.lib.calib_mfma_dma(cstream, dsrc._ptr(), dsrc_bytes, sink._ptr(), nld, window, d_iters, d_blocks))  # noqa: E731
                 _, ms = timer.time(fn, 10, 3)
                 fill = d_blocks * d_iters * 4.0 * nld * 1024
                 extras[f"calib_mfma_dma_{nld}_loads_per_16_mfma_window_{wname}"] = {
@@ -186,11 +188,11 @@ def main():
         nbytes = 1 << 30
         cx, cy = ag.Tensor.zeros((nbytes // 4,), "f32"), ag.Tensor.uninit((nbytes // 4,), "f32")
         for grid in (1024, 2048, 4096, 8192, 16384, 65536):
-            _, ms = timer.time(lambda: ag._ffi.check(ag.lib.agh_calib_copy(cx._ptr(), cy._ptr(), nbytes, grid)), 10, 3)
+            _, ms = timer.time(lambda: cal.check(cal.lib.calib_copy(cstream, cx._ptr(), cy._ptr(), nbytes, grid)), 10, 3)
             extras[f"calib_copy_1GiB_grid{grid}"] = {"ms": round(ms, 4), "rate": round(2.0 * nbytes / ms / 1e6, 1), "unit": "GB/s",
                                                      "bytes_read": nbytes, "bytes_written": nbytes}
             log(f"copy 1 GiB, grid {grid}: {ms:.3f} ms  {2.0 * nbytes / ms / 1e6:.0f} GB/s (read + write)")
-            _, ms = timer.time(lambda: ag._ffi.check(ag.lib.agh_calib_read(cx._ptr(), sink._ptr(), nbytes, grid)), 10, 3)
+            _, ms = timer.time(lambda: cal.check(cal.lib.calib_read(cstream, cx._ptr(), sink._ptr(), nbytes, grid)), 10, 3)
             extras[f"calib_read_1GiB_grid{grid}"] = {"ms": round(ms, 4), "rate": round(nbytes / ms / 1e6, 1), "unit": "GB/s"}
             log(f"read 1 GiB, grid {grid}: {ms:.3f} ms  {nbytes / ms / 1e6:.0f} GB/s")
         del cx, cy
@@ -199,7 +201,7 @@ def main():
             wbytes = 256 * 64 * 56 * 56 * es
             mx, my = ag.Tensor.zeros((9 * wbytes // 4,), "f32"), ag.Tensor.uninit((wbytes // 4,), "f32")
             for grid in (2048, 8192):
-                _, ms = timer.time(lambda: ag._ffi.check(ag.lib.agh_calib_mix(mx._ptr(), my._ptr(), wbytes, 9, grid)), 10, 3)
+                _, ms = timer.time(lambda: cal.check(cal.lib.calib_mix(cstream, mx._ptr(), my._ptr(), wbytes, 9, grid)), 10, 3)
                 extras[f"calib_mix_9to1_{dt}_sized_grid{grid}"] = {"ms": round(ms, 4), "rate": round(10.0 * wbytes / ms / 1e6, 1), "unit": "GB/s",
                                                                   "bytes_read": 9 * wbytes, "bytes_written": wbytes}
                 log(f"9 reads : 1 write, {wbytes >> 20} MiB written ({dt} col2im size), grid {grid}: {ms:.3f} ms  {10.0 * wbytes / ms / 1e6:.0f} GB/s (read + write)")

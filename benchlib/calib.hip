@@ -1,18 +1,46 @@
 // Calibration launches: what this GPU can do at best on the two resources the kernels of this library
 // are bound by, measured with the same stream, events and profiler as the kernels themselves.
-//   agh_calib_mfma_bf16  a loop of nothing but independent v_mfma_f32_32x32x16_bf16 or v_mfma_f32_16x16x32_bf16 (no memory traffic),
+//   calib_mfma_bf16  a loop of nothing but independent v_mfma_f32_32x32x16_bf16 or v_mfma_f32_16x16x32_bf16 (no memory traffic),
 //                        on all-zero operands or on operands shaped like N(0, 0.02^2) bf16 data: the matrix
 //                        pipes' sustained rate under the power limit, the ceiling of any bf16 GEMM on such data
-//   agh_calib_copy       a plain 16-byte copy with a chosen grid: the read+write HBM ceiling, and the pass of
+//   calib_copy       a plain 16-byte copy with a chosen grid: the read+write HBM ceiling, and the pass of
 //                        known size that FETCH_SIZE / WRITE_SIZE counter readings are scaled by
-//   agh_calib_read       a plain 16-byte read with a chosen grid: the read-only HBM ceiling
-//   agh_calib_mfma_dma   the MFMA-only loop with direct-to-LDS loads between the MFMAs, one workgroup of 4 waves per CU, every
+//   calib_read       a plain 16-byte read with a chosen grid: the read-only HBM ceiling
+//   calib_mfma_dma   the MFMA-only loop with direct-to-LDS loads between the MFMAs, one workgroup of 4 waves per CU, every
 //                        workgroup cycling through a window of its own: what the matrix pipes sustain while a CU pulls bytes
 //                        through its L1 at a chosen rate, from L2 (small windows) or from beyond it (large ones).  The bf16
 //                        GEMM's 256x256 tile needs 4 such loads per 16 MFMAs per wave (32 bytes per cycle and CU).
-//   agh_calib_mix        R 16-byte reads from R separate streams per 16-byte write: what the memory system sustains on
+//   calib_mix        R 16-byte reads from R separate streams per 16-byte write: what the memory system sustains on
 //                        the read:write mix of a gather kernel (col2im of a 3x3 filter reads 9 bytes per byte written)
-#include "agh_internal.h"
+// This library is measurement code for bench.py and is NOT part of libautograph_hip.so: every entry point takes the
+// hipStream_t to launch on (bench.py passes the product library's stream, so the same HIP events time both).
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "calib.h"
+
+namespace {
+
+thread_local char g_err[384] = "";
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+constexpr int CALIB_OK = 0, CALIB_EINVAL = -1, CALIB_ENULL = -3, CALIB_ERANGE = -4;
+
+#define CALIB_LAUNCH_CHECK(name)                                                        \
+    do {                                                                                \
+        hipError_t _e = hipGetLastError();                                              \
+        if (_e != hipSuccess) return fail((int)_e, "%s: %s", name, hipGetErrorString(_e)); \
+    } while (0)
+
+}  // namespace
+
 
 namespace {
 
@@ -178,65 +206,63 @@ __global__ __launch_bounds__(256) void mix16_kernel(const u32x4_t *__restrict__ 
 
 }  // namespace
 
-using namespace agh;
-
 extern "C" {
 
-int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks, int shape) {
-    AGH_API_ENTER();
-    if (!sink) return fail(AGH_ENULL, "agh_calib_mfma_bf16: null sink (1 KiB of device memory)");
+int calib_mfma_bf16(void *stream_handle, void *sink, int zero_operands, int iters, int blocks, int shape) {
+    hipStream_t st = (hipStream_t)stream_handle;
+    if (!sink) return fail(CALIB_ENULL, "calib_mfma_bf16: null sink (1 KiB of device memory)");
     if (iters < 1 || blocks < 1 || (shape != 0 && shape != 1))
-        return fail(AGH_EINVAL, "agh_calib_mfma_bf16: iters and blocks must be positive, shape 0 (32x32x16) or 1 (16x16x32)");
+        return fail(CALIB_EINVAL, "calib_mfma_bf16: iters and blocks must be positive, shape 0 (32x32x16) or 1 (16x16x32)");
     if (shape == 0)
-        hipLaunchKernelGGL(mfma_only_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, stream(), (float *)sink, iters, zero_operands);
+        hipLaunchKernelGGL(mfma_only_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, st, (float *)sink, iters, zero_operands);
     else
-        hipLaunchKernelGGL(mfma_only_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream(), (float *)sink, iters, zero_operands);
-    AGH_LAUNCH_CHECK("agh_calib_mfma_bf16");
-    return AGH_OK;
+        hipLaunchKernelGGL(mfma_only_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, (float *)sink, iters, zero_operands);
+    CALIB_LAUNCH_CHECK("calib_mfma_bf16");
+    return CALIB_OK;
 }
 
-int agh_calib_copy(const void *src, void *dst, size_t bytes, int blocks) {
-    AGH_API_ENTER();
-    if (bytes == 0) return AGH_OK;
-    if (!src || !dst) return fail(AGH_ENULL, "agh_calib_copy: null pointer");
+int calib_copy(void *stream_handle, const void *src, void *dst, size_t bytes, int blocks) {
+    hipStream_t st = (hipStream_t)stream_handle;
+    if (bytes == 0) return CALIB_OK;
+    if (!src || !dst) return fail(CALIB_ENULL, "calib_copy: null pointer");
     if (bytes % 16 != 0 || (((uintptr_t)src | (uintptr_t)dst) & 15) != 0 || blocks < 1)
-        return fail(AGH_EINVAL, "agh_calib_copy: 16-byte aligned pointers, a multiple of 16 bytes and blocks >= 1");
-    hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), (const u32x4_t *)src, (u32x4_t *)dst, bytes / 16);
-    AGH_LAUNCH_CHECK("agh_calib_copy");
-    return AGH_OK;
+        return fail(CALIB_EINVAL, "calib_copy: 16-byte aligned pointers, a multiple of 16 bytes and blocks >= 1");
+    hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const u32x4_t *)src, (u32x4_t *)dst, bytes / 16);
+    CALIB_LAUNCH_CHECK("calib_copy");
+    return CALIB_OK;
 }
 
-int agh_calib_read(const void *src, void *sink, size_t bytes, int blocks) {
-    AGH_API_ENTER();
-    if (bytes == 0) return AGH_OK;
-    if (!src || !sink) return fail(AGH_ENULL, "agh_calib_read: null pointer");
+int calib_read(void *stream_handle, const void *src, void *sink, size_t bytes, int blocks) {
+    hipStream_t st = (hipStream_t)stream_handle;
+    if (bytes == 0) return CALIB_OK;
+    if (!src || !sink) return fail(CALIB_ENULL, "calib_read: null pointer");
     if (bytes % 16 != 0 || ((uintptr_t)src & 15) != 0 || blocks < 1)
-        return fail(AGH_EINVAL, "agh_calib_read: a 16-byte aligned pointer, a multiple of 16 bytes and blocks >= 1");
-    hipLaunchKernelGGL(read16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream(), (const u32x4_t *)src, (uint32_t *)sink, bytes / 16);
-    AGH_LAUNCH_CHECK("agh_calib_read");
-    return AGH_OK;
+        return fail(CALIB_EINVAL, "calib_read: a 16-byte aligned pointer, a multiple of 16 bytes and blocks >= 1");
+    hipLaunchKernelGGL(read16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const u32x4_t *)src, (uint32_t *)sink, bytes / 16);
+    CALIB_LAUNCH_CHECK("calib_read");
+    return CALIB_OK;
 }
 
-int agh_calib_mfma_dma(const void *src, size_t src_bytes, void *sink, int loads_per_16_mfma, size_t window_bytes, int iters, int blocks) {
-    AGH_API_ENTER();
-    if (!sink) return fail(AGH_ENULL, "agh_calib_mfma_dma: null sink (1 KiB of device memory)");
+int calib_mfma_dma(void *stream_handle, const void *src, size_t src_bytes, void *sink, int loads_per_16_mfma, size_t window_bytes, int iters, int blocks) {
+    hipStream_t st = (hipStream_t)stream_handle;
+    if (!sink) return fail(CALIB_ENULL, "calib_mfma_dma: null sink (1 KiB of device memory)");
     const int nld = loads_per_16_mfma;
     if (iters < 1 || blocks < 1 || (nld != 0 && nld != 2 && nld != 4 && nld != 8 && nld != 16))
-        return fail(AGH_EINVAL, "agh_calib_mfma_dma: iters and blocks positive, loads_per_16_mfma one of 0, 2, 4, 8, 16");
+        return fail(CALIB_EINVAL, "calib_mfma_dma: iters and blocks positive, loads_per_16_mfma one of 0, 2, 4, 8, 16");
     const size_t step = (size_t)4 * nld * 1024;  // bytes per workgroup and iteration
     size_t wg_stride = 0;
     int wrap = 1;
     if (nld > 0) {
-        if (!src) return fail(AGH_ENULL, "agh_calib_mfma_dma: null src");
+        if (!src) return fail(CALIB_ENULL, "calib_mfma_dma: null src");
         if (((uintptr_t)src & 15) != 0 || window_bytes < step || window_bytes % step != 0 || window_bytes / step > (size_t)1 << 20)
-            return fail(AGH_EINVAL, "agh_calib_mfma_dma: src 16-byte aligned, window_bytes a multiple of 4096 * loads_per_16_mfma");
+            return fail(CALIB_EINVAL, "calib_mfma_dma: src 16-byte aligned, window_bytes a multiple of 4096 * loads_per_16_mfma");
         wg_stride = window_bytes + 896;  // windows of neighbouring workgroups start in different L2 channels
         if (src_bytes < (size_t)blocks * wg_stride)
-            return fail(AGH_ERANGE, "agh_calib_mfma_dma: src holds %zu bytes, %zu needed", src_bytes, (size_t)blocks * wg_stride);
+            return fail(CALIB_ERANGE, "calib_mfma_dma: src holds %zu bytes, %zu needed", src_bytes, (size_t)blocks * wg_stride);
         wrap = (int)(window_bytes / step);
     }
     auto launch = [&](auto kern) {
-        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, stream(), (const unsigned char *)src, (float *)sink, iters, wg_stride, wrap);
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, st, (const unsigned char *)src, (float *)sink, iters, wg_stride, wrap);
     };
     switch (nld) {
         case 0: launch(mfma_dma_kernel<0>); break;
@@ -245,19 +271,19 @@ int agh_calib_mfma_dma(const void *src, size_t src_bytes, void *sink, int loads_
         case 8: launch(mfma_dma_kernel<8>); break;
         default: launch(mfma_dma_kernel<16>); break;
     }
-    AGH_LAUNCH_CHECK("agh_calib_mfma_dma");
-    return AGH_OK;
+    CALIB_LAUNCH_CHECK("calib_mfma_dma");
+    return CALIB_OK;
 }
 
-int agh_calib_mix(const void *src, void *dst, size_t write_bytes, int reads_per_write, int blocks) {
-    AGH_API_ENTER();
-    if (write_bytes == 0) return AGH_OK;
-    if (!src || !dst) return fail(AGH_ENULL, "agh_calib_mix: null pointer");
+int calib_mix(void *stream_handle, const void *src, void *dst, size_t write_bytes, int reads_per_write, int blocks) {
+    hipStream_t st = (hipStream_t)stream_handle;
+    if (write_bytes == 0) return CALIB_OK;
+    if (!src || !dst) return fail(CALIB_ENULL, "calib_mix: null pointer");
     if (write_bytes % 16 != 0 || (((uintptr_t)src | (uintptr_t)dst) & 15) != 0 || blocks < 1 || reads_per_write < 0 || reads_per_write > 64)
-        return fail(AGH_EINVAL, "agh_calib_mix: 16-byte aligned pointers, a multiple of 16 bytes, 0 <= reads_per_write <= 64 and blocks >= 1");
+        return fail(CALIB_EINVAL, "calib_mix: 16-byte aligned pointers, a multiple of 16 bytes, 0 <= reads_per_write <= 64 and blocks >= 1");
     const size_t n16 = write_bytes / 16;
     auto launch = [&](auto kern) {
-        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, stream(), (const u32x4_t *)src, (u32x4_t *)dst, n16, reads_per_write);
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, st, (const u32x4_t *)src, (u32x4_t *)dst, n16, reads_per_write);
     };
     switch (reads_per_write) {
         case 1: launch(mix16_kernel<1>); break;
@@ -266,8 +292,10 @@ int agh_calib_mix(const void *src, void *dst, size_t write_bytes, int reads_per_
         case 9: launch(mix16_kernel<9>); break;
         default: launch(mix16_kernel<0>); break;
     }
-    AGH_LAUNCH_CHECK("agh_calib_mix");
-    return AGH_OK;
+    CALIB_LAUNCH_CHECK("calib_mix");
+    return CALIB_OK;
 }
+
+const char *calib_last_error_string(void) { return g_err; }
 
 }  // extern "C"

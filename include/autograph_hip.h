@@ -72,6 +72,10 @@ int agh_free(void *ptr);
 int agh_cache_release(void);
 /* Bytes and blocks held for reuse, blocks currently handed out (any pointer may be null). */
 int agh_cache_stats(size_t *cached_bytes, size_t *cached_blocks, size_t *live_blocks);
+/* Bytes of the library's own workspace (split-K partials, reordered filter banks; both streams' blocks) and the number of
+ * outgrown workspace blocks kept alive for live graphs.  None of this memory is the caller's; the figures let a caller
+ * that must not allocate verify that a call sequence did not grow it. */
+int agh_workspace_stats(size_t *workspace_bytes, size_t *retired_blocks);
 /* into_device / to_device (src/tensor.rs:1775-1833): host -> device, enqueued on the current stream
  * (the branch stream inside a branch, like every launch).
  * The host range must stay valid until the next agh_sync unless it is pageable memory. */
@@ -96,12 +100,16 @@ void *agh_stream(void);
 /* Launch-bound sequences (a LeNet5 forward pass is a dozen tiny kernels) can be recorded once
  * and replayed as one hipGraph: between agh_graph_begin and agh_graph_end every launch entry
  * point and agh_memcpy_d2h_async is captured instead of executed.  No entry point that
- * allocates, frees or waits (agh_malloc, agh_free, agh_sync, agh_memcpy_d2h, a first split-K
- * GEMM that has to grow the workspace) may be called while capturing (they return an error): run the
- * sequence once eagerly first.  The library's workspace (split-K partials, reordered filter banks) is
- * named by the captured nodes: while any graph from agh_graph_end is alive, a workspace block that
- * has to grow is retired, not freed, so replays stay valid after larger eager calls; retired blocks
- * are released when the last graph is destroyed or at agh_shutdown.
+ * allocates or waits (agh_malloc, agh_sync, agh_memcpy_d2h, a first split-K GEMM that has to grow the
+ * workspace) may be called while capturing (they return an error): run the sequence once eagerly first.
+ * agh_free is allowed while capturing (a host-side temporary may be dropped at any moment): the block is
+ * set aside and goes back to the cache in agh_graph_end; a block that recorded work touches must of course
+ * stay allocated for as long as the graph is replayed.  The library's workspace (split-K partials,
+ * reordered filter banks) is named by the captured nodes: while any graph from agh_graph_end is alive, a
+ * workspace block that has to grow is retired, not freed, so replays stay valid after larger eager calls;
+ * retired blocks are released when the last graph is destroyed or at agh_shutdown.  agh_graph_launch
+ * first joins any branch that is still open on the second stream (its work may use the workspace a
+ * captured arm names).
  * The reference has no counterpart (krnl dispatches kernel by kernel). */
 int agh_graph_begin(void);
 int agh_graph_end(void **graph_exec);
@@ -129,30 +137,6 @@ int agh_event_create(void **event);
 int agh_event_destroy(void *event);
 int agh_event_record(void *event);
 int agh_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for `stop` */
-
-/* Calibration launches on the library's stream, for measurement only (no counterpart in the
- * reference): what the part sustains at best on the two resources the kernels here are bound by.
- * agh_calib_mfma_bf16: `blocks` workgroups of 4 waves, each wave `iters` times 16 independent
- * v_mfma_f32_32x32x16_bf16 (shape 0) or 64 independent v_mfma_f32_16x16x32_bf16 (shape 1, the form the bf16
- * GEMM uses) on register operands (zero_operands != 0: all zero; else bf16 patterns shaped like N(0, 0.02^2)
- * samples), 2 * 32*32*16 * 16 * (1 + shape) * iters * 4 * blocks flop, no memory traffic; `sink` is
- * 1 KiB of device memory that is practically never written.  agh_calib_copy / agh_calib_read: a plain
- * 16-byte nontemporal copy / read of `bytes` bytes with a grid of `blocks` workgroups of 256 threads
- * (grid-stride); also the pass of known size that profiler byte counters are scaled by.  agh_calib_mix:
- * every 16 bytes of `dst` (`write_bytes` in all) receive the xor of the 16 bytes at the same offset of
- * `reads_per_write` consecutive source streams of `write_bytes` each (so `src` holds reads_per_write *
- * write_bytes bytes): the read:write mix of a gather kernel such as col2im in its simplest, fully coalesced form.
- * agh_calib_mfma_dma: the MFMA-only loop on zero operands (`blocks` workgroups of 4 waves that each take a whole CU,
- * `iters` times 16 MFMAs per wave) with `loads_per_16_mfma` (0, 2, 4, 8 or 16) direct-to-LDS loads of 1 KiB spread
- * between the MFMAs of every wave; every workgroup cycles through a window of `window_bytes` of its own inside `src`
- * (`src_bytes` >= blocks * (window_bytes + 896)), so small windows are served by L2 and large ones from beyond it:
- * what the matrix pipes sustain while a CU pulls bytes through its L1 at the rate a GEMM tile needs. */
-int agh_calib_mfma_bf16(void *sink, int zero_operands, int iters, int blocks, int shape);
-int agh_calib_copy(const void *src, void *dst, size_t bytes, int blocks);
-int agh_calib_read(const void *src, void *sink, size_t bytes, int blocks);
-int agh_calib_mix(const void *src, void *dst, size_t write_bytes, int reads_per_write, int blocks);
-int agh_calib_mfma_dma(const void *src, size_t src_bytes, void *sink, int loads_per_16_mfma, size_t window_bytes, int iters,
-                       int blocks);
 
 /* --------------------------------------------------------------------- gemm ---- */
 
@@ -426,6 +410,20 @@ int agh_assign_bf16(const void *x, int64_t off_x, int64_t sx0, int64_t sx1, int6
 int agh_scaled_add_f32(void *y, float alpha, const void *x, int64_t n);
 int agh_scaled_add_bf16(void *y, float alpha, const void *x, int64_t n);
 
+/* `scaled_add` on views (src/tensor/ops.rs:192-204 -> `assign(BinaryOp::Add, alpha, rhs, self)`, :257-318, eval
+ * :1319-1330; device kernels :1400-1438): y[i] = T(T(alpha) * x[i]) + y[i] over the index space d0..d3 (pad with 1),
+ * signed element strides, a stride 0 on x broadcasts (`rhs.broadcast(self.raw_dim())`, :287-291).  This is also
+ * `add_assign` (alpha = 1, :245-255), i.e. the un-fused `output.add_assign(&bias)` of Dense::forward
+ * (layer.rs:1138-1140, autograd.rs:571-599: y [m, n] strides (n, 1), x = bias [n] as strides (0, 1)), and gradient
+ * accumulation into a view.  The elements of y must be distinct addresses (no stride 0 along a dimension > 1, else
+ * AGH_EINVAL); x may alias y only element for element. */
+int agh_scaled_add_strided_f32(void *y, int64_t off_y, int64_t sy0, int64_t sy1, int64_t sy2, int64_t sy3, float alpha,
+                               const void *x, int64_t off_x, int64_t sx0, int64_t sx1, int64_t sx2, int64_t sx3,
+                               int64_t d0, int64_t d1, int64_t d2, int64_t d3);
+int agh_scaled_add_strided_bf16(void *y, int64_t off_y, int64_t sy0, int64_t sy1, int64_t sy2, int64_t sy3, float alpha,
+                                const void *x, int64_t off_x, int64_t sx0, int64_t sx1, int64_t sx2, int64_t sx3,
+                                int64_t d0, int64_t d1, int64_t d2, int64_t d3);
+
 /* SGD with momentum: in f32, v = momentum*v + dw; w -= learning_rate*v; both cast back
  * (optimizer.rs:430-465, kernel :509-512). */
 int agh_sgd_momentum_f32(void *w, const void *dw, float learning_rate, float momentum, void *velocity, int64_t n);
@@ -446,6 +444,13 @@ int agh_cross_entropy_loss_bf16(const void *x, const void *target_u8, int64_t bs
  * (src/learn/neural_network/criterion.rs:79-103). */
 int agh_cross_entropy_backward_f32(const void *x, const void *target_u8, float dy, void *dx, int64_t bs, int64_t classes);
 int agh_cross_entropy_backward_bf16(const void *x, const void *target_u8, float dy, void *dx, int64_t bs, int64_t classes);
+
+/* `Accuracy::accuracy` device branch (src/learn/criterion.rs:101-118, kernel :269-296; host rule :30-47): the number
+ * of rows of x [bs, classes] whose target score is strictly greater than every other score of the row (ties and
+ * NaNs do not count; a target >= classes does not count, where the host panics).  Targets are u8 class indices.
+ * `correct` is one uint32 in device memory or in memory from agh_host_alloc. */
+int agh_accuracy_f32(const void *x, const void *target_u8, int64_t bs, int64_t classes, void *correct);
+int agh_accuracy_bf16(const void *x, const void *target_u8, int64_t bs, int64_t classes, void *correct);
 
 #ifdef __cplusplus
 }

@@ -307,13 +307,35 @@ public:
         return dx;
     }
 
-    // -- scaled_add (src/tensor/ops.rs:294-296), sum_axis(Axis(0)) (reduce.rs:59-113) --
-    void scaled_add(float alpha, const Tensor &rhs) {
-        if (rhs.dim_ != dim_) bail("scaled_add: broadcast not possible " + shape_str(rhs.dim_) + " -> " + shape_str(dim_));
-        if (!is_standard_layout()) bail("scaled_add: destination must be in standard layout");
-        const Tensor x = rhs.as_standard_layout();
-        check((kBf16 ? agh_scaled_add_bf16 : agh_scaled_add_f32)(data_ptr(), alpha, x.data_ptr(), len()));
+    // -- broadcast (ndarray `broadcast`: trailing axes aligned, stride 0 where a dimension of 1 is stretched) --
+    bool broadcast(const Shape &shape, Tensor &out) const {
+        if (shape.size() < ndim()) return false;
+        const size_t pad = shape.size() - ndim();
+        Shape st(shape.size(), 0);
+        for (size_t i = 0; i < ndim(); ++i) {
+            if (dim_[i] == shape[pad + i]) st[pad + i] = strides_[i];
+            else if (dim_[i] != 1) return false;
+        }
+        out = Tensor(buffer_, shape, st, offset_);
+        return true;
     }
+    // -- scaled_add / add_assign (src/tensor/ops.rs:192-204, :245-255, :257-318), sum_axis(Axis(0)) (reduce.rs:59-113) --
+    void scaled_add(float alpha, const Tensor &rhs) {
+        Tensor x;
+        if (!rhs.broadcast(dim_, x)) bail("Broadcast not possible! " + shape_str(rhs.dim_) + " -> " + shape_str(dim_));
+        if (is_standard_layout() && rhs.dim_ == dim_ && rhs.is_standard_layout()) {
+            check((kBf16 ? agh_scaled_add_bf16 : agh_scaled_add_f32)(data_ptr(), alpha, rhs.data_ptr(), len()));
+            return;
+        }
+        if (ndim() > 4) bail("scaled_add: more than 4 dimensions");
+        int64_t d[4] = {1, 1, 1, 1}, sx[4] = {0, 0, 0, 0}, sy[4] = {0, 0, 0, 0};
+        const size_t pad = 4 - ndim();
+        for (size_t i = 0; i < ndim(); ++i) { d[pad + i] = dim_[i]; sx[pad + i] = x.strides_[i]; sy[pad + i] = strides_[i]; }
+        check((kBf16 ? agh_scaled_add_strided_bf16 : agh_scaled_add_strided_f32)(
+            buffer_ptr(), offset_, sy[0], sy[1], sy[2], sy[3], alpha, x.buffer_ptr(), x.offset_, sx[0], sx[1], sx[2], sx[3],
+            d[0], d[1], d[2], d[3]));
+    }
+    void add_assign(const Tensor &rhs) { scaled_add(1.0f, rhs); }
     Tensor sum_axis0() const {
         if (ndim() != 2) bail("sum_axis0: expected a 2-D tensor");
         const Tensor x = as_standard_layout();
@@ -402,6 +424,12 @@ template <typename T> struct Dense {
     Tensor<T> weight;
     std::shared_ptr<Tensor<T>> bias;
     Tensor<T> forward(const Tensor<T> &input, bool relu = false) const { return input.dot_bias_relu(weight, bias.get(), relu); }
+    // the reference's separate calls (layer.rs:1137-1140): dot, broadcast add_assign, then the Relu layer; same bits
+    Tensor<T> forward_unfused(const Tensor<T> &input, bool relu = false) const {
+        Tensor<T> out = input.dot(weight);
+        if (bias) out.add_assign(*bias);
+        return relu ? out.relu() : out;
+    }
 };
 // `MaxPool2` (layer.rs:1149-1216); the stride defaults to the filter (layer.rs:535-539)
 template <typename T> struct MaxPool2 {

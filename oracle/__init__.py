@@ -73,6 +73,10 @@ _sig("orc_max_threads", [], C.c_int)
 _sig("orc_assign4", [_p, _i64, _p, _p, _i64, _p, _p, _i64])
 _sig("orc_scaled_add_f32", [_p, C.c_float, _p, _i64])
 _sig("orc_scaled_add_bf16", [_p, C.c_float, _p, _i64])
+_sig("orc_scaled_add_strided_f32", [_p, _i64, _p, C.c_float, _p, _i64, _p, _p])
+_sig("orc_scaled_add_strided_bf16", [_p, _i64, _p, C.c_float, _p, _i64, _p, _p])
+_sig("orc_accuracy_f32", [_p, _p, _i64, _i64], _i64)
+_sig("orc_accuracy_bf16", [_p, _p, _i64, _i64], _i64)
 _sig("orc_sgd_momentum_f32", [_p, _p, C.c_float, C.c_float, _p, _i64])
 _sig("orc_sgd_momentum_bf16", [_p, _p, C.c_float, C.c_float, _p, _i64])
 _sig("orc_sum_axis0_f32", [_p, _p, _i64, _i64])
@@ -319,6 +323,38 @@ def scaled_add(y, alpha, x):
     return y
 
 
+def _base_off_strides(a):
+    """(base array, element offset, element strides) of a numpy view."""
+    base = a
+    while base.base is not None and isinstance(base.base, np.ndarray):
+        base = base.base
+    es = a.dtype.itemsize
+    off = (a.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // es
+    return base, off, [st // es for st in a.strides]
+
+
+def scaled_add_strided(y, alpha, x):
+    """IN PLACE on the numpy view `y` (<= 4-D, any strides): y += alpha * broadcast(x), product and sum each rounded to
+    the element type.  `x` is broadcast to y's shape as ndarray does (trailing axes aligned, stride 0)."""
+    assert y.ndim <= 4 and x.dtype == y.dtype
+    xb = np.broadcast_to(x, y.shape)
+    pad = 4 - y.ndim
+    yb, off_y, sy = _base_off_strides(y)
+    xbase, off_x, sx = _base_off_strides(xb) if xb.base is not None else (xb, 0, [st // xb.itemsize for st in xb.strides])
+    d = (C.c_int64 * 4)(*([1] * pad + list(y.shape)))
+    sxa = (C.c_int64 * 4)(*([0] * pad + sx))
+    sya = (C.c_int64 * 4)(*([0] * pad + sy))
+    fn = _lib.orc_scaled_add_strided_bf16 if _is_bf16(y) else _lib.orc_scaled_add_strided_f32
+    fn(_ptr(yb), off_y, sya, float(alpha), _ptr(xbase), off_x, sxa, d)
+    return y
+
+
+def accuracy(x, t):
+    x, t = np.ascontiguousarray(x), np.ascontiguousarray(t, dtype=np.uint8)
+    bs, classes = x.shape
+    return int((_lib.orc_accuracy_bf16 if _is_bf16(x) else _lib.orc_accuracy_f32)(_ptr(x), _ptr(t), bs, classes))
+
+
 def sgd_momentum(w, dw, lr, momentum, v):
     """Returns (w', v')."""
     w, v = np.array(w, order="C", copy=True), np.array(v, order="C", copy=True)
@@ -349,12 +385,13 @@ def cross_entropy_backward(x, t, dy=1.0):
     return dx
 
 
-def lenet5_train_step(x, t, params, lr=0.01, momentum=None, velocities=None):
+def lenet5_train_step(x, t, params, lr=0.01, momentum=None, velocities=None, intermediates=None):
     """One training step of the benchmark's LeNet5 (benches/neural-network-benches/src/autograph_backend.rs:70-86,
     layers :88-162) chained from the host ops above in the order the autograd edges run them
     (layer.rs:950-1005 conv, autograd.rs:607-627 dot, :571-599 bias, layer.rs:1253-1267 relu, :1193-1216 pool).
     GEMMs use f32 accumulation with one rounding (the numerics the tolerance is stated against).
-    params = [w1, w2, wd1, wd2, wd3, b3]; returns (loss, new_params, grads, new_velocities)."""
+    params = [w1, w2, wd1, wd2, wd3, b3]; returns (loss, new_params, grads, new_velocities).  A dict passed as
+    `intermediates` receives the masked gradients of the backward chain (g_logits, g_d2, g_d1, gm2, gm1)."""
     w1, w2, wd1, wd2, wd3, b3 = params
     bf = _is_bf16(w1)
     mm = gemm_bf16_f32acc if bf else (lambda a, b: gemm_f64acc(a, b).astype(np.float32))
@@ -382,20 +419,26 @@ def lenet5_train_step(x, t, params, lr=0.01, momentum=None, velocities=None):
     logits = bias_add_rows(mm(a2, wd3), b3)
     loss = cross_entropy_loss(logits, t)
 
+    keep = intermediates if intermediates is not None else {}
     g = cross_entropy_backward(logits, t, 1.0)
+    keep["g_logits"] = g
     db3 = sum_axis0(g)
     dwd3 = mm(a2.T, g)
     g = relu_backward(d2, mm(g, wd3.T))
+    keep["g_d2"] = g
     dwd2 = mm(a1.T, g)
     g = relu_backward(d1, mm(g, wd2.T))
+    keep["g_d1"] = g
     dwd1 = mm(f.T, g)
     g = mm(g, wd1.T).reshape(bs, 16, 4, 4)
     g = relu_backward(c2, max_pool2_backward(r2, g, (2, 2)))
     gm = to_standard_layout(g.transpose(0, 2, 3, 1)).reshape(bs * 64, 16)
+    keep["gm2"] = gm
     dw2 = mm(gm.T, cols2).reshape(w2.shape)
     g = col2im_conv2(mm(gm, w2.reshape(16, 150)), (8, 8), (5, 5))
     g = relu_backward(c1, max_pool2_backward(r1, g, (2, 2)))
     gm = to_standard_layout(g.transpose(0, 2, 3, 1)).reshape(bs * 576, 6)
+    keep["gm1"] = gm
     dw1 = mm(gm.T, cols1).reshape(w1.shape)
 
     grads = [dw1, dw2, dwd1, dwd2, dwd3, db3]

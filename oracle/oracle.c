@@ -578,6 +578,61 @@ void orc_scaled_add_bf16(bf16_t *y, float alpha, const bf16_t *x, i64 n) {
     for (i64 i = 0; i < n; ++i) y[i] = bf16_add(bf16_mul(a, x[i]), y[i]);
 }
 
+/* The same on views (src/tensor/ops.rs:192-204 `scaled_add` -> `assign(BinaryOp::Add, alpha, rhs, self)`, :257-318:
+ * `rhs.broadcast(self.raw_dim())` then `*y = op.eval(alpha * x.cast(), *y)` per element, eval = a + b at :1319-1330).
+ * Index space d[0..4], signed element strides, stride 0 on x = broadcast. */
+void orc_scaled_add_strided_f32(float *y, i64 off_y, const i64 *sy, float alpha, const float *x, i64 off_x, const i64 *sx,
+                                const i64 *d) {
+    for (i64 i0 = 0; i0 < d[0]; ++i0)
+        for (i64 i1 = 0; i1 < d[1]; ++i1)
+            for (i64 i2 = 0; i2 < d[2]; ++i2)
+                for (i64 i3 = 0; i3 < d[3]; ++i3) {
+                    const i64 ix = off_x + i0 * sx[0] + i1 * sx[1] + i2 * sx[2] + i3 * sx[3];
+                    const i64 iy = off_y + i0 * sy[0] + i1 * sy[1] + i2 * sy[2] + i3 * sy[3];
+                    volatile float prod = alpha * x[ix];
+                    y[iy] = prod + y[iy];
+                }
+}
+void orc_scaled_add_strided_bf16(bf16_t *y, i64 off_y, const i64 *sy, float alpha, const bf16_t *x, i64 off_x,
+                                 const i64 *sx, const i64 *d) {
+    const bf16_t a = f32_to_bf16(alpha);
+    for (i64 i0 = 0; i0 < d[0]; ++i0)
+        for (i64 i1 = 0; i1 < d[1]; ++i1)
+            for (i64 i2 = 0; i2 < d[2]; ++i2)
+                for (i64 i3 = 0; i3 < d[3]; ++i3) {
+                    const i64 ix = off_x + i0 * sx[0] + i1 * sx[1] + i2 * sx[2] + i3 * sx[3];
+                    const i64 iy = off_y + i0 * sy[0] + i1 * sy[1] + i2 * sy[2] + i3 * sy[3];
+                    y[iy] = bf16_add(bf16_mul(a, x[ix]), y[iy]);
+                }
+}
+
+/* accuracy_host (src/learn/criterion.rs:30-47): rows whose target score is strictly greater than every other
+ * score.  A target >= classes panics on the host; here it does not count (the device kernel's rule, :281-284). */
+i64 orc_accuracy_f32(const float *x, const uint8_t *t, i64 bs, i64 classes) {
+    i64 n = 0;
+    for (i64 i = 0; i < bs; ++i) {
+        if (t[i] >= classes) continue;
+        const float xt = x[i * classes + t[i]];
+        int ok = 1;
+        for (i64 j = 0; j < classes; ++j)
+            if (j != t[i] && !(xt > x[i * classes + j])) ok = 0;
+        n += ok;
+    }
+    return n;
+}
+i64 orc_accuracy_bf16(const bf16_t *x, const uint8_t *t, i64 bs, i64 classes) {
+    i64 n = 0;
+    for (i64 i = 0; i < bs; ++i) {
+        if (t[i] >= classes) continue;
+        const float xt = bf16_to_f32(x[i * classes + t[i]]);
+        int ok = 1;
+        for (i64 j = 0; j < classes; ++j)
+            if (j != t[i] && !(xt > bf16_to_f32(x[i * classes + j]))) ok = 0;
+        n += ok;
+    }
+    return n;
+}
+
 /* SGD with momentum (optimizer.rs:430-465, kernel :509-512): in f32, v = m*v + dw; w -= lr*v; then
  * both cast back to T. */
 void orc_sgd_momentum_f32(float *w, const float *dw, float lr, float m, float *v, i64 n) {

@@ -26,6 +26,7 @@ extern "C" {
     pub fn agh_free(ptr: *mut c_void) -> c_int;
     pub fn agh_cache_release() -> c_int;
     pub fn agh_cache_stats(cached_bytes: *mut usize, cached_blocks: *mut usize, live_blocks: *mut usize) -> c_int;
+    pub fn agh_workspace_stats(workspace_bytes: *mut usize, retired_blocks: *mut usize) -> c_int;
     pub fn agh_memcpy_h2d(dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     pub fn agh_memcpy_d2h(dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
     pub fn agh_memcpy_d2d(dst: *mut c_void, src: *const c_void, bytes: usize) -> c_int;
@@ -46,11 +47,6 @@ extern "C" {
     pub fn agh_event_destroy(event: *mut c_void) -> c_int;
     pub fn agh_event_record(event: *mut c_void) -> c_int;
     pub fn agh_event_elapsed_ms(start: *mut c_void, stop: *mut c_void, ms: *mut f32) -> c_int;
-    pub fn agh_calib_mfma_bf16(sink: *mut c_void, zero_operands: c_int, iters: c_int, blocks: c_int, shape: c_int) -> c_int;
-    pub fn agh_calib_copy(src: *const c_void, dst: *mut c_void, bytes: usize, blocks: c_int) -> c_int;
-    pub fn agh_calib_read(src: *const c_void, sink: *mut c_void, bytes: usize, blocks: c_int) -> c_int;
-    pub fn agh_calib_mix(src: *const c_void, dst: *mut c_void, write_bytes: usize, reads_per_write: c_int, blocks: c_int) -> c_int;
-    pub fn agh_calib_mfma_dma(src: *const c_void, src_bytes: usize, sink: *mut c_void, loads_per_16_mfma: c_int, window_bytes: usize, iters: c_int, blocks: c_int) -> c_int;
     pub fn agh_gemm_f32(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
     pub fn agh_gemm_bf16(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
     pub fn agh_gemm_bf16_noalloc(m: i64, k: i64, n: i64, alpha: f32, a: *const c_void, off_a: i64, rsa: i64, csa: i64, b: *const c_void, off_b: i64, rsb: i64, csb: i64, beta: f32, c: *mut c_void, off_c: i64, rsc: i64, csc: i64) -> c_int;
@@ -92,6 +88,8 @@ extern "C" {
     pub fn agh_assign_bf16(x: *const c_void, off_x: i64, sx0: i64, sx1: i64, sx2: i64, sx3: i64, y: *mut c_void, off_y: i64, sy0: i64, sy1: i64, sy2: i64, sy3: i64, d0: i64, d1: i64, d2: i64, d3: i64) -> c_int;
     pub fn agh_scaled_add_f32(y: *mut c_void, alpha: f32, x: *const c_void, n: i64) -> c_int;
     pub fn agh_scaled_add_bf16(y: *mut c_void, alpha: f32, x: *const c_void, n: i64) -> c_int;
+    pub fn agh_scaled_add_strided_f32(y: *mut c_void, off_y: i64, sy0: i64, sy1: i64, sy2: i64, sy3: i64, alpha: f32, x: *const c_void, off_x: i64, sx0: i64, sx1: i64, sx2: i64, sx3: i64, d0: i64, d1: i64, d2: i64, d3: i64) -> c_int;
+    pub fn agh_scaled_add_strided_bf16(y: *mut c_void, off_y: i64, sy0: i64, sy1: i64, sy2: i64, sy3: i64, alpha: f32, x: *const c_void, off_x: i64, sx0: i64, sx1: i64, sx2: i64, sx3: i64, d0: i64, d1: i64, d2: i64, d3: i64) -> c_int;
     pub fn agh_sgd_momentum_f32(w: *mut c_void, dw: *const c_void, learning_rate: f32, momentum: f32, velocity: *mut c_void, n: i64) -> c_int;
     pub fn agh_sgd_momentum_bf16(w: *mut c_void, dw: *const c_void, learning_rate: f32, momentum: f32, velocity: *mut c_void, n: i64) -> c_int;
     pub fn agh_sum_axis0_f32(x: *const c_void, y: *mut c_void, rows: i64, cols: i64) -> c_int;
@@ -100,4 +98,6 @@ extern "C" {
     pub fn agh_cross_entropy_loss_bf16(x: *const c_void, target_u8: *const c_void, bs: i64, classes: i64, loss: *mut f32) -> c_int;
     pub fn agh_cross_entropy_backward_f32(x: *const c_void, target_u8: *const c_void, dy: f32, dx: *mut c_void, bs: i64, classes: i64) -> c_int;
     pub fn agh_cross_entropy_backward_bf16(x: *const c_void, target_u8: *const c_void, dy: f32, dx: *mut c_void, bs: i64, classes: i64) -> c_int;
+    pub fn agh_accuracy_f32(x: *const c_void, target_u8: *const c_void, bs: i64, classes: i64, correct: *mut c_void) -> c_int;
+    pub fn agh_accuracy_bf16(x: *const c_void, target_u8: *const c_void, bs: i64, classes: i64, correct: *mut c_void) -> c_int;
 }

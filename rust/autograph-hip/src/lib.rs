@@ -128,6 +128,42 @@ pub fn gemm<T: Scalar>(m: usize, k: usize, n: usize, alpha: f32, a: MatrixView, 
     })
 }
 
+/// A strided view of up to four dimensions (pad leading dimensions with 1 and stride 0): buffer, element offset,
+/// signed element strides.  A stride of 0 on a source broadcasts it.
+#[derive(Clone, Copy)]
+pub struct View4 {
+    pub ptr: *const c_void,
+    pub offset: i64,
+    pub strides: [i64; 4],
+}
+
+/// `y += alpha * x` on views, the device branch of `assign(BinaryOp::Add, alpha, x, y)` behind `scaled_add` and
+/// `add_assign` (src/tensor/ops.rs:192-204, :245-255, :257-318): `x` already broadcast to `dims` by the caller
+/// (`rhs.broadcast(self.raw_dim())`, :287-291), product and sum each rounded to `T`.
+pub fn scaled_add<T: Scalar>(y_ptr: *mut c_void, y: View4, alpha: f32, x: View4, dims: [usize; 4]) -> Result<()> {
+    let d = [dims[0] as i64, dims[1] as i64, dims[2] as i64, dims[3] as i64];
+    let (sy, sx) = (y.strides, x.strides);
+    check(unsafe {
+        if T::IS_BF16 {
+            sys::agh_scaled_add_strided_bf16(y_ptr, y.offset, sy[0], sy[1], sy[2], sy[3], alpha, x.ptr, x.offset, sx[0], sx[1], sx[2], sx[3], d[0], d[1], d[2], d[3])
+        } else {
+            sys::agh_scaled_add_strided_f32(y_ptr, y.offset, sy[0], sy[1], sy[2], sy[3], alpha, x.ptr, x.offset, sx[0], sx[1], sx[2], sx[3], d[0], d[1], d[2], d[3])
+        }
+    })
+}
+
+/// `Accuracy::accuracy` device branch (src/learn/criterion.rs:101-118): writes the number of correct rows as one
+/// `u32` to `correct` (device memory or pinned host memory); u8 targets.
+pub fn accuracy<T: Scalar>(x: *const c_void, target_u8: *const c_void, batch_size: usize, classes: usize, correct: *mut c_void) -> Result<()> {
+    check(unsafe {
+        if T::IS_BF16 {
+            sys::agh_accuracy_bf16(x, target_u8, batch_size as i64, classes as i64, correct)
+        } else {
+            sys::agh_accuracy_f32(x, target_u8, batch_size as i64, classes as i64, correct)
+        }
+    })
+}
+
 /// Geometry of a 2-D convolution's patch extraction (`Im2ColConv2Options` / `Col2ImConv2Options`).
 #[derive(Clone, Copy, Debug)]
 pub struct ConvGeometry {

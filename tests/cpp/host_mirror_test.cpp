@@ -181,6 +181,28 @@ static int run_gpu(const char *in_path, const char *out_path) {
     REQUIRE(fused_grad.into_vec() == pre.relu_backward(grad).into_vec());
     REQUIRE(pre.max_pool2_relu_backward(ones, po, true).into_vec() ==
             fused_grad.permuted_axes({0, 2, 3, 1}).to_standard_layout().into_vec());
+    // Dense as the reference's separate calls (dot, broadcast add_assign, relu) equals the fused launch bit for bit
+    {
+        const Tensor<float> h = Tensor<float>::from_vec({37, 53}, a);
+        Dense<float> dn;
+        dn.weight = Tensor<float>::from_vec({53, 41}, b);
+        dn.bias = std::make_shared<Tensor<float>>(Tensor<float>::from_vec({41}, std::vector<float>(b.begin(), b.begin() + 41)));
+        REQUIRE(dn.forward(h, true).into_vec() == dn.forward_unfused(h, true).into_vec());
+        REQUIRE(dn.forward(h).into_vec() == dn.forward_unfused(h).into_vec());
+        // scaled_add into a transposed view: (y^T += 2 x) == (y += 2 x^T)
+        Tensor<float> y1 = Tensor<float>::from_vec({37, 53}, a), y2 = Tensor<float>::from_vec({37, 53}, a);
+        const Tensor<float> xs = Tensor<float>::from_vec({53, 37}, std::vector<float>(b.begin(), b.begin() + 53 * 37));
+        Tensor<float> y1t = y1.t();
+        y1t.scaled_add(2.0f, xs);
+        y2.scaled_add(2.0f, xs.t().to_standard_layout());
+        REQUIRE(y1.into_vec() == y2.into_vec());
+        try {
+            y1.scaled_add(1.0f, Tensor<float>::from_vec({5}, std::vector<float>(5, 1.0f)));
+            REQUIRE(false);
+        } catch (const Error &e) {
+            REQUIRE(std::string(e.what()).rfind("Broadcast not possible!", 0) == 0);
+        }
+    }
     // a permuted view copies into standard layout
     REQUIRE(act.permuted_axes({0, 2, 3, 1}).to_standard_layout().permuted_axes({0, 3, 1, 2}).into_vec() == act.into_vec());
     device.wait();

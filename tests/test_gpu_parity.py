@@ -5,6 +5,8 @@ generators (ramps, cycles), the same parameter grids, host result vs device resu
 Bars: im2col / col2im / pooling / relu bit-exact; f32 gemm within 1e-5*sqrt(K) relative;
 bf16 gemm within 1 bf16 ulp + 1e-2 relative of an f32-accumulated reference.
 """
+import ctypes as C  # noqa: F401
+
 import numpy as np
 import pytest
 
@@ -219,6 +221,84 @@ def test_gemm_random_views(ag):
             assert np.all(np.abs(got - want) <= bf16_ulp(want) + 1e-2 * np.abs(want) + 1e-5 * absprod), tag
         done += 1
     assert done >= 120
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_gemm_zero_stride_operands(ag, dtype):
+    """Broadcast views as operands of `fn gemm` (strides are taken as they come, src/tensor/linalg.rs:285-299; ndarray's
+    `broadcast` gives stride 0): every row of A the same vector, every column of B the same vector, an operand that is
+    one scalar, k broadcast.  Against the f64 product of the materialised arrays, at sizes that take the small and the
+    large tiles and split-K."""
+    rng = np.random.default_rng(271)
+
+    def check_case(av, bv, tag):
+        m, k = av.shape
+        n = bv.shape[1]
+        ta_base, oa, rsa, csa = orc._view(av)
+        tb_base, ob, rsb, csb = orc._view(bv)
+        ta, tb = ag.Tensor.from_array(ta_base), ag.Tensor.from_array(tb_base)
+        a = ag.Tensor(ta.buffer, (m, k), (rsa, csa), oa, dtype)
+        b = ag.Tensor(tb.buffer, (k, n), (rsb, csb), ob, dtype)
+        got = as_f32(a.dot(b).into_array()).astype(np.float64)
+        am, bm = np.ascontiguousarray(av), np.ascontiguousarray(bv)
+        want = orc.gemm_f64acc(am, bm)
+        absprod = np.abs(as_f32(am)).astype(np.float64) @ np.abs(as_f32(bm)).astype(np.float64)
+        if dtype == "f32":
+            assert np.all(np.abs(got - want) <= 1e-5 * np.sqrt(k) * absprod + 1e-30), tag
+        else:
+            assert np.all(np.abs(got - want) <= bf16_ulp(want) + 1e-2 * np.abs(want) + 1e-5 * absprod), tag
+
+    for m, k, n in [(5, 7, 3), (64, 96, 80), (300, 1024, 260), (16, 8192, 24), (1024, 256, 1024)]:
+        arow = to_dtype(rng.uniform(-1, 1, (1, k)), dtype)
+        acol = to_dtype(rng.uniform(-1, 1, (m, 1)), dtype)
+        a = to_dtype(rng.uniform(-1, 1, (m, k)), dtype)
+        b = to_dtype(rng.uniform(-1, 1, (k, n)), dtype)
+        bcol = to_dtype(rng.uniform(-1, 1, (k, 1)), dtype)
+        brow = to_dtype(rng.uniform(-1, 1, (1, n)), dtype)
+        one = to_dtype(rng.uniform(0.5, 1, (1, 1)), dtype)
+        check_case(np.broadcast_to(arow, (m, k)), b, ("A rows stride 0", m, k, n))
+        check_case(a, np.broadcast_to(bcol, (k, n)), ("B columns stride 0", m, k, n))
+        check_case(np.broadcast_to(acol, (m, k)), b, ("A along k stride 0", m, k, n))
+        check_case(a, np.broadcast_to(brow, (k, n)), ("B along k stride 0", m, k, n))
+        check_case(np.broadcast_to(one, (m, k)), b, ("A scalar", m, k, n))
+        check_case(a, np.broadcast_to(one, (k, n)), ("B scalar", m, k, n))
+        check_case(np.broadcast_to(arow, (m, k)), np.broadcast_to(bcol, (k, n)), ("both", m, k, n))
+
+
+def test_entry_points_from_two_threads(ag):
+    """Tensors are `Send + Sync` in the reference (autograd.rs:97) and the C ABI says any thread may call any entry
+    point: two host threads allocate, multiply and free concurrently (split-K shapes included, which share the
+    library's workspace); every product must equal the one a single thread gets, bit for bit."""
+    import threading
+    rng = np.random.default_rng(272)
+    shapes = [(128, 256, 64), (16, 8192, 24), (300, 200, 100), (6, 57600, 25), (1024, 512, 768), (64, 64, 64)]
+    data = {}
+    for dtype in ("f32", "bf16"):
+        for s in shapes:
+            data[(dtype, s)] = (to_dtype(rng.uniform(-1, 1, s[:2]), dtype), to_dtype(rng.uniform(-1, 1, s[1:]), dtype))
+    serial = {key: ag.Tensor.from_array(a).dot(ag.Tensor.from_array(b)).into_array() for key, (a, b) in data.items()}
+    errors = []
+
+    def worker(order):
+        try:
+            for _ in range(6):
+                for key in order:
+                    a, b = data[key]
+                    ta, tb = ag.Tensor.from_array(a), ag.Tensor.from_array(b)
+                    got = ta.dot(tb).into_array()
+                    if not np.array_equal(got, serial[key]):
+                        errors.append(key)
+                    del ta, tb
+        except Exception as e:  # noqa: BLE001
+            errors.append(repr(e))
+
+    keys = list(data)
+    threads = [threading.Thread(target=worker, args=(keys,)), threading.Thread(target=worker, args=(keys[::-1],))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:3]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])

@@ -196,22 +196,24 @@ def test_block_freed_under_an_unjoined_branch_is_reused_safely(ag):
 
 
 def test_calibration_launches(ag):
-    """The measurement-only launches behind `bench.py --calib`: the copy and the read:write mix move exactly the bytes
+    """The measurement-only launches behind `bench.py --calib` (benchlib/, a library of its own): the copy and the read:write mix move exactly the bytes
     they claim (checked bit for bit on a small buffer), the MFMA loops run in both instruction shapes with and without
     direct loads, and arguments that would leave the buffers are refused before anything is launched."""
-    lib, check = ag.lib, ag._ffi.check
+    import benchlib as cal
+    check, lib = cal.check, cal.lib
+    st = ag.lib.agh_stream()  # the product library's stream, as bench.py passes it
     rng = np.random.default_rng(5)
     n = 1 << 18  # 1 MiB of u32
     src = rng.integers(0, 2**32, 3 * n, dtype=np.uint32)
     tsrc = ag.Tensor.from_array(src.view(np.float32))
     tdst = ag.Tensor.zeros((n,), "f32")
-    check(lib.agh_calib_copy(tsrc._ptr(), tdst._ptr(), 4 * n, 64))
+    check(lib.calib_copy(st, tsrc._ptr(), tdst._ptr(), 4 * n, 64))
     assert np.array_equal(tdst.into_array().view(np.uint32), src[:n])
     sink = ag.Tensor.zeros((256,), "f32")
-    check(lib.agh_calib_read(tsrc._ptr(), sink._ptr(), 4 * n, 64))
+    check(lib.calib_read(st, tsrc._ptr(), sink._ptr(), 4 * n, 64))
     # every 16 bytes of dst: xor of the 16 bytes at the same offset of the streams, the first word also with the slot index
     for reads in (1, 2, 3):
-        check(lib.agh_calib_mix(tsrc._ptr(), tdst._ptr(), 4 * n, reads, 37))
+        check(lib.calib_mix(st, tsrc._ptr(), tdst._ptr(), 4 * n, reads, 37))
         want = np.zeros(n, np.uint32)
         for r in range(reads):
             want ^= src[r * n:(r + 1) * n]
@@ -219,16 +221,16 @@ def test_calibration_launches(ag):
         assert np.array_equal(tdst.into_array().view(np.uint32), want), reads
     for shape in (0, 1):
         for zero in (0, 1):
-            check(lib.agh_calib_mfma_bf16(sink._ptr(), zero, 4, 8, shape))
+            check(lib.calib_mfma_bf16(st, sink._ptr(), zero, 4, 8, shape))
     for nld in (0, 2, 4, 8, 16):
         window = 4096 * nld * 2 if nld else 0
-        check(lib.agh_calib_mfma_dma(tsrc._ptr(), 12 * n, sink._ptr(), nld, window, 8, 4))
-    check(lib.agh_sync())
+        check(lib.calib_mfma_dma(st, tsrc._ptr(), 12 * n, sink._ptr(), nld, window, 8, 4))
+    ag._ffi.check(ag.lib.agh_sync())
     assert not np.any(sink.into_array())  # the sinks are never written
     # AGH_EINVAL is -1, AGH_ERANGE -4
-    assert lib.agh_calib_mfma_bf16(sink._ptr(), 0, 4, 8, 2) == -1
-    assert lib.agh_calib_mfma_dma(tsrc._ptr(), 12 * n, sink._ptr(), 3, 4096 * 3, 8, 4) == -1
-    assert lib.agh_calib_mfma_dma(tsrc._ptr(), 12 * n, sink._ptr(), 4, 4096 * 4 + 16, 8, 4) == -1
-    assert lib.agh_calib_mfma_dma(tsrc._ptr(), 65536, sink._ptr(), 4, 65536, 8, 4) == -4
-    assert lib.agh_calib_mix(tsrc._ptr(), tdst._ptr(), 4 * n + 4, 2, 8) == -1
-    assert lib.agh_calib_copy(tsrc._ptr(), tdst._ptr(), 4 * n, 0) == -1
+    assert lib.calib_mfma_bf16(st, sink._ptr(), 0, 4, 8, 2) == -1
+    assert lib.calib_mfma_dma(st, tsrc._ptr(), 12 * n, sink._ptr(), 3, 4096 * 3, 8, 4) == -1
+    assert lib.calib_mfma_dma(st, tsrc._ptr(), 12 * n, sink._ptr(), 4, 4096 * 4 + 16, 8, 4) == -1
+    assert lib.calib_mfma_dma(st, tsrc._ptr(), 65536, sink._ptr(), 4, 65536, 8, 4) == -4
+    assert lib.calib_mix(st, tsrc._ptr(), tdst._ptr(), 4 * n + 4, 2, 8) == -1
+    assert lib.calib_copy(st, tsrc._ptr(), tdst._ptr(), 4 * n, 0) == -1

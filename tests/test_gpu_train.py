@@ -99,6 +99,112 @@ def test_scaled_add_sgd_sum_axis0_bit_exact(ag, dtype):
     assert np.array_equal(ag.Tensor.from_array(a).sum_axis0().into_array(), orc.sum_axis0(a))
 
 
+def _view_of(ag, t, a, base):
+    """The device Tensor that shows the same elements of `t` (uploaded from `base`) as the numpy view `a` of `base`."""
+    es = base.itemsize
+    off = (a.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // es
+    return ag.Tensor(t.buffer, a.shape, tuple(st // es for st in a.strides), off, t.dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_scaled_add_on_strided_and_broadcast_views(ag, dtype):
+    """`scaled_add` / `add_assign` on views (src/tensor/ops.rs:192-204, :245-255, :257-318): bit-exact against the
+    oracle, elements outside the destination view untouched; the 16-byte form (aligned, contiguous innermost axis) and
+    the element-wise one, negative strides, offsets, stride-0 sources, the Dense bias at full size."""
+    rng = np.random.default_rng(45)
+    base = to_dtype(rng.standard_normal((6, 10, 12, 16)), dtype)
+
+    def run(yview, x, alpha):
+        want = base.copy()
+        orc.scaled_add_strided(yview(want), alpha, x)
+        ty = ag.Tensor.from_array(base)
+        tx = ag.Tensor.from_array(x)
+        _view_of(ag, ty, yview(base), base).scaled_add(alpha, tx)
+        assert np.array_equal(ty.into_array(), want)
+
+    mk = lambda *shape: to_dtype(rng.standard_normal(shape) * 3, dtype)
+    run(lambda a: a, mk(16), 1.0)                                   # bias over the trailing axis, 16-byte groups
+    run(lambda a: a, mk(6, 1, 12, 1), -0.01)                        # stride-0 innermost source
+    run(lambda a: a[:, ::2, 1:9, :], mk(5, 8, 16), 0.3)             # sliced destination, still vectorisable
+    run(lambda a: a[:, :, :, 3:11], mk(12, 8), 0.3)                 # unaligned innermost window
+    run(lambda a: a.transpose(0, 3, 1, 2), mk(16, 10, 12), 2.0)     # permuted destination (NHWC buffer seen as NCHW)
+    run(lambda a: a[::-1, :, ::-1, ::-2], mk(1,), 0.5)              # negative strides, scalar source
+    run(lambda a: a[2, 3], mk(12, 16), -1.0)                        # 2-D window at an offset
+    # source given as a strided view itself (a transposed matrix), destination contiguous
+    y = to_dtype(rng.standard_normal((300, 70)), dtype)
+    x = to_dtype(rng.standard_normal((70, 300)), dtype)
+    ty, tx = ag.Tensor.from_array(y), ag.Tensor.from_array(x)
+    ty.scaled_add(0.25, tx.t())
+    want = y.copy()
+    orc.scaled_add_strided(want, 0.25, x.T)
+    assert np.array_equal(ty.into_array(), want)
+    # y += y (aliasing element for element)
+    ty = ag.Tensor.from_array(y)
+    tyt = ty.t()
+    tyt.add_assign(tyt)
+    want = y.copy()
+    orc.scaled_add_strided(want.T, 1.0, want.T.copy())
+    assert np.array_equal(ty.into_array(), want)
+    # shapes that cannot broadcast, a broadcast destination and a type mismatch are refused before any launch
+    with pytest.raises(ag.AghError, match="Broadcast not possible"):
+        ty.scaled_add(1.0, ag.Tensor.from_array(mk(7)))
+    with pytest.raises(ag.AghError, match="destination cannot be a broadcast view"):
+        ag.Tensor.from_array(mk(70)).broadcast((300, 70)).scaled_add(1.0, ty)
+    with pytest.raises(ag.AghError):
+        ty.scaled_add(1.0, ag.Tensor.from_array(to_dtype(rng.standard_normal((300, 70)), "f32" if dtype == "bf16" else "bf16")))
+    # the Dense-shaped bias add at full size, [16384, 4096] += [4096]
+    big = to_dtype(rng.standard_normal((16384, 4096), dtype=np.float32), dtype)
+    bias = mk(4096)
+    tb = ag.Tensor.from_array(big)
+    tb.add_assign(ag.Tensor.from_array(bias))
+    assert np.array_equal(tb.into_array(), orc.bias_add_rows(big, bias))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_dense_unfused_equals_fused_epilogue(ag, dtype):
+    """`Dense::forward` as the reference issues it (layer.rs:1137-1140: dot, `add_assign(&bias)`, then the Relu layer)
+    against the one-launch epilogue: the same bits."""
+    rng = np.random.default_rng(46)
+    for m, k, n in [(100, 84, 10), (1000, 256, 128), (257, 1000, 333), (2048, 512, 1024)]:
+        x = ag.Tensor.from_array(to_dtype(rng.standard_normal((m, k)), dtype))
+        layer = ag.Dense(ag.Tensor.from_array(to_dtype(rng.standard_normal((k, n)) * 0.1, dtype)),
+                         ag.Tensor.from_array(to_dtype(rng.standard_normal(n), dtype)))
+        for relu in (False, True):
+            a, b = layer.forward(x, relu=relu).into_array(), layer.forward(x, relu=relu, fused=False).into_array()
+            assert np.array_equal(a, b), (m, k, n, relu)
+        plain = x.dot(layer.weight).into_array()
+        assert np.array_equal(layer.forward(x, fused=False).into_array(), orc.bias_add_rows(plain, layer.bias.into_array()))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_accuracy(ag, dtype):
+    """`Accuracy` (src/learn/criterion.rs:22-118): the reference test's generator (tests/integration_tests.rs:767-793),
+    ties / NaNs / out-of-range targets, and random data with many ties at sizes that take one and several workgroups."""
+    for bs, classes in [(1, 8), (31, 16), (1000, 100)]:
+        flat = np.resize(np.arange(classes), bs * classes + classes // 2 + 1)[classes // 2 + 1:][: bs * classes]
+        x = to_dtype(flat.reshape(bs, classes), dtype)
+        t = (np.arange(bs) % classes).astype(np.uint8)
+        assert ag.Tensor.from_array(x).accuracy(labels(ag, t)) == orc.accuracy(x, t)
+    x = to_dtype(np.array([[1, 3, 2], [3, 3, 1], [np.nan, 1, 0], [0, np.nan, 5], [2, 1, 0], [-0.0, 0.0, -1]]), dtype)
+    t = np.array([1, 0, 0, 2, 7, 0], dtype=np.uint8)
+    assert ag.Tensor.from_array(x).accuracy(labels(ag, t)) == orc.accuracy(x, t) == 1
+    rng = np.random.default_rng(47)
+    for bs, classes in [(5000, 6), (300000, 10), (70000, 256)]:
+        x = to_dtype(rng.integers(0, 3 if classes < 100 else 4000, (bs, classes)), dtype)
+        t = rng.integers(0, classes, bs).astype(np.uint8)
+        want = orc.accuracy(x, t)
+        assert 0 < want < bs
+        assert ag.Tensor.from_array(x).accuracy(labels(ag, t)) == want
+    # the count may go straight to pinned host memory
+    hp = C.c_void_p()
+    ag._ffi.check(ag.lib.agh_host_alloc(C.byref(hp), 4))
+    tx = ag.Tensor.from_array(x)
+    ag._ffi.check(getattr(ag.lib, f"agh_accuracy_{dtype}")(tx._data_ptr(), labels(ag, t).ptr, bs, classes, hp))
+    ag._ffi.check(ag.lib.agh_sync())
+    assert C.cast(hp, C.POINTER(C.c_uint32))[0] == want
+    ag._ffi.check(ag.lib.agh_host_free(hp))
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_cross_entropy(ag, dtype):
     rng = np.random.default_rng(43)
@@ -239,7 +345,8 @@ def test_lenet5_train_step(ag, dtype, momentum, fused_forward, fused_backward):
     bs = 100
     x = to_dtype(rng.uniform(0, 1, (bs, 1, 28, 28)), dtype)
     t = rng.integers(0, 10, bs).astype(np.uint8)
-    want_loss, want_params, want_grads, want_v = orc.lenet5_train_step(x, t, params, lr=0.01, momentum=momentum)
+    inter = {}
+    want_loss, want_params, want_grads, want_v = orc.lenet5_train_step(x, t, params, lr=0.01, momentum=momentum, intermediates=inter)
 
     model = ag.LeNet5.from_arrays(*params)
     trainer = ag.LeNet5Trainer(model, bs, learning_rate=0.01, optimizer=ag.SGD(momentum), fused_forward=fused_forward,
@@ -259,6 +366,21 @@ def test_lenet5_train_step(ag, dtype, momentum, fused_forward, fused_backward):
             # decision moves single entries; the bulk has to agree
             assert np.abs(gf - wf).max() <= 0.1 * scale, name
             assert np.abs(gf - wf).mean() <= 0.01 * scale, name
+    # The masked gradients of the backward chain: a wrong relu or pooling mask moves whole cells between zero and
+    # non-zero, which the tolerances above would not see.  The zero pattern has to be the oracle's except where the
+    # last bit of a forward dot product decides a sign or a maximum (measured: under 0.1 % of the cells), and on the
+    # cells both call non-zero the values agree to a few bf16 steps of the tensor's scale.
+    for name in ("g_logits", "g_d2", "g_d1", "gm2", "gm1"):
+        g = as_f32(getattr(trainer, name).into_array()).astype(np.float64)
+        w = as_f32(inter[name]).astype(np.float64).reshape(g.shape)
+        flips = np.mean((g == 0) != (w == 0))
+        assert flips <= 2e-3, (name, flips)
+        assert 0.02 < np.mean(w == 0) < 0.98 or name == "g_logits", name  # the masks are really there
+        both = (g != 0) & (w != 0)
+        scale = np.abs(w).max()
+        err = np.abs(g - w)[both]
+        assert err.max() <= (1e-4 if dtype == "f32" else 2.0**-5) * scale, name
+        assert err.mean() <= (1e-6 if dtype == "f32" else 2.0**-10) * scale, name
     for name, p, w, old in zip(("w1", "w2", "wd1", "wd2", "wd3", "b3"), trainer.params, want_params, params):
         pf, wf, of = (as_f32(a).astype(np.float64) for a in (p.into_array(), w, old))
         step = np.abs(wf - of).max()

@@ -424,6 +424,74 @@ def test_scaled_add_vs_torch_per_op_rounding():
     assert np.array_equal(orc.scaled_add(yf, 0.3, xf), (np.float32(0.3) * xf) + yf)
 
 
+def test_scaled_add_strided_vs_torch_on_views():
+    """`scaled_add` on views (src/tensor/ops.rs:192-204, :257-318): torch evaluates `y_view += a * x` on strided and
+    broadcast operands with one bf16 rounding per operation; the oracle must leave every element outside the
+    destination view untouched and agree bit for bit inside it."""
+    rng = np.random.default_rng(132)
+    a_t = torch.tensor(0.3, dtype=torch.float32).to(torch.bfloat16)
+
+    def run(ybase, yview, x):
+        """yview(array) picks the destination view out of a base array; x is broadcast against it."""
+        for bf in (True, False):
+            yb = orc.f32_to_bf16(ybase) if bf else ybase.copy()
+            xv = orc.f32_to_bf16(x) if bf else x.copy()
+            want = yb.copy()
+            dst = yview(want)
+            if bf:  # torch rounds the product and the sum separately; done on contiguous copies of the view
+                prod = a_t * tbf(np.ascontiguousarray(np.broadcast_to(xv, dst.shape)))
+                dst[...] = tbits(prod + tbf(np.ascontiguousarray(dst)))
+            else:
+                dst[...] = (np.float32(0.3) * np.broadcast_to(xv, dst.shape)).astype(np.float32) + dst
+            orc.scaled_add_strided(yview(yb), 0.3, xv)
+            assert np.array_equal(yb, want)
+            assert not np.array_equal(yb, orc.f32_to_bf16(ybase) if bf else ybase)
+
+    base = rng.standard_normal((6, 10, 12)).astype(np.float32)
+    run(base, lambda t: t, rng.standard_normal(12).astype(np.float32))                       # bias over the trailing axis
+    run(base, lambda t: t[:, ::2, 1:9], rng.standard_normal((5, 8)).astype(np.float32))      # sliced destination
+    run(base, lambda t: t.transpose(2, 1, 0), rng.standard_normal((1, 10, 1)).astype(np.float32))  # permuted destination
+    run(base, lambda t: t[:, ::-1], rng.standard_normal((6, 1, 12)).astype(np.float32))      # negative stride
+    run(base, lambda t: t, rng.standard_normal((1,)).astype(np.float32))                     # scalar broadcast
+    # aliasing element for element: y += a * y
+    yb = orc.f32_to_bf16(base)
+    ty = tbf(yb).clone()
+    ty.add_(a_t * ty.clone())
+    got = yb.copy()
+    orc.scaled_add_strided(got, 0.3, got)
+    assert np.array_equal(got, tbits(ty))
+    # the contiguous entry is the same operation
+    x1 = orc.f32_to_bf16(rng.standard_normal(base.shape).astype(np.float32))
+    got = yb.copy()
+    orc.scaled_add_strided(got, -0.01, x1)
+    assert np.array_equal(got, orc.scaled_add(yb, -0.01, x1))
+
+
+def test_accuracy_reference_generator_and_rules():
+    """accuracy_host (src/learn/criterion.rs:30-47).  On the reference test's data (tests/integration_tests.rs:767-793:
+    rows are rotations of 0..classes starting at classes/2 + 1, targets cycle 0..classes) every row is a permutation,
+    so a row counts exactly when its target holds the row's maximum classes - 1: a closed form, not the oracle's loop."""
+    for bs, classes in [(1, 8), (31, 16), (1000, 100)]:
+        flat = np.resize(np.arange(classes), bs * classes + classes // 2 + 1)[classes // 2 + 1:][: bs * classes]
+        x = flat.reshape(bs, classes).astype(np.float32)
+        t = (np.arange(bs) % classes).astype(np.uint8)
+        want = int(np.sum(x[np.arange(bs), t] == classes - 1))
+        assert orc.accuracy(x, t) == want
+        assert orc.accuracy(orc.f32_to_bf16(x), t) == want
+    # ties, NaNs and out-of-range targets do not count; strictly greater does
+    x = np.array([[1, 3, 2], [3, 3, 1], [np.nan, 1, 0], [0, np.nan, 5], [2, 1, 0], [-0.0, 0.0, -1]], dtype=np.float32)
+    t = np.array([1, 0, 0, 2, 7, 0], dtype=np.uint8)
+    assert orc.accuracy(x, t) == 1
+    assert orc.accuracy(orc.f32_to_bf16(x), t) == 1
+    # against argmax with a uniqueness check on random data with many ties
+    rng = np.random.default_rng(133)
+    x = rng.integers(0, 4, (500, 6)).astype(np.float32)
+    t = rng.integers(0, 6, 500).astype(np.uint8)
+    top = x.max(axis=1)
+    want = int(np.sum((x[np.arange(500), t] == top) & ((x == top[:, None]).sum(axis=1) == 1)))
+    assert orc.accuracy(x, t) == want
+
+
 def test_sgd_momentum_vs_closed_form():
     rng = np.random.default_rng(33)
     w, dw, v = (rng.standard_normal(3000).astype(np.float32) for _ in range(3))

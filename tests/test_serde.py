@@ -100,14 +100,22 @@ def test_layer_values_follow_the_derived_field_lists():
     assert serde.max_pool2_to_value((2, 2), (2, 2)) == {"filter": [2, 2], "stride": [2, 2]}  # layer.rs:1152-1155
     assert serde.max_pool2_from_value({"filter": [3, 2], "stride": [1, 1]}) == dict(filter=(3, 2), stride=(1, 1))
     # an absent optimizer state is the default (none); a null one is no state (the deserializer reads a struct,
-    # autograd.rs:1141-1151); unknown or missing fields and wrong ranks are errors
+    # autograd.rs:1141-1151); missing non-optional fields and wrong ranks are errors
     assert serde.parameter_from_value({"value": json.loads(serde.to_json(b))}, 1).optim_state is None
     with pytest.raises(serde.SerdeError):
         serde.parameter_from_value({"value": json.loads(serde.to_json(b)), "optim_state": None}, 1)
-    for bad in ({"weight": v["weight"], "bias": None, "extra": 1}, {"weight": v["weight"]},
-                {"weight": {"value": json.loads(serde.to_json(b))}, "bias": None}):
+    for bad in ({"bias": None}, {"weight": {"value": json.loads(serde.to_json(b))}, "bias": None}):
         with pytest.raises(serde.SerdeError):
             serde.dense_from_value(bad)
+    # the derives set no `deny_unknown_fields` (layer.rs:833-848, :1069-1073, autograd.rs:639-656): a key they do not
+    # know is skipped and a missing `Option` field is None, at every level
+    lenient = serde.dense_from_value({"weight": {**d["weight"], "note": 1}, "extra": [1, 2]})
+    assert lenient["bias"] is None and np.array_equal(lenient["weight"][0], w.reshape(4, 75))
+    cv = {k: val for k, val in v.items() if k != "bias"}
+    assert serde.conv2_from_value({**cv, "future_field": None})["bias"] is None
+    assert serde.max_pool2_from_value({"filter": [2, 2], "stride": [2, 2], "x": 0}) == dict(filter=(2, 2), stride=(2, 2))
+    with pytest.raises(serde.SerdeError):
+        serde.conv2_from_value({k: val for k, val in v.items() if k != "stride"})
     with pytest.raises(serde.SerdeError):
         serde.conv2_from_value({**v, "padding": [1]})
     with pytest.raises(serde.SerdeError):

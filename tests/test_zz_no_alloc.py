@@ -30,6 +30,12 @@ def cache_stats(ag):
     return a.value, b.value, c.value
 
 
+def workspace_stats(ag):
+    a, b = C.c_size_t(), C.c_size_t()
+    ag._ffi.check(ag.lib.agh_workspace_stats(C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
 def test_noalloc_gemm_equals_gemm_on_calls_that_share_the_scratch(ag, monkeypatch):
     rng = np.random.default_rng(41)
     # k >> m*n: the split-K shapes of the LeNet5 weight gradients (256 and 25 k-groups), then smaller ones;
@@ -44,11 +50,15 @@ def test_noalloc_gemm_equals_gemm_on_calls_that_share_the_scratch(ag, monkeypatc
         run(ag, ag.lib.agh_gemm_bf16, ta, tb, want_t)
         cases.append((ta, tb, want_t.into_array(), dy, cols))
     outs = [ag.Tensor.zeros((m, n), "bf16") for m, _, n in shapes]
-    before = cache_stats(ag)
+    # The library's own workspace, which the agh_gemm_bf16 calls above have grown, is handed back (unless a graph of
+    # an earlier test still names it): a no-alloc call that fell back to it would have to grow it again.
+    ag._ffi.check(ag.lib.agh_cache_release())
+    before, ws_before = cache_stats(ag), workspace_stats(ag)
     # all calls queued back to back: each reuses the scratch the previous one has just read
     for (ta, tb, _, _, _), out in zip(cases, outs):
         run(ag, ag.lib.agh_gemm_bf16_noalloc, ta, tb, out)
     assert cache_stats(ag) == before, "no buffer was taken from or returned to the allocator"
+    assert workspace_stats(ag) == ws_before, "the library's workspace (hipMalloc) was not touched"
     for (ta, tb, want, dy, cols), out, shape in zip(cases, outs, shapes):
         got = out.into_array()
         assert np.array_equal(got, want), shape
