@@ -42,6 +42,20 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 // 32-byte group m (16 rows) of k-row kr sits at group slot m ^ (kr & 3) ^ (((kr >> 3) & 1) << 2): an involution in m
 __device__ __forceinline__ uint32_t rslot(uint32_t m, uint32_t kr) { return m ^ (kr & 3u) ^ (((kr >> 3) & 1u) << 2); }
 __device__ __forceinline__ uint32_t rslot_inv(uint32_t ms, uint32_t kr) { return rslot(ms, kr); }
+// The same for a tile of BR rows.  BR == 64: a k-row is 128 bytes, four groups, and covers only half of the LDS banks, so
+// the slot function has two bits, and k-rows 8 apart (which two neighbouring 16-lane groups of a transposing read
+// touch together) would meet on the same banks: k-rows with bit 3 set swap places with their even / odd neighbour
+// (krow_pos, an involution), which puts them on the other half of the banks.
+template <int BR>
+__device__ __forceinline__ uint32_t rslot_br(uint32_t m, uint32_t kr) {
+    if constexpr (BR == 64) return m ^ (kr & 3u);
+    else return rslot(m, kr);
+}
+template <int BR>
+__device__ __forceinline__ uint32_t krow_pos(uint32_t kr) {
+    if constexpr (BR == 64) return kr ^ ((kr >> 3) & 1u);
+    else return kr;
+}
 
 // 16-byte direct load: lane L's data lands at LDS address lds_base + 16*L (lds_base is
 // wave-uniform and travels in M0).  Issued as inline assembly on purpose: the compiler's
@@ -80,9 +94,9 @@ struct DirectLoad {
                 const int rowg = min(r0 + row, NR - 1);
                 off[i] = ((int64_t)rowg * rs + c * 8) * 2;
             } else {
-                const int kr = inst * KRPI + lane / CPR;
+                const int kr = (int)krow_pos<BR>((uint32_t)(inst * KRPI + lane / CPR));  // the k-row stored at this LDS row
                 const int pc = lane % CPR;
-                const uint32_t m = rslot_inv((uint32_t)(pc >> 1), (uint32_t)kr);
+                const uint32_t m = rslot_br<BR>((uint32_t)(pc >> 1), (uint32_t)kr);
                 int rowg = r0 + (int)(2 * m + (pc & 1)) * 8;
                 if (rowg >= NR) rowg = NR - 8;
                 off[i] = ((int64_t)kr * ks + rowg) * 2;
@@ -96,7 +110,7 @@ struct DirectLoad {
             const int row = inst * 8 + (lane >> 3);
             return (((lane & 7) ^ (int)swz((uint32_t)row)) * 8) < rem;
         } else {
-            return inst * KRPI + lane / CPR < rem;
+            return (int)krow_pos<BR>((uint32_t)(inst * KRPI + lane / CPR)) < rem;
         }
     }
 };
@@ -122,7 +136,7 @@ struct FragRead {
             } else {
                 const uint32_t j = (lane & 15) >> 2;
                 const uint32_t kr = 8u * (lane >> 4) + j;
-                off[i] = kr * PITCH + 32u * rslot((uint32_t)(rb >> 4), kr) + 8u * (lane & 3);
+                off[i] = krow_pos<BR>(kr) * PITCH + 32u * rslot_br<BR>((uint32_t)(rb >> 4), kr) + 8u * (lane & 3);
             }
         }
     }
@@ -233,7 +247,7 @@ __global__ __launch_bounds__(WGP *WGQ * 64) void gemm_bf16_dl_kernel(Args g) {
     // MFMAs, and the first MFMAs of substep 1 are followed by the reads of tile kt+1's substep 0 from `nxt` (set A).
     // sched_barrier(0) after every MFMA pins this interleaving.
     constexpr int NM = TP * TQ;
-    constexpr int RSTEP = 2;                                          // one fragment read every RSTEP MFMAs
+    constexpr int RSTEP = NU * 2 <= NM ? 2 : 1;                       // one fragment read every RSTEP MFMAs
     constexpr int NB = NU * RSTEP + NM / 16 < NM ? NU * RSTEP + NM / 16 : NM;  // barrier: a few MFMAs after the last read
     constexpr int LSTEP = NM / NLT > 0 ? NM / NLT : 1;                // one direct load every LSTEP MFMAs
     static_assert(NU * RSTEP <= NM, "fragment reads must fit behind the MFMAs of one substep");

@@ -30,6 +30,9 @@ static const TileCfg kCfgs[] = {
     {128, 32, 0.28f, 4, true},
 };
 static constexpr int kNumCfgs = sizeof(kCfgs) / sizeof(kCfgs[0]);
+// rate of a CU on 64 x 64 direct-to-LDS bf16 tiles relative to a 256 x 256 workgroup on a full chip: one workgroup with
+// the CU to itself (ring of eight stages), two sharing it (rings of four)
+static constexpr double kDirect64Alone = 0.27, kDirect64Shared = 0.19;
 
 template <typename T, int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
 int launch_one(const Args &g, int splits) {
@@ -63,18 +66,25 @@ inline int env_int(const char *name, int dflt);
 // AGH_GEMM_RING=2|4 forces either.
 template <int BP, int BQ, int WGP, int WGQ, int LP, int LQ>
 int launch_dl_ring(const Args &g, int splits) {
-    if constexpr (BP == 128 && BQ == 128) {
-        const int64_t wgs = (int64_t)g.tiles_p * g.tiles_q * splits * g.batch;
-        // split-K streams its operands from HBM once (no second workgroup re-reads them out of L2), where the deeper
-        // ring pays from 8 k-tiles on (128x4096x4096 in 8 splits: 19.5 against 20.5 us; in 4: 17.2 against 20.1)
-        const bool alone = wgs <= (compute_units() > 0 ? compute_units() : 256) &&
-                           (g.k_per_split >= 20 * 64 || (splits > 1 && g.k_per_split >= 8 * 64));
-        if (env_int("AGH_GEMM_RING", alone ? 4 : 2) == 4)
-            return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, 4>(g, splits);
+    if constexpr (BP == 64 && BQ == 64) {
+        // A k-tile of the 64 x 64 tile is eight MFMAs a wave, a small fraction of a load's latency: always a ring of
+        // four stages (64 KB, two workgroups per CU).  Eight stages measured slower at every size (1024^3: 6.2 against
+        // 5.6 us, 2048^3: 32.2 against 29.3 us).
+        return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, 4>(g, splits);
+    } else {
+        if constexpr (BP == 128 && BQ == 128) {
+            const int64_t wgs = (int64_t)g.tiles_p * g.tiles_q * splits * g.batch;
+            // split-K streams its operands from HBM once (no second workgroup re-reads them out of L2), where the deeper
+            // ring pays from 8 k-tiles on (128x4096x4096 in 8 splits: 19.5 against 20.5 us; in 4: 17.2 against 20.1)
+            const bool alone = wgs <= (compute_units() > 0 ? compute_units() : 256) &&
+                               (g.k_per_split >= 20 * 64 || (splits > 1 && g.k_per_split >= 8 * 64));
+            if (env_int("AGH_GEMM_RING", alone ? 4 : 2) == 4)
+                return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, 4>(g, splits);
+        }
+        // 128 x 256 and 256 x 128: three stages of 48 KB (a CU holds one such workgroup either way; 3 to 10 % faster than
+        // two at every size measured, 2048^3 to 8192^3)
+        return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, BP * BQ == 128 * 256 ? 3 : 2>(g, splits);
     }
-    // 128 x 256 and 256 x 128: three stages of 48 KB (a CU holds one such workgroup either way; 3 to 10 % faster than
-    // two at every size measured, 2048^3 to 8192^3)
-    return launch_one_dl<BP, BQ, WGP, WGQ, LP, LQ, BP * BQ == 128 * 256 ? 3 : 2>(g, splits);
 }
 #endif
 
@@ -125,8 +135,8 @@ int launch_loaders(const Args &g, int splits, int lp, int lq, bool direct) {
     }
 #endif
 #ifdef AGH_GEMM_WITH_BF16_DIRECT
-    if constexpr (std::is_same<T, uint16_t>::value && !SCALAR_OK) {
-        if (direct) {
+    if constexpr (std::is_same<T, uint16_t>::value && (!SCALAR_OK || (BP == 64 && BQ == 64))) {
+        if (direct && lp != LD_S && lq != LD_S) {
             switch (lp * 3 + lq) {
                 case LD_K * 3 + LD_K: return launch_dl_ring<BP, BQ, WGP, WGQ, LD_K, LD_K>(g, splits);
                 case LD_K * 3 + LD_R: return launch_dl_ring<BP, BQ, WGP, WGQ, LD_K, LD_R>(g, splits);
@@ -164,7 +174,7 @@ int launch_cfg(int cfg, const Args &g, int splits, int lp, int lq, bool direct) 
         case 1: return launch_loaders<T, 128, 256, 2, 2, false>(g, splits, lp, lq, direct);
         case 2: return launch_loaders<T, 256, 128, 2, 2, false>(g, splits, lp, lq, direct);
         case 3: return launch_loaders<T, 128, 128, 2, 2, false>(g, splits, lp, lq, direct);
-        case 4: return launch_loaders<T, 64, 64, 2, 2, true>(g, splits, lp, lq, false);
+        case 4: return launch_loaders<T, 64, 64, 2, 2, true>(g, splits, lp, lq, direct);
         case 5: return launch_loaders<T, 32, 128, 1, 4, true>(g, splits, lp, lq, false);
         case 6: return launch_loaders<T, 128, 32, 4, 1, true>(g, splits, lp, lq, false);
         default: return fail(AGH_EINVAL, "gemm: bad tile config %d", cfg);
@@ -269,6 +279,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
         // are a poor second: measured 2x slower at 1024^3 (16.4 us against 8.9 us) although they put four times as
         // many CUs to work
         double eff = (direct_ok && !kCfgs[i].scalar_ok) || !direct_ok ? t.eff : t.eff * 0.25;
+        const bool bf16_direct64 = direct_ok && t.bp == 64 && t.bq == 64;
         // the 64 x 64 direct tile is measured at 0.8 of the 256 x 256 tile's rate per CU (3072^3: 118 TFLOP/s, where
         // 144 tiles of 256 x 256 leave 112 CUs idle)
         // f32: the 64 x 64 and 128 x 128 tiles have direct-to-LDS kernels (agh_gemm_f32_dl.h)
@@ -310,6 +321,14 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
             };
             cost = ((double)(tiles / slots) * round_cost(slots) + (rest ? round_cost(rest) : 0.0)) *
                    (kt + (t.wgs_per_cu == 1 ? 4.0 : 2.0)) / kt;
+        }
+        // The 64 x 64 direct-to-LDS bf16 tile: a CU's fill path from L2 bounds it (16 KB per k-tile against the 32 KB a
+        // 128 x 128 tile moves for four times the flop), so a tile takes about half the time of a 128 x 128 one; filling
+        // its ring and storing the tile cost about six of its k-tiles.
+        if (bf16_direct64) {
+            const int64_t slots = (int64_t)cus * 2;
+            const double per_tile = (double)t.bp * t.bq / (tiles <= cus ? kDirect64Alone : kDirect64Shared);
+            cost = (double)((tiles + slots - 1) / slots) * (tiles <= cus ? 1 : 2) * per_tile * (kt + 6.0) / kt;
         }
         if (best < 0 || cost < best_cost) { best = i; best_cost = cost; }
     }
@@ -371,7 +390,7 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     g.store_mode = vec_store ? ST_VEC : ST_SCALAR;
     // the direct-to-LDS kernel can transpose its output tile through LDS and store full 16-byte
     // chunks when nothing has to be read back from C
-    if (direct && best <= 3 && vec_store && beta == 0.0f && g.NP % 8 == 0 && (g.dq % 8 == 0 || g.NQ == 1) &&
+    if (direct && best <= 4 && vec_store && beta == 0.0f && g.NP % 8 == 0 && (g.dq % 8 == 0 || g.NQ == 1) &&
         aligned(C, 16) && (batch == 1 || g.batch_d % 8 == 0))
         g.store_mode = ST_STAGED;
     return launch_cfg<T>(best, g, 1, lp, lq, direct);

@@ -368,31 +368,64 @@ def main():
                 model.replay()
                 ag._ffi.check(ag.lib.agh_sync())
 
+            def pipelined(launch, nwarm=100, nrep=1000):
+                """K launches back to back, one wait on each side: the way this bench times every step."""
+                for _ in range(nwarm):
+                    launch()
+                ag._ffi.check(sync_fn())
+                t0 = time.perf_counter()
+                for _ in range(nrep):
+                    launch()
+                ag._ffi.check(sync_fn())
+                return (time.perf_counter() - t0) * 1e3 / nrep
+
             gpu_ms = wall(infer)
             got = np.ctypeslib.as_array(C.cast(host.value, C.POINTER(C.c_float)), shape=(bsl, 10)).copy()
             graph_ms = wall(infer_graph, 50, 300)
+            gpu_pipe_ms = pipelined(lambda: lenet_fn(*lenet_args))
+            graph_pipe_ms = pipelined(model.replay, 50, 300)
             _, kernel_ms = timer.time(lambda: model.forward_single_launch(txl, host.value), 50, 20)
-            # layer-by-layer path (12 launches, im2col + gemm convolutions), eager
+            # layer-by-layer path (12 launches, im2col + gemm convolutions), eager, each layer allocating its output
             _, layered_ms = timer.time(lambda: model.forward(txl, algorithm="im2col"), 20, 5)
-            lenet = {"gpu_ms": round(gpu_ms, 4), "gpu_kernel_ms": round(kernel_ms, 4), "gpu_graph_5_launches_ms": round(graph_ms, 4),
+            # the same layer objects with each layer's own fused form (conv+relu+pool, dense+relu): 5 launches, eager
+            _, fused_eager_ms = timer.time(lambda: model.forward_fused(txl), 20, 5)
+            lenet = {"gpu_ms": round(gpu_ms, 4), "gpu_kernel_ms": round(kernel_ms, 4), "gpu_pipelined_ms": round(gpu_pipe_ms, 4),
+                     "gpu_graph_5_launches_ms": round(graph_ms, 4), "gpu_graph_5_launches_pipelined_ms": round(graph_pipe_ms, 4),
+                     "gpu_layered_5_launches_eager_ms": round(fused_eager_ms, 4),
                      "gpu_layered_im2col_eager_ms": round(layered_ms, 4),
                      "what": "gpu_ms: one launch of the whole-network kernel (input resident in HBM, [1000,10] logits written "
                              "into pinned host memory), wall clock per inference including the host-side wait; "
-                             "gpu_kernel_ms: the same launch between HIP events; gpu_graph_5_launches_ms: graph replay of "
-                             "conv+relu+pool x2 and 3 Dense GEMMs plus D2H; gpu_layered_im2col_eager_ms: the 12-launch "
-                             "layer-by-layer path, each layer allocating its output"}
+                             "gpu_kernel_ms: the same launch between HIP events; gpu_pipelined_ms: 1000 such launches back to "
+                             "back with one wait at the end, per launch; gpu_graph_5_launches_ms: graph replay of "
+                             "conv+relu+pool x2 and 3 Dense GEMMs plus D2H through the per-layer entry points, with the "
+                             "host-side wait (…_pipelined_ms: replays back to back); gpu_layered_5_launches_eager_ms: the "
+                             "same five per-layer calls issued eagerly, each allocating its output; "
+                             "gpu_layered_im2col_eager_ms: the 12-launch layer-by-layer path (im2col + gemm, relu, pool)"}
             if not args.no_cpu:
                 thr = orc.max_threads()
-                want = orc.lenet5_forward_f32(xl, *params, direct=True)
+                want = orc.lenet5_forward_f32(xl, *params, direct="packed")
                 t0 = time.perf_counter()
-                ncpu = 20
+                ncpu = 40
                 for _ in range(ncpu):
-                    orc.lenet5_forward_f32(xl, *params, direct=True)
+                    orc.lenet5_forward_f32(xl, *params, direct="packed")
                 cpu_ms = (time.perf_counter() - t0) * 1e3 / ncpu
-                lenet.update({"cpu_ms": round(cpu_ms, 3), "cpu_threads": thr, "speedup": round(cpu_ms / gpu_ms, 1),
+                t0 = time.perf_counter()
+                for _ in range(10):
+                    orc.lenet5_forward_f32(xl, *params, direct=True)
+                cpu_axpy_ms = (time.perf_counter() - t0) * 1e3 / 10
+                lenet.update({"cpu_ms": round(cpu_ms, 3), "cpu_threads": thr, "cpu_plain_direct_conv_ms": round(cpu_axpy_ms, 3),
+                              "speedup": round(cpu_ms / gpu_ms, 1),
+                              "speedup_single_kernel": round(cpu_ms / gpu_ms, 1),
+                              "speedup_single_kernel_pipelined": round(cpu_ms / gpu_pipe_ms, 1),
+                              "speedup_api_graph": round(cpu_ms / graph_ms, 1),
+                              "speedup_api_graph_pipelined": round(cpu_ms / graph_pipe_ms, 1),
+                              "speedup_api_eager": round(cpu_ms / fused_eager_ms, 1),
+                              "speedup_api_im2col_eager": round(cpu_ms / layered_ms, 1),
                               "max_abs_diff_vs_cpu": float(np.abs(got - want).max()),
-                              "cpu_what": "oracle port of the host path: direct f32 convolutions over the batch on all "
-                                          "cores (as conv_direct), blocked sgemm on <=4 threads for Dense"})
+                              "cpu_what": "oracle port of the host path: f32 convolutions packed to [f32; 8] and register-tiled as "
+                                          "conv_direct (AVX2 + FMA, images dealt to all cores), relu and pooling over all cores, "
+                                          "blocked sgemm on <=4 threads for Dense; cpu_plain_direct_conv_ms: the same with a plain "
+                                          "axpy convolution loop"})
             extras["lenet5_f32_infer_b1000"] = lenet
             log("lenet5 f32 b=1000:", lenet)
             del model

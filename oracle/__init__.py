@@ -69,6 +69,7 @@ _sig("orc_conv2_naive_f64", [_p, _p, _p] + [_i64] * 13)
 _sig("orc_lenet5_forward_f32", [_p, _i64, _p, _p, _p, _p, _p, _p, _p, C.c_int])
 _sig("orc_lenet5_forward_f32_alg", [_p, _i64, _p, _p, _p, _p, _p, _p, _p, C.c_int, C.c_int])
 _sig("orc_conv2_direct_f32", [_p, _p, _p] + [_i64] * 7)
+_sig("orc_conv2_direct_packed_f32", [_p, _p, _p] + [_i64] * 7 + [C.c_int])
 _sig("orc_max_threads", [], C.c_int)
 _sig("orc_assign4", [_p, _i64, _p, _p, _i64, _p, _p, _i64])
 _sig("orc_scaled_add_f32", [_p, C.c_float, _p, _i64])
@@ -284,14 +285,27 @@ def conv2_direct_f32(x, w):
     return y
 
 
+def conv2_direct_packed_f32(x, w, threads=0):
+    """The reference host's f32 Conv2 for default options as it runs it (conv_direct.rs:84-96, :760-946): packed
+    [f32; 8] layouts and a register-tiled AVX2/FMA kernel, images dealt to `threads` threads (0: all cores)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    bs, ic, ih, iw = x.shape
+    oc, _, fh, fw = w.shape
+    y = np.empty((bs, oc, ih - fh + 1, iw - fw + 1), dtype=np.float32)
+    _lib.orc_conv2_direct_packed_f32(_ptr(x), _ptr(w), _ptr(y), bs, ic, ih, iw, oc, fh, fw, threads)
+    return y
+
+
 def lenet5_forward_f32(x, w1, w2, wd1, wd2, wd3, b3, threads=None, direct=False):
     """Weights: w1 [6,1,5,5], w2 [16,6,5,5], wd* [in,out] (Dense layout, layer.rs:482-486), b3 [10].
-    direct=True runs the convolutions as the reference host does for f32 (conv_direct)."""
+    direct=True runs the convolutions as a plain direct loop, direct="packed" (or 2) as the reference host runs
+    them for f32 (conv_direct: packed layouts, register-tiled kernel)."""
     arrs = [np.ascontiguousarray(a, dtype=np.float32) for a in (x, w1, w2, wd1, wd2, wd3, b3)]
     bs = arrs[0].shape[0]
     out = np.empty((bs, 10), dtype=np.float32)
     _lib.orc_lenet5_forward_f32_alg(_ptr(arrs[0]), bs, *[_ptr(a) for a in arrs[1:]], _ptr(out),
-                                    threads or min(4, max_threads()), 1 if direct else 0)
+                                    threads or min(4, max_threads()), 2 if direct in ("packed", 2) else (1 if direct else 0))
     return out
 
 

@@ -509,8 +509,234 @@ void orc_conv2_direct_f32(const float *x, const float *w, float *y, i64 bs, i64 
         }
 }
 
-/* direct != 0: convolutions through orc_conv2_direct_f32 (what the reference host does for f32);
- * direct == 0: through im2col + sgemm (what conv2_im2col does). */
+/* ------------------------------------- conv_direct, packed and register-tiled ---- */
+
+/* The reference host's f32 Conv2 for default options as it actually runs (layer.rs:936-943 ->
+ * layer/conv_direct.rs:84-96 `conv2_direct_forward`): pack the input to [bs, ic/8, ih, iw][8 channels]
+ * (:368-437; not packed when ic == 1, :288-291), pack the weights to [oc/8, ic/TCX, fh, fw][TCX][8 output
+ * channels] (:487-557), run the register-tiled kernel (:760-946), unpack [bs, oc/8, oh, ow][8] to NCHW
+ * (:692-758).  The kernel keeps a TBY x TWY tile of 8-wide accumulators (TBY blocks of 8 output channels x TWY
+ * output columns; TBY = min(oc/8, 4), TWY = min(15 / (TBY + 1), ow) when compiled with FMA, :766-774, :925-926)
+ * and, per filter tap and input channel, broadcasts TWY input values and multiplies them into TBY weight
+ * vectors with `mul_add` (:799-820).  Images are dealt to threads round robin (`broadcast(Some(bs))`,
+ * tensor/parallel.rs:151-168).  `wide::f32x8` is __m256 here.  Summation order per output: (ic block, fi, fj,
+ * channel within the block), each step one fused multiply-add. */
+#include <immintrin.h>
+
+static inline i64 div_up(i64 a, i64 b) { return a / b + (a % b != 0); }
+
+/* f32x8::transpose of an 8 x 8 tile (rows in r[0..8]) */
+static inline void transpose8x8(__m256 r[8]) {
+    __m256 t0 = _mm256_unpacklo_ps(r[0], r[1]), t1 = _mm256_unpackhi_ps(r[0], r[1]);
+    __m256 t2 = _mm256_unpacklo_ps(r[2], r[3]), t3 = _mm256_unpackhi_ps(r[2], r[3]);
+    __m256 t4 = _mm256_unpacklo_ps(r[4], r[5]), t5 = _mm256_unpackhi_ps(r[4], r[5]);
+    __m256 t6 = _mm256_unpacklo_ps(r[6], r[7]), t7 = _mm256_unpackhi_ps(r[6], r[7]);
+    __m256 u0 = _mm256_shuffle_ps(t0, t2, 0x44), u1 = _mm256_shuffle_ps(t0, t2, 0xEE);
+    __m256 u2 = _mm256_shuffle_ps(t1, t3, 0x44), u3 = _mm256_shuffle_ps(t1, t3, 0xEE);
+    __m256 u4 = _mm256_shuffle_ps(t4, t6, 0x44), u5 = _mm256_shuffle_ps(t4, t6, 0xEE);
+    __m256 u6 = _mm256_shuffle_ps(t5, t7, 0x44), u7 = _mm256_shuffle_ps(t5, t7, 0xEE);
+    r[0] = _mm256_permute2f128_ps(u0, u4, 0x20); r[1] = _mm256_permute2f128_ps(u1, u5, 0x20);
+    r[2] = _mm256_permute2f128_ps(u2, u6, 0x20); r[3] = _mm256_permute2f128_ps(u3, u7, 0x20);
+    r[4] = _mm256_permute2f128_ps(u0, u4, 0x31); r[5] = _mm256_permute2f128_ps(u1, u5, 0x31);
+    r[6] = _mm256_permute2f128_ps(u2, u6, 0x31); r[7] = _mm256_permute2f128_ps(u3, u7, 0x31);
+}
+
+/* pack_input2_host_f32 (conv_direct.rs:368-437): x [bs, ic, ih, iw] -> xp [bs, ic_blocks, ih, iw][8], the eight
+ * channels of a block next to each other, missing channels zero; 8 x 8 tiles transposed in registers. */
+static void cd_pack_input(const float *x, float *xp, i64 bs, i64 ic, i64 ih, i64 iw, int threads) {
+    const i64 icb = div_up(ic, 8), plane = ih * iw;
+#pragma omp parallel num_threads(threads)
+    {
+        const i64 tid = omp_get_thread_num(), nt = omp_get_num_threads();
+        for (i64 b = tid; b < bs; b += nt)
+            for (i64 cb = 0; cb < icb; ++cb) {
+                const float *xs = x + (b * ic + cb * 8) * plane;
+                float *xd = xp + (b * icb + cb) * plane * 8;
+                const i64 nch = ic - cb * 8 < 8 ? ic - cb * 8 : 8;
+                for (i64 h = 0; h < ih; ++h) {
+                    i64 w0 = 0;
+                    for (; w0 + 8 <= iw; w0 += 8) {
+                        __m256 t[8];
+                        for (i64 c = 0; c < 8; ++c)
+                            t[c] = c < nch ? _mm256_loadu_ps(xs + c * plane + h * iw + w0) : _mm256_setzero_ps();
+                        transpose8x8(t);
+                        for (i64 j = 0; j < 8; ++j) _mm256_storeu_ps(xd + (h * iw + w0 + j) * 8, t[j]);
+                    }
+                    if (w0 < iw) {
+                        float tile[8][8];
+                        memset(tile, 0, sizeof(tile));
+                        for (i64 c = 0; c < nch; ++c)
+                            for (i64 j = 0; w0 + j < iw; ++j) tile[c][j] = xs[c * plane + h * iw + w0 + j];
+                        __m256 t[8];
+                        for (i64 c = 0; c < 8; ++c) t[c] = _mm256_loadu_ps(tile[c]);
+                        transpose8x8(t);
+                        for (i64 j = 0; w0 + j < iw; ++j) _mm256_storeu_ps(xd + (h * iw + w0 + j) * 8, t[j]);
+                    }
+                }
+            }
+    }
+}
+
+/* pack_weight2_host_f32<TCX> (conv_direct.rs:487-557): w [oc, ic, fh, fw] -> wp [oc_blocks, ic_blocks, fh, fw][TCX][8],
+ * lane ciy of vector cix = w[8*ob + ciy, TCX*cb + cix, fi, fj]; lanes and vectors beyond oc / ic are zero. */
+static void cd_pack_weight(const float *w, float *wp, i64 oc, i64 ic, i64 fh, i64 fw, i64 tcx) {
+    const i64 ocb = div_up(oc, 8), icb = div_up(ic, tcx);
+    memset(wp, 0, sizeof(float) * (size_t)(ocb * icb * fh * fw * tcx * 8));
+    for (i64 ob = 0; ob < ocb; ++ob)
+        for (i64 cb = 0; cb < icb; ++cb)
+            for (i64 fi = 0; fi < fh; ++fi)
+                for (i64 fj = 0; fj < fw; ++fj)
+                    for (i64 ciy = 0; ciy < 8 && ob * 8 + ciy < oc; ++ciy)
+                        for (i64 cix = 0; cix < tcx && cb * tcx + cix < ic; ++cix)
+                            wp[((((ob * icb + cb) * fh + fi) * fw + fj) * tcx + cix) * 8 + ciy] =
+                                w[(((ob * 8 + ciy) * ic + cb * tcx + cix) * fh + fi) * fw + fj];
+}
+
+/* unpack_output2_host_f32 (conv_direct.rs:692-758): yp [bs, oc_blocks, oh, ow][8] -> y [bs, oc, oh, ow] */
+static void cd_unpack_output(const float *yp, float *y, i64 bs, i64 oc, i64 oh, i64 ow, int threads) {
+    const i64 ocb = div_up(oc, 8), plane = oh * ow;
+#pragma omp parallel num_threads(threads)
+    {
+        const i64 tid = omp_get_thread_num(), nt = omp_get_num_threads();
+        for (i64 b = tid; b < bs; b += nt)
+            for (i64 ob = 0; ob < ocb; ++ob) {
+                const float *ys = yp + (b * ocb + ob) * plane * 8;
+                float *yd = y + (b * oc + ob * 8) * plane;
+                const i64 nch = oc - ob * 8 < 8 ? oc - ob * 8 : 8;
+                for (i64 h = 0; h < oh; ++h) {
+                    i64 w0 = 0;
+                    for (; w0 + 8 <= ow; w0 += 8) {
+                        __m256 t[8];
+                        for (i64 j = 0; j < 8; ++j) t[j] = _mm256_loadu_ps(ys + (h * ow + w0 + j) * 8);
+                        transpose8x8(t);
+                        for (i64 c = 0; c < nch; ++c) _mm256_storeu_ps(yd + c * plane + h * ow + w0, t[c]);
+                    }
+                    if (w0 < ow) {
+                        __m256 t[8];
+                        for (i64 j = 0; j < 8; ++j) t[j] = w0 + j < ow ? _mm256_loadu_ps(ys + (h * ow + w0 + j) * 8) : _mm256_setzero_ps();
+                        transpose8x8(t);
+                        float row[8];
+                        for (i64 c = 0; c < nch; ++c) {
+                            _mm256_storeu_ps(row, t[c]);
+                            for (i64 j = 0; w0 + j < ow; ++j) yd[c * plane + h * ow + w0 + j] = row[j];
+                        }
+                    }
+                }
+            }
+    }
+}
+
+/* `kernel` + the tile loops of `inner` (conv_direct.rs:778-922) for one image, with TCX, TBY, TWY compile-time
+ * constants at every call site (the function is inlined into cd_image_* below), so the accumulator tile lives in
+ * registers as in the reference's const-generic instantiations. */
+static inline __attribute__((always_inline)) void cd_image(const float *x, const float *wp, float *yp, i64 ic, i64 icb,
+                                                            i64 ih, i64 iw, i64 ocb, i64 fh, i64 fw, i64 oh, i64 ow,
+                                                            const int TCX, const int TBY, const int TWY) {
+    for (i64 chunk = 0; chunk * TBY < ocb; ++chunk) {
+        const i64 tby = ocb - chunk * TBY < TBY ? ocb - chunk * TBY : TBY;
+        const float *wc = wp + chunk * TBY * icb * fh * fw * TCX * 8;
+        float *yc = yp + chunk * TBY * oh * ow * 8;
+        for (i64 cb = 0; cb < icb; ++cb) {
+            const i64 tcx = ic - cb * TCX < TCX ? ic - cb * TCX : TCX;
+            const float *xb = x + cb * ih * iw * TCX;
+            for (i64 hy = 0; hy < oh; ++hy)
+                for (i64 wy = 0; wy < ow; wy += TWY) {
+                    const i64 twy = ow - wy < TWY ? ow - wy : TWY;
+                    __m256 acc[4][7];
+                    for (int b = 0; b < TBY; ++b)
+                        for (int t = 0; t < TWY; ++t) acc[b][t] = _mm256_setzero_ps();
+                    if (cb > 0)
+                        for (int b = 0; b < TBY && b < tby; ++b)
+                            for (int t = 0; t < TWY && t < twy; ++t)
+                                acc[b][t] = _mm256_loadu_ps(yc + ((b * oh + hy) * ow + wy + t) * 8);
+                    __m256 xv[7], wv[4];
+                    for (int t = 0; t < TWY; ++t) xv[t] = _mm256_setzero_ps();
+                    for (int b = 0; b < TBY; ++b) wv[b] = _mm256_setzero_ps();
+                    for (i64 fi = 0; fi < fh; ++fi)
+                        for (i64 fj = 0; fj < fw; ++fj)
+                            for (i64 cix = 0; cix < tcx; ++cix) {
+                                if (twy == TWY) {
+                                    for (int t = 0; t < TWY; ++t)
+                                        xv[t] = _mm256_broadcast_ss(xb + ((hy + fi) * iw + wy + fj + t) * TCX + cix);
+                                } else {
+                                    for (int t = 0; t < TWY && t < twy; ++t)
+                                        xv[t] = _mm256_broadcast_ss(xb + ((hy + fi) * iw + wy + fj + t) * TCX + cix);
+                                }
+                                for (int b = 0; b < TBY && b < tby; ++b)
+                                    wv[b] = _mm256_loadu_ps(wc + ((((b * icb + cb) * fh + fi) * fw + fj) * TCX + cix) * 8);
+                                for (int b = 0; b < TBY; ++b)
+                                    for (int t = 0; t < TWY; ++t) acc[b][t] = _mm256_fmadd_ps(xv[t], wv[b], acc[b][t]);
+                            }
+                    for (int b = 0; b < TBY && b < tby; ++b)
+                        for (int t = 0; t < TWY && t < twy; ++t)
+                            _mm256_storeu_ps(yc + ((b * oh + hy) * ow + wy + t) * 8, acc[b][t]);
+                }
+        }
+    }
+}
+
+#define CD_ARGS const float *x, const float *wp, float *yp, i64 ic, i64 icb, i64 ih, i64 iw, i64 ocb, i64 fh, i64 fw, i64 oh, i64 ow
+#define CD_PASS x, wp, yp, ic, icb, ih, iw, ocb, fh, fw, oh, ow
+#define CD_INST(TCX, TBY, TWY) \
+    static __attribute__((noinline)) void cd_image_##TCX##_##TBY##_##TWY(CD_ARGS) { cd_image(CD_PASS, TCX, TBY, TWY); }
+#define CD_INST_TCX(TCX)                                                                                              \
+    CD_INST(TCX, 1, 1) CD_INST(TCX, 1, 2) CD_INST(TCX, 1, 3) CD_INST(TCX, 1, 4) CD_INST(TCX, 1, 5) CD_INST(TCX, 1, 6)  \
+    CD_INST(TCX, 1, 7) CD_INST(TCX, 2, 1) CD_INST(TCX, 2, 2) CD_INST(TCX, 2, 3) CD_INST(TCX, 2, 4) CD_INST(TCX, 2, 5)  \
+    CD_INST(TCX, 3, 1) CD_INST(TCX, 3, 2) CD_INST(TCX, 3, 3) CD_INST(TCX, 4, 1) CD_INST(TCX, 4, 2) CD_INST(TCX, 4, 3)
+CD_INST_TCX(1)
+CD_INST_TCX(8)
+
+typedef void (*cd_image_fn)(CD_ARGS);
+#define CD_ROW(TCX, TBY) \
+    {cd_image_##TCX##_##TBY##_1, cd_image_##TCX##_##TBY##_2, cd_image_##TCX##_##TBY##_3, 0, 0, 0, 0}
+static cd_image_fn cd_pick(i64 tcx, i64 tby, i64 twy) {
+    static const cd_image_fn t1[4][7] = {
+        {cd_image_1_1_1, cd_image_1_1_2, cd_image_1_1_3, cd_image_1_1_4, cd_image_1_1_5, cd_image_1_1_6, cd_image_1_1_7},
+        {cd_image_1_2_1, cd_image_1_2_2, cd_image_1_2_3, cd_image_1_2_4, cd_image_1_2_5, 0, 0}, CD_ROW(1, 3), CD_ROW(1, 4)};
+    static const cd_image_fn t8[4][7] = {
+        {cd_image_8_1_1, cd_image_8_1_2, cd_image_8_1_3, cd_image_8_1_4, cd_image_8_1_5, cd_image_8_1_6, cd_image_8_1_7},
+        {cd_image_8_2_1, cd_image_8_2_2, cd_image_8_2_3, cd_image_8_2_4, cd_image_8_2_5, 0, 0}, CD_ROW(8, 3), CD_ROW(8, 4)};
+    return (tcx == 1 ? t1 : t8)[tby - 1][twy - 1];
+}
+
+/* conv2_direct_forward (conv_direct.rs:84-96) for default options: x [bs, ic, ih, iw], w [oc, ic, fh, fw] ->
+ * y [bs, oc, ih-fh+1, iw-fw+1].  threads <= 0: all cores (rayon's default pool). */
+void orc_conv2_direct_packed_f32(const float *x, const float *w, float *y, i64 bs, i64 ic, i64 ih, i64 iw, i64 oc,
+                                 i64 fh, i64 fw, int threads) {
+    const i64 oh = ih - fh + 1, ow = iw - fw + 1;
+    if (bs <= 0 || oc <= 0 || oh <= 0 || ow <= 0) return;
+    if (threads <= 0) threads = omp_get_max_threads();
+    if ((i64)threads > bs) threads = (int)bs;
+    const i64 tcx = ic == 1 ? 1 : 8;
+    const i64 icb = div_up(ic, tcx), ocb = div_up(oc, 8);
+    const i64 tby = ocb < 4 ? ocb : 4;
+    i64 twy = 15 / (tby + 1);
+    if (twy > ow) twy = ow;
+    float *xp = NULL;
+    if (tcx == 8) {
+        xp = (float *)aligned_alloc(64, sizeof(float) * (size_t)(bs * icb * ih * iw * 8));
+        cd_pack_input(x, xp, bs, ic, ih, iw, threads);
+    }
+    float *wp = (float *)aligned_alloc(64, (sizeof(float) * (size_t)(ocb * icb * fh * fw * tcx * 8) + 63) / 64 * 64);
+    cd_pack_weight(w, wp, oc, ic, fh, fw, tcx);
+    float *yp = (float *)aligned_alloc(64, (sizeof(float) * (size_t)(bs * ocb * oh * ow * 8) + 63) / 64 * 64);
+    const cd_image_fn fn = cd_pick(tcx, tby, twy);
+    const float *xs = tcx == 8 ? xp : x;
+    const i64 x_image = icb * ih * iw * tcx, y_image = ocb * oh * ow * 8;
+#pragma omp parallel num_threads(threads)
+    {
+        const i64 tid = omp_get_thread_num(), nt = omp_get_num_threads();
+        for (i64 b = tid; b < bs; b += nt) fn(xs + b * x_image, wp, yp + b * y_image, ic, icb, ih, iw, ocb, fh, fw, oh, ow);
+    }
+    cd_unpack_output(yp, y, bs, oc, oh, ow, threads);
+    free(xp);
+    free(wp);
+    free(yp);
+}
+
+/* direct == 2: convolutions through orc_conv2_direct_packed_f32, the packed register-tiled form the reference host
+ * runs for f32; direct == 1: through the plain axpy form orc_conv2_direct_f32; direct == 0: through im2col + sgemm
+ * (what conv2_im2col does). */
 void orc_lenet5_forward_f32_alg(const float *x, i64 bs, const float *w1, const float *w2, const float *wd1,
                                 const float *wd2, const float *wd3, const float *b3, float *logits, int threads,
                                 int direct);
@@ -529,11 +755,13 @@ void orc_lenet5_forward_f32_alg(const float *x, i64 bs, const float *w1, const f
     float *p2 = (float *)malloc(sizeof(float) * bs * 16 * 4 * 4);
     float *d1 = (float *)malloc(sizeof(float) * bs * 128);
     float *d2 = (float *)malloc(sizeof(float) * bs * 84);
-    if (direct) orc_conv2_direct_f32(x, w1, c1, bs, 1, 28, 28, 6, 5, 5);
+    if (direct == 2) orc_conv2_direct_packed_f32(x, w1, c1, bs, 1, 28, 28, 6, 5, 5, 0);
+    else if (direct) orc_conv2_direct_f32(x, w1, c1, bs, 1, 28, 28, 6, 5, 5);
     else conv_im2col_f32(x, w1, c1, bs, 1, 28, 28, 6, 5, 5, threads);
     orc_relu_f32(c1, c1, bs * 6 * 24 * 24);
     orc_max_pool2_f32(c1, p1, bs * 6, 24, 24, 2, 2, 2, 2);
-    if (direct) orc_conv2_direct_f32(p1, w2, c2, bs, 6, 12, 12, 16, 5, 5);
+    if (direct == 2) orc_conv2_direct_packed_f32(p1, w2, c2, bs, 6, 12, 12, 16, 5, 5, 0);
+    else if (direct) orc_conv2_direct_f32(p1, w2, c2, bs, 6, 12, 12, 16, 5, 5);
     else conv_im2col_f32(p1, w2, c2, bs, 6, 12, 12, 16, 5, 5, threads);
     orc_relu_f32(c2, c2, bs * 16 * 8 * 8);
     orc_max_pool2_f32(c2, p2, bs * 16, 8, 8, 2, 2, 2, 2);

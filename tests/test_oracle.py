@@ -388,6 +388,36 @@ def test_conv2_direct_host_vs_torch():
         assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(ic * f[0] * f[1]) * np.max(np.abs(want))
 
 
+def test_conv2_direct_packed_host_vs_torch_and_exact_on_integers():
+    """The packed, register-tiled restatement of conv2_direct_host_f32 (conv_direct.rs:760-946) against torch's
+    float64 convolution and, bit for bit, on small-integer data (every sum exact).  Shapes cover: ic == 1 (unpacked
+    input, TCX = 1) and ic > 1 (TCX = 8) with ic below, equal to and above a multiple of 8; oc below 8, a multiple
+    of 8 and above 32 (more than one chunk of four 8-channel blocks, a ragged last chunk); output rows shorter than
+    the column tile, equal to it and with a ragged last tile; one thread and many (images dealt round robin)."""
+    rng = np.random.default_rng(91)
+    shapes = [(3, 1, 28, 28, 6, (5, 5)), (5, 6, 12, 12, 16, (5, 5)), (2, 3, 9, 7, 4, (3, 2)), (2, 8, 6, 6, 8, (1, 1)),
+              (3, 11, 10, 13, 40, (3, 3)), (1, 17, 5, 9, 33, (2, 3)), (4, 1, 7, 3, 9, (2, 2)), (2, 16, 8, 11, 24, (3, 5)),
+              (7, 2, 6, 23, 20, (3, 3))]
+    for (bs, ic, ih, iw, oc, f) in shapes:
+        x = rng.standard_normal((bs, ic, ih, iw)).astype(np.float32)
+        w = rng.standard_normal((oc, ic) + f).astype(np.float32)
+        want = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double()).numpy()
+        for threads in (1, 0):
+            got = orc.conv2_direct_packed_f32(x, w, threads=threads)
+            assert got.shape == want.shape
+            assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(ic * f[0] * f[1]) * np.max(np.abs(want)), (bs, ic, oc, f)
+        xi = rng.integers(-4, 5, (bs, ic, ih, iw)).astype(np.float32)
+        wi = rng.integers(-4, 5, (oc, ic) + f).astype(np.float32)
+        exact = F.conv2d(torch.from_numpy(xi).double(), torch.from_numpy(wi).double()).numpy()
+        assert np.array_equal(orc.conv2_direct_packed_f32(xi, wi).astype(np.float64), exact), (bs, ic, oc, f)
+    # and the LeNet5 forward pass built on it agrees with the im2col + sgemm chain
+    x = rng.uniform(0, 1, (20, 1, 28, 28)).astype(np.float32)
+    params = [rng.standard_normal(s).astype(np.float32) * 0.1 for s in ((6, 1, 5, 5), (16, 6, 5, 5), (256, 128), (128, 84), (84, 10), (10,))]
+    a = orc.lenet5_forward_f32(x, *params, direct="packed")
+    b = orc.lenet5_forward_f32(x, *params)
+    assert np.max(np.abs(a - b)) <= 2e-5 * np.max(np.abs(b))
+
+
 # ------------------------------------------------------------ training tail ----
 def tbf(x):
     """numpy uint16 bf16 bits -> torch.bfloat16 tensor."""
