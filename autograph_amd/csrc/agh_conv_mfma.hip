@@ -57,6 +57,7 @@ struct ConvMfmaParams {
     int nchunk;    // 16-byte chunks per staged pixel
     int K;         // fh*fw*ic
     int per_xcd;   // workgroups per XCD when the grid divides by 8, else 0
+    int remap;     // staging takes the coalesced lane order where it applies (AGH_CONV_REMAP=0 switches it off)
     FastDiv div_ow, div_tiles, div_octiles, div_vec;
 };
 
@@ -116,7 +117,16 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
         // consecutive channel chunks of the same pixels, so a write instruction covers whole staged pixels
         // (contiguous bytes: no bank conflict).
         const int nvec = p.iw / PV, ngrp = p.icc / CPC;
-        const uint32_t items = (uint32_t)lrows * ngrp * nvec;
+        // Item order.  General: channel group fastest, so the lanes of an LDS write cover whole staged pixels.  With
+        // eight channel groups of 16-bit elements (64 channels per pass) the lanes are dealt differently: a wave takes
+        // eight consecutive 16-byte vectors of the rows (rows of a plane follow one another in memory, so the eight are
+        // contiguous) in all eight groups, lane = (vector & 1) + 2 * group + 16 * (vector >> 1).  A load instruction then
+        // touches 8 runs of 128 bytes instead of 64 separate 16-byte pieces in 64 cache lines, and the 16 lanes the LDS
+        // serves together still write 16 different 16-byte bank groups (two neighbouring vectors are 8 pixels = 72
+        // sixteen-byte units apart: 8 mod 16, the eight groups fill the gap).
+        const bool remap = ES == 2 && ngrp == 8 && p.remap;
+        const uint32_t nt = (uint32_t)lrows * nvec;  // 16-byte vectors of one channel plane in the staged rows
+        const uint32_t items = remap ? ((nt + 7) / 8) * 64 : (uint32_t)lrows * ngrp * nvec;
         const T *ximg = x + ((size_t)b * p.ic + (size_t)pass * p.icc) * p.ih * (size_t)p.iw;
         const size_t plane = (size_t)p.ih * p.iw;
         // SB items per thread and trip: all SB * CPC loads are requested before the first LDS write (with two, a
@@ -129,18 +139,25 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
             for (int u = 0; u < SB; ++u) {
                 const uint32_t it = it0 + u * kThreads;
                 uint32_t rv, v, lr, cg;
-                rv = it / (uint32_t)ngrp;
-                cg = it - rv * ngrp;
-                p.div_vec.divmod(rv, lr, v);
+                if (remap) {
+                    const uint32_t L = it & 63u;
+                    cg = (L >> 1) & 7u;
+                    rv = (it >> 6) * 8 + (((L >> 4) << 1) | (L & 1u));
+                } else {
+                    rv = it / (uint32_t)ngrp;
+                    cg = it - rv * ngrp;
+                }
+                const bool live = it < items && rv < nt;
+                p.div_vec.divmod(live ? rv : 0u, lr, v);
                 const int hi = ho_first - p.ph + (int)lr;
 #pragma unroll
                 for (int i = 0; i < CPC; ++i) r[u][i] = make_uint4(0, 0, 0, 0);
-                if (it < items && hi >= 0 && hi < p.ih) {
+                if (live && hi >= 0 && hi < p.ih) {
                     const T *src = ximg + ((size_t)(CPC * cg) * p.ih + hi) * (size_t)p.iw + v * PV;
 #pragma unroll
                     for (int i = 0; i < CPC; ++i) r[u][i] = *(const uint4 *)(src + i * plane);
                 }
-                dst[u] = it < items ? ((int)lr * p.lcols + p.pw + (int)v * PV) * pitch + ((int)cg << 4) : -1;
+                dst[u] = live ? ((int)lr * p.lcols + p.pw + (int)v * PV) * pitch + ((int)cg << 4) : -1;
             }
 #pragma unroll
             for (int u = 0; u < SB; ++u) {
@@ -396,6 +413,10 @@ static int conv2_mfma_launch(const char *name, const void *x, const void *w, con
     p.nchunk = icc / CPC;
     p.K = fh * fw * ic;
     p.per_xcd = blocks % 8 == 0 ? (int)(blocks / 8) : 0;
+    {
+        const char *e = getenv("AGH_CONV_REMAP");
+        p.remap = e && *e ? atoi(e) : 1;
+    }
     p.div_ow = FastDiv((uint32_t)ow);
     p.div_tiles = FastDiv((uint32_t)tiles);
     p.div_octiles = FastDiv((uint32_t)octiles);
