@@ -91,8 +91,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="only the headline GEMM")
     ap.add_argument("--no-graph", action="store_true",
-                    help="training section: time eager launches only, no graph capture / replay (rocprofv3 cannot "
-                         "follow the replay of that graph on this image)")
+                    help="LeNet5 sections: time eager launches only, no graph capture / replay (replaying a captured graph "
+                         "under rocprofv3 has ended in a segmentation fault inside the profiler on this image)")
     ap.add_argument("--sections", default="kernels,lenet,train",
                     help="which extras to run: kernels (other GEMMs, im2col/col2im/pool), lenet (inference), "
                          "train (training step); the last two replay captured graphs")
@@ -365,7 +365,8 @@ def main():
             ag._ffi.check(ag.lib.agh_host_alloc(C.byref(host), bsl * 10 * 4))
             host2 = C.c_void_p()
             ag._ffi.check(ag.lib.agh_host_alloc(C.byref(host2), bsl * 10 * 4))
-            model.capture(txl, host2.value)  # layered forward (5 launches) + D2H of the logits, as one graph
+            if not args.no_graph:
+                model.capture(txl, host2.value)  # layered forward (5 launches) + D2H of the logits, as one graph
 
             def wall(fn, nwarm=100, nrep=1000):
                 for _ in range(nwarm):
@@ -406,16 +407,20 @@ def main():
 
             gpu_ms = wall(infer)
             got = np.ctypeslib.as_array(C.cast(host.value, C.POINTER(C.c_float)), shape=(bsl, 10)).copy()
-            graph_ms = wall(infer_graph, 50, 300)
             gpu_pipe_ms = pipelined(lambda: lenet_fn(*lenet_args))
-            graph_pipe_ms = pipelined(model.replay, 50, 300)
+            if args.no_graph:
+                graph_ms = graph_pipe_ms = None
+            else:
+                graph_ms = wall(infer_graph, 50, 300)
+                graph_pipe_ms = pipelined(model.replay, 50, 300)
             _, kernel_ms = timer.time(lambda: model.forward_single_launch(txl, host.value), 50, 20)
             # layer-by-layer path (12 launches, im2col + gemm convolutions), eager, each layer allocating its output
             _, layered_ms = timer.time(lambda: model.forward(txl, algorithm="im2col"), 20, 5)
             # the same layer objects with each layer's own fused form (conv+relu+pool, dense+relu): 5 launches, eager
             _, fused_eager_ms = timer.time(lambda: model.forward_fused(txl), 20, 5)
             lenet = {"gpu_ms": round(gpu_ms, 4), "gpu_kernel_ms": round(kernel_ms, 4), "gpu_pipelined_ms": round(gpu_pipe_ms, 4),
-                     "gpu_graph_5_launches_ms": round(graph_ms, 4), "gpu_graph_5_launches_pipelined_ms": round(graph_pipe_ms, 4),
+                     "gpu_graph_5_launches_ms": None if graph_ms is None else round(graph_ms, 4),
+                     "gpu_graph_5_launches_pipelined_ms": None if graph_pipe_ms is None else round(graph_pipe_ms, 4),
                      "gpu_layered_5_launches_eager_ms": round(fused_eager_ms, 4),
                      "gpu_layered_im2col_eager_ms": round(layered_ms, 4),
                      "what": "gpu_ms: one launch of the whole-network kernel (input resident in HBM, [1000,10] logits written "
@@ -442,8 +447,8 @@ def main():
                               "speedup": round(cpu_ms / gpu_ms, 1),
                               "speedup_single_kernel": round(cpu_ms / gpu_ms, 1),
                               "speedup_single_kernel_pipelined": round(cpu_ms / gpu_pipe_ms, 1),
-                              "speedup_api_graph": round(cpu_ms / graph_ms, 1),
-                              "speedup_api_graph_pipelined": round(cpu_ms / graph_pipe_ms, 1),
+                              "speedup_api_graph": None if graph_ms is None else round(cpu_ms / graph_ms, 1),
+                              "speedup_api_graph_pipelined": None if graph_pipe_ms is None else round(cpu_ms / graph_pipe_ms, 1),
                               "speedup_api_eager": round(cpu_ms / fused_eager_ms, 1),
                               "speedup_api_im2col_eager": round(cpu_ms / layered_ms, 1),
                               "max_abs_diff_vs_cpu": float(np.abs(got - want).max()),
