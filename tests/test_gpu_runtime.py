@@ -195,6 +195,83 @@ def test_block_freed_under_an_unjoined_branch_is_reused_safely(ag):
         del res, again
 
 
+def test_free_during_capture_is_deferred_not_lost(ag):
+    """A host-side temporary may be dropped at any moment, also while a graph is being captured (the garbage collector
+    does not ask).  agh_free then sets the block aside: it is neither handed to the driver nor reused inside the
+    capture, and agh_graph_end files it with the cached blocks, so nothing leaks."""
+    rng = np.random.default_rng(61)
+    a = ag.Tensor.from_array(rng.uniform(-1, 1, (64, 64)).astype(np.float32))
+    out = ag.Tensor.uninit((64, 64), "f32")
+    victim = ag.Tensor.uninit((12345,), "f32")          # a size class of its own
+    ag.gemm(1.0, a, a, 0.0, out)                          # eager run first
+    ag._ffi.check(ag.lib.agh_sync())
+    cached0, blocks0, live0 = cache_stats(ag)
+    ag._ffi.check(ag.lib.agh_graph_begin())
+    try:
+        ag.gemm(1.0, a, a, 0.0, out)
+        ptr = victim.buffer.ptr
+        rc = ag.lib.agh_free(ptr)                         # what Buffer.__del__ does
+        victim.buffer.ptr = None
+        assert rc == 0
+        # not reusable yet, but no longer counted as handed out
+        assert cache_stats(ag)[2] == live0 - 1 and cache_stats(ag)[1] == blocks0
+    finally:
+        g = C.c_void_p()
+        ag._ffi.check(ag.lib.agh_graph_end(C.byref(g)))
+    try:
+        cached1, blocks1, live1 = cache_stats(ag)
+        assert live1 == live0 - 1 and blocks1 == blocks0 + 1 and cached1 > cached0
+        again = ag.Tensor.uninit((12345,), "f32")         # the same size class: the deferred block comes back
+        assert again.buffer.ptr == ptr
+        ag._ffi.check(ag.lib.agh_graph_launch(g))
+        ag._ffi.check(ag.lib.agh_sync())
+    finally:
+        ag._ffi.check(ag.lib.agh_graph_destroy(g))
+
+
+def test_graph_replay_joins_an_open_branch_first(ag, monkeypatch):
+    """A graph captured with a branch names the second stream's split-K workspace in its fork arm.  Eager split-K work
+    inside a branch that has not been joined may still be using that block when the graph is replayed: agh_graph_launch
+    orders the replay behind it.  Both products must come out as they do alone, on every repetition."""
+    rng = np.random.default_rng(62)
+    dy1, c1 = rng.normal(0, 1, (57600, 6)).astype(np.float32), rng.normal(0, 1, (57600, 25)).astype(np.float32)
+    dy2, c2 = rng.normal(0, 1, (36864, 48)).astype(np.float32), rng.normal(0, 1, (36864, 40)).astype(np.float32)
+    t1a, t1b, t2a, t2b = (ag.Tensor.from_array(v) for v in (dy1, c1, dy2, c2))
+    out1, out2 = ag.Tensor.uninit((6, 25), "f32"), ag.Tensor.uninit((48, 40), "f32")
+    # serial results; the second product also sizes the second stream's workspace for both
+    with ag.branch():
+        ag.gemm(1.0, t2a.t(), t2b, 0.0, out2)
+        ag.gemm(1.0, t1a.t(), t1b, 0.0, out1)
+    ag.join()
+    want1, want2 = out1.into_array(), out2.into_array()
+    ag._ffi.check(ag.lib.agh_graph_begin())
+    try:
+        with ag.branch():
+            ag.gemm(1.0, t1a.t(), t1b, 0.0, out1)
+        ag.join()
+    finally:
+        g = C.c_void_p()
+        ag._ffi.check(ag.lib.agh_graph_end(C.byref(g)))
+    try:
+        for i in range(6):
+            ag._ffi.check(ag.lib.agh_memset(out1._ptr(), 0xFF, 6 * 25 * 4))
+            ag._ffi.check(ag.lib.agh_memset(out2._ptr(), 0xFF, 48 * 40 * 4))
+            with ag.branch():                              # eager split-K product on the second stream, not joined
+                ag.gemm(1.0, t2a.t(), t2b, 0.0, out2)
+            ag._ffi.check(ag.lib.agh_graph_launch(g))      # the captured arm uses the same workspace
+            ag.join()
+            assert np.array_equal(out1.into_array(), want1), i
+            assert np.array_equal(out2.into_array(), want2), i
+        # a replay is refused inside a branch
+        ag._ffi.check(ag.lib.agh_branch_begin())
+        rc = ag.lib.agh_graph_launch(g)
+        ag._ffi.check(ag.lib.agh_branch_end())
+        ag.join()
+        assert rc == -1
+    finally:
+        ag._ffi.check(ag.lib.agh_graph_destroy(g))
+
+
 def test_calibration_launches(ag):
     """The measurement-only launches behind `bench.py --calib` (benchlib/, a library of its own): the copy and the read:write mix move exactly the bytes
     they claim (checked bit for bit on a small buffer), the MFMA loops run in both instruction shapes with and without
