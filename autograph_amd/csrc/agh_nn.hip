@@ -457,7 +457,7 @@ __global__ __launch_bounds__(kThreads) void col2im_ring_kernel(const T *__restri
             uint32_t wi, k;
             p.div_lw.divmod(e, wi, k);
             reg[i] = 0;
-            if (e < nwords) reg[i] = __builtin_nontemporal_load(src + (size_t)wi * ktotw + k);
+            if (e < nwords) reg[i] = src[(size_t)wi * ktotw + k];
         }
     };
     auto slot_to = [](uint32_t v) -> T {
@@ -607,7 +607,7 @@ __global__ __launch_bounds__(kThreads) void col2im_ring_unit_kernel(const T *__r
             // rows past the last one re-read it (never used): keeps the loads unconditional per row
             const int hr = min(hi + r, hi_hi);
             const uint32_t *src = (const uint32_t *)(x + ((size_t)b * p.gh + hr) * p.gw * p.ktot + (size_t)c0 * ff);
-            if (src_off[i] != 0xFFFFFFFFu) reg[i] = __builtin_nontemporal_load((const u32x4 *)(src + src_off[i]));
+            if (src_off[i] != 0xFFFFFFFFu) reg[i] = *(const u32x4 *)(src + src_off[i]);
         }
     };
 
@@ -1103,30 +1103,60 @@ __global__ __launch_bounds__(kThreads) void max_pool2_backward_kernel(T *__restr
 
 // 2x2 windows, stride 2, rows of whole 16-byte vectors: a work item is one 16-byte vector from each of the two
 // rows of a row pair (4 f32 / 8 bf16 elements: 2 / 4 neighbouring windows), so every load instruction of a wave
-// covers 1 KB of contiguous memory, and the 8 bytes of results leave as one streaming store.  The grid is sized to
+// covers 1 KB of the row pair's memory, and the 8 bytes of results leave as one store.  The grid is sized to
 // the chip and strides over the items two at a time: both items' loads are in flight before the first compare.
+// Loads and stores carry no streaming hint: a pooling layer sits between a producer and a consumer, and activations
+// of this size (a few hundred MB at most) are served from, and left in, the last-level cache.
 // Same visiting order inside a window as the general kernel: (0,0), (0,1), (1,0), (1,1), strictly-greater wins.
+//
+// The windows are worked on as f32 values throughout: a bf16 cell is its 16 bits in the high half of a dword (the low
+// half of a loaded dword shifted up, the high half masked), the winner's bits are the high half of the winning f32.
+// The launch streams 1.25 bytes per input byte and has nothing else to hide behind, so the instruction count per
+// window matters: with EVEN (ih == 2 * oh, no row left over at the bottom of a plane) row pairs follow one another
+// through the whole tensor and an item's place needs one division, not two.
 template <typename T>
 struct PoolVec {
     static constexpr int VEC = 16 / (int)sizeof(T), NW = VEC / 2;
-    T e[VEC];
 };
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 struct Pool2x2Item {
     size_t in_off, out_off;  // element offsets of the row pair's vector and of its outputs
 };
+template <bool EVEN>
 __device__ __forceinline__ Pool2x2Item pool2x2_item(const PoolParams &p, uint32_t g, int vec) {
-    uint32_t orow, gi, plane, ho;
-    p.div_gpr.divmod(g, orow, gi);     // orow = plane * oh + ho
-    p.div_oh.divmod(orow, plane, ho);
     Pool2x2Item it;
-    it.in_off = ((size_t)plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)gi * vec;
-    it.out_off = (size_t)orow * p.ow + (size_t)gi * (vec / 2);
+    if constexpr (EVEN) {
+        const uint32_t orow = p.div_gpr.div(g);  // row pair, counted through all planes
+        it.in_off = (size_t)(g + orow * p.div_gpr.d) * (size_t)vec;  // vectors before it: 2 * orow * gpr + gi
+        it.out_off = (size_t)g * (size_t)(vec / 2);
+    } else {
+        uint32_t orow, gi, plane, ho;
+        p.div_gpr.divmod(g, orow, gi);     // orow = plane * oh + ho
+        p.div_oh.divmod(orow, plane, ho);
+        it.in_off = ((size_t)plane * p.ih + (size_t)ho * 2) * p.iw + (size_t)gi * vec;
+        it.out_off = (size_t)orow * p.ow + (size_t)gi * (vec / 2);
+    }
     return it;
 }
 
+// window k of an item as four f32 values in visiting order, from the two rows' vectors
 template <typename T>
+__device__ __forceinline__ void pool2x2_window(const u32x4 &r0, const u32x4 &r1, int k, float (&f)[4]) {
+    if constexpr (sizeof(T) == 4) {
+        f[0] = __uint_as_float(r0[2 * k]); f[1] = __uint_as_float(r0[2 * k + 1]);
+        f[2] = __uint_as_float(r1[2 * k]); f[3] = __uint_as_float(r1[2 * k + 1]);
+    } else {
+        f[0] = __uint_as_float(r0[k] << 16); f[1] = __uint_as_float(r0[k] & 0xFFFF0000u);
+        f[2] = __uint_as_float(r1[k] << 16); f[3] = __uint_as_float(r1[k] & 0xFFFF0000u);
+    }
+}
+// two bf16 values, each the high half of an f32, as one dword (lo in the low half)
+__device__ __forceinline__ uint32_t pack_high_halves(float lo, float hi) {
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+
+template <typename T, bool EVEN>
 __global__ __launch_bounds__(kThreads) void max_pool2_2x2_kernel(const T *__restrict__ x, T *__restrict__ y,
                                                                   PoolParams p, uint32_t groups) {
     constexpr int VEC = PoolVec<T>::VEC, NW = PoolVec<T>::NW;
@@ -1134,34 +1164,37 @@ __global__ __launch_bounds__(kThreads) void max_pool2_2x2_kernel(const T *__rest
     for (uint32_t g0 = blockIdx.x * kThreads + threadIdx.x; g0 < groups; g0 += 2 * stride) {
         const uint32_t g1 = g0 + stride;
         const bool two = g1 < groups;
-        const Pool2x2Item it0 = pool2x2_item(p, g0, VEC), it1 = pool2x2_item(p, two ? g1 : g0, VEC);
-        PoolVec<T> r[2][2];
-        *(u32x4 *)r[0][0].e = __builtin_nontemporal_load((const u32x4 *)(x + it0.in_off));
-        *(u32x4 *)r[0][1].e = __builtin_nontemporal_load((const u32x4 *)(x + it0.in_off + p.iw));
-        *(u32x4 *)r[1][0].e = __builtin_nontemporal_load((const u32x4 *)(x + it1.in_off));
-        *(u32x4 *)r[1][1].e = __builtin_nontemporal_load((const u32x4 *)(x + it1.in_off + p.iw));
+        const Pool2x2Item it0 = pool2x2_item<EVEN>(p, g0, VEC), it1 = pool2x2_item<EVEN>(p, two ? g1 : g0, VEC);
+        u32x4 r[2][2];
+        r[0][0] = *(const u32x4 *)(x + it0.in_off);
+        r[0][1] = *(const u32x4 *)(x + it0.in_off + p.iw);
+        r[1][0] = *(const u32x4 *)(x + it1.in_off);
+        r[1][1] = *(const u32x4 *)(x + it1.in_off + p.iw);
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             if (u == 1 && !two) break;
-            __align__(8) T out[NW];
+            float mf[NW];
 #pragma unroll
             for (int k = 0; k < NW; ++k) {
-                T m = r[u][0].e[2 * k];
-                float mf = Elem<T>::raw(m);
-                const T c[3] = {r[u][0].e[2 * k + 1], r[u][1].e[2 * k], r[u][1].e[2 * k + 1]};
+                float f[4];
+                pool2x2_window<T>(r[u][0], r[u][1], k, f);
+                mf[k] = f[0];
 #pragma unroll
-                for (int q = 0; q < 3; ++q) {
-                    const float vf = Elem<T>::raw(c[q]);
-                    if (vf > mf) { m = c[q]; mf = vf; }
-                }
-                out[k] = m;
+                for (int q = 1; q < 4; ++q)
+                    if (f[q] > mf[k]) mf[k] = f[q];
             }
-            __builtin_nontemporal_store(*(const u32x2 *)out, (u32x2 *)(y + (u ? it1.out_off : it0.out_off)));
+            u32x2 out;
+            if constexpr (sizeof(T) == 4) {
+                out[0] = __float_as_uint(mf[0]); out[1] = __float_as_uint(mf[1]);
+            } else {
+                out[0] = pack_high_halves(mf[0], mf[1]); out[1] = pack_high_halves(mf[2], mf[3]);
+            }
+            *(u32x2 *)(y + (u ? it1.out_off : it0.out_off)) = out;
         }
     }
 }
 
-template <typename T>
+template <typename T, bool EVEN>
 __global__ __launch_bounds__(kThreads) void max_pool2_backward_2x2_kernel(T *__restrict__ dx, const T *__restrict__ dy,
                                                                            PoolParams p, uint32_t groups) {
     constexpr int VEC = PoolVec<T>::VEC, NW = PoolVec<T>::NW;
@@ -1169,38 +1202,49 @@ __global__ __launch_bounds__(kThreads) void max_pool2_backward_2x2_kernel(T *__r
     for (uint32_t g0 = blockIdx.x * kThreads + threadIdx.x; g0 < groups; g0 += 2 * stride) {
         const uint32_t g1 = g0 + stride;
         const bool two = g1 < groups;
-        const Pool2x2Item it0 = pool2x2_item(p, g0, VEC), it1 = pool2x2_item(p, two ? g1 : g0, VEC);
-        PoolVec<T> r[2][2];
-        __align__(8) T gy[2][NW];
-        *(u32x4 *)r[0][0].e = __builtin_nontemporal_load((const u32x4 *)(dx + it0.in_off));
-        *(u32x4 *)r[0][1].e = __builtin_nontemporal_load((const u32x4 *)(dx + it0.in_off + p.iw));
-        *(u32x2 *)gy[0] = __builtin_nontemporal_load((const u32x2 *)(dy + it0.out_off));
-        *(u32x4 *)r[1][0].e = __builtin_nontemporal_load((const u32x4 *)(dx + it1.in_off));
-        *(u32x4 *)r[1][1].e = __builtin_nontemporal_load((const u32x4 *)(dx + it1.in_off + p.iw));
-        *(u32x2 *)gy[1] = __builtin_nontemporal_load((const u32x2 *)(dy + it1.out_off));
+        const Pool2x2Item it0 = pool2x2_item<EVEN>(p, g0, VEC), it1 = pool2x2_item<EVEN>(p, two ? g1 : g0, VEC);
+        u32x4 r[2][2];
+        u32x2 gy[2];
+        r[0][0] = *(const u32x4 *)(dx + it0.in_off);
+        r[0][1] = *(const u32x4 *)(dx + it0.in_off + p.iw);
+        gy[0] = *(const u32x2 *)(dy + it0.out_off);
+        r[1][0] = *(const u32x4 *)(dx + it1.in_off);
+        r[1][1] = *(const u32x4 *)(dx + it1.in_off + p.iw);
+        gy[1] = *(const u32x2 *)(dy + it1.out_off);
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             if (u == 1 && !two) break;
+            u32x4 o0, o1;
 #pragma unroll
             for (int k = 0; k < NW; ++k) {
-                float mf = Elem<T>::raw(r[u][0].e[2 * k]);
-                int am = 0;
-                const T c[3] = {r[u][0].e[2 * k + 1], r[u][1].e[2 * k], r[u][1].e[2 * k + 1]};
-#pragma unroll
-                for (int q = 0; q < 3; ++q) {
-                    const float vf = Elem<T>::raw(c[q]);
-                    if (vf > mf) { mf = vf; am = q + 1; }
+                float f[4];
+                pool2x2_window<T>(r[u][0], r[u][1], k, f);
+                // `0 + dy` in T, as the host's `+=` on the zeroed cell computes it.  c[q]: what the window's dwords
+                // hold if cell q wins (f32: the cell itself; bf16: the pair of cells of its row)
+                uint32_t gbits;
+                if constexpr (sizeof(T) == 4) {
+                    gbits = __float_as_uint(0.0f + __uint_as_float(gy[u][k]));
+                } else {
+                    const uint32_t gd = gy[u][k >> 1];
+                    gbits = f32_to_bf16(0.0f + __uint_as_float((k & 1) ? (gd & 0xFFFF0000u) : (gd << 16)));
                 }
-                // `0 + dy` in T, as the host's `+=` on the zeroed cell computes it
-                const T gv = Elem<T>::from_f32(0.0f + Elem<T>::raw(gy[u][k]));
-                r[u][0].e[2 * k] = am == 0 ? gv : Elem<T>::zero();
-                r[u][0].e[2 * k + 1] = am == 1 ? gv : Elem<T>::zero();
-                r[u][1].e[2 * k] = am == 2 ? gv : Elem<T>::zero();
-                r[u][1].e[2 * k + 1] = am == 3 ? gv : Elem<T>::zero();
+                float mf = f[0];
+                int am = 0;
+#pragma unroll
+                for (int q = 1; q < 4; ++q)
+                    if (f[q] > mf) { mf = f[q]; am = q; }
+                if constexpr (sizeof(T) == 4) {
+                    o0[2 * k] = am == 0 ? gbits : 0u; o0[2 * k + 1] = am == 1 ? gbits : 0u;
+                    o1[2 * k] = am == 2 ? gbits : 0u; o1[2 * k + 1] = am == 3 ? gbits : 0u;
+                } else {
+                    const uint32_t placed = (am & 1) ? (gbits << 16) : gbits;
+                    o0[k] = am < 2 ? placed : 0u;
+                    o1[k] = am < 2 ? 0u : placed;
+                }
             }
             T *win = dx + (u ? it1.in_off : it0.in_off);
-            __builtin_nontemporal_store(*(const u32x4 *)r[u][0].e, (u32x4 *)win);
-            __builtin_nontemporal_store(*(const u32x4 *)r[u][1].e, (u32x4 *)(win + p.iw));
+            *(u32x4 *)win = o0;
+            *(u32x4 *)(win + p.iw) = o1;
         }
     }
 }
@@ -1276,8 +1320,12 @@ int max_pool2_launch(const char *name, const void *x, void *y, int64_t bc, int64
         constexpr int VEC = 16 / (int)sizeof(T);
         const size_t groups = total / (VEC / 2);
         p.div_gpr = FastDiv((uint32_t)(p.iw / VEC));
-        hipLaunchKernelGGL(max_pool2_2x2_kernel<T>, dim3(pool_2x2_grid(groups)), dim3(kThreads),
-                           0, stream(), (const T *)x, (T *)y, p, (uint32_t)groups);
+        if (p.ih == 2 * p.oh)
+            hipLaunchKernelGGL((max_pool2_2x2_kernel<T, true>), dim3(pool_2x2_grid(groups)), dim3(kThreads),
+                               0, stream(), (const T *)x, (T *)y, p, (uint32_t)groups);
+        else
+            hipLaunchKernelGGL((max_pool2_2x2_kernel<T, false>), dim3(pool_2x2_grid(groups)), dim3(kThreads),
+                               0, stream(), (const T *)x, (T *)y, p, (uint32_t)groups);
         AGH_LAUNCH_CHECK(name);
         return AGH_OK;
     }
@@ -1300,8 +1348,12 @@ int max_pool2_backward_launch(const char *name, void *dx, const void *dy, int64_
         constexpr int VEC = 16 / (int)sizeof(T);
         const size_t groups = total / (VEC / 2);
         p.div_gpr = FastDiv((uint32_t)(p.iw / VEC));
-        hipLaunchKernelGGL(max_pool2_backward_2x2_kernel<T>, dim3(pool_2x2_grid(groups)),
-                           dim3(kThreads), 0, stream(), (T *)dx, (const T *)dy, p, (uint32_t)groups);
+        if (p.ih == 2 * p.oh)
+            hipLaunchKernelGGL((max_pool2_backward_2x2_kernel<T, true>), dim3(pool_2x2_grid(groups)),
+                               dim3(kThreads), 0, stream(), (T *)dx, (const T *)dy, p, (uint32_t)groups);
+        else
+            hipLaunchKernelGGL((max_pool2_backward_2x2_kernel<T, false>), dim3(pool_2x2_grid(groups)),
+                               dim3(kThreads), 0, stream(), (T *)dx, (const T *)dy, p, (uint32_t)groups);
     } else if (sh >= h && sw >= w) {
         size_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > 0x7FFFFFFFull) return fail(AGH_ERANGE, "%s: too many elements", name);
