@@ -42,6 +42,52 @@ __device__ __forceinline__ T round_bias_relu(float acc, bool has_bias, T bias, i
     return (act == AGH_ACT_RELU && neg) ? Elem<T>::zero() : r;
 }
 
+// Fills n LDS slots from global memory with U reads of a thread in flight at a time: `get(e)` reads (it is called
+// with e < n only and must not fault), `put(e, v)` stores.  Written as two unrolled passes because a plain
+// `for (e...) lds[e] = g[...]` loop compiles to one read, one wait and one store per trip, and a workgroup that stages
+// a few thousand values that way spends most of its life in a dozen memory round trips one after another.
+template <int U, typename V, typename Get, typename Put>
+__device__ __forceinline__ void staged_fill(int n, Get get, Put put) {
+    const int step = (int)blockDim.x;
+    for (int base = (int)threadIdx.x; base < n; base += U * step) {
+        V v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = get(min(base + u * step, n - 1));
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (base + u * step < n) put(base + u * step, v[u]);
+    }
+}
+
+// The two halves of staged_fill for one batch of U slots starting at slot `first`, so that a kernel can put the
+// reads of several regions (filter bank, images) in flight before it stores any of them.
+template <int U, typename V, typename Get>
+__device__ __forceinline__ void batch_read(V (&v)[U], int first, int n, Get get) {
+    const int step = (int)blockDim.x, base = first + (int)threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = get(min(base + u * step, n - 1));
+}
+template <int U, typename V, typename Put>
+__device__ __forceinline__ void batch_store(const V (&v)[U], int first, int n, Put put) {
+    const int step = (int)blockDim.x, base = first + (int)threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+        if (base + u * step < n) put(base + u * step, v[u]);
+}
+// slots [first, n) by staged_fill
+template <int U, typename V, typename Get, typename Put>
+__device__ __forceinline__ void staged_fill_from(int first, int n, Get get, Put put) {
+    const int step = (int)blockDim.x;
+    for (int base = first + (int)threadIdx.x; base < n; base += U * step) {
+        V v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = get(min(base + u * step, n - 1));
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (base + u * step < n) put(base + u * step, v[u]);
+    }
+}
+
 template <typename T, int OCT, bool POOL>
 __global__ __launch_bounds__(256) void conv2_direct_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                             const T *__restrict__ bias, T *__restrict__ y,
@@ -54,12 +100,15 @@ __global__ __launch_bounds__(256) void conv2_direct_kernel(const T *__restrict__
     const int b0 = blockIdx.x * p.imgs;
     const int nimg = min(p.imgs, p.bs - b0);
 
-    for (int e = threadIdx.x; e < taps * p.ocpad; e += blockDim.x) {
-        const int tap = e / p.ocpad, o = e - tap * p.ocpad;
-        ws[e] = o < p.oc ? Elem<T>::to_f32(w[(size_t)o * taps + tap]) : 0.0f;
-    }
+    staged_fill<8, T>(
+        taps * p.ocpad,
+        [&](int e) {
+            const int tap = e / p.ocpad, o = min(e - tap * p.ocpad, p.oc - 1);
+            return w[(size_t)o * taps + tap];
+        },
+        [&](int e, T v) { ws[e] = (e % p.ocpad) < p.oc ? Elem<T>::to_f32(v) : 0.0f; });
     const T *xb = x + (size_t)b0 * img_sz;
-    for (int e = threadIdx.x; e < nimg * img_sz; e += blockDim.x) xs[e] = Elem<T>::to_f32(xb[e]);
+    staged_fill<8, T>(nimg * img_sz, [&](int e) { return xb[e]; }, [&](int e, T v) { xs[e] = Elem<T>::to_f32(v); });
     __syncthreads();
 
     constexpr int NPIX = POOL ? 4 : 1;
@@ -157,21 +206,39 @@ __global__ __launch_bounds__(256) void conv2_rowtile_kernel(const T *__restrict_
     const int b0 = blockIdx.x * p.imgs;
     const int nimg = min(p.imgs, p.bs - b0);
 
-    for (int e = threadIdx.x; e < taps * p.ocpad; e += blockDim.x) {
-        uint32_t tap, o;
-        p.div_ocpad.divmod((uint32_t)e, tap, o);
-        ws[e] = (int)o < p.oc ? Elem<T>::to_f32(w[(size_t)o * taps + tap]) : 0.0f;
-    }
-    for (int e = threadIdx.x; e < nimg * img_sz; e += blockDim.x) {
+    staged_fill<8, T>(
+        taps * p.ocpad,
+        [&](int e) {
+            uint32_t tap, o;
+            p.div_ocpad.divmod((uint32_t)e, tap, o);
+            return w[(size_t)min((int)o, p.oc - 1) * taps + tap];
+        },
+        [&](int e, T v) {
+            uint32_t tap, o;
+            p.div_ocpad.divmod((uint32_t)e, tap, o);
+            ws[e] = (int)o < p.oc ? Elem<T>::to_f32(v) : 0.0f;
+        });
+    // the padding cells read the nearest cell of the image (a valid address) and store zero
+    auto cell = [&](int e, int &hi, int &wi) -> size_t {
         uint32_t r1, col, r2, row;  // r2 = img * ic + channel
         p.div_pitch.divmod((uint32_t)e, r1, col);
         p.div_ihp.divmod(r1, r2, row);
-        const int hi = (int)row - p.ph, wi = (int)col - p.pw;
-        float v = 0.0f;
-        if (hi >= 0 && hi < p.ih && wi >= 0 && wi < p.iw)
-            v = Elem<T>::to_f32(x[((size_t)b0 * p.ic + r2) * p.ih * p.iw + (size_t)hi * p.iw + wi]);
-        xs[e] = v;
-    }
+        hi = (int)row - p.ph;
+        wi = (int)col - p.pw;
+        return ((size_t)b0 * p.ic + r2) * p.ih * p.iw;
+    };
+    staged_fill<8, T>(
+        nimg * img_sz,
+        [&](int e) {
+            int hi, wi;
+            const size_t plane = cell(e, hi, wi);
+            return x[plane + (size_t)min(max(hi, 0), p.ih - 1) * p.iw + min(max(wi, 0), p.iw - 1)];
+        },
+        [&](int e, T v) {
+            int hi, wi;
+            cell(e, hi, wi);
+            xs[e] = (hi >= 0 && hi < p.ih && wi >= 0 && wi < p.iw) ? Elem<T>::to_f32(v) : 0.0f;
+        });
     __syncthreads();
 
     const int total = nimg * p.items_per_img;
@@ -252,6 +319,179 @@ __global__ __launch_bounds__(256) void conv2_rowtile_kernel(const T *__restrict_
                 for (int t = 0; t < WT; ++t) {
                     const int px = wb * WT + t;
                     if (live && px < p.yw) yp[px] = round_bias_relu<T>(acc[0][t][o], p.has_bias != 0, bv, p.act);
+                }
+            }
+        }
+    }
+}
+
+// ---- few channels, small images: implicit GEMM on v_mfma_f32_16x16x4_f32 ----
+//
+// The layers of small networks (LeNet5's conv2: 6 -> 16 channels on 12 x 12 images) have too few outputs per image to
+// fill the chip with register tiles and too many multiply-adds per output (150) for one thread each: the row-tiled
+// kernel spends 17 us on conv2 at batch 1000, three quarters of it a single wave per SIMD walking its 2400 FMAs.
+// Here the same staged (zero-padded) images feed the matrix pipes: a 16 x 16 x 4 MFMA takes 16 output positions of one
+// image (rows), up to 16 output channels (columns) and 4 taps.  The A operand is gathered straight from the staged
+// image, one 4-byte LDS read per lane (position base + tap offset; the offsets of all taps sit in a small LDS table);
+// the B operand is the filter bank as [tap][16] in LDS.  With the pool fused, the 16 rows of a tile are 4 whole 2 x 2
+// windows, cell-minor: the accumulator layout (lane group g holds rows 4g .. 4g+3) then leaves each lane one complete
+// window of one channel, and bias, ReLU and the first-strict-maximum pooling happen in registers.
+// A wave takes (image, TG consecutive tiles) units; the k loop runs in chunks of 8 steps whose B values and tap
+// offsets are fetched one chunk ahead.  f32 accumulation like every other kernel here; the summation order over the
+// taps differs from the row-tiled kernel's (4 partial chains), which the f32 tolerance of the tests covers.
+struct SmallMfmaParams {
+    int bs, ic, ih, iw, oc, oh, ow, fh, fw, ph, pw;
+    int act, has_bias;
+    int imgs;           // images per workgroup
+    int ihp, pitch;     // staged rows per channel and their pitch (floats)
+    int ktot, ksteps;   // taps; k steps of 4 (a multiple of 8, the taps beyond ktot multiply zeros)
+    int nout;           // results per image and channel: positions, or windows with the pool
+    int mtiles;         // 16-row tiles per image
+    int units_per_img;  // ceil(mtiles / TG)
+    int yw;             // width of the result (pooled or not)
+    FastDiv div_pitch, div_ihp, div_yw, div_fw, div_fhfw, div_upi;
+};
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <typename T, bool POOL, int TG>
+__global__ __launch_bounds__(256) void conv2_small_mfma_kernel(const T *__restrict__ x, const T *__restrict__ w,
+                                                                const T *__restrict__ bias, T *__restrict__ y,
+                                                                SmallMfmaParams p) {
+    extern __shared__ __align__(16) float smem_f[];
+    const int kpad = p.ksteps * 4;
+    float *Bs = smem_f;                          // [kpad][16]
+    int *tapoff = (int *)(smem_f + kpad * 16);   // [kpad], byte offsets into a staged image
+    float *xs = smem_f + kpad * 17;              // [imgs][ic][ihp][pitch], zero padded
+    const int ch_sz = p.ihp * p.pitch, img_sz = p.ic * ch_sz;
+    const int b0 = blockIdx.x * p.imgs;
+    const int nimg = min(p.imgs, p.bs - b0);
+
+    for (int k = threadIdx.x; k < kpad; k += blockDim.x) {
+        uint32_t ci, rem, fi, fj;
+        p.div_fhfw.divmod((uint32_t)min(k, p.ktot - 1), ci, rem);
+        p.div_fw.divmod(rem, fi, fj);
+        tapoff[k] = (int)(ci * ch_sz + fi * p.pitch + fj) * 4;
+    }
+    // a padding cell reads the nearest cell of the image (a valid address) and stores zero
+    auto cell = [&](int e, int &hi, int &wi) -> size_t {
+        uint32_t r1, col, r2, row;  // r2 = img * ic + channel
+        p.div_pitch.divmod((uint32_t)e, r1, col);
+        p.div_ihp.divmod(r1, r2, row);
+        hi = (int)row - p.ph;
+        wi = (int)col - p.pw;
+        return ((size_t)b0 * p.ic + r2) * p.ih * p.iw;
+    };
+    const int nw = kpad * 16, nx = nimg * img_sz;
+    auto get_w = [&](int e) { return w[(size_t)min(e & 15, p.oc - 1) * p.ktot + min(e >> 4, p.ktot - 1)]; };
+    auto put_w = [&](int e, T v) { Bs[e] = ((e & 15) < p.oc && (e >> 4) < p.ktot) ? Elem<T>::to_f32(v) : 0.0f; };
+    constexpr int WU = 12, XU = 8;
+    T wv[WU], xv[XU];
+    batch_read<WU>(wv, 0, nw, get_w);
+    if (p.ph == 0 && p.pw == 0) {  // nothing to pad: the staged images are a copy
+        const T *xb = x + (size_t)b0 * img_sz;
+        auto get_x = [&](int e) { return xb[e]; };
+        auto put_x = [&](int e, T v) { xs[e] = Elem<T>::to_f32(v); };
+        batch_read<XU>(xv, 0, nx, get_x);
+        batch_store<WU>(wv, 0, nw, put_w);
+        batch_store<XU>(xv, 0, nx, put_x);
+        staged_fill_from<8, T>(XU * (int)blockDim.x, nx, get_x, put_x);
+    } else {
+        auto get_x = [&](int e) {
+            int hi, wi;
+            const size_t plane = cell(e, hi, wi);
+            return x[plane + (size_t)min(max(hi, 0), p.ih - 1) * p.iw + min(max(wi, 0), p.iw - 1)];
+        };
+        auto put_x = [&](int e, T v) {
+            int hi, wi;
+            cell(e, hi, wi);
+            xs[e] = (hi >= 0 && hi < p.ih && wi >= 0 && wi < p.iw) ? Elem<T>::to_f32(v) : 0.0f;
+        };
+        batch_read<XU>(xv, 0, nx, get_x);
+        batch_store<WU>(wv, 0, nw, put_w);
+        batch_store<XU>(xv, 0, nx, put_x);
+        staged_fill_from<8, T>(XU * (int)blockDim.x, nx, get_x, put_x);
+    }
+    staged_fill_from<8, T>(WU * (int)blockDim.x, nw, get_w, put_w);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, i = lane & 15;
+    const int nunits = nimg * p.units_per_img;
+    const char *Bl = (const char *)(Bs + lane);
+    const char *tl = (const char *)(tapoff + g);
+    for (int u = wave; u < nunits; u += 4) {
+        uint32_t img, ug;
+        p.div_upi.divmod((uint32_t)u, img, ug);
+        const int tile0 = (int)ug * TG;
+        // this lane's A row of every tile: byte offset of the position's top-left input cell in LDS
+        const char *abase[TG];
+#pragma unroll
+        for (int t = 0; t < TG; ++t) {
+            const int tile = min(tile0 + t, p.mtiles - 1);
+            uint32_t oy, ox;
+            if (POOL) {
+                uint32_t py, px;
+                p.div_yw.divmod((uint32_t)min(tile * 4 + (i >> 2), p.nout - 1), py, px);
+                oy = 2 * py + ((i >> 1) & 1);
+                ox = 2 * px + (i & 1);
+            } else {
+                p.div_yw.divmod((uint32_t)min(tile * 16 + i, p.nout - 1), oy, ox);
+            }
+            abase[t] = (const char *)(xs + (size_t)img * img_sz + oy * p.pitch + ox);
+        }
+        f32x4_t acc[TG];
+#pragma unroll
+        for (int t = 0; t < TG; ++t) acc[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        float bq[8];
+        int tq[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            bq[q] = *(const float *)(Bl + q * 256);
+            tq[q] = *(const int *)(tl + q * 16);
+        }
+        for (int s0 = 0; s0 < p.ksteps; s0 += 8) {
+            float bc[8];
+            int tc[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) { bc[q] = bq[q]; tc[q] = tq[q]; }
+            if (s0 + 8 < p.ksteps) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    bq[q] = *(const float *)(Bl + (s0 + 8 + q) * 256);
+                    tq[q] = *(const int *)(tl + (s0 + 8 + q) * 16);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+#pragma unroll
+                for (int t = 0; t < TG; ++t) {
+                    const float a = *(const float *)(abase[t] + tc[q]);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bc[q], acc[t], 0, 0, 0);
+                }
+        }
+        // lane (g, i) holds rows 4g .. 4g+3 of column i: one window (pool) or 4 consecutive positions of channel i
+        const bool live = i < p.oc;
+        const T bv = (p.has_bias && live) ? bias[i] : Elem<T>::zero();
+        T *yc = y + ((size_t)(b0 + img) * p.oc + (live ? i : 0)) * p.nout;
+#pragma unroll
+        for (int t = 0; t < TG; ++t) {
+            const int tile = tile0 + t;
+            if (tile >= p.mtiles) break;
+            if (POOL) {
+                T m = round_bias_relu<T>(acc[t][0], p.has_bias != 0, bv, p.act);
+                float mf = Elem<T>::to_f32(m);
+#pragma unroll
+                for (int r = 1; r < 4; ++r) {
+                    const T v = round_bias_relu<T>(acc[t][r], p.has_bias != 0, bv, p.act);
+                    const float f = Elem<T>::to_f32(v);
+                    if (f > mf) { m = v; mf = f; }
+                }
+                const int wi = tile * 4 + g;
+                if (live && wi < p.nout) yc[wi] = m;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int pos = tile * 16 + 4 * g + r;
+                    if (live && pos < p.nout) yc[pos] = round_bias_relu<T>(acc[t][r], p.has_bias != 0, bv, p.act);
                 }
             }
         }
@@ -1109,6 +1349,61 @@ int conv2_direct_entry(const char *name, const void *x, const void *w, const voi
     if (sh == 1 && sw == 1 && dh == 1 && dw == 1 && !pool2x2) {
         const int rc = conv2_mfma_try<T>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
         if (rc != 1) return rc;
+    }
+
+    // up to 16 output channels over enough taps on small images: matrix cores fed from the staged image
+    if (sh == 1 && sw == 1 && dh == 1 && dw == 1 && oc <= 16) {
+        const char *env = getenv("AGH_CONV_SMALL");  // 0 / 1 forces the choice (measurements)
+        const int64_t taps = ic * fh * fw;
+        const bool want = env ? atoi(env) != 0 : (oc >= 8 && taps >= 32);
+        SmallMfmaParams q;
+        q.bs = (int)bs; q.ic = (int)ic; q.ih = (int)ih; q.iw = (int)iw; q.oc = (int)oc; q.oh = (int)oh; q.ow = (int)ow;
+        q.fh = (int)fh; q.fw = (int)fw; q.ph = (int)ph; q.pw = (int)pw;
+        q.act = act; q.has_bias = bias != nullptr;
+        q.ihp = (int)(ih + 2 * ph);
+        q.pitch = (int)(iw + 2 * pw);
+        q.ktot = (int)taps;
+        q.ksteps = (int)((taps + 31) / 32 * 8);
+        const int64_t yh = pool2x2 ? oh / 2 : oh, yw = pool2x2 ? ow / 2 : ow;
+        q.nout = (int)(yh * yw);
+        q.yw = (int)yw;
+        q.mtiles = (int)(pool2x2 ? (yh * yw + 3) / 4 : (yh * yw + 15) / 16);
+        const int tg = q.mtiles >= 8 ? 4 : 2;
+        q.units_per_img = (q.mtiles + tg - 1) / tg;
+        const int64_t kpad = (int64_t)q.ksteps * 4;
+        const int64_t fixed_bytes = kpad * 17 * 4, img_bytes = ic * (int64_t)q.ihp * q.pitch * 4;
+        constexpr int64_t kLds = 64 * 1024;
+        if (want && taps <= 2048 && fixed_bytes + img_bytes <= kLds && yh * yw <= ((int64_t)1 << 20)) {
+            const int64_t cus = compute_units() > 0 ? compute_units() : 256;
+            // a workgroup's four waves want a unit each; more images per workgroup only while the grid still
+            // covers the chip twice
+            int64_t imgs = std::max<int64_t>(1, 4 / q.units_per_img);
+            while (fixed_bytes + (imgs + 1) * img_bytes <= kLds && (imgs + 1) * q.units_per_img <= 8 &&
+                   (bs + imgs) / (imgs + 1) >= 2 * cus)
+                ++imgs;
+            while (imgs > 1 && fixed_bytes + imgs * img_bytes > kLds) --imgs;
+            if (imgs > bs) imgs = bs;
+            q.imgs = (int)imgs;
+            q.div_pitch = FastDiv((uint32_t)q.pitch);
+            q.div_ihp = FastDiv((uint32_t)q.ihp);
+            q.div_yw = FastDiv((uint32_t)yw);
+            q.div_fw = FastDiv((uint32_t)fw);
+            q.div_fhfw = FastDiv((uint32_t)(fh * fw));
+            q.div_upi = FastDiv((uint32_t)q.units_per_img);
+            const int64_t blocks = (bs + imgs - 1) / imgs;
+            if (blocks > 0x7FFFFFFF) return fail(AGH_ERANGE, "%s: too many workgroups", name);
+            const size_t smem = (size_t)(fixed_bytes + imgs * img_bytes);
+            const dim3 grid((unsigned)blocks), block(256);
+            const T *xp = (const T *)x, *wp = (const T *)w, *bp = (const T *)bias;
+            T *yp = (T *)y;
+#define AGH_SM(POOLV, TGV) \
+    hipLaunchKernelGGL((conv2_small_mfma_kernel<T, POOLV, TGV>), grid, block, smem, stream(), xp, wp, bp, yp, q)
+            if (pool2x2) { if (tg == 4) AGH_SM(true, 4); else AGH_SM(true, 2); }
+            else { if (tg == 4) AGH_SM(false, 4); else AGH_SM(false, 2); }
+#undef AGH_SM
+            AGH_LAUNCH_CHECK(name);
+            return AGH_OK;
+        }
     }
 
     // stride 1, dilation 1, filter width 3 or 5: row-tiled kernel

@@ -162,6 +162,63 @@ def test_conv2_direct_bf16_matrix_core_path(ag, case):
     assert np.array_equal(yi, orc.f32_to_bf16(exact.astype(np.float32)))
 
 
+CONV_FEW_CHANNELS = [
+    # bs, ic, ih, iw, oc, filter, padding: layers the 16-channel-wide matrix-core kernel takes (or can be made to)
+    (100, 6, 12, 12, 16, (5, 5), (0, 0)),    # LeNet5 conv2: 150 taps (5 chunks, 10 padded), 4 tiles of 4 windows
+    (100, 1, 28, 28, 6, (5, 5), (0, 0)),     # LeNet5 conv1: 6 of 16 columns live, 25 taps in one chunk, 36 tiles
+    (7, 3, 11, 9, 10, (3, 3), (1, 1)),       # padding, odd sizes: last tile partly empty, pooling drops a row and a column
+    (5, 8, 9, 14, 16, (3, 5), (2, 1)),       # rectangular filter, padding larger than half the filter
+    (3, 20, 6, 6, 12, (1, 1), (0, 0)),       # 1x1: the tap table is the channel stride
+    (2, 4, 40, 36, 9, (3, 3), (0, 0)),       # many tiles per image: 4 tiles per unit
+    (300, 2, 5, 5, 3, (2, 2), (0, 0)),       # tiny images, many per workgroup
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("case", CONV_FEW_CHANNELS)
+def test_conv2_direct_few_channels_matrix_core_path(ag, monkeypatch, dtype, case):
+    """AGH_CONV_SMALL=1 sends every layer with at most 16 output channels through the 16x16x4 MFMA kernel (by itself
+    the library picks it from 8 output channels and 32 taps).  Checked against the f64 convolution, exactly on integer
+    data, and its fused bias / ReLU / 2x2 pool against the separate layers applied to its own plain result."""
+    bs, ic, ih, iw, oc, f, p = case
+    monkeypatch.setenv("AGH_CONV_SMALL", "1")
+    rng = np.random.default_rng(27)
+    x = to_dtype(rng.standard_normal((bs, ic, ih, iw)), dtype)
+    w = to_dtype(rng.standard_normal((oc, ic) + f) * np.sqrt(2.0 / (ic * f[0] * f[1])), dtype)
+    b = to_dtype(rng.standard_normal(oc) * 0.1, dtype)
+    tx, tw, tb = ag.Tensor.from_array(x), ag.Tensor.from_array(w), ag.Tensor.from_array(b)
+    y = ag.conv2_direct_forward(tx, tw, padding=p).into_array()
+    want = orc.conv2_naive_f64(as_f32(x), as_f32(w), p, (1, 1), (1, 1))
+    scale = orc.conv2_naive_f64(np.abs(as_f32(x)), np.abs(as_f32(w)), p, (1, 1), (1, 1))
+    assert y.shape == want.shape
+    k = ic * f[0] * f[1]
+    got = as_f32(y).astype(np.float64)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0**-126))) - (7 if dtype == "bf16" else 23))
+    assert np.all(np.abs(got - want) <= ulp + 8 * np.sqrt(k) * 2.0**-24 * scale)
+    # the other kernel (register tiles on the vector units) sums the same products in another order
+    monkeypatch.setenv("AGH_CONV_SMALL", "0")
+    other = as_f32(ag.conv2_direct_forward(tx, tw, padding=p).into_array()).astype(np.float64)
+    monkeypatch.setenv("AGH_CONV_SMALL", "1")
+    assert np.all(np.abs(got - other) <= 2 * ulp + 16 * np.sqrt(k) * 2.0**-24 * scale)
+    # epilogues, bit for bit on this kernel's own sums
+    yb = ag.conv2_direct_forward(tx, tw, padding=p, bias=tb, relu=True).into_array()
+    n, c, h, wd = y.shape
+    flat = np.ascontiguousarray(y.transpose(0, 2, 3, 1).reshape(-1, c))
+    ref = orc.relu(orc.bias_add_rows(flat, b)).reshape(n, h, wd, c).transpose(0, 3, 1, 2)
+    assert np.array_equal(yb, ref)
+    if h >= 2 and wd >= 2:
+        fused = ag.conv2_direct_forward(tx, tw, padding=p, relu=True, pool2x2=True).into_array()
+        assert np.array_equal(fused, orc.max_pool2(orc.relu(y), (2, 2)))
+        fused_b = ag.conv2_direct_forward(tx, tw, padding=p, bias=tb, relu=True, pool2x2=True).into_array()
+        assert np.array_equal(fused_b, orc.max_pool2(ref, (2, 2)))
+    # exact-integer data: every sum is exact in f32
+    xi = to_dtype(((np.arange(x.size) % 10) + 1).astype(np.float32).reshape(x.shape), dtype)
+    wi = to_dtype(((np.arange(w.size) % 7) - 3).astype(np.float32).reshape(w.shape), dtype)
+    yi = ag.conv2_direct_forward(ag.Tensor.from_array(xi), ag.Tensor.from_array(wi), padding=p).into_array()
+    exact = orc.conv2_naive_f64(as_f32(xi), as_f32(wi), p, (1, 1), (1, 1)).astype(np.float32)
+    assert np.array_equal(yi, to_dtype(exact, dtype))
+
+
 CONV_MFMA_F32 = [
     # the f32 variant steps 8 channels at a time
     (2, 64, 56, 56, 128, (3, 3), (1, 1)),    # config-3 layer, small batch: two passes of 32 channels
