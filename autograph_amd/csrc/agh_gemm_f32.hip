@@ -1,6 +1,8 @@
 // f32 GEMM entry points (v_mfma_f32_32x32x2_f32: full f32 multiplies and accumulation).
 #define AGH_GEMM_WITH_F32_DIRECT
+#define AGH_GEMM_WITH_F32_SMALL
 #include "agh_gemm_f32_dl.h"
+#include "agh_gemm_f32_small.h"
 #include "agh_gemm_host.h"
 
 extern "C" {

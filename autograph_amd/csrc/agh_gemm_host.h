@@ -262,6 +262,13 @@ int gemm_entry(const char *name, int64_t m, int64_t k, int64_t n, float alpha, c
     const bool vec_store = g.dp == 1 && g.NP % 4 == 0 && (g.dq % 4 == 0 || g.NQ == 1) && aligned(C, 4 * sizeof(T)) &&
                            (batch == 1 || g.batch_d % 4 == 0);
 
+#ifdef AGH_GEMM_WITH_F32_SMALL
+    if constexpr (sizeof(T) == 4) {
+        const int rc = gemm_f32_small_try(g, lp, lq, vec_store, batch);
+        if (rc != 1) return rc;
+    }
+#endif
+
     // ---- tile shape: minimise (rounds of workgroups) x (tile area) / efficiency ----
     const int cus = compute_units() > 0 ? compute_units() : 256;
     // (any k: a last k-tile shorter than 64 is loaded with zeros behind k = K)

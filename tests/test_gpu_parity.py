@@ -116,8 +116,18 @@ def test_dot_seeded_all_transposes(ag, dtype, mkn):
                 assert_bf16_gemm_close(out, orc.gemm_bf16_f32acc(av, bv), av, bv)
 
 
+@pytest.fixture(params=["tiled", "default"])
+def f32_small_kernel(request, monkeypatch):
+    """f32 products of few tiles and short k have a kernel of their own, which by default takes most shapes of the
+    view / stride / broadcast tests below: each of those runs once with it switched off (the tiled kernels and their
+    loaders) and once as the library chooses."""
+    if request.param == "tiled":
+        monkeypatch.setenv("AGH_GEMM_SMALL", "0")
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-def test_gemm_strides_offsets_alpha_beta(ag, dtype):
+def test_gemm_strides_offsets_alpha_beta(ag, dtype, f32_small_kernel):
     """fn gemm with the full (offset, rs, cs) tuple for all three operands (linalg.rs:281-299):
     sub-views with offsets, negative strides, a column-major C, alpha and beta."""
     rng = np.random.default_rng(11)
@@ -224,7 +234,7 @@ def test_gemm_random_views(ag):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-def test_gemm_zero_stride_operands(ag, dtype):
+def test_gemm_zero_stride_operands(ag, dtype, f32_small_kernel):
     """Broadcast views as operands of `fn gemm` (strides are taken as they come, src/tensor/linalg.rs:285-299; ndarray's
     `broadcast` gives stride 0): every row of A the same vector, every column of B the same vector, an operand that is
     one scalar, k broadcast.  Against the f64 product of the materialised arrays, at sizes that take the small and the
@@ -746,6 +756,46 @@ def test_gemm_f32_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
             assert np.abs(C.into_array() - want).max() <= tol, (m, k, n, ta, tb, alpha, beta, cfg)
     monkeypatch.delenv("AGH_GEMM_CFG", raising=False)
     assert ran[None] == 150 and min(ran.values()) >= 30, ran
+
+
+def test_gemm_f32_few_tiles_short_k_kernel(ag, monkeypatch):
+    """Products of a few hundred 16 x 16 tiles with k <= 512 and both operands k-contiguous go to a kernel of their own
+    (one tile per workgroup, k split over its four waves).  AGH_GEMM_SMALL=1 sends every eligible product there,
+    =0 none: both against the f64 product, bias / ReLU epilogues bit for bit against the separate ops on the plain
+    result, exact on integers.  Shapes: the LeNet5 Dense layers at batch 1000 and 100, k not a multiple of 16 or 64,
+    k = 4, n = 10 (no 16-byte stores), one row, beta and alpha."""
+    rng = np.random.default_rng(321)
+    shapes = [(1000, 256, 128), (1000, 128, 84), (1000, 84, 10), (100, 256, 128), (7, 4, 3), (1, 40, 50), (33, 20, 1),
+              (130, 500, 36), (16, 16, 16), (250, 1028, 20)]
+    for (m, k, n) in shapes:
+        a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        w = rng.uniform(-1, 1, (n, k)).astype(np.float32)     # Dense weight [out, in]: the product is a . w^T
+        bias = rng.uniform(-1, 1, n).astype(np.float32)
+        c0 = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+        A, W, Bv = ag.Tensor.from_array(a), ag.Tensor.from_array(w), ag.Tensor.from_array(bias)
+        got = {}
+        for small in ("1", "0"):
+            monkeypatch.setenv("AGH_GEMM_SMALL", small)
+            for alpha, beta in ((1.0, 0.0), (0.5, -0.5)):
+                C = ag.Tensor.from_array(c0)
+                ag.gemm(alpha, A, W.t(), beta, C)
+                want = alpha * (a.astype(np.float64) @ w.T.astype(np.float64)) + beta * c0
+                tol = 1e-5 * np.sqrt(k) * max(np.abs(want).max(), 1e-3) + 1e-6
+                assert np.abs(C.into_array() - want).max() <= tol, (m, k, n, small, alpha, beta)
+                got[small, alpha] = C.into_array()
+            plain = got[small, 1.0]
+            fused = ag.Tensor.from_array(a).dot(W.t(), bias=Bv, relu=True).into_array()
+            assert np.array_equal(fused, orc.relu(orc.bias_add_rows(plain, bias))), (m, k, n, small)
+            # c = a^T-free column-major output: p runs along m, the bias along q
+            Ct = ag.Tensor.uninit((n, m), "f32")
+            ag.gemm(1.0, A, W.t(), 0.0, Ct.t(), bias=Bv, relu=False)
+            assert np.array_equal(Ct.into_array().T, orc.bias_add_rows(plain, bias)), (m, k, n, small)
+        assert np.abs(got["1", 1.0] - got["0", 1.0]).max() <= 2e-5 * np.sqrt(k), (m, k, n)
+        ai = rng.integers(-8, 9, (m, k)).astype(np.float32)
+        wi = rng.integers(-8, 9, (n, k)).astype(np.float32)
+        monkeypatch.setenv("AGH_GEMM_SMALL", "1")
+        assert np.array_equal(ag.Tensor.from_array(ai).dot(ag.Tensor.from_array(wi).t()).into_array(), ai @ wi.T)
+    monkeypatch.delenv("AGH_GEMM_SMALL")
 
 
 def test_gemm_bf16_seeded_shapes_in_every_tile_configuration(ag, monkeypatch):
