@@ -599,6 +599,19 @@ __device__ __forceinline__ void store_rounded(T *dst, const float (&v)[N]) {
     }
 }
 
+// 16 bytes per lane from global memory straight into LDS: lane L's data lands at lds_base + 16 L (lds_base is
+// wave-uniform and travels in M0).  Inline assembly, so the compiler's wait counting does not know it: whoever reads
+// the destination waits with s_waitcnt vmcnt(0) and a barrier first.
+__device__ __forceinline__ void lds_direct_load16(const void *gptr, uint32_t lds_base_uniform) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(__builtin_amdgcn_readfirstlane((int)lds_base_uniform))
+                 : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_address_of(const void *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char *)p;
+}
+
 // waves_per_eu(2, 2): eight waves per workgroup are two per SIMD whatever the register count; without the hint the
 // compiler aimed the bf16 training instantiation at 128 registers and gave up the early weight loads for it (30 us
 // instead of 20)
@@ -607,24 +620,59 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                                               const T *__restrict__ w2, const T *__restrict__ wd1,
                                                               const T *__restrict__ wd2, const T *__restrict__ wd3,
                                                               const T *__restrict__ b3, T *__restrict__ out, int bs,
-                                                              LenetSaves<T> sv) {
+                                                              LenetSaves<T> sv, int w23_aligned) {
     constexpr int IMGS = 4;
     __shared__ __align__(16) float xs[IMGS * 28 * 28];     // input images, pitch 28
     __shared__ __align__(16) float w1s[25 * 6];            // [tap][oc]
     __shared__ __align__(16) float p1[IMGS * 6 * 12 * 12]; // after conv1 + relu + pool
-    __shared__ __align__(16) float w2s[150 * 16];          // [ci][fi][fj][oc]
+    __shared__ __align__(16) float w2s[160 * 16];          // [ci][fi][fj][oc], ten rows of zeros behind the 150 taps
+    __shared__ int tap2[160];                              // byte offset of tap k inside an image of p1 (0 behind the taps)
     __shared__ __align__(16) float p2[IMGS * 256];         // after conv2 + relu + pool, flattened [c][h][w]
     __shared__ __align__(16) float d1[IMGS * 128];
     __shared__ __align__(16) float d2[IMGS * 84];
     __shared__ __align__(16) float parts[16 * IMGS * 128];  // dense1 partial sums
+    __shared__ __align__(16) T wd2s[128 * 84];              // dense2 / dense3 weights as they lie in memory
+    __shared__ __align__(16) T wd3s[1024];                  // (84 * 10, rounded up to whole KB)
     constexpr int NT = 512;  // 8 waves: two per SIMD, so one can wait on LDS while the other multiplies
     const int tid = threadIdx.x;
     const int b0 = blockIdx.x * IMGS;
     const int nimg = min(IMGS, bs - b0);
 
-    for (int e = tid; e < 150; e += NT) { const int tap = e / 6, o = e - tap * 6; w1s[e] = Elem<T>::to_f32(w1[o * 25 + tap]); }
-    for (int e = tid; e < 2400; e += NT) { const int tap = e >> 4, o = e & 15; w2s[e] = Elem<T>::to_f32(w2[o * 150 + tap]); }
-    for (int e = tid; e < IMGS * 784; e += NT) xs[e] = e < nimg * 784 ? Elem<T>::to_f32(x[(size_t)b0 * 784 + e]) : 0.0f;
+    // Everything staged is read first and stored afterwards, so that the reads are all in flight together: written as
+    // `lds[e] = global[...]` loops they compile to one read, one wait and one store per trip (a dozen memory round trips
+    // one after another, 3 of the launch's 16 us).  Addresses are clamped, what lies outside is stored as zero.
+    {
+        constexpr int XU = (IMGS * 784 + NT - 1) / NT;  // 7 image values a thread
+        const int nx = nimg * 784;
+        T w1v, w2v[5], xv[XU];
+        {
+            const int e = min(tid, 149), tap = e / 6, o = e - tap * 6;
+            w1v = w1[o * 25 + tap];
+        }
+#pragma unroll
+        for (int u = 0; u < 5; ++u) {
+            const int e = tid + u * NT, tap = e >> 4, o = e & 15;
+            w2v[u] = w2[o * 150 + min(tap, 149)];
+        }
+        const T *xb = x + (size_t)b0 * 784;
+#pragma unroll
+        for (int u = 0; u < XU; ++u) xv[u] = xb[min(tid + u * NT, nx - 1)];
+        if (tid < 150) w1s[tid] = Elem<T>::to_f32(w1v);
+#pragma unroll
+        for (int u = 0; u < 5; ++u) {
+            const int e = tid + u * NT;
+            w2s[e] = (e >> 4) < 150 ? Elem<T>::to_f32(w2v[u]) : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < XU; ++u) {
+            const int e = tid + u * NT;
+            if (e < IMGS * 784) xs[e] = e < nx ? Elem<T>::to_f32(xv[u]) : 0.0f;
+        }
+    }
+    if (tid < 160) {
+        const int k = min(tid, 149), ci = k / 25, rem = k - ci * 25, fi = rem / 5, fj = rem - fi * 5;
+        tap2[tid] = tid < 150 ? (ci * 144 + fi * 12 + fj) * 4 : 0;
+    }
     // dense1 weights of this thread (see the dense1 stage below), requested now, used much later
     float4 wreg[16];
     {
@@ -639,6 +687,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 wreg[kk] = make_float4(bf16_to_f32((uint16_t)(raw.x & 0xFFFF)), bf16_to_f32((uint16_t)(raw.x >> 16)),
                                        bf16_to_f32((uint16_t)(raw.y & 0xFFFF)), bf16_to_f32((uint16_t)(raw.y >> 16)));
             }
+        }
+    }
+    // The weights of the last two dense layers travel into LDS behind everything requested so far, 1 KB per
+    // instruction without passing through registers, while the convolution stages run: read where they are used
+    // (130 loads per thread, each waiting on L2) they cost the launch 3 of its 16 us.
+    {
+        constexpr int kW2Bytes = 128 * 84 * (int)sizeof(T), kW3Bytes = 84 * 10 * (int)sizeof(T);
+        static_assert(kW2Bytes % 1024 == 0 && kW3Bytes % 16 == 0, "whole direct loads");
+        const int lane = tid & 63, wave = tid >> 6;
+        if (w23_aligned) {
+            for (int c = wave; c < kW2Bytes / 1024; c += NT / 64)
+                lds_direct_load16((const char *)wd2 + c * 1024 + lane * 16, lds_address_of(wd2s) + c * 1024);
+            for (int c = wave; c < (kW3Bytes + 1023) / 1024; c += NT / 64)
+                lds_direct_load16((const char *)wd3 + min(c * 1024 + lane * 16, kW3Bytes - 16), lds_address_of(wd3s) + c * 1024);
+        } else {  // views at odd offsets: element copies
+            for (int e = tid; e < 128 * 84; e += NT) wd2s[e] = wd2[e];
+            for (int e = tid; e < 840; e += NT) wd3s[e] = wd3[e];
         }
     }
     __syncthreads();
@@ -677,26 +742,66 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     __syncthreads();
 
-    // conv2 (6->16, 5x5) + relu + pool: items = img x 16 channels x 4 row pairs x 2 column blocks of 4
+    // conv2 (6->16, 5x5) + relu + pool on v_mfma_f32_16x16x4_f32, as conv2_small_mfma_kernel does it: an MFMA takes the
+    // 4 pool windows of one pooled row (16 positions, cell-minor) x 16 channels x 4 taps, the A operand gathered from
+    // p1 through the tap table.  Wave w: image w / 2, pooled rows 2 (w % 2) and 2 (w % 2) + 1; 40 steps of 4 taps.
     {
-        const int img = tid >> 7, r0 = tid & 127;
-        const int oc = r0 >> 3, row = (r0 >> 1) & 3, wb = r0 & 1;
-        float acc[2][4][1];
-        rowpair_conv<5, 1, 4>(p1 + img * 864 + 2 * row * 12 + wb * 4, 144, 12, 6, 5, w2s + oc, 16, acc);
+        const int lane = tid & 63, wave = tid >> 6, g = lane >> 4, i = lane & 15;
+        const int img = wave >> 1, tile0 = (wave & 1) * 2;
+        const char *abase[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) p2[img * 256 + (oc * 4 + row) * 4 + wb * 2 + j] = relu_pool_window<T, 1, 4>(acc, j, 0);
-        if constexpr (SAVE) {
-            if (img < nimg) {
-                const size_t plane = (size_t)(b0 + img) * 16 + oc;
+        for (int t = 0; t < 2; ++t)
+            abase[t] = (const char *)(p1 + img * 864 + (2 * (tile0 + t) + ((i >> 1) & 1)) * 12 + 2 * (i >> 2) + (i & 1));
+        const char *Bl = (const char *)(w2s + lane), *tl = (const char *)(tap2 + g);
+        f32x4_t acc[2] = {f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}};
+        float bq[8];
+        int tq[8];
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    float v[4];
+        for (int q = 0; q < 8; ++q) {
+            bq[q] = *(const float *)(Bl + q * 256);
+            tq[q] = *(const int *)(tl + q * 16);
+        }
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) v[t] = acc[a][t][0];
-                    store_rounded<T, 4>(sv.c2 + (plane * 8 + 2 * row + a) * 8 + wb * 4, v);
+        for (int s0 = 0; s0 < 40; s0 += 8) {
+            float bc[8];
+            int tc[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) { bc[q] = bq[q]; tc[q] = tq[q]; }
+            if (s0 + 8 < 40) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    bq[q] = *(const float *)(Bl + (s0 + 8 + q) * 256);
+                    tq[q] = *(const int *)(tl + (s0 + 8 + q) * 16);
                 }
-                const float q[2] = {p2[img * 256 + (oc * 4 + row) * 4 + wb * 2], p2[img * 256 + (oc * 4 + row) * 4 + wb * 2 + 1]};
-                store_rounded<T, 2>(sv.p2 + (plane * 4 + row) * 4 + wb * 2, q);
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(*(const float *)(abase[t] + tc[q]), bc[q], acc[t], 0, 0, 0);
+        }
+        // lane (g, i): channel i, pooled column g; acc[t][2 dy + dx] is cell (dy, dx) of the window in pooled row tile0 + t
+        const T zero = Elem<T>::zero();
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int row = tile0 + t;
+            float mf = Elem<T>::to_f32(round_bias_relu<T>(acc[t][0], false, zero, AGH_ACT_RELU));
+#pragma unroll
+            for (int r = 1; r < 4; ++r) {
+                const float f = Elem<T>::to_f32(round_bias_relu<T>(acc[t][r], false, zero, AGH_ACT_RELU));
+                if (f > mf) mf = f;
+            }
+            p2[img * 256 + (i * 4 + row) * 4 + g] = mf;
+            if constexpr (SAVE) {
+                if (img < nimg) {
+                    const size_t plane = (size_t)(b0 + img) * 16 + i;
+#pragma unroll
+                    for (int dy = 0; dy < 2; ++dy) {
+                        const float v[2] = {acc[t][2 * dy], acc[t][2 * dy + 1]};
+                        store_rounded<T, 2>(sv.c2 + (plane * 8 + 2 * row + dy) * 8 + 2 * g, v);
+                    }
+                    sv.p2[(plane * 4 + row) * 4 + g] = Elem<T>::from_f32(mf);
+                }
             }
         }
     }
@@ -752,14 +857,42 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the direct loads of wd2s / wd3s (not known to the compiler)
     __syncthreads();
-    // dense2 128 -> 84 + relu (weights straight from L2, 32 loads in flight per thread)
+    // dense2 128 -> 84 + relu, weights from LDS.  Thread (c, kq) forms the partial sums of output c over a quarter of k
+    // for all four images (four independent chains of 32, each weight read once); the quarters are then added in order
+    // through LDS (`parts` is free again).  One thread per output over all of k is a chain of 128 dependent FMAs behind
+    // 256 LDS reads: 1.6 us of the launch.
+    if (tid < 4 * 84) {
+        const int kq = tid / 84, c = tid - kq * 84;
+        float part[IMGS];
+#pragma unroll
+        for (int r = 0; r < IMGS; ++r) part[r] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < 32; kk += 4) {
+            const int k = kq * 32 + kk;
+            float4 xk[IMGS];
+#pragma unroll
+            for (int r = 0; r < IMGS; ++r) xk[r] = *(const float4 *)(d1 + r * 128 + k);
+            const float w0 = Elem<T>::to_f32(wd2s[k * 84 + c]), w1v = Elem<T>::to_f32(wd2s[(k + 1) * 84 + c]);
+            const float w2v = Elem<T>::to_f32(wd2s[(k + 2) * 84 + c]), w3v = Elem<T>::to_f32(wd2s[(k + 3) * 84 + c]);
+#pragma unroll
+            for (int r = 0; r < IMGS; ++r) {
+                part[r] = __builtin_fmaf(xk[r].x, w0, part[r]);
+                part[r] = __builtin_fmaf(xk[r].y, w1v, part[r]);
+                part[r] = __builtin_fmaf(xk[r].z, w2v, part[r]);
+                part[r] = __builtin_fmaf(xk[r].w, w3v, part[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < IMGS; ++r) parts[(kq * IMGS + r) * 84 + c] = part[r];
+    }
+    __syncthreads();
     if (tid < IMGS * 84) {
-        const int r = tid / 84, c = tid - r * 84;
-        float a = 0.0f;
-        const float *xr = d1 + r * 128;
-#pragma unroll 32
-        for (int k = 0; k < 128; ++k) a = __builtin_fmaf(xr[k], Elem<T>::to_f32(wd2[k * 84 + c]), a);
+        const int r = tid / 84;
+        float a = parts[tid];
+#pragma unroll
+        for (int kq = 1; kq < 4; ++kq) a += parts[kq * IMGS * 84 + tid];
         const T act = round_bias_relu<T>(a, false, Elem<T>::zero(), AGH_ACT_RELU);
         d2[tid] = Elem<T>::to_f32(act);
         if constexpr (SAVE) {
@@ -770,13 +903,28 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
     __syncthreads();
-    // dense3 84 -> 10 + bias
+    // dense3 84 -> 10 + bias: thread (kp, r, c) sums 12 of the 84 products, the seven parts are added in order
+    if (tid < 7 * IMGS * 10) {
+        const int kp = tid / (IMGS * 10), rc = tid - kp * (IMGS * 10), r = rc / 10, c = rc - r * 10;
+        float a = 0.0f;
+        const float *xr = d2 + r * 84 + kp * 12;
+#pragma unroll
+        for (int kk = 0; kk < 12; kk += 4) {
+            const float4 xk = *(const float4 *)(xr + kk);
+            const int k = kp * 12 + kk;
+            a = __builtin_fmaf(xk.x, Elem<T>::to_f32(wd3s[k * 10 + c]), a);
+            a = __builtin_fmaf(xk.y, Elem<T>::to_f32(wd3s[(k + 1) * 10 + c]), a);
+            a = __builtin_fmaf(xk.z, Elem<T>::to_f32(wd3s[(k + 2) * 10 + c]), a);
+            a = __builtin_fmaf(xk.w, Elem<T>::to_f32(wd3s[(k + 3) * 10 + c]), a);
+        }
+        parts[2048 + tid] = a;  // behind the dense2 partials, which other waves may still be reading
+    }
+    __syncthreads();
     if (tid < IMGS * 10) {
         const int r = tid / 10, c = tid - r * 10;
-        float a = 0.0f;
-        const float *xr = d2 + r * 84;
-#pragma unroll 28
-        for (int k = 0; k < 84; ++k) a = __builtin_fmaf(xr[k], Elem<T>::to_f32(wd3[k * 10 + c]), a);
+        float a = parts[2048 + tid];
+#pragma unroll
+        for (int kp = 1; kp < 7; ++kp) a += parts[2048 + kp * IMGS * 10 + tid];
         if (r < nimg) out[(size_t)(b0 + r) * 10 + c] = round_bias_relu<T>(a, true, b3[c], AGH_ACT_NONE);
     }
 }
@@ -1525,17 +1673,18 @@ int lenet5_forward_entry(const char *name, const void *x, const void *w1, const 
     if (bs == 0) return AGH_OK;
     if (!x || !w1 || !w2 || !wd1 || !wd2 || !wd3 || !b3 || !logits) return fail(AGH_ENULL, "%s: null buffer", name);
     LenetSaves<T> sv = {};
+    const int w23_aligned = (((uintptr_t)wd2 | (uintptr_t)wd3) & 15) == 0;
     if (saves) {
         for (int i = 0; i < 8; ++i)
             if (!saves[i]) return fail(AGH_ENULL, "%s: null buffer for a saved activation", name);
         sv = {(T *)saves[0], (T *)saves[1], (T *)saves[2], (T *)saves[3], (T *)saves[4], (T *)saves[5], (T *)saves[6], (T *)saves[7]};
         hipLaunchKernelGGL((lenet5_forward_kernel<T, true>), dim3((unsigned)((bs + 3) / 4)), dim3(512), 0, stream(), (const T *)x,
                            (const T *)w1, (const T *)w2, (const T *)wd1, (const T *)wd2, (const T *)wd3, (const T *)b3,
-                           (T *)logits, (int)bs, sv);
+                           (T *)logits, (int)bs, sv, w23_aligned);
     } else {
         hipLaunchKernelGGL((lenet5_forward_kernel<T, false>), dim3((unsigned)((bs + 3) / 4)), dim3(512), 0, stream(), (const T *)x,
                            (const T *)w1, (const T *)w2, (const T *)wd1, (const T *)wd2, (const T *)wd3, (const T *)b3,
-                           (T *)logits, (int)bs, sv);
+                           (T *)logits, (int)bs, sv, w23_aligned);
     }
     AGH_LAUNCH_CHECK(name);
     return AGH_OK;
