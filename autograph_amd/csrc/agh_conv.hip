@@ -193,13 +193,17 @@ struct RowTileParams {
     FastDiv div_items, div_rowsxwb, div_nwb, div_ocpad, div_pitch, div_ihp;
 };
 
-template <typename T, int FW, int OCT, bool POOL>
+template <typename T, int FW, int OCT, bool POOL, int FHC>  // FHC: the filter height when it equals FW, else 0 (run time)
 __global__ __launch_bounds__(256) void conv2_rowtile_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                              const T *__restrict__ bias, T *__restrict__ y,
                                                              RowTileParams p) {
     constexpr int WT = 8, NR = POOL ? 2 : 1, XW = WT + FW - 1, XV = (XW + 3) / 4;
     extern __shared__ __align__(16) float smem_f[];
-    const int taps = p.ic * p.fh * FW;
+    // a filter height known at compile time unrolls the row loop: which filter row an input row meets is then decided
+    // at compile time, not by branches around every group of FMAs (LeNet5 conv1: 10.3 -> 9.0 us)
+    constexpr int kUnrollRows = FHC ? FHC + (POOL ? 1 : 0) : 1;
+    const int fh = FHC ? FHC : p.fh;
+    const int taps = p.ic * fh * FW;
     float *ws = smem_f;                                         // [ic][fh][FW][ocpad]
     float *xs = smem_f + (((size_t)taps * p.ocpad + 3) & ~(size_t)3);  // [imgs][ic][ihp][pitch], zero padded
     const int ch_sz = p.ihp * p.pitch, img_sz = p.ic * ch_sz;
@@ -261,9 +265,10 @@ __global__ __launch_bounds__(256) void conv2_rowtile_kernel(const T *__restrict_
 
         for (int ci = 0; ci < p.ic; ++ci) {
             const float *xc = xi + ci * ch_sz;
-            const float *wc = wg + (size_t)ci * p.fh * FW * p.ocpad;
+            const float *wc = wg + (size_t)ci * fh * FW * p.ocpad;
             // input row r (relative to ho0) meets filter row r of output row 0 and r-1 of output row 1
-            for (int r = 0; r < p.fh + NR - 1; ++r) {
+#pragma unroll kUnrollRows
+            for (int r = 0; r < fh + NR - 1; ++r) {
                 float xin[XV * 4];
 #pragma unroll
                 for (int v = 0; v < XV; ++v) {
@@ -273,7 +278,7 @@ __global__ __launch_bounds__(256) void conv2_rowtile_kernel(const T *__restrict_
 #pragma unroll
                 for (int a = 0; a < NR; ++a) {
                     const int fi = r - a;
-                    if (fi >= 0 && fi < p.fh) {
+                    if (fi >= 0 && fi < fh) {
                         const float *wr = wc + fi * FW * p.ocpad;
 #pragma unroll
                         for (int fj = 0; fj < FW; ++fj) {
@@ -1603,7 +1608,10 @@ int conv2_direct_entry(const char *name, const void *x, const void *w, const voi
             const T *xp = (const T *)x, *wp = (const T *)w, *bp = (const T *)bias;
             T *yp = (T *)y;
 #define AGH_RT(FWV, OCTV, POOLV) \
-    hipLaunchKernelGGL((conv2_rowtile_kernel<T, FWV, OCTV, POOLV>), grid, block, smem, stream(), xp, wp, bp, yp, q)
+    do { \
+        if (fh == FWV) hipLaunchKernelGGL((conv2_rowtile_kernel<T, FWV, OCTV, POOLV, FWV>), grid, block, smem, stream(), xp, wp, bp, yp, q); \
+        else hipLaunchKernelGGL((conv2_rowtile_kernel<T, FWV, OCTV, POOLV, 0>), grid, block, smem, stream(), xp, wp, bp, yp, q); \
+    } while (0)
             if (fw == 3) {
                 if (oct == 1) { if (pool2x2) AGH_RT(3, 1, true); else AGH_RT(3, 1, false); }
                 else { if (pool2x2) AGH_RT(3, 2, true); else AGH_RT(3, 2, false); }
