@@ -465,11 +465,15 @@ __global__ __launch_bounds__(256) void conv2_small_mfma_kernel(const T *__restri
                     tq[q] = *(const int *)(tl + (s0 + 8 + q) * 16);
                 }
             }
+            // the taps behind ktot multiply zeros of the bank; their A values are zeroed too (0 * inf would poison the
+            // sum), which only the last chunk has to look at
+            const bool tail = s0 + 8 >= p.ksteps;
 #pragma unroll
             for (int q = 0; q < 8; ++q)
 #pragma unroll
                 for (int t = 0; t < TG; ++t) {
-                    const float a = *(const float *)(abase[t] + tc[q]);
+                    float a = *(const float *)(abase[t] + tc[q]);
+                    if (tail && 4 * (s0 + q) + g >= p.ktot) a = 0.0f;
                     acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bc[q], acc[t], 0, 0, 0);
                 }
         }
@@ -782,8 +786,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
             for (int q = 0; q < 8; ++q)
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(*(const float *)(abase[t] + tc[q]), bc[q], acc[t], 0, 0, 0);
+                for (int t = 0; t < 2; ++t) {
+                    float a = *(const float *)(abase[t] + tc[q]);
+                    if (4 * (s0 + q) + g >= 150) a = 0.0f;  // behind the taps: zero times zero, whatever p1 holds (s0, q constants)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, bc[q], acc[t], 0, 0, 0);
+                }
         }
         // lane (g, i): channel i, pooled column g; acc[t][2 dy + dx] is cell (dy, dx) of the window in pooled row tile0 + t
         const T zero = Elem<T>::zero();

@@ -217,6 +217,16 @@ def test_conv2_direct_few_channels_matrix_core_path(ag, monkeypatch, dtype, case
     yi = ag.conv2_direct_forward(ag.Tensor.from_array(xi), ag.Tensor.from_array(wi), padding=p).into_array()
     exact = orc.conv2_naive_f64(as_f32(xi), as_f32(wi), p, (1, 1), (1, 1)).astype(np.float32)
     assert np.array_equal(yi, to_dtype(exact, dtype))
+    # an infinite input value reaches exactly the outputs whose window covers it: the padded taps behind the last one
+    # (zeros of the filter bank) must not turn it into NaN anywhere
+    xinf = np.abs(as_f32(x)).copy()
+    xinf[0, ic - 1, ih // 2, iw // 2] = np.inf
+    wpos = np.abs(as_f32(w)) + 0.01
+    yinf = as_f32(ag.conv2_direct_forward(ag.Tensor.from_array(to_dtype(xinf, dtype)), ag.Tensor.from_array(to_dtype(wpos, dtype)),
+                                          padding=p).into_array())
+    want_inf = np.isinf(orc.conv2_naive_f64(as_f32(to_dtype(xinf, dtype)), as_f32(to_dtype(wpos, dtype)), p, (1, 1), (1, 1)))
+    assert not np.isnan(yinf).any()
+    assert np.array_equal(np.isinf(yinf), want_inf) and want_inf.any()
 
 
 CONV_MFMA_F32 = [
