@@ -57,6 +57,7 @@ struct ConvMfmaParams {
     int nchunk;    // 16-byte chunks per staged pixel
     int K;         // fh*fw*ic
     int per_xcd;   // workgroups per XCD when the grid divides by 8, else 0
+    int nt_store;  // output stores carry the streaming hint
     int remap;     // staging takes the coalesced lane order where it applies (AGH_CONV_REMAP=0 switches it off)
     FastDiv div_ow, div_tiles, div_octiles, div_vec;
 };
@@ -363,7 +364,11 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
                 if (TOTAL % 64 != 0 && idx >= TOTAL) continue;
                 const uint4 v = *(const uint4 *)(region + row * kEpitch + chunk * 16);
                 const int pos = p0 + part * kEpiPos + chunk * CPC, o = oc0 + row;
-                if (pos < p.npos && o < p.oc) *(uint4 *)(y + ((size_t)b * p.oc + o) * p.npos + pos) = v;
+                if (pos < p.npos && o < p.oc) {
+                    typedef uint32_t u32x4_nt __attribute__((ext_vector_type(4)));
+                    if (p.nt_store) __builtin_nontemporal_store(u32x4_nt{v.x, v.y, v.z, v.w}, (u32x4_nt *)(y + ((size_t)b * p.oc + o) * p.npos + pos));
+                    else *(uint4 *)(y + ((size_t)b * p.oc + o) * p.npos + pos) = v;
+                }
             }
         });
     }
@@ -416,6 +421,12 @@ static int conv2_mfma_launch(const char *name, const void *x, const void *w, con
     {
         const char *e = getenv("AGH_CONV_REMAP");
         p.remap = e && *e ? atoi(e) : 1;
+        // An output that could not stay in the 256 MB last-level cache next to the input anyway is stored with the
+        // streaming hint, which leaves that cache to the input rows neighbouring tiles share (config 3 in bf16: 0.135 ->
+        // 0.124 ms); a smaller one is stored plainly, for the layer that reads it next.  AGH_CONV_NT=0|1 overrides.
+        const char *nt = getenv("AGH_CONV_NT");
+        const size_t out_bytes = (size_t)bs * oc * npos * sizeof(T);
+        p.nt_store = nt && *nt ? atoi(nt) : out_bytes > ((size_t)64 << 20);
     }
     p.div_ow = FastDiv((uint32_t)ow);
     p.div_tiles = FastDiv((uint32_t)tiles);
