@@ -142,10 +142,6 @@ def test_conv2_direct_bf16_matrix_core_path(ag, monkeypatch, case, grid):
     b = orc.f32_to_bf16((rng.standard_normal(oc) * 0.1).astype(np.float32))
     tx, tw, tb = ag.Tensor.from_array(x), ag.Tensor.from_array(w), ag.Tensor.from_array(b)
     y = ag.conv2_direct_forward(tx, tw, padding=p).into_array()
-    if grid == "1x4":  # every output sums the same products in the same order in both arrangements
-        monkeypatch.delenv("AGH_CONV_GRID")
-        assert np.array_equal(y, ag.conv2_direct_forward(tx, tw, padding=p).into_array())
-        monkeypatch.setenv("AGH_CONV_GRID", "1")
     want = orc.conv2_naive_f64(orc.bf16_to_f32(x), orc.bf16_to_f32(w), p, (1, 1), (1, 1))
     scale = orc.conv2_naive_f64(np.abs(orc.bf16_to_f32(x)), np.abs(orc.bf16_to_f32(w)), p, (1, 1), (1, 1))
     assert y.shape == want.shape
