@@ -82,22 +82,17 @@ __global__ __launch_bounds__(kThreads) void pack_filter_kernel(const T *__restri
 }
 
 // kTilePos output positions per workgroup (kMT MFMA tiles of 32), kWgs workgroups per CU, kBRing register sets of B
-// fragments (requested kBRing - 1 steps ahead).  kOT = 1: a wave owns all position tiles and one tile of 32 output
-// channels (the four waves read every A fragment from LDS, four times in all); kOT = 2: the waves form a 2 x 2 grid, a
-// wave owns half of the position tiles and two channel tiles, so an A fragment is read by two waves and feeds two MFMAs
-// each time: half the LDS bytes per flop, twice the (cache-resident) filter fragments.
-template <typename T, int kTilePos, int kWgs, int kBRing, int kOT>
-__global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__restrict__ x, const T *__restrict__ wpk,
+// fragments (requested kBRing - 1 steps ahead).
+template <typename T, int kTilePos, int kWgs, int kBRing>
+__global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__restrict__ x, const T *__restrict__ wp,
                                                                                   const T *__restrict__ bias, T *__restrict__ y,
                                                                                   ConvMfmaParams p) {
     extern __shared__ __align__(16) unsigned char lds[];
     constexpr int ES = Geo<T>::ES, CPC = Geo<T>::CPC, PV = Geo<T>::CPC, kEpitch = Geo<T>::EPITCH, kEpiPos = Geo<T>::EPI_POS;
     constexpr int kMT = kTilePos / 32, kEpiMT = kEpiPos / 32, kBAhead = kBRing - 1;
-    constexpr int kMTW = kMT / kOT;  // position tiles of a wave
-    static_assert(kTilePos % 32 == 0 && (kOT == 1 || kOT == 2) && kMT % kOT == 0, "whole MFMA tiles");
+    static_assert(kTilePos % 32 == 0, "whole MFMA tiles");
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wrow = kOT == 2 ? (wave & 1) : 0, wcol = kOT == 2 ? (wave >> 1) : wave;  // the wave's place in the grid
     uint32_t t0, oct, b, tile;
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a run of consecutive
     // tiles, so that the input rows two neighbouring position tiles share are fetched from HBM once
@@ -203,31 +198,26 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
 
     // ---- per-lane operand addressing ----
     const int kg = lane >> 5, l32 = lane & 31;
-    int abase[kMTW];  // byte address of the lane's chunk (half-wave kg) of its staged pixel for tap (0,0), per position tile
+    int abase[kMT];  // byte address of the lane's chunk (half-wave kg) of its staged pixel for tap (0,0), per position tile
 #pragma unroll
-    for (int mt = 0; mt < kMTW; ++mt) {
-        const int pp = min(p0 + (wrow * kMTW + mt) * 32 + l32, p.npos - 1);  // clamped: a duplicate, never stored
+    for (int mt = 0; mt < kMT; ++mt) {
+        const int pp = min(p0 + mt * 32 + l32, p.npos - 1);  // clamped: a duplicate, never stored
         uint32_t ho, wo;
         p.div_ow.divmod((uint32_t)pp, ho, wo);
         abase[mt] = (((int)ho - ho_first) * p.lcols + (int)wo) * pitch + (kg << 4);
     }
     const int ncc = p.icc / (2 * CPC);          // k steps per tap in one pass
     const int nsteps = p.fh * p.fw * ncc;       // k steps per pass
-    const int oc0 = oct * kTileOc + wcol * 32 * kOT;
+    const int oc0 = oct * kTileOc + wave * 32;
     const bool wave_live = oc0 < p.oc;  // oc is a multiple of 64
     // fragment-ordered bank: block (tile of 32 channels, step), 16 bytes per lane.  The block address is
     // wave-uniform (scalar registers), the lane adds 16 * lane.
-    const unsigned char *bbank[kOT];
-#pragma unroll
-    for (int ot = 0; ot < kOT; ++ot)
-        bbank[ot] = (const unsigned char *)wpk + (size_t)(min(oc0 + 32 * ot, p.oc - 32) >> 5) * nsteps * p.npass * 1024;
+    const unsigned char *bbank = (const unsigned char *)wp + (size_t)(min(oc0, p.oc - 32) >> 5) * nsteps * p.npass * 1024;
     const uint32_t blane = (uint32_t)lane * 16u;
 
-    f32x16 acc[kMTW][kOT];
+    f32x16 acc[kMT];
 #pragma unroll
-    for (int mt = 0; mt < kMTW; ++mt)
-#pragma unroll
-        for (int ot = 0; ot < kOT; ++ot) acc[mt][ot] = (f32x16)(0.0f);
+    for (int mt = 0; mt < kMT; ++mt) acc[mt] = (f32x16)(0.0f);
 
     // ---- k loop of a pass: taps outer, 2*CPC channels per step ----
     int fi = 0, fj = 0, cc = 0;  // position of the NEXT step to load
@@ -241,7 +231,7 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
     // group, which serialises the L2 latency into each step).
     int aoff_next = 0;  // wave-uniform byte offset of the step the next load_a calls will fetch
     auto prepare_a = [&](int s) { aoff_next = s < nsteps ? (fi * p.lcols + fj) * pitch + (cc << 5) : 0; };
-    auto load_a = [&](uint4(&a)[kMTW], auto mtc) {
+    auto load_a = [&](uint4(&a)[kMT], auto mtc) {
         constexpr int mt = decltype(mtc)::value;
         a[mt] = *(const uint4 *)(lds + abase[mt] + aoff_next);
     };
@@ -251,35 +241,30 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
             if (++fj == p.fw) { fj = 0; ++fi; }
         }
     };
-    auto load_b = [&](uint4 &bq, int ot, int s) { bq = *(const uint4 *)(bbank[ot] + (size_t)min(s, nsteps - 1) * 1024 + blane); };
-    auto mma = [&](const uint4(&a)[kMTW], const uint4 &bq, auto mtc, auto otc) {
-        constexpr int mt = decltype(mtc)::value, ot = decltype(otc)::value;
+    auto load_b = [&](uint4 &bq, int s) { bq = *(const uint4 *)(bbank + (size_t)min(s, nsteps - 1) * 1024 + blane); };
+    auto mma = [&](const uint4(&a)[kMT], const uint4 &bq, auto mtc) {
+        constexpr int mt = decltype(mtc)::value;
         if constexpr (ES == 2) {
-            acc[mt][ot] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[mt]), __builtin_bit_cast(bf16x8_t, bq), acc[mt][ot], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[mt]), __builtin_bit_cast(bf16x8_t, bq), acc[mt], 0, 0, 0);
         } else {  // lanes 0-31 hold channels c..c+3, lanes 32-63 channels c+4..c+7: element j of both is one k pair
-            acc[mt][ot] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].x), __uint_as_float(bq.x), acc[mt][ot], 0, 0, 0);
-            acc[mt][ot] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].y), __uint_as_float(bq.y), acc[mt][ot], 0, 0, 0);
-            acc[mt][ot] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].z), __uint_as_float(bq.z), acc[mt][ot], 0, 0, 0);
-            acc[mt][ot] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].w), __uint_as_float(bq.w), acc[mt][ot], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].x), __uint_as_float(bq.x), acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].y), __uint_as_float(bq.y), acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].z), __uint_as_float(bq.z), acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[mt].w), __uint_as_float(bq.w), acc[mt], 0, 0, 0);
         }
     };
     // One step: the eight MFMA groups of step s on (a, bq); the A fragment of each tile is refreshed for step s+1
     // right behind its MFMA, the B fragment of the step kBAhead ahead is requested (into bn) in the middle; the
     // tap bookkeeping for step s+2 runs at the end of the step, after the last refresh.  sched_barrier pins the order, so the matrix pipe gets
     // new work back to back while the other requests trickle out.
-    auto step = [&](uint4(&a)[kMTW], const uint4(&bq)[kOT], uint4(&bn)[kOT], int s) {
+    auto step = [&](uint4(&a)[kMT], const uint4 &bq, uint4 &bn, int s) {
         prepare_a(s + 1);
-        static_for<kMTW>([&](auto mtc) {
+        static_for<kMT>([&](auto mtc) {
             constexpr int mt = decltype(mtc)::value;
-            static_for<kOT>([&](auto otc) { mma(a, bq[decltype(otc)::value], mtc, otc); });
+            mma(a, bq, mtc);
             load_a(a, mtc);
-            if constexpr (kOT == 1) {
-                if constexpr (mt == 3) load_b(bn[0], 0, s + kBAhead);
-            } else {
-                if constexpr (mt == kMTW / 2 - 1) load_b(bn[0], 0, s + kBAhead);
-                if constexpr (mt == kMTW - 1) load_b(bn[1], 1, s + kBAhead);
-            }
-            if constexpr (mt == kMTW - 1) advance_a();
+            if constexpr (mt == 3) load_b(bn, s + kBAhead);
+            if constexpr (mt == kMT - 1) advance_a();
             __builtin_amdgcn_sched_barrier(0);
         });
     };
@@ -289,13 +274,11 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
         stage(pass);
         __syncthreads();
         if (wave_live) {
-            uint4 a[kMTW], bf[kBRing][kOT];
-            static_for<kBAhead>([&](auto ic) {
-                static_for<kOT>([&](auto otc) { load_b(bf[decltype(ic)::value][decltype(otc)::value], decltype(otc)::value, decltype(ic)::value); });
-            });
+            uint4 a[kMT], bf[kBRing];
+            static_for<kBAhead>([&](auto ic) { load_b(bf[decltype(ic)::value], decltype(ic)::value); });
             fi = 0; fj = 0; cc = 0;
             prepare_a(0);
-            static_for<kMTW>([&](auto mtc) { load_a(a, mtc); });
+            static_for<kMT>([&](auto mtc) { load_a(a, mtc); });
             advance_a();
             int s = 0;
             for (; s + kBRing <= nsteps; s += kBRing)
@@ -310,8 +293,7 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
                 constexpr int i = decltype(ic)::value;
                 if (i < left) step(a, bf[i], bf[kBRing - 1], s + i);
             });
-#pragma unroll
-            for (int ot = 0; ot < kOT; ++ot) bbank[ot] += (size_t)nsteps * 1024;
+            bbank += (size_t)nsteps * 1024;
         }
     }
     __syncthreads();  // every wave is done with the staged image: LDS becomes the epilogue's transposition space
@@ -320,16 +302,13 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
     if (wave_live) {
         unsigned char *region = lds + wave * 32 * kEpitch;
         const bool relu = p.act == AGH_ACT_RELU;
-        static_for<kOT>([&](auto otc) {
-        constexpr int ot = decltype(otc)::value;
-        const int oct0 = oc0 + 32 * ot;  // first channel of this tile
-        const int o_lane = oct0 + l32;
+        const int o_lane = oc0 + l32;
         float bq = 0.0f;
         if (p.has_bias) bq = Elem<T>::to_f32(bias[min(o_lane, p.oc - 1)]);
         // the position tiles leave in groups of kEpiMT (256 bytes of every output row), the last group may be smaller
-        static_for<(kMTW + kEpiMT - 1) / kEpiMT>([&](auto partc) {
+        static_for<(kMT + kEpiMT - 1) / kEpiMT>([&](auto partc) {
             constexpr int part = decltype(partc)::value;
-            constexpr int NMT = (kMTW - part * kEpiMT) < kEpiMT ? (kMTW - part * kEpiMT) : kEpiMT;
+            constexpr int NMT = (kMT - part * kEpiMT) < kEpiMT ? (kMT - part * kEpiMT) : kEpiMT;
 #pragma unroll
             for (int m4 = 0; m4 < NMT; ++m4)
 #pragma unroll
@@ -338,8 +317,8 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
                     const int pl = m4 * 32 + blk * 8 + kg * 4;  // position inside this part
                     if constexpr (ES == 2) {
                         // two packed conversions give the four rounded values as two dwords
-                        uint32_t w[2] = {f32x2_to_bf16x2(acc[mt][ot][blk * 4 + 0], acc[mt][ot][blk * 4 + 1]),
-                                         f32x2_to_bf16x2(acc[mt][ot][blk * 4 + 2], acc[mt][ot][blk * 4 + 3])};
+                        uint32_t w[2] = {f32x2_to_bf16x2(acc[mt][blk * 4 + 0], acc[mt][blk * 4 + 1]),
+                                         f32x2_to_bf16x2(acc[mt][blk * 4 + 2], acc[mt][blk * 4 + 3])};
                         if (p.has_bias || relu) {  // wave-uniform
 #pragma unroll
                             for (int h = 0; h < 2; ++h) {
@@ -363,7 +342,7 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
                     } else {
                         float v[4];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = acc[mt][ot][blk * 4 + e];
+                        for (int e = 0; e < 4; ++e) v[e] = acc[mt][blk * 4 + e];
                         if (p.has_bias) {
 #pragma unroll
                             for (int e = 0; e < 4; ++e) v[e] = bq + v[e];
@@ -384,14 +363,13 @@ __global__ __launch_bounds__(kThreads, kWgs) void conv2_mfma_kernel(const T *__r
                 const int idx = r * 64 + lane, row = idx / CPRW, chunk = idx % CPRW;
                 if (TOTAL % 64 != 0 && idx >= TOTAL) continue;
                 const uint4 v = *(const uint4 *)(region + row * kEpitch + chunk * 16);
-                const int pos = p0 + wrow * kMTW * 32 + part * kEpiPos + chunk * CPC, o = oct0 + row;
+                const int pos = p0 + part * kEpiPos + chunk * CPC, o = oc0 + row;
                 if (pos < p.npos && o < p.oc) {
                     typedef uint32_t u32x4_nt __attribute__((ext_vector_type(4)));
                     if (p.nt_store) __builtin_nontemporal_store(u32x4_nt{v.x, v.y, v.z, v.w}, (u32x4_nt *)(y + ((size_t)b * p.oc + o) * p.npos + pos));
                     else *(uint4 *)(y + ((size_t)b * p.oc + o) * p.npos + pos) = v;
                 }
             }
-        });
         });
     }
 }
@@ -402,7 +380,7 @@ namespace agh {
 
 // Returns 1 when the geometry is not one this kernel takes (the caller goes on to its other paths),
 // otherwise a status code.  The API lock is held by the caller.
-template <typename T, int kTilePos, int kWgs, int kBRing, int kOT>
+template <typename T, int kTilePos, int kWgs, int kBRing>
 static int conv2_mfma_launch(const char *name, const void *x, const void *w, const void *bias, void *y, int64_t bs, int64_t ic, int64_t ih,
                    int64_t iw, int64_t oc, int64_t fh, int64_t fw, int64_t ph, int64_t pw, int64_t oh, int64_t ow, int act) {
     constexpr int ES = Geo<T>::ES, CPC = Geo<T>::CPC;
@@ -456,10 +434,10 @@ static int conv2_mfma_launch(const char *name, const void *x, const void *w, con
     p.div_vec = FastDiv((uint32_t)(iw / CPC));
     static bool attr_done = false;
     if (!attr_done) {
-        AGH_HIP(hipFuncSetAttribute((const void *)(conv2_mfma_kernel<T, kTilePos, kWgs, kBRing, kOT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
+        AGH_HIP(hipFuncSetAttribute((const void *)(conv2_mfma_kernel<T, kTilePos, kWgs, kBRing>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
         attr_done = true;
     }
-    hipLaunchKernelGGL((conv2_mfma_kernel<T, kTilePos, kWgs, kBRing, kOT>), dim3((unsigned)blocks), dim3(kThreads), (size_t)smem, stream(), (const T *)x,
+    hipLaunchKernelGGL((conv2_mfma_kernel<T, kTilePos, kWgs, kBRing>), dim3((unsigned)blocks), dim3(kThreads), (size_t)smem, stream(), (const T *)x,
                        (const T *)wperm, (const T *)bias, (T *)y, p);
     AGH_LAUNCH_CHECK(name);
     return AGH_OK;
@@ -475,12 +453,8 @@ int conv2_mfma_try(const char *name, const void *x, const void *w, const void *b
     const char *e = getenv("AGH_CONV_TILE");
     const int tile = e && *e ? atoi(e) : (sizeof(T) == 4 ? 128 : 256);
     if (tile == 128)
-        return conv2_mfma_launch<T, 128, 3, 8, 1>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
-    // 256 positions: the waves as a 2 x 2 grid (AGH_CONV_GRID=1 puts them back into one column of four)
-    const char *g = getenv("AGH_CONV_GRID");
-    if (g && *g && atoi(g) == 1)
-        return conv2_mfma_launch<T, 256, 2, 8, 1>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
-    return conv2_mfma_launch<T, 256, 2, 6, 2>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
+        return conv2_mfma_launch<T, 128, 3, 8>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
+    return conv2_mfma_launch<T, 256, 2, 8>(name, x, w, bias, y, bs, ic, ih, iw, oc, fh, fw, ph, pw, oh, ow, act);
 }
 
 template int conv2_mfma_try<uint16_t>(const char *, const void *, const void *, const void *, void *, int64_t, int64_t, int64_t, int64_t,

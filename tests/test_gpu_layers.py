@@ -128,14 +128,9 @@ CONV_MFMA = [
 ]
 
 
-@pytest.mark.parametrize("grid", ["2x2", "1x4"])
 @pytest.mark.parametrize("case", CONV_MFMA)
-def test_conv2_direct_bf16_matrix_core_path(ag, monkeypatch, case, grid):
-    """Both arrangements of a workgroup's four waves: 2 x 2 (half of the positions x 64 channels each, the default at 256
-    positions per workgroup) and one column of four (all positions x 32 channels each, AGH_CONV_GRID=1)."""
+def test_conv2_direct_bf16_matrix_core_path(ag, case):
     bs, ic, ih, iw, oc, f, p = case
-    if grid == "1x4":
-        monkeypatch.setenv("AGH_CONV_GRID", "1")
     rng = np.random.default_rng(25)
     x = orc.f32_to_bf16(rng.standard_normal((bs, ic, ih, iw)).astype(np.float32))
     w = orc.f32_to_bf16((rng.standard_normal((oc, ic) + f) * np.sqrt(2.0 / (ic * f[0] * f[1]))).astype(np.float32))
